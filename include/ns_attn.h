@@ -1,0 +1,133 @@
+/* ns_attn.h - the LLM attention path of libnextsycl-llm.so on one AMD MI355X (gfx950): KV-cache stores, split-K decode
+ * (one row, or the few rows of a speculative verify pass), causal flash-attention prefill, absorbed MLA decode.
+ *
+ * The entry points named ns_q35_*, ns_mg_*, ns_ds2_*, ns_llm_minimaxm3_*, ns_mla_*, ns_to_q8row are the ones the
+ * reference engines bind by name (llm/<arch>/src/ffi.rs) - same names, argument order, layouts and error behaviour, so
+ * an engine's ffi table resolves against this library unchanged. Each declaration cites the reference interface it
+ * replaces. The ns_attn_* / ns_mla_decode_latent entry points are this library's own: the same operations with typed
+ * (f32 / f16 / bf16) query and output rows, any G = Hq / Hkv, either cache layout and a bfloat16 cache form.
+ *
+ * Conventions (reference: kernels/llm/qwen35/q35.h:1-4): rows q/out are [T][Hq*D]; row t sits at absolute position
+ * p0 + t and sees keys 0 .. p0 + t (causal); query head hq reads key head hq / (Hq / Hkv). Everything is queued on the
+ * ns_gpu's compute stream and returns at once; 0, or -1 with the reason in ns_last_error(). The caller owns every
+ * buffer; `scratch` may be NULL only when the matching *_scratch() returns 0. No call allocates device memory.
+ *
+ * Cache forms `kt` (reference: llm/qwen35/src/engine.rs:44-60, kernels/llm/qwen35/silo/attn.cpp:43-46):
+ *   0  half       [D] half                                  2 D bytes a (head, position)
+ *   1  q8_0       [D int8][D/32 half scales]                D + D/16 bytes   (D 128: 136, D 256: 272)
+ *   2  q4_0       [D/2 bytes][D/32 half scales]             D/2 + D/16 bytes (D 128: 72,  D 256: 144)
+ *   3  bfloat16   [D] bfloat16 (this library's addition)    2 D bytes
+ * Cache layouts: head-major [Hkv][cap][row] (qwen35, museglimmer: slot = position, or position % cap for a ring) and
+ * position-major [position][Hkv][row] (minimaxm3: kernels/llm/minimaxm3/mm3.h:33-36).
+ */
+#ifndef NS_ATTN_H
+#define NS_ATTN_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ns_gpu ns_gpu;
+
+/* element types of query / output rows for the typed entry points */
+#define NS_F32 0
+#define NS_F16 1
+#define NS_BF16 2
+/* cache forms */
+#define NS_KV_F16 0
+#define NS_KV_Q8_0 1
+#define NS_KV_Q4_0 2
+#define NS_KV_BF16 3
+
+/* ---- KV-cache stores ------------------------------------------------------------------------------------------ */
+
+/* float32 rows k [T, Hkv x D] (ks floats apart) and v (vs apart) into the half caches [Hkv][cap][D] at positions
+ * p0.. ; -1 past the capacity. Replaces: kernels/llm/qwen35/q35.h:55-57 (q35.cpp:573-588) */
+int ns_q35_kv_store(ns_gpu* g, const float* k, int64_t ks, const float* v, int64_t vs, int64_t T, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
+                    void* kc, void* vc);
+/* the same rows as q8_0 (kt 1) or q4_0 (kt 2) rows, bit for bit ggml's quantize_row_q8_0_ref / _q4_0_ref with the
+ * scales behind the row's values; D a multiple of 32 (the reference: 256 only). Replaces:
+ * kernels/llm/qwen35/q35.h:37-42 (q35.cpp:281-326) */
+int ns_q35_kv_store_q(ns_gpu* g, int kt, const float* k, int64_t ks, const float* v, int64_t vs, int64_t T, int64_t Hkv, int64_t D, int64_t cap,
+                      int64_t p0, void* kc, void* vc);
+/* float32 rows k, v [T, Hkv x D] into half ring caches, slot (p0 + t) % cap. Replaces: kernels/llm/museglimmer/mg.h:25-26
+ * (mg.cpp:192-206) */
+int ns_mg_kv_store(ns_gpu* g, const float* k, const float* v, int64_t T, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, void* kc, void* vc);
+/* this library's typed store: any cache form (kt 0..3), ring != 0 for slot = position % cap (forms 0 and 3 only) */
+int ns_attn_kv_store(ns_gpu* g, int kt, int ring, const float* k, int64_t ks, const float* v, int64_t vs, int64_t T, int64_t Hkv, int64_t D,
+                     int64_t cap, int64_t p0, void* kc, void* vc);
+/* n cache rows of form kt (`stride` bytes apart) widened to float32 [n][D] exactly as the attention kernels read them
+ * into float32 (kernels/llm/qwen35/q35.cpp:19-25): the check of the byte formats. This library's own */
+int ns_attn_kv_dequant(ns_gpu* g, int kt, const void* rows, int64_t n, int64_t D, int64_t stride, float* out);
+/* normalized 32-point Walsh-Hadamard transform of each block of 32 in place (a quantized cache's optional rotation).
+ * Replaces: kernels/llm/qwen35/q35.h:43-45 (q35.cpp:328-348) */
+int ns_q35_fwht32(ns_gpu* g, float* x, int64_t rows, int64_t n, int64_t stride);
+
+/* ---- decode / verify attention (1..16 rows), split over the keys ------------------------------------------------ */
+
+/* Typed decode: rows q [T][Hq*D] (element type qt, rows qs elements apart) at positions p0.. against caches of form kt;
+ * pm 0 head-major [Hkv][cap][row] (slot = position % cap), 1 position-major [position][Hkv][row]; window win (<= 0:
+ * all earlier keys); scale <= 0: 1/sqrt(D). out [T][Hq*D] of type qt. The keys are cut at absolute multiples of the
+ * split size into ~1024 work-groups, every row of the pass riding on each key tile (a key is read once for all T x G
+ * rows of its key head); partials (values, max in log2 units, sum) [T][Hq][ns][D + 2] go through `scratch`
+ * (ns_attn_decode_scratch floats) and are merged by a second kernel. A row's result does not depend on which other
+ * rows share its pass, bit for bit. D 128 or 256, T 1..16 */
+int64_t ns_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win);
+int ns_attn_decode_t(ns_gpu* g, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq,
+                     int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out, float* scratch);
+
+/* Replaces: kernels/llm/qwen35/silo/silo.h:46-59 (silo/attn.cpp:375-435). The reference covers D 256 with 6 query
+ * heads a key head and 1..8 rows; here D 128 or 256, any Hq a multiple of Hkv, 1..16 rows */
+int ns_q35_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);
+int64_t ns_q35_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0);
+int ns_q35_attn_decode(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
+                       int64_t cap, int64_t p0, float* out, float* scratch);
+int ns_q35_attn_decode_kv(ns_gpu* g, int kt, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv,
+                          int64_t D, int64_t cap, int64_t p0, float* out, float* scratch);
+/* Replaces: kernels/llm/museglimmer/silo/silo.h:50-56 (silo/attn.cpp:317-375): ring caches and a window */
+int ns_mg_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);
+int64_t ns_mg_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win);
+int ns_mg_attn_decode(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap,
+                      int64_t p0, int64_t win, float* out, float* scratch);
+
+/* ---- prompt (prefill) attention ---------------------------------------------------------------------------------- */
+
+/* Typed causal flash attention of T rows at positions p0.. against caches that already hold positions 0 .. p0 + T - 1
+ * (the engine stores a pass's keys first: llm/museglimmer/src/engine.rs:856-860). kt 0 (half) or 3 (bfloat16). No
+ * scratch. D 128 */
+int ns_attn_prompt_t(ns_gpu* g, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq,
+                     int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out);
+/* Replaces: kernels/llm/museglimmer/silo/silo.h:44-48 (silo/attn.cpp:378-392) */
+int ns_mg_attn_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);
+int ns_mg_attn_prompt(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap,
+                      int64_t p0, int64_t win, float* out);
+/* Replaces: kernels/llm/qwen35/silo/silo.h:43-45,57-58 (silo/attn.cpp:375-400) */
+int ns_q35_attn_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);
+int ns_q35_attn_prompt(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
+                       int64_t cap, int64_t p0, float* out);
+int ns_q35_attn_prompt_kv(ns_gpu* g, int kt, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv,
+                          int64_t D, int64_t cap, int64_t p0, float* out);
+
+/* ---- the engines' own ("exact") attention entry points, routed to the kernels above ----------------------------- */
+
+/* Replaces: kernels/llm/qwen35/q35.h:61-66 (q35.cpp:590-612) */
+int64_t ns_q35_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0);
+int ns_q35_attn(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
+                int64_t cap, int64_t p0, float* out, float* scratch);
+/* Replaces: kernels/llm/museglimmer/mg.h:27-33 (mg.cpp:208-253). causal 0 (the drafter's block: every row sees to the
+ * pass's last key) is accepted for T <= 16 */
+int64_t ns_mg_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win, int causal);
+int ns_mg_attn(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
+               int64_t win, int causal, float* out, float* scratch);
+/* GQA over a position-major half cache [position][G][128], q [T][H][128], explicit scale; dense (sel must be NULL).
+ * Replaces: kernels/llm/minimaxm3/mm3.h:33-37 (mm3.cpp:118-190). Needs scratch: this library keeps
+ * ns_attn_decode_scratch(T, H, G, 128, pos0, 0) floats per ns_gpu for it (allocated at ns_gpu_open, 16 MiB) */
+int ns_llm_minimaxm3_attend(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
+                            int64_t H, int64_t G, int64_t pos0, float scale);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,232 @@
+"""The attention ABI (include/ns_attn.h) bound by name, and the size-checked wrappers an engine calls.
+
+`Kernels` is the table of function pointers - the counterpart of an engine's `ffi.rs` (llm/qwen35/src/ffi.rs:42-52,
+70-136; llm/museglimmer/src/ffi.rs; llm/deepseek2/src/ffi.rs:36-39): every entry point looked up by name when the table
+is built, a missing symbol being a load error. `Ops` is the counterpart of `ops.rs` (llm/deepseek2/src/ops.rs:391-445):
+each wrapper checks that its buffers hold what the kernel will touch, then makes the C call and turns -1 into
+Error("<what>: <ns_last_error>"). The call order of a pass is the engines': kv_store -> *_scratch -> attention
+(llm/museglimmer/src/engine.rs:856-873). Nothing here computes: the HIP library does, or the call fails."""
+import ctypes as C
+
+from .core import Error, api
+from .sys import P, f32, i32, i64
+
+F32, F16, BF16 = 0, 1, 2                       # q / out element types (NS_F32, NS_F16, NS_BF16)
+KV_F16, KV_Q8_0, KV_Q4_0, KV_BF16 = 0, 1, 2, 3   # cache forms
+ELT = {F32: 4, F16: 2, BF16: 2}
+
+
+def kv_row_bytes(kt, D):
+    """Bytes of one (head, position) row of a cache of form kt (llm/qwen35/src/engine.rs:54-60)."""
+    if kt == KV_Q8_0:
+        return D + D // 32 * 2
+    if kt == KV_Q4_0:
+        return D // 2 + D // 32 * 2
+    if kt in (KV_F16, KV_BF16):
+        return 2 * D
+    raise Error("a cache form 0 (half), 1 (q8_0), 2 (q4_0) or 3 (bfloat16)")
+
+
+# name -> (restype, argtypes): include/ns_attn.h
+ATTN_H = {
+    "ns_q35_kv_store": (i32, [P, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_q35_kv_store_q": (i32, [P, i32, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_mg_kv_store": (i32, [P, P, P, i64, i64, i64, i64, i64, P, P]),
+    "ns_attn_kv_store": (i32, [P, i32, i32, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_attn_kv_dequant": (i32, [P, i32, P, i64, i64, i64, P]),
+    "ns_q35_fwht32": (i32, [P, P, i64, i64, i64]),
+    "ns_attn_decode_scratch": (i64, [i64, i64, i64, i64, i64, i64]),
+    "ns_attn_decode_t": (i32, [P, i32, i32, i32, P, i64, P, P, i64, i64, i64, i64, i64, i64, i64, f32, P, P]),
+    "ns_q35_attn_decode_supported": (i32, [i64, i64, i64, i64]),
+    "ns_q35_attn_decode_scratch": (i64, [i64, i64, i64, i64, i64]),
+    "ns_q35_attn_decode": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_q35_attn_decode_kv": (i32, [P, i32, P, i64, P, P, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_mg_attn_decode_supported": (i32, [i64, i64, i64, i64]),
+    "ns_mg_attn_decode_scratch": (i64, [i64, i64, i64, i64, i64, i64]),
+    "ns_mg_attn_decode": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_attn_prompt_t": (i32, [P, i32, i32, i32, P, i64, P, P, i64, i64, i64, i64, i64, i64, i64, f32, P]),
+    "ns_mg_attn_prompt_supported": (i32, [i64, i64, i64, i64]),
+    "ns_mg_attn_prompt": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, P]),
+    "ns_q35_attn_prompt_supported": (i32, [i64, i64, i64, i64]),
+    "ns_q35_attn_prompt": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P]),
+    "ns_q35_attn_prompt_kv": (i32, [P, i32, P, i64, P, P, i64, i64, i64, i64, i64, i64, P]),
+    "ns_q35_attn_scratch": (i64, [i64, i64, i64, i64, i64]),
+    "ns_q35_attn": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_mg_attn_scratch": (i64, [i64, i64, i64, i64, i64, i64, i32]),
+    "ns_mg_attn": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, i32, P, P]),
+    "ns_llm_minimaxm3_attend": (i32, [P, P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
+}
+
+
+class Kernels:
+    """Every attention entry point bound by name; a missing symbol fails the load."""
+
+    def __init__(self, a=None):
+        self.api = a or api()
+        for name, (res, args) in ATTN_H.items():
+            setattr(self, name[3:], self.api.symbol(name, res, args))
+
+
+_k = None
+
+
+def kernels():
+    global _k
+    if _k is None:
+        _k = Kernels()
+    return _k
+
+
+def _need(buf, nbytes, what):
+    if buf is None:
+        raise Error("%s: no buffer" % what)
+    if buf.len < nbytes:
+        raise Error("%s: %d bytes, needs %d" % (what, buf.len, nbytes))
+
+
+class Ops:
+    """Checked wrappers over one GPU: the buffers' sizes against what the kernel reads and writes, then the call."""
+
+    def __init__(self, gpu, k=None):
+        self.gpu = gpu
+        self.k = k or kernels()
+
+    def raw(self):
+        return self.gpu.raw
+
+    def ok(self, rc, what):
+        if rc != 0:
+            raise Error("%s: %s" % (what, self.k.api.error()))
+
+    # ---- caches
+    def cache_bytes(self, kt, Hkv, cap, D):
+        return Hkv * cap * kv_row_bytes(kt, D)
+
+    def kv_store(self, kt, k, ks, v, vs, T, Hkv, D, cap, p0, kc, vc, ring=False):
+        """float32 rows k, v [T][Hkv*D] (strides ks, vs floats) into caches of form kt at positions p0.."""
+        if T > 0:
+            _need(k, ((T - 1) * ks + Hkv * D) * 4, "kv_store k")
+            _need(v, ((T - 1) * vs + Hkv * D) * 4, "kv_store v")
+        _need(kc, self.cache_bytes(kt, Hkv, cap, D), "kv_store key cache")
+        _need(vc, self.cache_bytes(kt, Hkv, cap, D), "kv_store value cache")
+        self.ok(self.k.attn_kv_store(self.raw(), kt, int(ring), k.ptr, ks, v.ptr, vs, T, Hkv, D, cap, p0, kc.ptr, vc.ptr), "kv_store")
+
+    def q35_kv_store(self, k, ks, v, vs, T, Hkv, D, cap, p0, kc, vc):
+        if T > 0:
+            _need(k, ((T - 1) * ks + Hkv * D) * 4, "kv_store k")
+            _need(v, ((T - 1) * vs + Hkv * D) * 4, "kv_store v")
+        _need(kc, self.cache_bytes(0, Hkv, cap, D), "kv_store key cache")
+        _need(vc, self.cache_bytes(0, Hkv, cap, D), "kv_store value cache")
+        self.ok(self.k.q35_kv_store(self.raw(), k.ptr, ks, v.ptr, vs, T, Hkv, D, cap, p0, kc.ptr, vc.ptr), "kv_store")
+
+    def q35_kv_store_q(self, kt, k, ks, v, vs, T, Hkv, D, cap, p0, kc, vc):
+        if T > 0:
+            _need(k, ((T - 1) * ks + Hkv * D) * 4, "kv_store_q k")
+            _need(v, ((T - 1) * vs + Hkv * D) * 4, "kv_store_q v")
+        if kt in (1, 2):
+            _need(kc, self.cache_bytes(kt, Hkv, cap, D), "kv_store_q key cache")
+            _need(vc, self.cache_bytes(kt, Hkv, cap, D), "kv_store_q value cache")
+        self.ok(self.k.q35_kv_store_q(self.raw(), kt, k.ptr, ks, v.ptr, vs, T, Hkv, D, cap, p0, kc.ptr, vc.ptr), "kv_store_q")
+
+    def mg_kv_store(self, k, v, T, Hkv, D, cap, p0, kc, vc):
+        _need(k, T * Hkv * D * 4, "kv_store k")
+        _need(v, T * Hkv * D * 4, "kv_store v")
+        _need(kc, self.cache_bytes(0, Hkv, cap, D), "kv_store key cache")
+        _need(vc, self.cache_bytes(0, Hkv, cap, D), "kv_store value cache")
+        self.ok(self.k.mg_kv_store(self.raw(), k.ptr, v.ptr, T, Hkv, D, cap, p0, kc.ptr, vc.ptr), "kv_store")
+
+    def kv_dequant(self, kt, rows, n, D, out):
+        rb = kv_row_bytes(kt, D)
+        _need(rows, n * rb, "kv_dequant rows")
+        _need(out, n * D * 4, "kv_dequant out")
+        self.ok(self.k.attn_kv_dequant(self.raw(), kt, rows.ptr, n, D, rb, out.ptr), "kv_dequant")
+
+    def fwht32(self, x, rows, n, stride):
+        if rows > 0:
+            _need(x, ((rows - 1) * stride + n) * 4, "fwht32 x")
+        self.ok(self.k.q35_fwht32(self.raw(), x.ptr, rows, n, stride), "fwht32")
+
+    # ---- decode / verify
+    def decode_scratch(self, T, Hq, Hkv, D, p0, win=0):
+        return self.k.attn_decode_scratch(T, Hq, Hkv, D, p0, win)
+
+    def decode(self, qt, kt, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, out, scratch, win=0, pm=False, scale=0.0):
+        """Typed split-K decode of T rows (ns_attn_decode_t)."""
+        if T > 0:
+            _need(q, ((T - 1) * qs + Hq * D) * ELT[qt], "decode q")
+            _need(out, T * Hq * D * ELT[qt], "decode out")
+            _need(scratch, self.decode_scratch(T, Hq, Hkv, D, p0, win) * 4, "decode scratch")
+        _need(kc, self.cache_bytes(kt, Hkv, cap, D), "decode key cache")
+        _need(vc, self.cache_bytes(kt, Hkv, cap, D), "decode value cache")
+        self.ok(self.k.attn_decode_t(self.raw(), qt, kt, int(pm), q.ptr, qs, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, scale, out.ptr,
+                                     scratch.ptr if scratch is not None else None), "attention decode")
+
+    def q35_attn_decode_kv(self, kt, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, out, scratch):
+        if T > 0:
+            _need(q, ((T - 1) * qs + Hq * D) * 4, "decode q")
+            _need(out, T * Hq * D * 4, "decode out")
+        if kt in (0, 1, 2):
+            _need(kc, self.cache_bytes(kt, Hkv, cap, D), "decode key cache")
+            _need(vc, self.cache_bytes(kt, Hkv, cap, D), "decode value cache")
+        sc = self.k.q35_attn_decode_scratch(T, Hq, Hkv, D, p0)
+        if scratch is not None:
+            _need(scratch, sc * 4, "decode scratch")
+        self.ok(self.k.q35_attn_decode_kv(self.raw(), kt, q.ptr, qs, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, out.ptr,
+                                          scratch.ptr if scratch is not None else None), "attention decode")
+
+    def mg_attn_decode(self, q, kc, vc, T, Hq, Hkv, D, cap, p0, win, out, scratch):
+        _need(q, T * Hq * D * 4, "decode q")
+        _need(out, T * Hq * D * 4, "decode out")
+        _need(kc, self.cache_bytes(0, Hkv, cap, D), "decode key cache")
+        _need(vc, self.cache_bytes(0, Hkv, cap, D), "decode value cache")
+        if scratch is not None:
+            _need(scratch, self.k.mg_attn_decode_scratch(T, Hq, Hkv, D, p0, win) * 4, "decode scratch")
+        self.ok(self.k.mg_attn_decode(self.raw(), q.ptr, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, out.ptr,
+                                      scratch.ptr if scratch is not None else None), "attention decode")
+
+    # ---- prompt
+    def prompt(self, qt, kt, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, out, win=0, pm=False, scale=0.0):
+        """Typed causal flash attention of T prompt rows (ns_attn_prompt_t)."""
+        if T > 0:
+            _need(q, ((T - 1) * qs + Hq * D) * ELT[qt], "prompt q")
+            _need(out, T * Hq * D * ELT[qt], "prompt out")
+        _need(kc, self.cache_bytes(kt, Hkv, cap, D), "prompt key cache")
+        _need(vc, self.cache_bytes(kt, Hkv, cap, D), "prompt value cache")
+        self.ok(self.k.attn_prompt_t(self.raw(), qt, kt, int(pm), q.ptr, qs, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, scale, out.ptr),
+                "attention prompt")
+
+    def mg_attn_prompt(self, q, kc, vc, T, Hq, Hkv, D, cap, p0, win, out):
+        _need(q, T * Hq * D * 4, "prompt q")
+        _need(out, T * Hq * D * 4, "prompt out")
+        _need(kc, self.cache_bytes(0, Hkv, cap, D), "prompt key cache")
+        _need(vc, self.cache_bytes(0, Hkv, cap, D), "prompt value cache")
+        self.ok(self.k.mg_attn_prompt(self.raw(), q.ptr, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, out.ptr), "attention prompt")
+
+    # ---- the engines' own entry points
+    def mg_attn(self, q, kc, vc, T, Hq, Hkv, D, cap, p0, win, causal, out, scratch):
+        _need(q, T * Hq * D * 4, "attention q")
+        _need(out, T * Hq * D * 4, "attention out")
+        _need(kc, self.cache_bytes(0, Hkv, cap, D), "attention key cache")
+        _need(vc, self.cache_bytes(0, Hkv, cap, D), "attention value cache")
+        if scratch is not None:
+            _need(scratch, self.k.mg_attn_scratch(T, Hq, Hkv, D, p0, win, int(causal)) * 4, "attention scratch")
+        self.ok(self.k.mg_attn(self.raw(), q.ptr, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, int(causal), out.ptr,
+                               scratch.ptr if scratch is not None else None), "attention")
+
+    def q35_attn(self, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, out, scratch):
+        if T > 0:
+            _need(q, ((T - 1) * qs + Hq * D) * 4, "attention q")
+            _need(out, T * Hq * D * 4, "attention out")
+        _need(kc, self.cache_bytes(0, Hkv, cap, D), "attention key cache")
+        _need(vc, self.cache_bytes(0, Hkv, cap, D), "attention value cache")
+        if scratch is not None:
+            _need(scratch, self.k.q35_attn_scratch(T, Hq, Hkv, D, p0) * 4, "attention scratch")
+        self.ok(self.k.q35_attn(self.raw(), q.ptr, qs, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, out.ptr,
+                                scratch.ptr if scratch is not None else None), "attention")
+
+    def minimaxm3_attend(self, q, kc, vc, out, T, H, G, pos0, scale):
+        _need(q, T * H * 128 * 4, "attend q")
+        _need(out, T * H * 128 * 4, "attend out")
+        _need(kc, (pos0 + T) * G * 128 * 2, "attend key cache")
+        _need(vc, (pos0 + T) * G * 128 * 2, "attend value cache")
+        self.ok(self.k.llm_minimaxm3_attend(self.raw(), q.ptr, kc.ptr, vc.ptr, None, 0, out.ptr, T, H, G, pos0, scale), "attend")

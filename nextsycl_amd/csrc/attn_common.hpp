@@ -1,0 +1,66 @@
+// attn_common.hpp: MFMA operand types and small device helpers shared by the attention kernels (gfx950, wave64).
+//
+// v_mfma_f32_16x16x32_{f16,bf16}: D[16x16] += A[16x32] B[32x16]. Per lane l (n = l % 16, g = l / 16):
+//   A operand: row m = n, the 8 values k = 8 g .. 8 g + 7        B operand: column n, the same 8 k
+//   D / C:     column n, rows m = 4 g .. 4 g + 3 (4 floats)
+// v_mfma_f32_32x32x16_{f16,bf16}: D[32x32] += A[32x16] B[16x32]. Per lane l (n = l % 32, g = l / 32):
+//   A operand: row m = n, k = 8 g .. 8 g + 7                     B operand: column n, the same 8 k
+//   D / C:     column n, rows m = 8 (i / 4) + 4 g + i % 4 for register i = 0..15
+// ds_read_b64_tr_b16 (the transposing LDS read): in each group of 16 lanes, lane s supplies the address of 4
+// consecutive 16-bit values; lane i receives element i % 4 of the rows of lanes i / 4, 4 + i / 4, 8 + i / 4, 12 + i / 4.
+// With lane s pointing at &M[k0 + s / 4][m0 + 4 (s % 4)] of a row-major M[k][m], lane i receives M[k0 .. k0 + 3][m0 + i]:
+// the four k of one m - an MFMA operand's packing read out of the other-major matrix.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+typedef short s8v __attribute__((ext_vector_type(8)));
+typedef short s4v __attribute__((ext_vector_type(4)));
+typedef _Float16 h8v __attribute__((ext_vector_type(8)));
+typedef __bf16 b8v __attribute__((ext_vector_type(8)));
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+template <bool BF>
+__device__ __forceinline__ f4v mfma16(s8v a, s8v b, f4v c) {
+    if constexpr (BF) return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8v, a), __builtin_bit_cast(b8v, b), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8v, a), __builtin_bit_cast(h8v, b), c, 0, 0, 0);
+}
+template <bool BF>
+__device__ __forceinline__ f16v mfma32(s8v a, s8v b, f16v c) {
+    if constexpr (BF) return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(b8v, a), __builtin_bit_cast(b8v, b), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8v, a), __builtin_bit_cast(h8v, b), c, 0, 0, 0);
+}
+
+// float -> the kernel's 16-bit operand type, round to nearest even
+template <bool BF>
+__device__ __forceinline__ short to16(float f) {
+    if constexpr (BF) {
+        const __bf16 b = (__bf16) f;
+        return __builtin_bit_cast(short, b);
+    } else {
+        const _Float16 h = (_Float16) f;
+        return __builtin_bit_cast(short, h);
+    }
+}
+
+// the transposing LDS read of 4 x 16 bits
+__device__ __forceinline__ s4v lds_read_tr16(void* lds_addr) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) lds_addr);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// element i of a row of query / output type QT (0 float32, 1 half, 2 bfloat16)
+template <int QT>
+__device__ __forceinline__ float load_q(const void* p, int64_t i) {
+    if constexpr (QT == 0) return reinterpret_cast<const float*>(p)[i];
+    else if constexpr (QT == 1) return (float) reinterpret_cast<const _Float16*>(p)[i];
+    else return (float) reinterpret_cast<const __bf16*>(p)[i];
+}
+template <int QT>
+__device__ __forceinline__ void store_o(void* p, int64_t i, float v) {
+    if constexpr (QT == 0) reinterpret_cast<float*>(p)[i] = v;
+    else if constexpr (QT == 1) reinterpret_cast<_Float16*>(p)[i] = (_Float16) v;
+    else reinterpret_cast<__bf16*>(p)[i] = (__bf16) v;
+}

@@ -1,0 +1,655 @@
+// attn_decode.hip: split-K GQA decode / verify attention over the KV cache (half, bfloat16, q8_0, q4_0 rows) for gfx950.
+//
+// Bound: HBM. A decode pass reads every visible key and value once (2 x row bytes a key and key head) and computes
+// 4 D flops a (row, key): at most 32 flop/byte for a 4-row verify pass - far under the MFMA ridge, so the kernel is
+// built to keep HBM reads in flight and everything else out of their way.
+//
+// Work split: grid (key split, key head, row chunk). A work-group of 4 waves owns the keys [s kbs, (s + 1) kbs) of one
+// key head - kbs a multiple of 128 chosen so the grid has ~NS_DEC_WGS work-groups whatever the context - and ALL the
+// pass's T x G query rows of that key head ride on every key tile, so a key is read from HBM once. Wave w takes the
+// 32-key tiles with (tile index % 4 == w): tiles and splits sit at absolute key positions, which (with MFMA columns
+// being independent) makes a row's arithmetic the same whatever rows share its pass - the verify invariant.
+//
+// A wave's tile step (32 keys), all in the transposed orientation so no row statistic ever crosses lanes through LDS:
+//   K:  global -> registers straight in MFMA A-operand layout (lane = key, 16 bytes of its row per k-block)
+//   S^T[key][row] = K Q^T           v_mfma_f32_16x16x32 (rows padded to 16-row tiles; Q^T lives in registers)
+//   online softmax, base 2, float32: a lane holds 8 keys of one row; row max / sum = 8 in-lane + 2 xor-shuffles
+//   P^T -> 16 bit: it already IS the B operand of the next product (k-slot i of lane group g <-> key 4 g + i | 16 + 4 g + i)
+//   V:  half / bfloat16 rows: global -> LDS directly (global_load_lds_dwordx4, 1 KiB contiguous per instruction), the
+//       16-byte chunks of a row XOR-swizzled by the key so the transposing reads meet no bank conflicts; q8_0 / q4_0
+//       rows: global -> registers -> dequantized -> LDS [key][D] (rows padded by 32 bytes);
+//       then ds_read_b64_tr_b16 gives V^T in A-operand layout
+//   O^T[d][row] = O^T c + V^T P^T   v_mfma_f32_16x16x32, float32 accumulators in registers
+// The next tile's K (registers) and V (second LDS buffer) loads are issued before the current tile's math: ~16 KiB in
+// flight per wave, 8 waves a CU. The 4 waves' (O, m, l) are merged through LDS in a fixed order and written as the split's partial
+// {O[D], m (log2 units), l}; a second kernel merges the splits: out = sum O_s 2^(m_s - M) / sum l_s 2^(m_s - M).
+//
+// Reference behaviour kept: kernels/llm/qwen35/silo/attn.cpp:100-104,261-290,321-370 (split form, partial layout,
+// merge, one launch when the rows' split sizes agree else a row at a time), kernels/llm/museglimmer/silo/attn.cpp:51-55,
+// 86-92,120-127 (absolute split positions, ring slots, window), and the rounding model of both (16-bit operands,
+// float32 scores, softmax and accumulation; quantized values rounded to half as staged).
+#include "ns_internal.hpp"
+#include "ns_attn.h"
+#include "attn_common.hpp"
+#include "kv_formats.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+#include <type_traits>
+
+namespace {
+
+constexpr int WAVES = 4, TILE = 32;
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+
+struct DecodeParams {
+    const void* q;
+    int qt;                     // element type of q: 0 float32, 1 half, 2 bfloat16
+    int64_t qs;                 // elements between query rows
+    const uint8_t* kc;
+    const uint8_t* vc;
+    int64_t head_stride, row_stride;   // bytes between key heads / between slots
+    int64_t cap;
+    int wrap;                   // slots are position % cap (a ring that has wrapped); else slot = position
+    int T, Hq, G;
+    int causal;                 // 0: every row sees to the pass's last key (the drafter's block)
+    int64_t p0, win;
+    int64_t kbs, sp0;           // keys a split, the first split's index (absolute position / kbs)
+    int ns;
+    float sl2;                  // scale x log2(e)
+    float* part;                // [T][Hq][ns][D + 2]
+};
+
+template <int D, int KT>
+struct TileRegs {
+    static constexpr bool DMA = KT == 0 || KT == 3;                      // 16-bit value rows go global -> LDS directly
+    static constexpr int KB = D / 32;                                    // k-blocks of 32 features
+    static constexpr int KW = DMA ? 4 : 2;                               // words a lane loads per (key tile, k-block)
+    static constexpr int CPR = KT == 1 ? D / 16 : KT == 2 ? D / 32 : D / 8;   // 16-byte chunks a value row
+    static constexpr int KPI = 64 / CPR;                                 // keys a wave covers per V load
+    static constexpr int NLV = TILE / KPI;                               // V loads a lane per tile
+    u4v k4[2][DMA ? KB : 1];                                             // 16-bit rows: 8 features per (key tile, k-block)
+    uint32_t k[2][DMA ? 1 : KB][KW];                                     // quantized rows: 8 int8 / 8 nibbles
+    uint16_t ksc[2][DMA ? 1 : KB];
+    uint4 v[DMA ? 1 : NLV];                                              // quantized forms only
+    uint16_t vsc[DMA ? 1 : NLV];
+};
+
+// 4 int8 in a word -> 4 halfs x scale; each product is exact in float32, so one rounding to half (what the reference
+// stages: half((float) q * (float) d))
+__device__ __forceinline__ void dq8x4(uint32_t w, _Float16 d, short* o) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const _Float16 h = (_Float16) (short) (int8_t) (w >> (8 * b)) * d;
+        o[b] = __builtin_bit_cast(short, h);
+    }
+}
+// 4 nibbles (bits sh .. sh + 3 of each byte) -> 4 halfs: (nibble - 8) x scale
+__device__ __forceinline__ void dq4x4(uint32_t w, int sh, _Float16 d, short* o) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const _Float16 h = (_Float16) (short) ((int) ((w >> (8 * b + sh)) & 15u) - 8) * d;
+        o[b] = __builtin_bit_cast(short, h);
+    }
+}
+
+template <int D, int RT, int KT>
+__global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kernel(const DecodeParams p) {
+    constexpr bool BF = KT == 3;
+    using R = TileRegs<D, KT>;
+    constexpr bool DMA = R::DMA;
+    constexpr int KB = R::KB, DT = D / 16;
+    // a wave's value stage: DMA: two unpadded swizzled tiles [32][2 D bytes]; else one padded tile (rows + 32 bytes)
+    constexpr int RS = DMA ? D * 2 : D * 2 + 32;
+    constexpr int VTILE = TILE * RS;
+    constexpr int STAGE = DMA ? 2 * VTILE : VTILE;
+    constexpr int OROW = D + 4;                                    // floats a row of the merge buffer
+    constexpr int MERGE = RT * 16 * OROW * 4;
+    constexpr int LDS_MAIN = WAVES * STAGE > MERGE ? WAVES * STAGE : MERGE;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_MAIN];
+    __shared__ float ml[WAVES][RT * 16][2];
+    __shared__ float ML[RT * 16][2];
+
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // the wave's index, known uniform to the compiler
+    const int split = blockIdx.x, hk = blockIdx.y, z = blockIdx.z;
+    const int rows = p.T * p.G;
+    const int64_t pass_end = p.p0 + p.T;
+    const int64_t fmin = p.win > 0 ? std::max<int64_t>(0, p.p0 + 1 - p.win) : 0;
+    const int64_t jb = std::max((p.sp0 + split) * p.kbs, fmin), je = std::min((p.sp0 + split + 1) * p.kbs, pass_end);
+
+    // ---- this lane's rows (one per row tile): their key ranges and Q^T operands
+    int64_t lo_r[RT], hi_r[RT];
+    s8v qreg[RT][KB];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int ri = (z * RT + rt) * 16 + n;
+        const bool live = ri < rows;
+        const int t = live ? ri / p.G : 0, gq = live ? ri % p.G : 0;
+        const int64_t pos = p.p0 + t, first = p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0;
+        lo_r[rt] = live ? std::max(first, jb) : 1;
+        hi_r[rt] = live ? std::min(p.causal ? pos : pass_end - 1, je - 1) : 0;
+        // 8 consecutive features per k-block, vector loads all issued before any is used (rows are 16-byte aligned:
+        // checked on the host); a dead row reads row 0's and is zeroed
+        const int64_t qoff = (int64_t) t * p.qs + ((int64_t) hk * p.G + gq) * D + g4 * 8;
+        if (p.qt == 0) {
+            float4 raw[KB][2];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                raw[kb][0] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.q) + qoff + kb * 32);
+                raw[kb][1] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.q) + qoff + kb * 32 + 4);
+            }
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const float f[8] = {raw[kb][0].x, raw[kb][0].y, raw[kb][0].z, raw[kb][0].w, raw[kb][1].x, raw[kb][1].y, raw[kb][1].z, raw[kb][1].w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = live ? to16<BF>(f[i]) : (short) 0;
+            }
+        } else {
+            uint4 raw[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) raw[kb] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.q) + qoff + kb * 32);
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const uint32_t ww[4] = {raw[kb].x, raw[kb].y, raw[kb].z, raw[kb].w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint16_t b16 = (uint16_t) (ww[i >> 1] >> (16 * (i & 1)));
+                    // the same 16-bit type as the kernel's operands passes through; the other is converted
+                    const short v = (p.qt == 2) == BF ? (short) b16 : to16<BF>(p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16));
+                    qreg[rt][kb][i] = live ? v : (short) 0;
+                }
+            }
+        }
+    }
+
+    float m_r[RT], l_r[RT];
+    f4v o[RT][DT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        m_r[rt] = -INFINITY;
+        l_r[rt] = 0.0f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[rt][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
+    const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
+    const uint8_t* vbase = p.vc + (int64_t) hk * p.head_stride;
+    uint8_t* stage = lds + w * STAGE;
+
+    // a key's row offset: keys outside [jb, je) are clamped into it (their scores are masked, their values meet P = 0).
+    // A wrapped ring's slot is position % cap: the split's first key's slot once, then offsets from it with at most two
+    // wraps (a pass's keys span less than two rings). 32-bit arithmetic relative to the split's first key.
+    const int64_t jb_slot = p.wrap && jb < je ? jb % p.cap : jb;
+    const int span = (int) (je - jb) - 1;
+    auto row_off = [&](int rel) -> int64_t {
+        const int rc = std::min(std::max(rel, 0), span);
+        int64_t slot = jb_slot + rc;
+        if (p.wrap) {
+            slot = slot >= p.cap ? slot - p.cap : slot;
+            slot = slot >= p.cap ? slot - p.cap : slot;
+        }
+        return slot * p.row_stride;
+    };
+    // the tile's keys into registers (MFMA A layout) and its values on their way: DMA into LDS buffer `buf`, chunk
+    // position cp of key kk holding the row's chunk cp ^ 2 (kk % 8); or raw into registers
+    auto load_tile = [&](R& r, int64_t ti, int buf) {
+        const int j0 = (int) (ti * TILE - jb);                 // the tile's first key relative to the split's
+#pragma unroll
+        for (int kt2 = 0; kt2 < 2; ++kt2) {
+            const uint8_t* kr = kbase + row_off(j0 + kt2 * 16 + n);
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                if constexpr (DMA) {
+                    r.k4[kt2][kb] = *reinterpret_cast<const u4v*>(kr + kb * 64 + g4 * 16);
+                } else if constexpr (KT == 1) {
+                    const uint2 x = *reinterpret_cast<const uint2*>(kr + kb * 32 + g4 * 8);
+                    r.k[kt2][kb][0] = x.x; r.k[kt2][kb][1] = x.y;
+                    r.ksc[kt2][kb] = *reinterpret_cast<const uint16_t*>(kr + D + 2 * kb);
+                } else {
+                    const uint2 x = *reinterpret_cast<const uint2*>(kr + kb * 16 + (g4 & 1) * 8);
+                    r.k[kt2][kb][0] = x.x; r.k[kt2][kb][1] = x.y;
+                    r.ksc[kt2][kb] = *reinterpret_cast<const uint16_t*>(kr + D / 2 + 2 * kb);
+                }
+            }
+        }
+        const int cp = lane % R::CPR, kr0 = lane / R::CPR;
+#pragma unroll
+        for (int i = 0; i < R::NLV; ++i) {
+            const int kk = kr0 + R::KPI * i;
+            const uint8_t* vr = vbase + row_off(j0 + kk);
+            if constexpr (DMA) {
+                const int c = cp ^ (2 * (kk & 7));
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (vr + c * 16),
+                                                 (__attribute__((address_space(3))) void*) (stage + buf * VTILE + i * 1024), 16, 0, 0);
+            } else {
+                r.v[i] = *reinterpret_cast<const uint4*>(vr + cp * 16);
+                if constexpr (KT == 1) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D + 2 * (cp / 2));
+                if constexpr (KT == 2) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D / 2 + 2 * cp);
+            }
+        }
+    };
+
+    // MORE: how many tiles' loads were issued after this tile's (0 or 1) - what the DMA wait may leave in flight
+    auto process_tile = [&](R& r, int64_t ti, int buf, auto more_c) {
+        constexpr bool more = decltype(more_c)::value;
+        const int64_t j0 = ti * TILE;
+        if constexpr (!DMA) {
+            // ---- the value tile dequantized into this wave's LDS stage, [key][D] halfs
+            const int c = lane % R::CPR, kr0 = lane / R::CPR;
+#pragma unroll
+            for (int i = 0; i < R::NLV; ++i) {
+                uint8_t* dst = stage + (kr0 + R::KPI * i) * RS;
+                const _Float16 d = __builtin_bit_cast(_Float16, r.vsc[i]);
+                if constexpr (KT == 1) {
+                    short tmp[16];
+                    dq8x4(r.v[i].x, d, tmp); dq8x4(r.v[i].y, d, tmp + 4); dq8x4(r.v[i].z, d, tmp + 8); dq8x4(r.v[i].w, d, tmp + 12);
+                    s8v a, b;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) { a[e] = tmp[e]; b[e] = tmp[8 + e]; }
+                    *reinterpret_cast<s8v*>(dst + c * 32) = a;
+                    *reinterpret_cast<s8v*>(dst + c * 32 + 16) = b;
+                } else {
+                    short tmp[32];
+                    dq4x4(r.v[i].x, 0, d, tmp); dq4x4(r.v[i].y, 0, d, tmp + 4); dq4x4(r.v[i].z, 0, d, tmp + 8); dq4x4(r.v[i].w, 0, d, tmp + 12);
+                    dq4x4(r.v[i].x, 4, d, tmp + 16); dq4x4(r.v[i].y, 4, d, tmp + 20); dq4x4(r.v[i].z, 4, d, tmp + 24); dq4x4(r.v[i].w, 4, d, tmp + 28);
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; ++q4) {
+                        s8v a;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) a[e] = tmp[q4 * 8 + e];
+                        *reinterpret_cast<s8v*>(dst + c * 64 + q4 * 16) = a;
+                    }
+                }
+            }
+        }
+        // ---- S^T = K Q^T for both 16-key tiles and every row tile
+        f4v s[RT][2];
+#pragma unroll
+        for (int kt2 = 0; kt2 < 2; ++kt2) {
+            s8v ka[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                if constexpr (DMA) {
+                    ka[kb] = __builtin_bit_cast(s8v, r.k4[kt2][kb]);
+                } else {
+                    const _Float16 d = __builtin_bit_cast(_Float16, r.ksc[kt2][kb]);
+                    short tmp[8];
+                    if constexpr (KT == 1) {
+                        dq8x4(r.k[kt2][kb][0], d, tmp);
+                        dq8x4(r.k[kt2][kb][1], d, tmp + 4);
+                    } else {
+                        const int sh = g4 >= 2 ? 4 : 0;
+                        dq4x4(r.k[kt2][kb][0], sh, d, tmp);
+                        dq4x4(r.k[kt2][kb][1], sh, d, tmp + 4);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) ka[kb][e] = tmp[e];
+                }
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
+                s[rt][kt2] = acc;
+            }
+        }
+        // ---- online softmax a row (this lane: row n of each row tile, keys j0 + 16 kt2 + 4 g4 + i)
+        s8v pb[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            float x[8], mx = -INFINITY;
+#pragma unroll
+            for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int64_t j = j0 + kt2 * 16 + g4 * 4 + i;
+                    const float v = (j >= lo_r[rt] && j <= hi_r[rt]) ? s[rt][kt2][i] * p.sl2 : -INFINITY;
+                    x[kt2 * 4 + i] = v;
+                    mx = fmaxf(mx, v);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float mn = fmaxf(m_r[rt], mx);
+            const float c = mn == -INFINITY ? 1.0f : fast_exp2(m_r[rt] - mn);
+            float sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float pv = x[e] == -INFINITY ? 0.0f : fast_exp2(x[e] - mn);
+                sum += pv;
+                pb[rt][e] = to16<BF>(pv);
+            }
+            sum += __shfl_xor(sum, 16);
+            sum += __shfl_xor(sum, 32);
+            m_r[rt] = mn;
+            l_r[rt] = l_r[rt] * c + sum;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
+        }
+        // ---- O^T += V^T P^T: the value tile read back transposed. The reads and their waits are written in assembly:
+        // the compiler's own tracking of LDS writes by DMA would wait for EVERY outstanding load here (the next tile's
+        // too) before any LDS read it can see. DMA: this tile's loads are older than the next tile's 2 KB + NLV
+        // (issued after them, in order), so waiting until only those remain makes the tile visible
+        if constexpr (DMA) {
+            if constexpr (more) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * KB + R::NLV) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+        const int kk = g4 * 4 + (n >> 2);                      // the key row this lane's address names (and + 16)
+        constexpr int HALF = DT / 2;
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+            s4v lo[HALF], hi[HALF];
+#pragma unroll
+            for (int d2 = 0; d2 < HALF; ++d2) {
+                const int dt = h2 * HALF + d2;
+                uint32_t src;
+                if constexpr (DMA) {
+                    const int c = (dt * 2 + ((n & 3) >> 1)) ^ (2 * (kk & 7));
+                    src = (uint32_t) (uintptr_t) (stage + buf * VTILE + kk * RS + c * 16 + (n & 1) * 8);
+                } else {
+                    src = (uint32_t) (uintptr_t) (stage + kk * RS + (dt * 16 + 4 * (n & 3)) * 2);
+                }
+                asm volatile("ds_read_b64_tr_b16 %0, %2\n\tds_read_b64_tr_b16 %1, %2 offset:%3" : "=&v"(lo[d2]), "=&v"(hi[d2]) : "v"(src), "n"(16 * RS));
+            }
+#pragma unroll
+            for (int d2 = 0; d2 < HALF; ++d2) {
+                const int dt = h2 * HALF + d2;
+                // reads return in order: 2 (HALF - 1 - d2) may still be out when this pair is needed
+                asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(lo[d2]), "+v"(hi[d2]) : "n"(2 * (HALF - 1 - d2)));
+                const s8v va = {lo[d2][0], lo[d2][1], lo[d2][2], lo[d2][3], hi[d2][0], hi[d2][1], hi[d2][2], hi[d2][3]};
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
+            }
+        }
+        // every read of the stage has returned: it is free for the next loads
+        asm volatile("" ::: "memory");
+    };
+
+    // ---- this wave's tiles: absolute tile index % 4 == w, over [jb, je). The steady state is its own loop so that
+    // every wait in it knows exactly which loads were issued after the ones it needs
+    if (jb < je) {
+        const int64_t tb = jb / TILE, te = (je + TILE - 1) / TILE;
+        int64_t ti = tb + ((w - (int) (tb % WAVES) + WAVES) % WAVES);
+        if (ti < te) {
+            R ra, rb;
+            const std::true_type more;
+            const std::false_type last;
+            load_tile(ra, ti, 0);
+            while (ti + 2 * WAVES < te) {
+                load_tile(rb, ti + WAVES, 1);
+                process_tile(ra, ti, 0, more);
+                load_tile(ra, ti + 2 * WAVES, 0);
+                process_tile(rb, ti + WAVES, 1, more);
+                ti += 2 * WAVES;
+            }
+            if (ti + WAVES < te) {
+                load_tile(rb, ti + WAVES, 1);
+                process_tile(ra, ti, 0, more);
+                process_tile(rb, ti + WAVES, 1, last);
+            } else {
+                process_tile(ra, ti, 0, last);
+            }
+        }
+    }
+
+    // ---- the 4 waves' partials merged in wave order, then written as the split's partial
+    if (g4 == 0)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            ml[w][rt * 16 + n][0] = m_r[rt];
+            ml[w][rt * 16 + n][1] = l_r[rt];
+        }
+    __syncthreads();
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = rt * 16 + n;
+        float M = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < WAVES; ++k) M = fmaxf(M, ml[k][row][0]);
+        float L = 0.0f;
+#pragma unroll
+        for (int k = 0; k < WAVES; ++k) L += ml[k][row][0] == -INFINITY ? 0.0f : ml[k][row][1] * fast_exp2(ml[k][row][0] - M);
+        const float f = m_r[rt] == -INFINITY ? 0.0f : fast_exp2(m_r[rt] - M);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= f;
+        if (w == 0 && g4 == 0) {
+            ML[row][0] = M;
+            ML[row][1] = L;
+        }
+    }
+    float* obuf = reinterpret_cast<float*>(lds);
+    for (int k = 0; k < WAVES; ++k) {
+        if (w == k) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    f4v* dst = reinterpret_cast<f4v*>(obuf + (rt * 16 + n) * OROW + dt * 16 + g4 * 4);
+                    if (k == 0) *dst = o[rt][dt];
+                    else *dst = *dst + o[rt][dt];
+                }
+        }
+        __syncthreads();
+    }
+    const int live_rows = std::min(RT * 16, rows - z * RT * 16);
+    for (int idx = tid; idx < live_rows * D; idx += WAVES * 64) {
+        const int row = idx / D, d = idx % D, ri = z * RT * 16 + row;
+        const int t = ri / p.G, gq = ri % p.G;
+        float* pr = p.part + (((int64_t) t * p.Hq + hk * p.G + gq) * p.ns + split) * (D + 2);
+        pr[d] = obuf[row * OROW + d];
+        if (d == 0) {
+            pr[D] = ML[row][0];
+            pr[D + 1] = ML[row][1];
+        }
+    }
+}
+
+// the splits of a (row, head) merged: a work-group per (row, head), a thread per feature
+template <int D, int QT>
+__global__ __launch_bounds__(D) void attn_merge_kernel(const float* __restrict__ part, int ns, void* __restrict__ out) {
+    const int64_t rh = blockIdx.x;
+    const int d = threadIdx.x;
+    const float* pr = part + rh * ns * (D + 2);
+    float mx = -INFINITY;
+    for (int s = 0; s < ns; ++s) mx = fmaxf(mx, pr[s * (D + 2) + D]);
+    float L = 0.0f, A = 0.0f;
+    if (mx != -INFINITY) {
+        for (int s = 0; s < ns; ++s) {
+            const float e = fast_exp2(pr[s * (D + 2) + D] - mx);
+            L += pr[s * (D + 2) + D + 1] * e;
+            A += pr[s * (D + 2) + d] * e;
+        }
+    }
+    store_o<QT>(out, rh * D + d, L > 0.0f ? A / L : 0.0f);
+}
+
+// ---- host side ----------------------------------------------------------------------------------------------------
+
+// work-groups the key splits aim for (key heads x splits); NS_DEC_WGS overrides (tuning)
+int64_t target_wgs() {
+    static const int64_t v = [] {
+        const char* e = getenv("NS_DEC_WGS");
+        const int64_t x = e ? atoll(e) : 0;
+        return x > 0 ? x : 1024;
+    }();
+    return v;
+}
+// keys a split for a row that sees `keys` keys: a multiple of 128 (4 waves x 32-key tiles)
+int64_t dec_kbs(int64_t keys, int64_t Hkv) {
+    const int64_t t = target_wgs(), want = (keys * Hkv + t - 1) / t;
+    return std::max<int64_t>(128, (want + 127) / 128 * 128);
+}
+inline int64_t row_first(int64_t pos, int64_t win) { return win > 0 ? std::max<int64_t>(0, pos - win + 1) : 0; }
+
+// the pass's T x G rows of a key head ride in row tiles of 16: one tile up to 16 rows, else chunks of two tiles (more
+// rows than 32 re-read the keys once per chunk)
+template <int D, int KT>
+int launch_rt(ns_gpu* g, const DecodeParams& p, int rows, dim3 grid_xy) {
+    const int RT = rows <= 16 ? 1 : 2;
+    dim3 grid(grid_xy.x, grid_xy.y, (unsigned) ((rows + RT * 16 - 1) / (RT * 16)));
+    if (RT == 1) attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(p);
+    else attn_decode_kernel<D, 2, KT><<<grid, WAVES * 64, 0, g->q>>>(p);
+    NS_LAUNCHED("attn_decode");
+    return 0;
+}
+
+template <int D>
+int launch_kt(ns_gpu* g, int kt, const DecodeParams& p, int rows, dim3 grid_xy) {
+    switch (kt) {
+        case 0: return launch_rt<D, 0>(g, p, rows, grid_xy);
+        case 1: return launch_rt<D, 1>(g, p, rows, grid_xy);
+        case 2: return launch_rt<D, 2>(g, p, rows, grid_xy);
+        default: return launch_rt<D, 3>(g, p, rows, grid_xy);
+    }
+}
+
+template <int D, int QT>
+int launch_merge(ns_gpu* g, const float* part, int ns, int64_t rh, void* out) {
+    attn_merge_kernel<D, QT><<<(unsigned) rh, D, 0, g->q>>>(part, ns, out);
+    NS_LAUNCHED("attn_merge");
+    return 0;
+}
+
+template <int D, int QT>
+int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv,
+                 int64_t cap, int64_t p0, int64_t win, int causal, float scale, void* out, float* scratch) {
+    const int64_t rb = kv_row_bytes(kt, D);
+    const int esz = QT == 0 ? 4 : 2;
+    DecodeParams p{};
+    p.qt = QT;
+    p.kc = (const uint8_t*) kc;
+    p.vc = (const uint8_t*) vc;
+    p.head_stride = pm ? rb : cap * rb;
+    p.row_stride = pm ? Hkv * rb : rb;
+    p.cap = cap;
+    p.wrap = !pm && p0 + T > cap;
+    p.Hq = (int) Hq;
+    p.G = (int) (Hq / Hkv);
+    p.causal = causal;
+    p.win = win;
+    p.sl2 = (scale > 0.0f ? scale : 1.0f / sqrtf((float) D)) * 1.4426950408889634f;
+    const int64_t last = p0 + T - 1;
+    auto kb_of = [&](int64_t r) {
+        const int64_t pos = causal ? p0 + r : last;
+        return dec_kbs(pos + 1 - row_first(p0 + r, win), Hkv);
+    };
+    bool same = true;
+    for (int64_t r = 1; r < T; ++r) same = same && kb_of(r) == kb_of(0);
+    const int64_t nsa = ns_attn_decode_scratch(T, Hq, Hkv, D, p0, win) / (T * Hq * (D + 2));
+    auto launch = [&](int64_t r0, int64_t nr, int64_t kb) -> int {
+        const int64_t pp = p0 + r0, sp0 = row_first(pp, win) / kb, ns = (pp + nr - 1) / kb - sp0 + 1;
+        if (ns > nsa) return ns_fail("ns_attn_decode: internal: more splits than the scratch holds");
+        DecodeParams c = p;
+        c.q = (const uint8_t*) q + r0 * qs * esz;
+        c.qs = qs;
+        c.T = (int) nr;
+        c.p0 = pp;
+        c.kbs = kb;
+        c.sp0 = sp0;
+        c.ns = (int) ns;
+        c.part = scratch + r0 * Hq * nsa * (D + 2);
+        if (launch_kt<D>(g, kt, c, (int) (nr * c.G), dim3((unsigned) ns, (unsigned) Hkv))) return -1;
+        return launch_merge<D, QT>(g, c.part, (int) ns, nr * Hq, (uint8_t*) out + r0 * Hq * D * esz);
+    };
+    if (same) return launch(0, T, kb_of(0));
+    for (int64_t r = 0; r < T; ++r)
+        if (launch(r, 1, kb_of(r))) return -1;
+    return 0;
+}
+
+int decode_checked(ns_gpu* g, const char* who, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T,
+                   int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, int causal, float scale, void* out, float* scratch) {
+    NS_TRY
+    const std::string w(who);
+    if (T <= 0) return 0;
+    if (T > 16) return ns_fail(w + ": 1..16 rows (a decode or verify pass)");
+    if (D != 128 && D != 256) return ns_fail(w + ": heads of 128 or 256");
+    if (Hkv <= 0 || Hq <= 0 || Hq % Hkv) return ns_fail(w + ": query heads a multiple of the key heads");
+    if (kt < 0 || kt > 3) return ns_fail(w + ": a cache form 0 (half), 1 (q8_0), 2 (q4_0) or 3 (bfloat16)");
+    if (qt < 0 || qt > 2) return ns_fail(w + ": rows of type 0 (float32), 1 (half) or 2 (bfloat16)");
+    if (p0 < 0 || cap <= 0) return ns_fail(w + ": a position and a capacity");
+    const int64_t need = pm ? p0 + T : (win > 0 ? std::min(p0 + T, win + T - 1) : p0 + T);
+    if (need > cap) return ns_fail(w + (win > 0 ? ": the cache's ring is shorter than the window and the pass" : ": past the cache's capacity"));
+    if (!scratch) return ns_fail(w + ": no scratch");
+    if (!q || !kc || !vc || !out) return ns_fail(w + ": a null buffer");
+    if ((uintptr_t) q % 16 || qs % (qt == 0 ? 4 : 8)) return ns_fail(w + ": query rows 16-byte aligned");
+    if (((uintptr_t) kc | (uintptr_t) vc) % 16 && (kt == 0 || kt == 3)) return ns_fail(w + ": caches 16-byte aligned");
+    if (((uintptr_t) kc | (uintptr_t) vc) % 8) return ns_fail(w + ": caches 8-byte aligned");
+    NS_HIP(hipSetDevice(g->dev));
+#define NS_DISPATCH(DD, QQ) return decode_typed<DD, QQ>(g, kt, pm, q, qs, kc, vc, T, Hq, Hkv, cap, p0, win, causal, scale, out, scratch)
+    if (D == 128) {
+        if (qt == 0) NS_DISPATCH(128, 0);
+        if (qt == 1) NS_DISPATCH(128, 1);
+        NS_DISPATCH(128, 2);
+    } else {
+        if (qt == 0) NS_DISPATCH(256, 0);
+        if (qt == 1) NS_DISPATCH(256, 1);
+        NS_DISPATCH(256, 2);
+    }
+#undef NS_DISPATCH
+    NS_CATCH
+}
+
+}  // namespace
+
+// used by the exact-API routing in attn_api.cpp
+int ns_attn_decode_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T,
+                       int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, int causal, float scale, void* out,
+                       float* scratch) {
+    return decode_checked(g, who, qt, kt, pm, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, win, causal, scale, out, scratch);
+}
+
+extern "C" {
+
+int64_t ns_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win) {
+    if (T <= 0 || Hq <= 0 || Hkv <= 0) return 0;
+    int64_t ns = 1;
+    // a row launched alone: its own split size over its own keys
+    for (int64_t r = 0; r < T; ++r) {
+        const int64_t pos = p0 + r, first = row_first(pos, win), kb = dec_kbs(pos + 1 - first, Hkv);
+        ns = std::max(ns, pos / kb - first / kb + 1);
+    }
+    // the pass in one launch: from its first row's first key to its last row's last; causal or not, the last row's
+    // key count bounds every row's
+    const int64_t f0 = row_first(p0, win), last = p0 + T - 1;
+    for (int64_t r = 0; r < T; ++r) {
+        const int64_t kb = dec_kbs(last + 1 - row_first(p0 + r, win), Hkv), kb2 = dec_kbs(p0 + r + 1 - row_first(p0 + r, win), Hkv);
+        ns = std::max(ns, last / kb - f0 / kb + 1);
+        ns = std::max(ns, last / kb2 - f0 / kb2 + 1);
+    }
+    return T * Hq * ns * (D + 2);
+}
+
+int ns_attn_decode_t(ns_gpu* g, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq,
+                     int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out, float* scratch) {
+    return decode_checked(g, "ns_attn_decode_t", qt, kt, pm, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, win, 1, scale, out, scratch);
+}
+
+int ns_q35_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) {
+    return T >= 1 && T <= 16 && (D == 128 || D == 256) && Hkv > 0 && Hq > 0 && Hq % Hkv == 0;
+}
+int64_t ns_q35_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0) { return ns_attn_decode_scratch(T, Hq, Hkv, D, p0, 0); }
+int ns_q35_attn_decode(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
+                       int64_t cap, int64_t p0, float* out, float* scratch) {
+    return decode_checked(g, "ns_q35_attn_decode", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, 1, 0.0f, out, scratch);
+}
+int ns_q35_attn_decode_kv(ns_gpu* g, int kt, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv,
+                          int64_t D, int64_t cap, int64_t p0, float* out, float* scratch) {
+    if (kt < 0 || kt > 2) return ns_fail("ns_q35_attn_decode_kv: a cache form 0 (half), 1 (q8_0) or 2 (q4_0)");
+    return decode_checked(g, "ns_q35_attn_decode_kv", 0, kt, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, 1, 0.0f, out, scratch);
+}
+
+int ns_mg_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) { return ns_q35_attn_decode_supported(T, Hq, Hkv, D); }
+int64_t ns_mg_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win) {
+    return ns_attn_decode_scratch(T, Hq, Hkv, D, p0, win);
+}
+int ns_mg_attn_decode(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap,
+                      int64_t p0, int64_t win, float* out, float* scratch) {
+    return decode_checked(g, "ns_mg_attn_decode", 0, 0, 0, q, Hq * D, kc, vc, T, Hq, Hkv, D, cap, p0, win, 1, 0.0f, out, scratch);
+}
+
+}  // extern "C"

@@ -1,0 +1,34 @@
+// kv_formats.hpp: device helpers for the cache row formats and 16-bit float conversions (shared by the store and the
+// attention kernels).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+// float -> half bits, round to nearest even (v_cvt_f16_f32 under the default rounding mode)
+__device__ __forceinline__ uint16_t f32_to_f16(float f) {
+    const _Float16 h = (_Float16) f;
+    return __builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ float f16_to_f32(uint16_t b) { return (float) __builtin_bit_cast(_Float16, b); }
+// float -> bfloat16 bits, round to nearest even; NaN stays NaN
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+    uint32_t x = __builtin_bit_cast(uint32_t, f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t) ((x >> 16) | 0x40u);
+    x += 0x7fffu + ((x >> 16) & 1u);
+    return (uint16_t) (x >> 16);
+}
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __builtin_bit_cast(float, (uint32_t) b << 16); }
+
+__host__ __device__ constexpr int64_t kv_row_bytes(int kt, int64_t D) {
+    return kt == 1 ? D + D / 32 * 2 : kt == 2 ? D / 2 + D / 32 * 2 : 2 * D;
+}
+
+// value i of a cache row of form kt as float32: (float) q x (float) half scale for the quantized forms
+__device__ __forceinline__ float kv_value_f32(const uint8_t* row, int kt, int D, int i) {
+    if (kt == 0) return f16_to_f32(*reinterpret_cast<const uint16_t*>(row + 2 * i));
+    if (kt == 3) return bf16_to_f32(*reinterpret_cast<const uint16_t*>(row + 2 * i));
+    const int b = i / 32, j = i % 32;
+    if (kt == 1) return (float) (int8_t) row[i] * f16_to_f32(*reinterpret_cast<const uint16_t*>(row + D + 2 * b));
+    const uint8_t w = row[b * 16 + (j & 15)];
+    return (float) ((int) (j < 16 ? w & 15 : w >> 4) - 8) * f16_to_f32(*reinterpret_cast<const uint16_t*>(row + D / 2 + 2 * b));
+}

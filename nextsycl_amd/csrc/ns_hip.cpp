@@ -1,0 +1,290 @@
+// ns_hip.cpp: devices, memory, copies, tickets and stamps of the C ABI (ns.h) over HIP.
+#include "ns_internal.hpp"
+
+#include <cstdio>
+#include <cstring>
+
+namespace {
+thread_local std::string g_err;
+constexpr size_t EV_RING = 1 << 16;
+constexpr size_t OWN_SCRATCH_FLOATS = (size_t) 4 << 20;   // 16 MiB
+
+int bad_index(int index, int n) { return ns_fail("no GPU " + std::to_string(index) + " (" + std::to_string(n) + " found)"); }
+
+// the event of ticket slot t, created on first use
+hipEvent_t* slot(ns_gpu* g, int64_t t) {
+    hipEvent_t* e = &g->ev[(size_t) t % EV_RING];
+    if (!*e && hipEventCreate(e) != hipSuccess) return nullptr;
+    return e;
+}
+}  // namespace
+
+int ns_fail(const std::string& what) {
+    g_err = what;
+    return -1;
+}
+
+int ns_hip_check(hipError_t e, const char* what) {
+    if (e == hipSuccess) return 0;
+    return ns_fail(std::string("hip: ") + what + ": " + hipGetErrorString(e));
+}
+
+extern "C" {
+
+const char* ns_last_error(void) { return g_err.c_str(); }
+const char* ns_version(void) { return "nextsycl-amd 0.1 (hip, gfx950)"; }
+
+int ns_gpu_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+int ns_gpu_name(int index, char* buf, size_t len) {
+    NS_TRY
+    const int n = ns_gpu_count();
+    if (index < 0 || index >= n) return bad_index(index, n);
+    hipDeviceProp_t p;
+    NS_HIP(hipGetDeviceProperties(&p, index));
+    std::snprintf(buf, len, "%s", p.name[0] ? p.name : p.gcnArchName);
+    return 0;
+    NS_CATCH
+}
+
+int ns_gpu_pci(int index, char* buf, size_t len) {
+    NS_TRY
+    const int n = ns_gpu_count();
+    if (index < 0 || index >= n) return bad_index(index, n);
+    hipDeviceProp_t p;
+    NS_HIP(hipGetDeviceProperties(&p, index));
+    std::snprintf(buf, len, "%04x:%02x:%02x.0", p.pciDomainID, p.pciBusID, p.pciDeviceID);
+    return 0;
+    NS_CATCH
+}
+
+int ns_gpu_units(int index, int* units, int* mhz) {
+    NS_TRY
+    const int n = ns_gpu_count();
+    if (index < 0 || index >= n) return bad_index(index, n);
+    hipDeviceProp_t p;
+    NS_HIP(hipGetDeviceProperties(&p, index));
+    *units = p.multiProcessorCount;
+    *mhz = p.clockRate / 1000;
+    return 0;
+    NS_CATCH
+}
+
+int ns_gpu_open(int index, ns_gpu** out) {
+    NS_TRY
+    const int n = ns_gpu_count();
+    if (index < 0 || index >= n) return bad_index(index, n);
+    NS_HIP(hipSetDevice(index));
+    ns_gpu* g = new ns_gpu;
+    g->dev = index;
+    g->ev.assign(EV_RING, nullptr);
+    // default priority on all three: streams of unequal priority are not used anywhere in this library
+    if (ns_hip_check(hipStreamCreateWithFlags(&g->q, hipStreamNonBlocking), "compute stream") ||
+        ns_hip_check(hipStreamCreateWithFlags(&g->cq, hipStreamNonBlocking), "copy stream 0") ||
+        ns_hip_check(hipStreamCreateWithFlags(&g->cq2, hipStreamNonBlocking), "copy stream 1") ||
+        ns_hip_check(hipMalloc((void**) &g->own_scratch, OWN_SCRATCH_FLOATS * sizeof(float)), "library scratch")) {
+        ns_gpu_close(g);
+        return -1;
+    }
+    g->own_scratch_floats = OWN_SCRATCH_FLOATS;
+    *out = g;
+    return 0;
+    NS_CATCH
+}
+
+void ns_gpu_close(ns_gpu* g) {
+    if (!g) return;
+    (void) hipSetDevice(g->dev);
+    if (g->q) (void) hipStreamSynchronize(g->q);
+    if (g->cq) (void) hipStreamSynchronize(g->cq);
+    if (g->cq2) (void) hipStreamSynchronize(g->cq2);
+    for (hipEvent_t e : g->ev)
+        if (e) (void) hipEventDestroy(e);
+    if (g->own_scratch) (void) hipFree(g->own_scratch);
+    if (g->q) (void) hipStreamDestroy(g->q);
+    if (g->cq) (void) hipStreamDestroy(g->cq);
+    if (g->cq2) (void) hipStreamDestroy(g->cq2);
+    delete g;
+}
+
+void* ns_gpu_queue(ns_gpu* g) { return &g->q; }
+
+int ns_gpu_memory(ns_gpu* g, uint64_t* total, int64_t* free_bytes) {
+    NS_TRY
+    NS_HIP(hipSetDevice(g->dev));
+    size_t f = 0, t = 0;
+    NS_HIP(hipMemGetInfo(&f, &t));
+    *total = t;
+    *free_bytes = (int64_t) f;
+    return 0;
+    NS_CATCH
+}
+
+int ns_alloc(ns_gpu* g, size_t bytes, void** out) {
+    NS_TRY
+    NS_HIP(hipSetDevice(g->dev));
+    *out = nullptr;
+    if (hipMalloc(out, bytes ? bytes : 1) != hipSuccess || !*out) {
+        (void) hipGetLastError();
+        return ns_fail("device allocation of " + std::to_string(bytes) + " bytes failed");
+    }
+    return 0;
+    NS_CATCH
+}
+
+int ns_free(ns_gpu* g, void* p) {
+    NS_TRY
+    NS_HIP(hipSetDevice(g->dev));
+    NS_HIP(hipFree(p));
+    return 0;
+    NS_CATCH
+}
+
+int ns_alloc_host(ns_gpu* g, size_t bytes, void** out) {
+    NS_TRY
+    NS_HIP(hipSetDevice(g->dev));
+    *out = nullptr;
+    if (hipHostMalloc(out, bytes ? bytes : 1, hipHostMallocDefault) != hipSuccess || !*out) {
+        (void) hipGetLastError();
+        return ns_fail("pinned host allocation of " + std::to_string(bytes) + " bytes failed");
+    }
+    return 0;
+    NS_CATCH
+}
+
+int ns_free_host(ns_gpu* g, void* p) {
+    NS_TRY
+    NS_HIP(hipSetDevice(g->dev));
+    NS_HIP(hipHostFree(p));
+    return 0;
+    NS_CATCH
+}
+
+int ns_copy_to(ns_gpu* g, void* dst, const void* src, size_t bytes) {
+    NS_TRY
+    if (!bytes) return 0;
+    NS_HIP(hipSetDevice(g->dev));
+    NS_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g->q));
+    return 0;
+    NS_CATCH
+}
+
+int ns_copy_from(ns_gpu* g, void* dst, const void* src, size_t bytes) {
+    NS_TRY
+    if (!bytes) return 0;
+    NS_HIP(hipSetDevice(g->dev));
+    NS_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g->q));
+    return 0;
+    NS_CATCH
+}
+
+int ns_copy_dev(ns_gpu* g, void* dst, const void* src, size_t bytes) {
+    NS_TRY
+    if (!bytes) return 0;
+    NS_HIP(hipSetDevice(g->dev));
+    NS_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g->q));
+    return 0;
+    NS_CATCH
+}
+
+int ns_copy_2d(ns_gpu* g, void* dst, size_t dst_pitch, const void* src, size_t src_pitch, size_t width, size_t height) {
+    NS_TRY
+    if (width == 0 || height == 0) return 0;
+    NS_HIP(hipSetDevice(g->dev));
+    NS_HIP(hipMemcpy2DAsync(dst, dst_pitch, src, src_pitch, width, height, hipMemcpyDeviceToDevice, g->q));
+    return 0;
+    NS_CATCH
+}
+
+int ns_mark(ns_gpu* g, int64_t* ticket) {
+    NS_TRY
+    NS_HIP(hipSetDevice(g->dev));
+    const int64_t t = g->next_ev++;
+    hipEvent_t* e = slot(g, t);
+    if (!e) return ns_fail("ns_mark: no event");
+    NS_HIP(hipEventRecord(*e, g->q));
+    *ticket = t;
+    return 0;
+    NS_CATCH
+}
+
+int ns_stream_copy(ns_gpu* g, void* dst, const void* src, size_t bytes, const int64_t* after, int ndeps, int lane, int64_t* ticket) {
+    NS_TRY
+    NS_HIP(hipSetDevice(g->dev));
+    hipStream_t s = lane ? g->cq2 : g->cq;
+    for (int i = 0; i < ndeps; ++i) {
+        hipEvent_t e = g->ev[(size_t) after[i] % EV_RING];
+        if (!e) return ns_fail("ns_stream_copy: ticket " + std::to_string(after[i]) + " was never issued");
+        NS_HIP(hipStreamWaitEvent(s, e, 0));
+    }
+    if (bytes) NS_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, s));
+    const int64_t t = g->next_ev++;
+    hipEvent_t* e = slot(g, t);
+    if (!e) return ns_fail("ns_stream_copy: no event");
+    NS_HIP(hipEventRecord(*e, s));
+    *ticket = t;
+    return 0;
+    NS_CATCH
+}
+
+int ns_await(ns_gpu* g, int64_t t) {
+    NS_TRY
+    NS_HIP(hipSetDevice(g->dev));
+    hipEvent_t e = t >= 0 ? g->ev[(size_t) t % EV_RING] : nullptr;
+    if (!e) return ns_fail("ns_await: ticket " + std::to_string(t) + " was never issued");
+    NS_HIP(hipStreamWaitEvent(g->q, e, 0));
+    return 0;
+    NS_CATCH
+}
+
+int ns_stamp(ns_gpu* g, int64_t* ticket) { return ns_mark(g, ticket); }
+
+int ns_elapsed(ns_gpu* g, int64_t t0, int64_t t1, double* ns) {
+    NS_TRY
+    NS_HIP(hipSetDevice(g->dev));
+    hipEvent_t a = t0 >= 0 ? g->ev[(size_t) t0 % EV_RING] : nullptr, b = t1 >= 0 ? g->ev[(size_t) t1 % EV_RING] : nullptr;
+    if (!a || !b) return ns_fail("ns_elapsed: a ticket that was never issued");
+    NS_HIP(hipEventSynchronize(a));
+    NS_HIP(hipEventSynchronize(b));
+    float ms = 0.0f;
+    NS_HIP(hipEventElapsedTime(&ms, a, b));
+    *ns = (double) ms * 1.0e6;
+    return 0;
+    NS_CATCH
+}
+
+int ns_fill(ns_gpu* g, void* dst, uint8_t value, size_t bytes) {
+    NS_TRY
+    if (!bytes) return 0;
+    NS_HIP(hipSetDevice(g->dev));
+    NS_HIP(hipMemsetAsync(dst, value, bytes, g->q));
+    return 0;
+    NS_CATCH
+}
+
+int ns_sync(ns_gpu* g) {
+    NS_TRY
+    NS_HIP(hipSetDevice(g->dev));
+    NS_HIP(hipStreamSynchronize(g->q));
+    return 0;
+    NS_CATCH
+}
+
+int ns_copy_peer(ns_gpu* to, void* dst, ns_gpu* from, const void* src, size_t bytes, void* staging) {
+    NS_TRY
+    if (!bytes) return 0;
+    NS_HIP(hipSetDevice(from->dev));
+    NS_HIP(hipMemcpyAsync(staging, src, bytes, hipMemcpyDeviceToHost, from->q));
+    NS_HIP(hipStreamSynchronize(from->q));
+    NS_HIP(hipSetDevice(to->dev));
+    NS_HIP(hipMemcpyAsync(dst, staging, bytes, hipMemcpyHostToDevice, to->q));
+    NS_HIP(hipStreamSynchronize(to->q));
+    return 0;
+    NS_CATCH
+}
+
+}  // extern "C"

@@ -1,0 +1,43 @@
+// ns_internal.hpp: what the library's translation units share; not part of the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "ns.h"
+
+// One opened device: the in-order compute stream every kernel and queued copy goes to, two copy streams for copies
+// that overlap it, and a ring of events - the "tickets" of ns_mark / ns_stream_copy / ns_stamp.
+struct ns_gpu {
+    int dev = 0;
+    hipStream_t q = nullptr;     // compute, in order
+    hipStream_t cq = nullptr;    // copy lane 0
+    hipStream_t cq2 = nullptr;   // copy lane 1
+    std::vector<hipEvent_t> ev;  // created on first use of a slot, re-recorded when the ring wraps
+    int64_t next_ev = 0;
+    // scratch the library keeps for entry points whose reference signature has no scratch argument
+    // (ns_llm_minimaxm3_attend); allocated once at ns_gpu_open, never inside a kernel call
+    float* own_scratch = nullptr;
+    size_t own_scratch_floats = 0;
+};
+
+// sets the calling thread's error text (ns_last_error) and returns -1
+int ns_fail(const std::string& what);
+// -1 with "hip: <what>: <error string>" when e is an error, else 0
+int ns_hip_check(hipError_t e, const char* what);
+
+#define NS_HIP(call)                                        \
+    do {                                                    \
+        if (ns_hip_check((call), #call) != 0) return -1;    \
+    } while (0)
+
+// every entry point runs with its device current (a caller's thread may have switched) and turns C++ exceptions into -1
+#define NS_TRY try {
+#define NS_CATCH                                                      \
+    }                                                                 \
+    catch (const std::exception& e) { return ns_fail(e.what()); }     \
+    catch (...) { return ns_fail("unknown C++ exception"); }
+
+// after a kernel launch: launch errors (bad configuration) surface here, not at the next sync
+#define NS_LAUNCHED(name) NS_HIP(hipGetLastError())

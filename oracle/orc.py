@@ -1,0 +1,269 @@
+"""ctypes binding of the CPU oracle (oracle.c -> liboracle.so). TEST INFRASTRUCTURE: imported only by tests/,
+__graft_entry__.smoke() and bench.py's cpu_baseline leg; the product (nextsycl_amd) never imports it."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB = os.path.join(HERE, "liboracle.so")
+
+
+def build(force=False):
+    """Compile oracle.c with gcc (the recipe is oracle/Makefile)."""
+    if force or not os.path.exists(LIB) or os.path.getmtime(LIB) < os.path.getmtime(os.path.join(HERE, "oracle.c")):
+        subprocess.run(["make", "-C", HERE, "-B", "liboracle.so"], check=True, capture_output=True)
+    return LIB
+
+
+_lib = None
+i64, f32, f64, u64 = C.c_int64, C.c_float, C.c_double, C.c_uint64
+P = C.c_void_p
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB):
+            build()
+        L = C.CDLL(LIB)
+        sig = {
+            "orc_f2h": (C.c_uint16, [f32]), "orc_h2f": (f32, [C.c_uint16]), "orc_f2bf": (C.c_uint16, [f32]), "orc_bf2f": (f32, [C.c_uint16]),
+            "orc_f2h_n": (None, [P, P, i64]), "orc_h2f_n": (None, [P, P, i64]), "orc_f2bf_n": (None, [P, P, i64]), "orc_bf2f_n": (None, [P, P, i64]),
+            "orc_uniform_f32": (None, [u64, P, i64]), "orc_randn_f32": (None, [u64, f64, P, i64]),
+            "orc_kv_row_bytes": (i64, [C.c_int, i64]),
+            "orc_kv_dequant": (None, [P, C.c_int, i64, i64, i64, P]),
+            "orc_kv_store": (C.c_int, [C.c_int, P, i64, P, i64, i64, i64, i64, i64, i64, C.c_int, P, P]),
+            "orc_kv_store_q": (C.c_int, [C.c_int, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]),
+            "orc_fwht32": (None, [P, i64, i64, i64]),
+            "orc_glm_to_q8row": (None, [P, P, i64, i64]),
+            "orc_q35_split_keys": (i64, [i64, i64, i64]), "orc_q35_splits": (i64, [i64, i64, i64]),
+            "orc_mg_split_keys": (i64, [i64, i64, i64]), "orc_mg_splits": (i64, [i64, i64, i64]), "orc_mg_seen": (i64, [i64, i64, i64, C.c_int]),
+            "orc_dec_split": (i64, [i64, i64]), "orc_dec_splits": (i64, [i64, i64]),
+            "orc_q35_attn_decode_scratch": (i64, [i64, i64, i64, i64, i64]),
+            "orc_attn_exact": (C.c_int, [P, i64, P, P, C.c_int, C.c_int, i64, i64, i64, i64, i64, i64, i64, C.c_int, i64, C.c_int, P]),
+            "orc_attn_f64": (C.c_int, [P, i64, P, P, C.c_int, C.c_int, i64, i64, i64, i64, i64, i64, i64, C.c_int, f64, P]),
+            "orc_attn_flash_model": (C.c_int, [P, i64, P, P, C.c_int, C.c_int, i64, i64, i64, i64, i64, i64, i64, i64, P]),
+            "orc_mm3_attend": (C.c_int, [P, P, P, P, i64, i64, i64, i64, f32]),
+            "orc_ds2_kv_store": (C.c_int, [P, P, f32, P, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32]),
+            "orc_mla_absorb": (None, [P, P, P, i64, i64, i64, i64, i64]),
+            "orc_mla_decode_u": (None, [P, P, P, i64, i64, i64, i64, i64, f32]),
+            "orc_mla_vb": (None, [P, P, P, i64, i64, i64, i64]),
+            "orc_mla_f64": (None, [P, P, P, i64, i64, i64, i64, i64, f64]),
+            "orc_glm_mla_attend": (None, [P, P, C.c_int, P, i64, i64, i64, i64, f32]),
+            "orc_compare": (None, [P, P, i64, P, P, P]),
+            "orc_threads": (C.c_int, []),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(L, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(P)
+
+
+def _c(a, dt):
+    a = np.ascontiguousarray(a, dtype=dt)
+    return a
+
+
+# ---- conversions -------------------------------------------------------------------------------------------------
+def f2h(x):
+    x = _c(x, np.float32)
+    y = np.empty(x.shape, np.uint16)
+    lib().orc_f2h_n(_p(x), _p(y), x.size)
+    return y
+
+
+def h2f(x):
+    x = _c(x, np.uint16)
+    y = np.empty(x.shape, np.float32)
+    lib().orc_h2f_n(_p(x), _p(y), x.size)
+    return y
+
+
+def f2bf(x):
+    x = _c(x, np.float32)
+    y = np.empty(x.shape, np.uint16)
+    lib().orc_f2bf_n(_p(x), _p(y), x.size)
+    return y
+
+
+def bf2f(x):
+    x = _c(x, np.uint16)
+    y = np.empty(x.shape, np.float32)
+    lib().orc_bf2f_n(_p(x), _p(y), x.size)
+    return y
+
+
+# ---- seeded inputs -----------------------------------------------------------------------------------------------
+def uniform(seed, n):
+    y = np.empty(n, np.float32)
+    lib().orc_uniform_f32(seed, _p(y), n)
+    return y
+
+
+def randn(seed, shape, sigma=1.0):
+    n = int(np.prod(shape))
+    y = np.empty(n, np.float32)
+    lib().orc_randn_f32(seed, float(sigma), _p(y), n)
+    return y.reshape(shape)
+
+
+def randn_f16(seed, shape, sigma=1.0):
+    """N(0, sigma) rounded to half: (bits uint16, the rounded values as float32)."""
+    b = f2h(randn(seed, shape, sigma))
+    return b, h2f(b)
+
+
+def randn_bf16(seed, shape, sigma=1.0):
+    b = f2bf(randn(seed, shape, sigma))
+    return b, bf2f(b)
+
+
+# ---- cache rows --------------------------------------------------------------------------------------------------
+def kv_row_bytes(kt, D):
+    return lib().orc_kv_row_bytes(kt, D)
+
+
+def kv_store(kt, k, v, Hkv, D, cap, p0, kc=None, vc=None, ring=False):
+    """k, v float32 [T][Hkv*D] -> caches (uint8 [Hkv][cap][row bytes]); kt 0 half, 3 bfloat16, 1 q8_0, 2 q4_0."""
+    k, v = _c(k, np.float32), _c(v, np.float32)
+    T = k.shape[0]
+    rb = kv_row_bytes(kt, D)
+    if kc is None:
+        kc = np.zeros((Hkv, cap, rb), np.uint8)
+        vc = np.zeros((Hkv, cap, rb), np.uint8)
+    if kt in (0, 3):
+        rc = lib().orc_kv_store(kt, _p(k), k.shape[1], _p(v), v.shape[1], T, Hkv, D, cap, p0, int(ring), _p(kc), _p(vc))
+    else:
+        rc = lib().orc_kv_store_q(kt, _p(k), k.shape[1], _p(v), v.shape[1], T, Hkv, D, cap, p0, _p(kc), _p(vc))
+    if rc:
+        raise ValueError("orc_kv_store: bad arguments")
+    return kc, vc
+
+
+def kv_dequant(rows, kt, D):
+    rows = _c(rows, np.uint8)
+    rb = kv_row_bytes(kt, D)
+    n = rows.size // rb
+    out = np.empty((n, D), np.float32)
+    lib().orc_kv_dequant(_p(rows), kt, D, n, rb, _p(out))
+    return out.reshape(rows.shape[:-1] + (D,))
+
+
+def fwht32(x):
+    x = _c(x, np.float32).copy()
+    rows, n = x.reshape(-1, x.shape[-1]).shape
+    lib().orc_fwht32(_p(x), rows, n, n)
+    return x
+
+
+def glm_to_q8row(x, L):
+    x = _c(x, np.float32)
+    n = x.size // L
+    y = np.zeros((n, L // 32 * 2 + L), np.uint8)
+    lib().orc_glm_to_q8row(_p(x), _p(y), n, L)
+    return y
+
+
+# ---- attention ---------------------------------------------------------------------------------------------------
+def attn_exact(q, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=0, causal=True, pm=False, groups=None, split_single_only=False):
+    q = _c(q, np.float32).reshape(T, Hq * D)
+    out = np.empty((T, Hq * D), np.float32)
+    g = groups if groups is not None else max(1, Hq // 4)
+    rc = lib().orc_attn_exact(_p(q), Hq * D, _p(kc), _p(vc), kt, int(pm), T, Hq, Hkv, D, cap, p0, win, int(causal), g, int(split_single_only), _p(out))
+    if rc:
+        raise ValueError("orc_attn_exact: bad arguments")
+    return out
+
+
+def attn_f64(q, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=0, causal=True, pm=False, scale=0.0):
+    q = _c(q, np.float32).reshape(T, Hq * D)
+    out = np.empty((T, Hq * D), np.float64)
+    rc = lib().orc_attn_f64(_p(q), Hq * D, _p(kc), _p(vc), kt, int(pm), T, Hq, Hkv, D, cap, p0, win, int(causal), float(scale), _p(out))
+    if rc:
+        raise ValueError("orc_attn_f64: bad arguments")
+    return out
+
+
+def attn_flash_model(q, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=0, kbs=0, pm=False):
+    q = _c(q, np.float32).reshape(T, Hq * D)
+    out = np.empty((T, Hq * D), np.float32)
+    rc = lib().orc_attn_flash_model(_p(q), Hq * D, _p(kc), _p(vc), kt, int(pm), T, Hq, Hkv, D, cap, p0, win, kbs, _p(out))
+    if rc:
+        raise ValueError("orc_attn_flash_model: bad arguments")
+    return out
+
+
+def mm3_attend(q, kc, vc, T, H, G, pos0, scale):
+    q = _c(q, np.float32)
+    out = np.empty((T, H * 128), np.float32)
+    rc = lib().orc_mm3_attend(_p(q), _p(kc), _p(vc), _p(out), T, H, G, pos0, float(scale))
+    if rc:
+        raise ValueError("orc_mm3_attend: bad arguments")
+    return out
+
+
+# ---- MLA ---------------------------------------------------------------------------------------------------------
+def ds2_kv_store(kv, w, eps, cache, T, L, R, pos0, freq_base, freq_scale, ext_factor, mscale, corr0, corr1):
+    kv, w = _c(kv, np.float32), _c(w, np.float32)
+    rc = lib().orc_ds2_kv_store(_p(kv), _p(w), eps, _p(cache), T, L, R, pos0, freq_base, freq_scale, ext_factor, mscale, corr0, corr1)
+    if rc:
+        raise ValueError("orc_ds2_kv_store: bad arguments")
+    return cache
+
+
+def mla_absorb(q, kb, T, H, L=512, R=64, NOPE=128):
+    q, kb = _c(q, np.float32), _c(kb, np.uint16)
+    qa = np.empty((T, H, L + R), np.float32)
+    lib().orc_mla_absorb(_p(q), _p(kb), _p(qa), T, H, L, R, NOPE)
+    return qa
+
+
+def mla_decode_u(qa, cache, T, H, pos0, scale, L=512, R=64):
+    qa, cache = _c(qa, np.float32), _c(cache, np.uint16)
+    u = np.empty((T, H, L), np.float32)
+    lib().orc_mla_decode_u(_p(qa), _p(cache), _p(u), T, H, L, R, pos0, float(scale))
+    return u
+
+
+def mla_vb(u, vb, T, H, L=512, V=128):
+    u, vb = _c(u, np.float32), _c(vb, np.uint16)
+    out = np.empty((T, H, V), np.float32)
+    lib().orc_mla_vb(_p(u), _p(vb), _p(out), T, H, L, V)
+    return out
+
+
+def mla_f64(qa, cache, T, H, pos0, scale, L=512, R=64):
+    qa, cache = _c(qa, np.float32), _c(cache, np.uint16)
+    u = np.empty((T, H, L), np.float64)
+    lib().orc_mla_f64(_p(qa), _p(cache), _p(u), T, H, L, R, pos0, float(scale))
+    return u
+
+
+def glm_mla_attend(qa, cache, q8, T, H, L, pos0, scale):
+    qa = _c(qa, np.float32)
+    cache = np.ascontiguousarray(cache)
+    u = np.empty((T, H, L), np.float32)
+    lib().orc_glm_mla_attend(_p(qa), _p(cache), int(q8), _p(u), T, H, L, pos0, float(scale))
+    return u
+
+
+# ---- comparisons -------------------------------------------------------------------------------------------------
+def compare(a, b):
+    """(max-abs, relative L2, cosine) of a (float32) against b (float64) - the reference's `kernels` check's measures."""
+    a = _c(a, np.float32).ravel()
+    b = _c(b, np.float64).ravel()
+    assert a.size == b.size
+    m, r, c = f64(), f64(), f64()
+    lib().orc_compare(_p(a), _p(b), a.size, C.byref(m), C.byref(r), C.byref(c))
+    return m.value, r.value, c.value
+
+
+def threads():
+    return lib().orc_threads()
