@@ -448,23 +448,56 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     }
 }
 
-// the splits of a (row, head) merged: a work-group per (row, head), a thread per feature
+// The splits of a (row, head) merged: out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M). A work-group of 512 threads per
+// (row, head): the splits' maxima and weights first (a thread a split), then 512 / D groups of D threads each take every
+// (512 / D)-th split's values, and the groups' sums are added pairwise. Every sum runs over a fixed shape (slots past the
+// last split hold zeros), so the result does not depend on how many empty splits a pass appends to a row's own.
+constexpr int MERGE_T = 512, MERGE_MAX_NS = 2048;
+
+__device__ __forceinline__ float block_reduce(float v, float* red, int tid, bool is_max) {
+    red[tid] = v;
+    __syncthreads();
+#pragma unroll
+    for (int o = MERGE_T / 2; o > 0; o >>= 1) {
+        if (tid < o) red[tid] = is_max ? fmaxf(red[tid], red[tid + o]) : red[tid] + red[tid + o];
+        __syncthreads();
+    }
+    const float r = red[0];
+    __syncthreads();
+    return r;
+}
+
 template <int D, int QT>
-__global__ __launch_bounds__(D) void attn_merge_kernel(const float* __restrict__ part, int ns, void* __restrict__ out) {
+__global__ __launch_bounds__(MERGE_T) void attn_merge_kernel(const float* __restrict__ part, int ns, void* __restrict__ out) {
+    constexpr int GROUPS = MERGE_T / D;
+    __shared__ float wsh[MERGE_MAX_NS];
+    __shared__ float red[MERGE_T];
     const int64_t rh = blockIdx.x;
-    const int d = threadIdx.x;
+    const int tid = threadIdx.x;
     const float* pr = part + rh * ns * (D + 2);
     float mx = -INFINITY;
-    for (int s = 0; s < ns; ++s) mx = fmaxf(mx, pr[s * (D + 2) + D]);
-    float L = 0.0f, A = 0.0f;
-    if (mx != -INFINITY) {
-        for (int s = 0; s < ns; ++s) {
-            const float e = fast_exp2(pr[s * (D + 2) + D] - mx);
-            L += pr[s * (D + 2) + D + 1] * e;
-            A += pr[s * (D + 2) + d] * e;
-        }
+    for (int s = tid; s < ns; s += MERGE_T) mx = fmaxf(mx, pr[s * (D + 2) + D]);
+    mx = block_reduce(mx, red, tid, true);
+    float ls = 0.0f;
+    for (int s = tid; s < ns; s += MERGE_T) {
+        const float m = pr[s * (D + 2) + D];
+        const float wgt = m == -INFINITY ? 0.0f : fast_exp2(m - mx);
+        wsh[s] = wgt;
+        ls += pr[s * (D + 2) + D + 1] * wgt;
     }
-    store_o<QT>(out, rh * D + d, L > 0.0f ? A / L : 0.0f);
+    const float L = block_reduce(ls, red, tid, false);   // its barriers also publish wsh
+    const int grp = tid / D, d = tid % D;
+    float acc = 0.0f;
+#pragma unroll 8
+    for (int s = grp; s < ns; s += GROUPS) acc += pr[s * (D + 2) + d] * wsh[s];
+    red[tid] = acc;
+    __syncthreads();
+    if (grp == 0) {
+        float A;
+        if constexpr (GROUPS == 4) A = (red[d] + red[D + d]) + (red[2 * D + d] + red[3 * D + d]);
+        else A = red[d] + red[D + d];
+        store_o<QT>(out, rh * D + d, L > 0.0f ? A / L : 0.0f);
+    }
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------------
@@ -509,7 +542,8 @@ int launch_kt(ns_gpu* g, int kt, const DecodeParams& p, int rows, dim3 grid_xy) 
 
 template <int D, int QT>
 int launch_merge(ns_gpu* g, const float* part, int ns, int64_t rh, void* out) {
-    attn_merge_kernel<D, QT><<<(unsigned) rh, D, 0, g->q>>>(part, ns, out);
+    if (ns > MERGE_MAX_NS) return ns_fail("ns_attn_decode: more key splits than the merge holds");
+    attn_merge_kernel<D, QT><<<(unsigned) rh, MERGE_T, 0, g->q>>>(part, ns, out);
     NS_LAUNCHED("attn_merge");
     return 0;
 }
