@@ -66,7 +66,8 @@ class Api:
                     continue
                 raise OSError("%s: missing symbol %s" % (self.path, name))
             fn.restype, fn.argtypes = res, args
-            setattr(self, name[3:], fn)
+            # `await` is a keyword: bound as await_, as the reference's table names it (crates/sys/src/lib.rs:54)
+            setattr(self, "await_" if name == "ns_await" else name[3:], fn)
 
     def symbol(self, name, restype, argtypes):
         """An engine's own entry point by name; a missing one is a load error (llm/qwen35/src/ffi.rs:139-145)."""

@@ -76,12 +76,14 @@ def gpu_prompt(ops, qt, kt, q_dev_arr, kc, vc, T, Hq, Hkv, D, cap, p0, win=0, pm
     return out_to_f32(qt, raw).reshape(T, Hq * D), raw
 
 
-def check_close(got, ref64, qt=F32, what=""):
-    """The path's bar against the float64 closed form."""
+def check_close(got, ref64, qt=F32, what="", kt=0):
+    """The path's bar against the float64 closed form: max-abs 2e-3, relative L2 1e-3. Where bfloat16 enters - output
+    rows of that type, or a bfloat16 cache (the kernel's MFMA operands are then bfloat16: the query and the softmax
+    weights are rounded to 8 significant bits) - the bound of that rounding, 2^-9 relative, is added: a correctly
+    rounded bfloat16 copy of the exact result already sits at ~1.6e-3 relative L2."""
     mx, rel, cos = orc.compare(got, ref64)
     tol_abs, tol_rel = MAX_ABS, REL_L2
-    if qt == BF16:
-        # the output's own rounding to bfloat16: relative 2^-9 a value on top of the kernel's error
+    if qt == BF16 or kt == 3:
         tol_abs = MAX_ABS + BF16_ROUND * float(np.abs(ref64).max())
         tol_rel = REL_L2 + BF16_ROUND
     assert np.isfinite(got).all(), "%s: non-finite output" % what

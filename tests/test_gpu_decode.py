@@ -38,7 +38,7 @@ def test_decode_small(ops, T, Hq, Hkv, D, p0, win, kt, qt):
     qd, qf = make_q(qt, T, Hq, D)
     got, _ = gpu_decode(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
     ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
-    check_close(got, ref, qt, "decode vs float64 closed form")
+    check_close(got, ref, qt, "decode vs float64 closed form", kt=kt)
     if kt != 3:
         # and the reference's exact kernel (float32, its own summation order) sits as close to the closed form
         ex = orc.attn_exact(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)

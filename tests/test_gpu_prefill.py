@@ -1,0 +1,99 @@
+"""Parity of the causal flash-attention prefill kernel (ns_attn_prompt_t and the reference-named entry points over it)
+against the oracle's float64 closed form, through the C ABI, on seeded inputs."""
+import numpy as np
+import pytest
+
+from helpers import check_close, gpu_decode, gpu_prompt, make_kv, make_q
+from nextsycl_amd import DevBuf
+from nextsycl_amd.attn import BF16, F16, F32
+from oracle import orc
+
+pytestmark = pytest.mark.gpu
+
+SMALL = [
+    # T, Hq, Hkv, p0, win, kt, qt
+    (17, 4, 1, 0, 0, 0, F32),        # the shortest prompt pass
+    (128, 4, 2, 0, 0, 0, F32),       # one row block exactly
+    (129, 4, 2, 0, 0, 0, F16),       # one row into the second
+    (300, 10, 2, 0, 0, 3, BF16),     # G 5, bfloat16 cache and rows (BASELINE config 2's types)
+    (200, 8, 2, 1000, 0, 0, F32),    # a later chunk of a prompt: p0 > 0
+    (333, 16, 1, 77, 0, 0, F16),     # G 16 (museglimmer's ratio)
+    (260, 4, 1, 500, 256, 0, F32),   # a window
+    (96, 6, 6, 31, 0, 3, F32),       # G 1
+]
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,p0,win,kt,qt", SMALL)
+def test_prefill_small(ops, T, Hq, Hkv, p0, win, kt, qt):
+    D = 128
+    cap = p0 + T + 5
+    kc, vc = make_kv(kt, Hkv, D, cap, p0 + T)
+    qd, qf = make_q(qt, T, Hq, D)
+    got, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got, ref, qt, "prefill vs float64 closed form", kt=kt)
+
+
+def test_prefill_ring(ops):
+    T, Hq, Hkv, D, cap, win, p0 = 150, 4, 2, 128, 512, 300, 900
+    k = orc.randn(11, (p0 + T, Hkv * D))
+    v = orc.randn(12, (p0 + T, Hkv * D))
+    kc = np.zeros((Hkv, cap, 2 * D), np.uint8)
+    vc = np.zeros((Hkv, cap, 2 * D), np.uint8)
+    for s in range(0, p0 + T, 128):
+        e = min(p0 + T, s + 128)
+        orc.kv_store(0, k[s:e], v[s:e], Hkv, D, cap, s, kc, vc, ring=True)
+    qd, qf = make_q(F32, T, Hq, D)
+    got, _ = gpu_prompt(ops, F32, 0, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got, ref, F32, "ring prefill")
+
+
+def test_prompt_rows_agree_with_decode_rows(ops):
+    """The reference's --prompt-decode check (cli/nextsycl/src/main.rs:869-917): a prompt pass's row t against the
+    decode pass at position p0 + t - two kernels, one result within the path's tolerance."""
+    T, Hq, Hkv, D, p0 = 64, 8, 2, 128, 200
+    cap = p0 + T
+    kc, vc = make_kv(0, Hkv, D, cap, cap)
+    qd, qf = make_q(F32, T, Hq, D)
+    g = ops.gpu
+    bufs = (DevBuf.of(g, kc), DevBuf.of(g, vc))
+    pr, _ = gpu_prompt(ops, F32, 0, qd, kc, vc, T, Hq, Hkv, D, cap, p0, bufs=bufs)
+    for t in (0, 1, 31, 63):
+        de, _ = gpu_decode(ops, F32, 0, qd[t:t + 1], kc, vc, 1, Hq, Hkv, D, cap, p0 + t, bufs=bufs)
+        mx, rel, _ = orc.compare(pr[t:t + 1], de.astype(np.float64))
+        assert mx <= 2e-3 and rel <= 1e-3, (t, mx, rel)
+
+
+def test_softmax_weights_sum_to_one(ops):
+    """V = 1 everywhere -> every output is 1: a row's weights sum to one (to the rounding of the weights to half)."""
+    T, Hq, Hkv, D = 400, 4, 1, 128
+    kc, vc = make_kv(0, Hkv, D, T, T)
+    vc = np.ascontiguousarray(np.broadcast_to(np.array([0x3C00], np.uint16).view(np.uint8), (Hkv, T, D, 2)).reshape(Hkv, T, 2 * D))
+    qd, _ = make_q(F32, T, Hq, D)
+    got, _ = gpu_prompt(ops, F32, 0, qd, kc, vc, T, Hq, Hkv, D, T, 0)
+    assert np.abs(got - 1.0).max() < 5e-4
+
+
+def test_reference_named_prompt_entry_points(ops):
+    T, Hq, Hkv, D, p0 = 70, 8, 2, 128, 10
+    cap = p0 + T
+    kc, vc = make_kv(0, Hkv, D, cap, cap)
+    qd, _ = make_q(F32, T, Hq, D)
+    g = ops.gpu
+    bufs = (DevBuf.of(g, kc), DevBuf.of(g, vc))
+    want, _ = gpu_prompt(ops, F32, 0, qd, kc, vc, T, Hq, Hkv, D, cap, p0, bufs=bufs)
+    qb, ob = DevBuf.of(g, qd), DevBuf(g, T * Hq * D * 4)
+    k = ops.k
+    assert k.mg_attn_prompt_supported(T, Hq, Hkv, D) == 1 and k.mg_attn_prompt_supported(16, Hq, Hkv, D) == 0
+    ops.mg_attn_prompt(qb, bufs[0], bufs[1], T, Hq, Hkv, D, cap, p0, 0, ob)
+    assert np.array_equal(ob.read(np.float32).reshape(T, -1), want)
+    ob.fill(0)
+    ops.mg_attn(qb, bufs[0], bufs[1], T, Hq, Hkv, D, cap, p0, 0, True, ob, None)
+    assert np.array_equal(ob.read(np.float32).reshape(T, -1), want)
+    ob.fill(0)
+    ops.q35_attn(qb, Hq * D, bufs[0], bufs[1], T, Hq, Hkv, D, cap, p0, ob, None)
+    assert np.array_equal(ob.read(np.float32).reshape(T, -1), want)
+    assert k.q35_attn_prompt_kv(g.raw, 1, qb.ptr, Hq * D, bufs[0].ptr, bufs[1].ptr, T, Hq, Hkv, D, cap, p0, ob.ptr) == -1
+    assert k.attn_prompt_t(g.raw, 0, 0, 0, qb.ptr, Hq * D, bufs[0].ptr, bufs[1].ptr, T, Hq, Hkv, 256, cap, p0, 0, 0.0, ob.ptr) == -1
+    assert "heads of 128" in k.api.error()
