@@ -1,0 +1,235 @@
+#!/usr/bin/env python3
+"""bench.py - the attention hot path on one MI355X, one JSON line on stdout.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload prefill8k|decode32k|...] [--no-cpu] [--no-extra]
+
+A step is one pass of the hot path over one batch of synthetic input, inputs resident in HBM when the timed region
+starts. The default workload is BASELINE.json's configs[1] - causal GQA flash-attention prefill, batch 1, 8192 rows, 40
+query heads / 8 key heads, head 128, bfloat16 Q / K / V / output - and `value` is its TFLOP/s counted on the causal
+flops 4 D Hq S (S + 1) / 2. The line also carries:
+  roofline      the dominant kernel's algorithmic flops (or bytes) per launch over its device time, measured with HIP
+                events on the library's own compute stream (ns_attn_profile), against MI355X's published peak;
+  cpu_baseline  the CPU oracle (a port of the reference's exact kernel, OpenMP) timed on this host on a bounded sample;
+  others        the decode-side workloads of the same metric (GB/s of algorithmic KV bytes, % of 8 TB/s): the 32K GQA
+                decode target, BASELINE configs 1, 3, 5 - unless --no-extra.
+Decode workloads rotate over several distinct caches (> 512 MB in all) so the keys come from HBM, not from the 256 MB
+Infinity Cache."""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS_BF16 = 2500.0   # MI355X dense bf16 / fp16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+# name -> (kind, T, Hq, Hkv, D, kv_len, kt, qt, description)
+WORKLOADS = {
+    "prefill8k": ("prefill", 8192, 40, 8, 128, 8192, 3, 2, "causal GQA flash-attention prefill, batch 1, seq 8192, 40 q heads / 8 kv heads, head_dim 128, bf16 (BASELINE configs[1])"),
+    "decode4k": ("decode", 1, 32, 8, 128, 4096, 0, 1, "GQA decode, batch 1, 32 q heads / 8 kv heads, head_dim 128, KV 4096, f16 (BASELINE configs[0])"),
+    "decode32k": ("decode", 1, 32, 8, 128, 32768, 0, 1, "GQA decode, batch 1, 32 q heads / 8 kv heads, head_dim 128, KV 32768, f16 (the north star's 32K target)"),
+    "decode128k_q8": ("decode", 1, 64, 4, 128, 131072, 1, 1, "GQA decode, q8_0 KV cache, 64 q heads / 4 kv heads, head_dim 128, KV 131072 (BASELINE configs[2])"),
+    "verify64k": ("decode", 4, 32, 4, 128, 65540, 0, 1, "MTP verify, 4 draft rows on a 65536-token f16 KV cache, 32 q heads / 4 kv heads, head_dim 128 (BASELINE configs[4])"),
+}
+
+
+def kv_bytes(kt, D):
+    return {0: 2 * D, 1: D + D // 16, 2: D // 2 + D // 16, 3: 2 * D}[kt]
+
+
+def algorithmic(kind, T, Hq, Hkv, D, kv, kt, qt):
+    """(flops, bytes) of one step: the accounting of the reference's own probe (llm/qwen35/src/engine.rs:1540-1541,1591):
+    flops 4 keys Hq D with keys = rows x visible keys; bytes = every visible K and V row once + q + out."""
+    p0 = kv - T
+    keys = T * p0 + T * (T + 1) // 2
+    esz = 4 if qt == 0 else 2
+    return 4 * keys * Hq * D, 2 * Hkv * kv * kv_bytes(kt, D) + 2 * T * Hq * D * esz
+
+
+class Workload:
+    """Synthetic inputs of one workload resident on the GPU: seeded N(0, 1) K / V rows packed by the library's own
+    store kernel into `nbuf` distinct caches, query rows of the workload's type."""
+
+    def __init__(self, ops, name, nbuf):
+        from nextsycl_amd import DevBuf
+        from oracle import orc
+
+        self.ops, self.name = ops, name
+        self.kind, self.T, self.Hq, self.Hkv, self.D, self.kv, self.kt, self.qt, self.desc = WORKLOADS[name]
+        g = ops.gpu
+        T, Hq, Hkv, D, kv, kt, qt = self.T, self.Hq, self.Hkv, self.D, self.kv, self.kt, self.qt
+        self.p0 = kv - T
+        rb = kv_bytes(kt, D)
+        self.caches = []
+        chunk = 8192
+        for b in range(nbuf):
+            kc, vc = DevBuf(g, Hkv * kv * rb), DevBuf(g, Hkv * kv * rb)
+            if b == 0:
+                for s in range(0, kv, chunk):
+                    n = min(chunk, kv - s)
+                    k = DevBuf.of(g, orc.randn(0xB0B + s, (n, Hkv * D)))
+                    v = DevBuf.of(g, orc.randn(0xC0FFEE + s, (n, Hkv * D)))
+                    ops.kv_store(kt, k, Hkv * D, v, Hkv * D, n, Hkv, D, kv, s, kc, vc)
+            else:
+                # further caches: the same rows at other addresses (what the rotation needs is distinct memory)
+                g.api.copy_dev(g.raw, kc.ptr, self.caches[0][0].ptr, kc.len)
+                g.api.copy_dev(g.raw, vc.ptr, self.caches[0][1].ptr, vc.len)
+            g.sync()
+            self.caches.append((kc, vc))
+        q = orc.randn(0xA11CE, (T, Hq * D))
+        qd = q if qt == 0 else (orc.f2h(q) if qt == 1 else orc.f2bf(q))
+        self.q = DevBuf.of(g, qd)
+        self.out = DevBuf(g, T * Hq * D * (4 if qt == 0 else 2))
+        self.scratch = DevBuf(g, max(4, 4 * ops.decode_scratch(T, Hq, Hkv, D, self.p0))) if self.kind == "decode" else None
+        self.flops, self.bytes = algorithmic(self.kind, T, Hq, Hkv, D, kv, kt, qt)
+        self.i = 0
+
+    def step(self):
+        kc, vc = self.caches[self.i % len(self.caches)]
+        self.i += 1
+        o = self.ops
+        if self.kind == "prefill":
+            o.prompt(self.qt, self.kt, self.q, self.Hq * self.D, kc, vc, self.T, self.Hq, self.Hkv, self.D, self.kv, 0, self.out)
+        else:
+            o.decode(self.qt, self.kt, self.q, self.Hq * self.D, kc, vc, self.T, self.Hq, self.Hkv, self.D, self.kv, self.p0, self.out, self.scratch)
+
+
+def timed(w, steps, warmup):
+    """(ms per step over exactly `steps` steps, average device ns of the dominant kernel, of the merge kernel)."""
+    g = w.ops.gpu
+    for _ in range(warmup):
+        w.step()
+    g.sync()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        w.step()
+    g.sync()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    # the dominant kernel alone: HIP events on the library's compute stream around each launch (a pass of its own:
+    # the events open gaps between the launches that the throughput pass must not see)
+    w.ops.profile(True)
+    main = merge = 0.0
+    n = max(3, min(steps, 20))
+    for _ in range(n):
+        w.step()
+        a, b = w.ops.profile_last()
+        main += a
+        merge += b
+    w.ops.profile(False)
+    return ms, main / n, merge / n
+
+
+def roofline(w, main_ns):
+    if w.kind == "prefill":
+        ach = w.flops / main_ns / 1e3
+        return {"bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_TFLOPS_BF16, "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS_BF16, 4),
+                "traffic": None, "kernel": "attn_prefill_kernel", "kernel_us": round(main_ns / 1e3, 2)}
+    ach = w.bytes / main_ns
+    return {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+            "kernel": "attn_decode_kernel", "kernel_us": round(main_ns / 1e3, 2)}
+
+
+def cpu_baseline(name):
+    """The CPU oracle on a bounded sample of the workload, timed on this host's cores."""
+    from oracle import orc
+
+    kind, T, Hq, Hkv, D, kv, kt, qt, _ = WORKLOADS[name]
+    k = orc.randn(0xB0B, (kv, Hkv * D))
+    v = orc.randn(0xC0FFEE, (kv, Hkv * D))
+    kc, vc = orc.kv_store(kt, k, v, Hkv, D, kv, 0)
+    if kind == "prefill":
+        rows = 1024          # the last 1024 query rows against the whole cache (~10-20 s on 16 cores)
+        p0 = kv - rows
+        q = orc.bf2f(orc.f2bf(orc.randn(0xA11CE, (rows, Hq * D))))
+        sample = "last %d of %d query rows (positions %d..%d), all %d heads, full %d-key cache, reference-order float32 kernel" % (rows, T, p0, kv - 1, Hq, kv)
+        flops = 4 * D * Hq * (rows * p0 + rows * (rows + 1) // 2)
+        t0 = time.perf_counter()
+        orc.attn_exact(q, kc, vc, kt, rows, Hq, Hkv, D, kv, p0, groups=max(1, Hq // 4))
+        dt = time.perf_counter() - t0
+        return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": orc.threads(), "kind": "port", "sample": sample, "seconds": round(dt, 2)}
+    reps = 3
+    q = orc.randn(0xA11CE, (T, Hq * D))
+    flops, nbytes = algorithmic(kind, T, Hq, Hkv, D, kv, kt, qt)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        orc.attn_exact(q, kc, vc, kt, T, Hq, Hkv, D, kv, kv - T, groups=max(1, Hq // 4))
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": orc.threads(), "kind": "port",
+            "sample": "the whole workload, %d passes, reference-order float32 kernel" % reps, "seconds": round(dt * reps, 2)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="prefill8k", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the decode-side workloads of the metric")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (the path shards by key head or by context, see DESIGN.md)" % a.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+
+    from nextsycl_amd import Gpu, library_path
+    from nextsycl_amd.attn import Ops
+
+    if not os.path.exists(library_path()):
+        from nextsycl_amd.build import build
+        build()
+    g = Gpu.open(0)
+    ops = Ops(g)
+
+    def run(name, steps, warmup):
+        kind = WORKLOADS[name][0]
+        # decode: rotate distinct caches totalling > 512 MB so the keys are read from HBM
+        nbuf = 1 if kind == "prefill" else max(4, int(np.ceil(600e6 / (2 * WORKLOADS[name][3] * WORKLOADS[name][5] * kv_bytes(WORKLOADS[name][6], WORKLOADS[name][4])))))
+        nbuf = min(nbuf, 40)
+        w = Workload(ops, name, nbuf)
+        ms, main_ns, merge_ns = timed(w, steps, warmup)
+        return w, ms, main_ns, merge_ns
+
+    w, ms, main_ns, merge_ns = run(a.workload, a.steps, a.warmup)
+    if w.kind == "prefill":
+        metric, unit, value = "prefill attention TFLOP/s (causal flops), 1 MI355X", "TFLOP/s", w.flops / (ms * 1e-3) / 1e12
+    else:
+        metric, unit, value = "decode attention HBM GB/s (algorithmic KV bytes), 1 MI355X", "GB/s", w.bytes / (ms * 1e-3) / 1e9
+    line = {
+        "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": {0: "f32", 1: "f16", 2: "bf16"}[w.qt] if w.kt in (0, 3) else "q8_0/f16",
+        "data": "synthetic (seeded xorshift64* + Box-Muller N(0,1))",
+        "config": {"workload": w.desc, "name": a.workload, "rows": w.T, "q_heads": w.Hq, "kv_heads": w.Hkv, "head_dim": w.D, "kv_len": w.kv,
+                   "kv_form": {0: "f16", 1: "q8_0", 2: "q4_0", 3: "bf16"}[w.kt], "flops_per_step": w.flops, "bytes_per_step": w.bytes},
+        "tokens_per_s": round(w.T / (ms * 1e-3), 1),
+        "roofline": roofline(w, main_ns),
+    }
+    if merge_ns:
+        line["merge_kernel_us"] = round(merge_ns / 1e3, 2)
+    del w
+    if not a.no_extra:
+        others = {}
+        for name in ("decode32k", "decode4k", "decode128k_q8", "verify64k", "prefill8k"):
+            if name == a.workload:
+                continue
+            ww, m2, k2, g2 = run(name, max(10, a.steps), a.warmup)
+            r = roofline(ww, k2)
+            others[name] = {"ms_per_step": round(m2, 5), "step_" + ("TFLOP/s" if ww.kind == "prefill" else "GB/s"):
+                            round((ww.flops / (m2 * 1e-3) / 1e12) if ww.kind == "prefill" else (ww.bytes / (m2 * 1e-3) / 1e9), 2), "roofline": r,
+                            "merge_kernel_us": round(g2 / 1e3, 2)}
+            del ww
+        line["others"] = others
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(a.workload)
+    print(json.dumps(line))
+    g.close()
+
+
+if __name__ == "__main__":
+    main()

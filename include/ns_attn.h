@@ -127,6 +127,15 @@ int ns_mg_attn(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_
 int ns_llm_minimaxm3_attend(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
                             int64_t H, int64_t G, int64_t pos0, float scale);
 
+/* ---- measurement ---------------------------------------------------------------------------------------------------- */
+
+/* This library's own (the reference times kernels from the host side: llm/qwen35/src/probe.rs:105-113). on != 0: every
+ * attention call records HIP events on the compute stream before its main kernel, between it and the merge kernel, and
+ * after; ns_attn_profile_last waits for the last call's and returns the two kernels' device times in nanoseconds
+ * (merge_ns 0 for a call without a merge). Off by default: the events add gaps between the launches */
+int ns_attn_profile(ns_gpu* g, int on);
+int ns_attn_profile_last(ns_gpu* g, double* main_ns, double* merge_ns);
+
 #ifdef __cplusplus
 }
 #endif

@@ -55,6 +55,8 @@ ATTN_H = {
     "ns_mg_attn_scratch": (i64, [i64, i64, i64, i64, i64, i64, i32]),
     "ns_mg_attn": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, i32, P, P]),
     "ns_llm_minimaxm3_attend": (i32, [P, P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
+    "ns_attn_profile": (i32, [P, i32]),
+    "ns_attn_profile_last": (i32, [P, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
 }
 
 
@@ -97,6 +99,16 @@ class Ops:
     def ok(self, rc, what):
         if rc != 0:
             raise Error("%s: %s" % (what, self.k.api.error()))
+
+    # ---- measurement
+    def profile(self, on):
+        self.ok(self.k.attn_profile(self.raw(), int(on)), "profile")
+
+    def profile_last(self):
+        """(main kernel ns, merge kernel ns) of the last attention call made with profiling on; waits for it."""
+        a, b = C.c_double(), C.c_double()
+        self.ok(self.k.attn_profile_last(self.raw(), C.byref(a), C.byref(b)), "profile_last")
+        return a.value, b.value
 
     # ---- caches
     def cache_bytes(self, kt, Hkv, cap, D):

@@ -586,8 +586,11 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
         c.sp0 = sp0;
         c.ns = (int) ns;
         c.part = scratch + r0 * Hq * nsa * (D + 2);
+        if (ns_profile_mark(g, 0)) return -1;
         if (launch_kt<D>(g, kt, c, (int) (nr * c.G), dim3((unsigned) ns, (unsigned) Hkv))) return -1;
-        return launch_merge<D, QT>(g, c.part, (int) ns, nr * Hq, (uint8_t*) out + r0 * Hq * D * esz);
+        if (ns_profile_mark(g, 1)) return -1;
+        if (launch_merge<D, QT>(g, c.part, (int) ns, nr * Hq, (uint8_t*) out + r0 * Hq * D * esz)) return -1;
+        return ns_profile_mark(g, 2);
     };
     if (same) return launch(0, T, kb_of(0));
     for (int64_t r = 0; r < T; ++r)

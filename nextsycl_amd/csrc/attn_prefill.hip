@@ -292,10 +292,11 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     p.sl2 = (scale > 0.0f ? scale : 1.0f / sqrtf((float) D)) * 1.4426950408889634f;
     p.out = out;
     dim3 grid((unsigned) ((T + ROWS - 1) / ROWS), (unsigned) Hq);
+    if (ns_profile_mark(g, 0)) return -1;
     if (kt == 3) attn_prefill_kernel<128, true><<<grid, PW * 64, 0, g->q>>>(p);
     else attn_prefill_kernel<128, false><<<grid, PW * 64, 0, g->q>>>(p);
     NS_LAUNCHED("attn_prefill");
-    return 0;
+    return ns_profile_mark(g, 1);
     NS_CATCH
 }
 

@@ -29,7 +29,38 @@ int ns_hip_check(hipError_t e, const char* what) {
     return ns_fail(std::string("hip: ") + what + ": " + hipGetErrorString(e));
 }
 
+int ns_profile_mark(ns_gpu* g, int i) {
+    if (!g->profile) return 0;
+    if (!g->pev[i]) NS_HIP(hipEventCreate(&g->pev[i]));
+    NS_HIP(hipEventRecord(g->pev[i], g->q));
+    if (i + 1 > g->pev_used) g->pev_used = i + 1;
+    return 0;
+}
+
 extern "C" {
+
+int ns_attn_profile(ns_gpu* g, int on) {
+    g->profile = on != 0;
+    g->pev_used = 0;
+    return 0;
+}
+
+int ns_attn_profile_last(ns_gpu* g, double* main_ns, double* merge_ns) {
+    NS_TRY
+    *main_ns = *merge_ns = 0.0;
+    if (g->pev_used < 2) return ns_fail("ns_attn_profile_last: no profiled attention call yet");
+    NS_HIP(hipSetDevice(g->dev));
+    NS_HIP(hipEventSynchronize(g->pev[g->pev_used - 1]));
+    float ms = 0.0f;
+    NS_HIP(hipEventElapsedTime(&ms, g->pev[0], g->pev[1]));
+    *main_ns = (double) ms * 1.0e6;
+    if (g->pev_used > 2) {
+        NS_HIP(hipEventElapsedTime(&ms, g->pev[1], g->pev[2]));
+        *merge_ns = (double) ms * 1.0e6;
+    }
+    return 0;
+    NS_CATCH
+}
 
 const char* ns_last_error(void) { return g_err.c_str(); }
 const char* ns_version(void) { return "nextsycl-amd 0.1 (hip, gfx950)"; }
@@ -103,6 +134,8 @@ void ns_gpu_close(ns_gpu* g) {
     if (g->cq) (void) hipStreamSynchronize(g->cq);
     if (g->cq2) (void) hipStreamSynchronize(g->cq2);
     for (hipEvent_t e : g->ev)
+        if (e) (void) hipEventDestroy(e);
+    for (hipEvent_t e : g->pev)
         if (e) (void) hipEventDestroy(e);
     if (g->own_scratch) (void) hipFree(g->own_scratch);
     if (g->q) (void) hipStreamDestroy(g->q);

@@ -20,7 +20,14 @@ struct ns_gpu {
     // (ns_llm_minimaxm3_attend); allocated once at ns_gpu_open, never inside a kernel call
     float* own_scratch = nullptr;
     size_t own_scratch_floats = 0;
+    // ns_attn_profile: events around the kernels of the last attention call (measurement only; off by default)
+    bool profile = false;
+    hipEvent_t pev[3] = {nullptr, nullptr, nullptr};
+    int pev_used = 0;
 };
+
+// records profile event i on the compute stream when profiling is on (creates it on first use); 0 or -1
+int ns_profile_mark(ns_gpu* g, int i);
 
 // sets the calling thread's error text (ns_last_error) and returns -1
 int ns_fail(const std::string& what);
