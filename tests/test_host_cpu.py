@@ -1,0 +1,88 @@
+"""What needs no GPU: the library loads and exports every symbol the headers declare, the host wrappers' own logic
+(row sizes, error classification, scratch sizing through the C ABI's pure functions)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from nextsycl_amd import Error, library_path
+from nextsycl_amd.attn import ATTN_H, kv_row_bytes
+from nextsycl_amd.sys import NS_H
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def handle():
+    if not os.path.exists(library_path()):
+        from nextsycl_amd.build import build
+        build()
+    return C.CDLL(library_path())
+
+
+def _declared(header):
+    """extern "C" function names a header declares."""
+    src = open(os.path.join(ROOT, "include", header)).read()
+    src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
+    return set(re.findall(r"\b(ns_[a-z0-9_]+)\s*\(", src))
+
+
+def test_library_exports_every_declared_symbol(handle):
+    declared = _declared("ns.h") | _declared("ns_attn.h")
+    assert len(_declared("ns.h")) == 26                      # the reference's 26 (kernels/ns/ns.h:18-56)
+    missing = [n for n in sorted(declared) if not hasattr(handle, n)]
+    assert not missing, missing
+    # and the host tables bind exactly the declared set
+    assert set(NS_H) == _declared("ns.h")
+    assert set(ATTN_H) == _declared("ns_attn.h")
+
+
+def test_pure_functions_without_a_gpu(handle):
+    f = handle.ns_attn_decode_scratch
+    f.restype, f.argtypes = C.c_int64, [C.c_int64] * 6
+    # one row, 32 / 8 heads, 4096 keys: splits of 128 -> 32 partials of D + 2 floats a head
+    assert f(1, 32, 8, 128, 4095, 0) == 32 * 32 * 130
+    assert f(0, 32, 8, 128, 4095, 0) == 0
+    # a verify pass needs at least its rows' own
+    assert f(4, 32, 4, 128, 65536, 0) >= 4 * f(1, 32, 4, 128, 65536, 0)
+    # a window bounds the splits whatever the position
+    assert f(1, 16, 1, 128, 10 ** 6, 2048) <= 16 * 17 * 130
+    s = handle.ns_q35_attn_decode_supported
+    s.restype, s.argtypes = C.c_int, [C.c_int64] * 4
+    assert s(1, 12, 2, 256) == 1 and s(8, 32, 8, 128) == 1 and s(17, 32, 8, 128) == 0 and s(1, 12, 5, 128) == 0 and s(1, 12, 2, 96) == 0
+    p = handle.ns_mg_attn_prompt_supported
+    p.restype, p.argtypes = C.c_int, [C.c_int64] * 4
+    assert p(17, 64, 4, 128) == 1 and p(16, 64, 4, 128) == 0 and p(100, 64, 4, 256) == 0
+    handle.ns_version.restype = C.c_char_p
+    assert b"gfx950" in handle.ns_version()
+    handle.ns_last_error.restype = C.c_char_p
+    assert handle.ns_last_error() is not None
+
+
+def test_row_bytes_and_errors():
+    assert [kv_row_bytes(k, 128) for k in (0, 1, 2, 3)] == [256, 136, 72, 256]
+    assert [kv_row_bytes(k, 256) for k in (0, 1, 2)] == [512, 272, 144]      # llm/qwen35/src/engine.rs:54-60
+    with pytest.raises(Error):
+        kv_row_bytes(4, 128)
+    # crates/core/src/lib.rs:509-516
+    assert Error("copying to the GPU: hip: hipMemcpyAsync: hipErrorOutOfMemory").is_no_room()
+    assert Error("device allocation of 1024 bytes failed").is_no_room()
+    assert Error.no_room("needs 2.0 GiB more").is_no_room()
+    assert not Error("hip: hipStreamSynchronize: unspecified launch failure").is_no_room()
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    from nextsycl_amd.sys import Api
+    monkeypatch.setenv("NEXTSYCL_LIB", str(tmp_path / "nope.so"))
+    with pytest.raises(OSError):
+        Api()
+
+
+def test_product_never_imports_the_oracle():
+    """The oracle is test infrastructure: nothing under nextsycl_amd/ may import, load or link it."""
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "nextsycl_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".cpp", ".hpp", ".h")):
+                src = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in src and "liboracle" not in src, os.path.join(dirpath, f)
