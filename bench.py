@@ -35,6 +35,8 @@ WORKLOADS = {
     "decode32k": ("decode", 1, 32, 8, 128, 32768, 0, 1, "GQA decode, batch 1, 32 q heads / 8 kv heads, head_dim 128, KV 32768, f16 (the north star's 32K target)"),
     "decode128k_q8": ("decode", 1, 64, 4, 128, 131072, 1, 1, "GQA decode, q8_0 KV cache, 64 q heads / 4 kv heads, head_dim 128, KV 131072 (BASELINE configs[2])"),
     "verify64k": ("decode", 4, 32, 4, 128, 65540, 0, 1, "MTP verify, 4 draft rows on a 65536-token f16 KV cache, 32 q heads / 4 kv heads, head_dim 128 (BASELINE configs[4])"),
+    # MLA: Hq = heads, Hkv unused (one latent row a position), D = 512 latent + 64 rope
+    "mla32k": ("mla", 1, 128, 1, 576, 32768, 0, 1, "DeepSeek-style absorbed MLA decode, 128 heads, 512 latent + 64 rope, f16 latent cache, KV 32768 (BASELINE configs[3])"),
 }
 
 
@@ -48,6 +50,9 @@ def algorithmic(kind, T, Hq, Hkv, D, kv, kt, qt):
     p0 = kv - T
     keys = T * p0 + T * (T + 1) // 2
     esz = 4 if qt == 0 else 2
+    if kind == "mla":
+        # scores over 576 features, the latent sum over 512; the cache once; q (576) and u (512) a head
+        return 2 * keys * Hq * (576 + 512), kv * 576 * 2 + T * Hq * (576 + 512) * esz
     return 4 * keys * Hq * D, 2 * Hkv * kv * kv_bytes(kt, D) + 2 * T * Hq * D * esz
 
 
@@ -64,6 +69,17 @@ class Workload:
         g = ops.gpu
         T, Hq, Hkv, D, kv, kt, qt = self.T, self.Hq, self.Hkv, self.D, self.kv, self.kt, self.qt
         self.p0 = kv - T
+        self.flops, self.bytes = algorithmic(self.kind, T, Hq, Hkv, D, kv, kt, qt)
+        self.i = 0
+        if self.kind == "mla":
+            self.caches = []
+            host = orc.f2h(orc.randn(0xB0B, (kv, 576), 0.5))
+            for b in range(nbuf):
+                self.caches.append((DevBuf.of(g, host), None))
+            self.q = DevBuf.of(g, orc.f2h(orc.randn(0xA11CE, (T, Hq, 576))))
+            self.out = DevBuf(g, T * Hq * 512 * 2)
+            self.scratch = DevBuf(g, 4 * ops.mla_latent_scratch(T, Hq, self.p0))
+            return
         rb = kv_bytes(kt, D)
         self.caches = []
         chunk = 8192
@@ -86,14 +102,14 @@ class Workload:
         self.q = DevBuf.of(g, qd)
         self.out = DevBuf(g, T * Hq * D * (4 if qt == 0 else 2))
         self.scratch = DevBuf(g, max(4, 4 * ops.decode_scratch(T, Hq, Hkv, D, self.p0))) if self.kind == "decode" else None
-        self.flops, self.bytes = algorithmic(self.kind, T, Hq, Hkv, D, kv, kt, qt)
-        self.i = 0
 
     def step(self):
         kc, vc = self.caches[self.i % len(self.caches)]
         self.i += 1
         o = self.ops
-        if self.kind == "prefill":
+        if self.kind == "mla":
+            o.mla_decode_latent(1, self.q, kc, self.out, self.T, self.Hq, 64, self.p0, 192.0 ** -0.5, self.scratch)
+        elif self.kind == "prefill":
             o.prompt(self.qt, self.kt, self.q, self.Hq * self.D, kc, vc, self.T, self.Hq, self.Hkv, self.D, self.kv, 0, self.out)
         else:
             o.decode(self.qt, self.kt, self.q, self.Hq * self.D, kc, vc, self.T, self.Hq, self.Hkv, self.D, self.kv, self.p0, self.out, self.scratch)
@@ -125,6 +141,10 @@ def timed(w, steps, warmup):
 
 
 def roofline(w, main_ns):
+    if w.kind == "mla":
+        ach = w.flops / main_ns / 1e3
+        return {"bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_TFLOPS_BF16, "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS_BF16, 4),
+                "traffic": None, "kernel": "mla_decode_kernel", "kernel_us": round(main_ns / 1e3, 2), "hbm_GB/s": round(w.bytes / main_ns, 1)}
     if w.kind == "prefill":
         ach = w.flops / main_ns / 1e3
         return {"bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_TFLOPS_BF16, "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS_BF16, 4),
@@ -189,14 +209,16 @@ def main():
     def run(name, steps, warmup):
         kind = WORKLOADS[name][0]
         # decode: rotate distinct caches totalling > 512 MB so the keys are read from HBM
-        nbuf = 1 if kind == "prefill" else max(4, int(np.ceil(600e6 / (2 * WORKLOADS[name][3] * WORKLOADS[name][5] * kv_bytes(WORKLOADS[name][6], WORKLOADS[name][4])))))
+        nbuf = 1 if kind == "prefill" else 16 if kind == "mla" else max(4, int(np.ceil(600e6 / (2 * WORKLOADS[name][3] * WORKLOADS[name][5] * kv_bytes(WORKLOADS[name][6], WORKLOADS[name][4])))))
         nbuf = min(nbuf, 40)
         w = Workload(ops, name, nbuf)
         ms, main_ns, merge_ns = timed(w, steps, warmup)
         return w, ms, main_ns, merge_ns
 
     w, ms, main_ns, merge_ns = run(a.workload, a.steps, a.warmup)
-    if w.kind == "prefill":
+    if w.kind == "mla":
+        metric, unit, value = "MLA decode attention TFLOP/s, 1 MI355X", "TFLOP/s", w.flops / (ms * 1e-3) / 1e12
+    elif w.kind == "prefill":
         metric, unit, value = "prefill attention TFLOP/s (causal flops), 1 MI355X", "TFLOP/s", w.flops / (ms * 1e-3) / 1e12
     else:
         metric, unit, value = "decode attention HBM GB/s (algorithmic KV bytes), 1 MI355X", "GB/s", w.bytes / (ms * 1e-3) / 1e9
@@ -215,13 +237,13 @@ def main():
     del w
     if not a.no_extra:
         others = {}
-        for name in ("decode32k", "decode4k", "decode128k_q8", "verify64k", "prefill8k"):
+        for name in ("decode32k", "decode4k", "decode128k_q8", "verify64k", "mla32k", "prefill8k"):
             if name == a.workload:
                 continue
             ww, m2, k2, g2 = run(name, max(10, a.steps), a.warmup)
             r = roofline(ww, k2)
-            others[name] = {"ms_per_step": round(m2, 5), "step_" + ("TFLOP/s" if ww.kind == "prefill" else "GB/s"):
-                            round((ww.flops / (m2 * 1e-3) / 1e12) if ww.kind == "prefill" else (ww.bytes / (m2 * 1e-3) / 1e9), 2), "roofline": r,
+            others[name] = {"ms_per_step": round(m2, 5), "step_" + ("TFLOP/s" if ww.kind != "decode" else "GB/s"):
+                            round((ww.flops / (m2 * 1e-3) / 1e12) if ww.kind != "decode" else (ww.bytes / (m2 * 1e-3) / 1e9), 2), "roofline": r,
                             "merge_kernel_us": round(g2 / 1e3, 2)}
             del ww
         line["others"] = others

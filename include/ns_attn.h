@@ -1,10 +1,10 @@
 /* ns_attn.h - the LLM attention path of libnextsycl-llm.so on one AMD MI355X (gfx950): KV-cache stores, split-K decode
- * (one row, or the few rows of a speculative verify pass), causal flash-attention prefill, absorbed MLA decode.
+ * (one row, or the few rows of a speculative verify pass), causal flash-attention prefill. (MLA: ns_mla.h.)
  *
- * The entry points named ns_q35_*, ns_mg_*, ns_ds2_*, ns_llm_minimaxm3_*, ns_mla_*, ns_to_q8row are the ones the
+ * The entry points named ns_q35_*, ns_mg_*, ns_llm_minimaxm3_* are the ones the
  * reference engines bind by name (llm/<arch>/src/ffi.rs) - same names, argument order, layouts and error behaviour, so
  * an engine's ffi table resolves against this library unchanged. Each declaration cites the reference interface it
- * replaces. The ns_attn_* / ns_mla_decode_latent entry points are this library's own: the same operations with typed
+ * replaces. The ns_attn_* entry points are this library's own: the same operations with typed
  * (f32 / f16 / bf16) query and output rows, any G = Hq / Hkv, either cache layout and a bfloat16 cache form.
  *
  * Conventions (reference: kernels/llm/qwen35/q35.h:1-4): rows q/out are [T][Hq*D]; row t sits at absolute position
@@ -123,7 +123,7 @@ int ns_mg_attn(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_
                int64_t win, int causal, float* out, float* scratch);
 /* GQA over a position-major half cache [position][G][128], q [T][H][128], explicit scale; dense (sel must be NULL).
  * Replaces: kernels/llm/minimaxm3/mm3.h:33-37 (mm3.cpp:118-190). Needs scratch: this library keeps
- * ns_attn_decode_scratch(T, H, G, 128, pos0, 0) floats per ns_gpu for it (allocated at ns_gpu_open, 16 MiB) */
+ * ns_attn_decode_scratch(T, H, G, 128, pos0, 0) floats per ns_gpu for it (allocated at ns_gpu_open, 64 MiB) */
 int ns_llm_minimaxm3_attend(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
                             int64_t H, int64_t G, int64_t pos0, float scale);
 

@@ -1,0 +1,56 @@
+/* ns_mla.h - multi-head latent attention (DeepSeek-V3 / R1's absorbed form, GLM-5.3's latent-only form) of
+ * libnextsycl-llm.so on one AMD MI355X (gfx950). Conventions as ns_attn.h: everything queued on the ns_gpu's compute
+ * stream, 0 or -1 with the reason in ns_last_error(), the caller owns every buffer.
+ *
+ * The latent cache (reference: kernels/llm/deepseek2/ds2.h:28-31): one row a position, shared by all heads,
+ *   DeepSeek   [512 latent | 64 rope-rotated key] half         1152 bytes
+ *   GLM        [512 latent] half                               1024 bytes
+ *   GLM q8     [16 half scales][512 int8]                       544 bytes   (kernels/llm/glm5next/glm.cpp:1074-1077)
+ * Row t of a pass sits at position pos0 + t and reads cells 0 .. pos0 + t.
+ */
+#ifndef NS_MLA_H
+#define NS_MLA_H
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ns_gpu ns_gpu;
+
+/* The absorbed decode up to the latent sum (BASELINE's MLA configuration ends here): qa [T][H][512 + R] already absorbed
+ * and rotated ([k_b q_nope | q_pe]), element type qt (0 float32, 1 half); cache rows [512 + R] half; u [T][H][512] of
+ * type qt = softmax_i(scale qa . c_i) c_i[:512]. R 64 or 0; T 1..16. `scratch`: ns_mla_decode_latent_scratch floats.
+ * This library's own entry point (the reference computes u inside ns_ds2_mla_decode / ns_mla_attend_sel) */
+int64_t ns_mla_decode_latent_scratch(int64_t T, int64_t H, int64_t pos0);
+int ns_mla_decode_latent(ns_gpu* g, int qt, const void* qa, const uint16_t* cache, void* u, int64_t T, int64_t H, int64_t R, int64_t pos0,
+                         float scale, float* scratch);
+
+/* MLA at decode widths in one call: q [T][H][128 nope + 64 rope] (rope part rotated), k_b [H][512][128] and v_b
+ * [H][128][512] half, cache [n][576] half -> out [T][H][128] = v_b u. Runs absorb, the latent decode and the value
+ * up-projection; its scratch is the library's own (kept per ns_gpu, 64 MiB). Replaces:
+ * kernels/llm/deepseek2/ds2.h:32-37 (ds2.cpp:139-258, 262-270) */
+int ns_ds2_mla_decode(ns_gpu* g, const float* q, const uint16_t* kb, const uint16_t* vb, const uint16_t* cache, float* out, int64_t T, int64_t H,
+                      int64_t pos0, float scale);
+/* The latent cache's rows pos0 .. pos0 + T - 1 from kv [T][L + R] float32: the first L RMS-normed with w (eps), the last
+ * R rotated by ggml's YaRN rope on adjacent pairs. Replaces: kernels/llm/deepseek2/ds2.h:28-31 (ds2.cpp:85-112) */
+int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint16_t* cache, int64_t T, int64_t L, int64_t R, int64_t pos0,
+                    float freq_base, float freq_scale, float ext_factor, float mscale, float corr0, float corr1);
+
+/* GLM-5.3's latent-only MLA over a half cache [n][512]: qa [T][H][512] float32 -> u [T][H][512] float32. Dense rows
+ * only: sel and sel_cnt must be NULL (the sparse cell selection is not built). Replaces:
+ * kernels/llm/glm5next/glm.h:65-66 (glm.cpp:1252-1264) */
+int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
+                      const int32_t* sel, const int32_t* sel_cnt, int64_t K);
+/* the same over q8 latent rows, at most 8 rows. Replaces: kernels/llm/glm5next/glm.h:79-80 (glm.cpp:1267-1276) */
+int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
+                         const int32_t* sel, const int32_t* sel_cnt, int64_t K);
+/* rows x [n][512] float32 -> q8 latent rows y [n][544]: a block's scale amax / 127 rounded to half BEFORE the values are
+ * divided by it, round half away from zero, clamp to +-127. Replaces: kernels/llm/glm5next/glm.h:77 (glm.cpp:1282-1299) */
+int ns_to_q8row(ns_gpu* g, const float* x, void* y, int64_t n, int64_t L);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

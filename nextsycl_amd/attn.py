@@ -60,12 +60,24 @@ ATTN_H = {
 }
 
 
+# include/ns_mla.h
+MLA_H = {
+    "ns_mla_decode_latent_scratch": (i64, [i64, i64, i64]),
+    "ns_mla_decode_latent": (i32, [P, i32, P, P, P, i64, i64, i64, i64, f32, P]),
+    "ns_ds2_mla_decode": (i32, [P, P, P, P, P, P, i64, i64, i64, f32]),
+    "ns_ds2_kv_store": (i32, [P, P, P, f32, P, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32]),
+    "ns_mla_attend_sel": (i32, [P, P, P, P, i64, i64, i64, i64, f32, P, P, i64]),
+    "ns_mla_attend_sel_q8": (i32, [P, P, P, P, i64, i64, i64, i64, f32, P, P, i64]),
+    "ns_to_q8row": (i32, [P, P, P, i64, i64]),
+}
+
+
 class Kernels:
     """Every attention entry point bound by name; a missing symbol fails the load."""
 
     def __init__(self, a=None):
         self.api = a or api()
-        for name, (res, args) in ATTN_H.items():
+        for name, (res, args) in list(ATTN_H.items()) + list(MLA_H.items()):
             setattr(self, name[3:], self.api.symbol(name, res, args))
 
 
@@ -235,6 +247,48 @@ class Ops:
             _need(scratch, self.k.q35_attn_scratch(T, Hq, Hkv, D, p0) * 4, "attention scratch")
         self.ok(self.k.q35_attn(self.raw(), q.ptr, qs, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, out.ptr,
                                 scratch.ptr if scratch is not None else None), "attention")
+
+    # ---- MLA (include/ns_mla.h; wrappers as llm/deepseek2/src/ops.rs:409-445)
+    def mla_latent_scratch(self, T, H, pos0):
+        return self.k.mla_decode_latent_scratch(T, H, pos0)
+
+    def mla_decode_latent(self, qt, qa, cache, u, T, H, R, pos0, scale, scratch):
+        """qa [T][H][512 + R] (absorbed) over the cache's cells 0 .. pos0 + T - 1 -> u [T][H][512]."""
+        e = ELT[qt]
+        _need(qa, T * H * (512 + R) * e, "mla_decode_latent qa")
+        _need(cache, (pos0 + T) * (512 + R) * 2, "mla_decode_latent cache")
+        _need(u, T * H * 512 * e, "mla_decode_latent u")
+        _need(scratch, self.mla_latent_scratch(T, H, pos0) * 4, "mla_decode_latent scratch")
+        self.ok(self.k.mla_decode_latent(self.raw(), qt, qa.ptr, cache.ptr, u.ptr, T, H, R, pos0, scale, scratch.ptr), "mla_decode_latent")
+
+    def mla_decode(self, q, kb, vb, cache, out, T, H, pos0, scale):
+        """ns_ds2_mla_decode: q [T][H][192], k_b / v_b half, cache half [.., 576] -> out [T][H][128]."""
+        _need(q, T * H * 192 * 4, "mla_decode q")
+        _need(kb, H * 512 * 128 * 2, "mla_decode k_b")
+        _need(vb, H * 128 * 512 * 2, "mla_decode v_b")
+        _need(cache, (pos0 + T) * 576 * 2, "mla_decode cache")
+        _need(out, T * H * 128 * 4, "mla_decode out")
+        self.ok(self.k.ds2_mla_decode(self.raw(), q.ptr, kb.ptr, vb.ptr, cache.ptr, out.ptr, T, H, pos0, scale), "mla_decode")
+
+    def ds2_kv_store(self, kv, w, eps, cache, T, L, R, pos0, freq_base, freq_scale, ext_factor, mscale, corr0, corr1):
+        _need(kv, T * (L + R) * 4, "kv_store kv")
+        _need(w, L * 4, "kv_store w")
+        _need(cache, (pos0 + T) * (L + R) * 2, "kv_store cache")
+        self.ok(self.k.ds2_kv_store(self.raw(), kv.ptr, w.ptr, eps, cache.ptr, T, L, R, pos0, freq_base, freq_scale, ext_factor, mscale, corr0, corr1),
+                "kv_store")
+
+    def mla_attend(self, qa, c, u, T, H, L, pos0, scale, q8=False):
+        """GLM's latent-only MLA (dense): ns_mla_attend_sel / ns_mla_attend_sel_q8 with no selection."""
+        _need(qa, T * H * L * 4, "mla_attend qa")
+        _need(c, (pos0 + T) * ((L // 32 * 2 + L) if q8 else 2 * L), "mla_attend cache")
+        _need(u, T * H * L * 4, "mla_attend u")
+        f = self.k.mla_attend_sel_q8 if q8 else self.k.mla_attend_sel
+        self.ok(f(self.raw(), qa.ptr, c.ptr, u.ptr, T, H, L, pos0, scale, None, None, 0), "mla_attend")
+
+    def to_q8row(self, x, y, n, L):
+        _need(x, n * L * 4, "to_q8row x")
+        _need(y, n * (L // 32 * 2 + L), "to_q8row y")
+        self.ok(self.k.to_q8row(self.raw(), x.ptr, y.ptr, n, L), "to_q8row")
 
     def minimaxm3_attend(self, q, kc, vc, out, T, H, G, pos0, scale):
         _need(q, T * H * 128 * 4, "attend q")

@@ -1,0 +1,544 @@
+// mla.hip: DeepSeek-style absorbed MLA decode over the latent cache for gfx950, and its neighbours: the absorb (q~ = k_b
+// q_nope), the value up-projection (out = v_b u), the latent cache store (RMS norm + YaRN rope) and GLM's q8 latent rows.
+//
+// The absorbed decode is one dense contraction per cell tile with "the key is the value": every head scores a cell with
+// its 512 latent + 64 rope features and then accumulates the same 512 latent features. Per cell: H x (576 + 512) x 2
+// flops against 1152 bytes - ~240 flop/byte at H = 128: the kernel is MFMA-bound and is built so that a cell is read
+// from HBM once for ALL heads.
+//
+// Work split: grid (cell split, row group). A work-group of 8 waves owns 128 (row, head) pairs - one decode row's 128
+// heads - a wave 16 of them (one 16-row MFMA tile: 72 registers of queries, 128 of accumulators), and a split of the
+// cells in 32-cell tiles. A tile is fetched by all 512 threads (16-byte chunks, global -> registers one tile ahead ->
+// LDS, two LDS buffers, one barrier a tile; GLM's q8 rows are widened to half on the way) and shared by the 8 waves. LDS rows are 72 chunks; chunk c of row r sits at
+// position c ^ g(r), g(r) = 2 ((r >> 1) & 3) | ((r >> 3) & 1), which spreads both access patterns over the banks: 16
+// rows x 16 bytes of one column (the score product's operand) and 8 rows x 32 bytes (the transposing read).
+//
+// A wave's tile step (transposed orientation: a lane owns one row of each row tile):
+//   S^T[cell][row] = C Q^T          A = cache rows from LDS (ds_read_b128), B = absorbed queries, in registers
+//   base-2 online softmax in float32 (scale folded in), causal edge masked per row
+//   P^T -> half = the B operand of the second product
+//   O^T[latent][row] += C^T P^T     A = the same tile through ds_read_b64_tr_b16; 128 float32 accumulators a lane
+// Each wave owns its rows outright, so a split's partial {O[L], m (log2 units), l} goes from registers to scratch
+// [row][split][L + 4]; the splits are merged by a second kernel.
+//
+// Reference behaviour kept: kernels/llm/deepseek2/ds2.cpp:139-258 (q~, scores over [latent | rope] x scale, online
+// softmax, u = sum p c / sum p, out = v_b u; L 512, R 64, nope = V = 128), :85-112 (cache rows), and
+// kernels/llm/glm5next/glm.cpp:1079-1186,1282-1299 (latent-only MLA, q8 rows [16 half scales][512 int8]).
+#include "ns_internal.hpp"
+#include "ns_mla.h"
+#include "attn_common.hpp"
+#include "kv_formats.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
+
+namespace {
+
+constexpr int MW = 8, MTILE = 32, MROWS = 128, ML = 512;
+constexpr int PSTRIDE = ML + 4;   // floats a partial: O[512], m, l, 2 of padding (rows stay 16-byte aligned)
+
+struct MlaParams {
+    const void* qa;      // [T][H][L + R] absorbed queries
+    int qt;              // 0 float32, 1 half
+    const uint8_t* cache;
+    int T, H;
+    int64_t pos0;
+    int64_t kbs;         // cells a split
+    int ns;
+    float sl2;
+    float* part;         // [T * H][ns][PSTRIDE]
+};
+
+__device__ __forceinline__ int swz(int r) { return (((r >> 1) & 3) << 1) | ((r >> 3) & 1); }
+
+// R: rope features (64: DeepSeek's [512 | 64] rows; 0: GLM's latent-only rows); Q8: GLM's q8 rows
+template <int R, bool Q8>
+__global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams p) {
+    constexpr int DK = ML + R, KB = DK / 32, DT = ML / 16;
+    constexpr int RSTRIDE = 72 * 16;                     // bytes a staged row (72 chunks, whatever DK)
+    constexpr int TILEB = MTILE * RSTRIDE;
+    constexpr int64_t CROW = Q8 ? ML / 32 * 2 + ML : DK * 2;   // bytes a cache row
+    constexpr int CPR = Q8 ? ML / 16 : DK / 8;           // 16-byte loads a cache row
+    constexpr int NCH = MTILE * CPR;                     // loads a tile
+    constexpr int NLD = (NCH + MW * 64 - 1) / (MW * 64); // loads a thread per tile (the last may be idle)
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * TILEB];
+
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int split = blockIdx.x, z = blockIdx.y;
+    const int rows = p.T * p.H;
+    const int64_t n_all = p.pos0 + p.T;                                  // cells the pass's last row sees
+    const int64_t jb = (int64_t) split * p.kbs, je = std::min(jb + p.kbs, n_all);
+
+    // ---- this lane's row
+    const int ri = z * MROWS + w * 16 + n;
+    const bool live = ri < rows;
+    const int rr = live ? ri : rows - 1;
+    const int64_t hi_r = live ? std::min(p.pos0 + rr / p.H, je - 1) : -1;
+    s8v qreg[KB];
+    {
+        const int64_t qoff = (int64_t) rr * DK + g4 * 8;
+        if (p.qt == 0) {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const float4 a = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.qa) + qoff + kb * 32);
+                const float4 b = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.qa) + qoff + kb * 32 + 4);
+                const float f[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) qreg[kb][i] = live ? to16<false>(f[i]) : (short) 0;
+            }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const s8v raw = *reinterpret_cast<const s8v*>(reinterpret_cast<const uint16_t*>(p.qa) + qoff + kb * 32);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) qreg[kb][i] = live ? raw[i] : (short) 0;
+            }
+        }
+    }
+    float m_r = -INFINITY, l_r = 0.0f;
+    f4v o[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+
+    // ---- tile traffic: chunk id = tid + 512 i -> row id / CPR, piece id % CPR; cells past the split's end are clamped
+    // to its last (a valid row; their scores are masked)
+    uint4 st[NLD];
+    uint16_t stsc[Q8 ? NLD : 1];
+    auto fetch = [&](int64_t j0) {
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int id = tid + MW * 64 * i, r = id / CPR, c = id % CPR;
+            if (NCH % (MW * 64) != 0 && id >= NCH) continue;
+            const uint8_t* row = p.cache + std::min(j0 + r, je - 1) * CROW;
+            if constexpr (Q8) {
+                st[i] = *reinterpret_cast<const uint4*>(row + ML / 32 * 2 + c * 16);
+                stsc[i] = *reinterpret_cast<const uint16_t*>(row + 2 * (c / 2));
+            } else {
+                st[i] = *reinterpret_cast<const uint4*>(row + c * 16);
+            }
+        }
+    };
+    auto stash = [&](int buf) {
+        uint8_t* base = lds + buf * TILEB;
+#pragma unroll
+        for (int i = 0; i < NLD; ++i) {
+            const int id = tid + MW * 64 * i, r = id / CPR, c = id % CPR;
+            if (NCH % (MW * 64) != 0 && id >= NCH) continue;
+            if constexpr (Q8) {
+                // 16 int8 x one half scale -> 16 halfs = chunks 2c, 2c + 1; value = half(scale) x q, one rounding to
+                // half (the reference widens half(scale) x q in float32: kernels/llm/glm5next/glm.cpp:1116-1124)
+                const _Float16 d = __builtin_bit_cast(_Float16, stsc[i]);
+                const uint32_t ww[4] = {st[i].x, st[i].y, st[i].z, st[i].w};
+                s8v a, b;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const _Float16 x0 = (_Float16) (short) (int8_t) (ww[e >> 2] >> (8 * (e & 3))) * d;
+                    const _Float16 x1 = (_Float16) (short) (int8_t) (ww[2 + (e >> 2)] >> (8 * (e & 3))) * d;
+                    a[e] = __builtin_bit_cast(short, x0);
+                    b[e] = __builtin_bit_cast(short, x1);
+                }
+                *reinterpret_cast<s8v*>(base + r * RSTRIDE + ((2 * c) ^ swz(r)) * 16) = a;
+                *reinterpret_cast<s8v*>(base + r * RSTRIDE + ((2 * c + 1) ^ swz(r)) * 16) = b;
+            } else {
+                *reinterpret_cast<uint4*>(base + r * RSTRIDE + (c ^ swz(r)) * 16) = st[i];
+            }
+        }
+    };
+
+    const int64_t nt = jb < je ? (je - jb + MTILE - 1) / MTILE : 0;
+    if (nt > 0) {
+        fetch(jb);
+        stash(0);
+    }
+    __syncthreads();
+    for (int64_t it = 0; it < nt; ++it) {
+        const int buf = (int) (it & 1);
+        const int64_t j0 = jb + it * MTILE;
+        if (it + 1 < nt) fetch(j0 + MTILE);
+        uint8_t* tile = lds + buf * TILEB;
+        // ---- S^T = C Q^T
+        f4v s[2];
+#pragma unroll
+        for (int ct = 0; ct < 2; ++ct) {
+            const int r = ct * 16 + n;
+            f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const s8v a = *reinterpret_cast<const s8v*>(tile + r * RSTRIDE + ((kb * 4 + g4) ^ swz(r)) * 16);
+                acc = mfma16<false>(a, qreg[kb], acc);
+            }
+            s[ct] = acc;
+        }
+        // ---- softmax of this lane's row
+        s8v pb;
+        {
+            float x[8], mx = -INFINITY;
+#pragma unroll
+            for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int64_t j = j0 + ct * 16 + g4 * 4 + i;
+                    const float v = j <= hi_r ? s[ct][i] * p.sl2 : -INFINITY;
+                    x[ct * 4 + i] = v;
+                    mx = fmaxf(mx, v);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float mn = fmaxf(m_r, mx);
+            const float c = mn == -INFINITY ? 1.0f : fast_exp2(m_r - mn);
+            float sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float pv = x[e] == -INFINITY ? 0.0f : fast_exp2(x[e] - mn);
+                sum += pv;
+                pb[e] = to16<false>(pv);
+            }
+            sum += __shfl_xor(sum, 16);
+            sum += __shfl_xor(sum, 32);
+            m_r = mn;
+            l_r = l_r * c + sum;
+            // the 128 accumulators are rescaled only when some row's maximum moved
+            if (__any(c != 1.0f)) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o[dt] *= c;
+            }
+        }
+        // ---- O^T += C^T P^T
+        const int kk = g4 * 4 + (n >> 2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            const int c = (dt * 2 + ((n & 3) >> 1)) ^ swz(kk);    // swz(kk + 16) == swz(kk)
+            uint8_t* src = tile + kk * RSTRIDE + c * 16 + (n & 1) * 8;
+            const s4v lo = lds_read_tr16(src), hi = lds_read_tr16(src + 16 * RSTRIDE);
+            const s8v va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            o[dt] = mfma16<false>(va, pb, o[dt]);
+        }
+        if (it + 1 < nt) stash(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- the split's partial, straight from the registers: a lane holds latents 16 dt + 4 g4 .. + 3 of its row
+    if (live) {
+        float* pr = p.part + ((int64_t) ri * p.ns + split) * PSTRIDE;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f4v*>(pr + dt * 16 + g4 * 4) = o[dt];
+        if (g4 == 0) {
+            pr[ML] = m_r;
+            pr[ML + 1] = l_r;
+        }
+    }
+}
+
+// the splits of a row merged: u = sum O_s 2^(m_s - M) / sum l_s 2^(m_s - M); a work-group of 512 threads a row
+template <int QT>
+__global__ __launch_bounds__(ML) void mla_merge_kernel(const float* __restrict__ part, int ns, void* __restrict__ u) {
+    __shared__ float wsh[1024];
+    __shared__ float red[ML];
+    const int64_t row = blockIdx.x;
+    const int tid = threadIdx.x;
+    const float* pr = part + row * ns * PSTRIDE;
+    float mx = -INFINITY;
+    for (int s = tid; s < ns; s += ML) mx = fmaxf(mx, pr[s * PSTRIDE + ML]);
+    red[tid] = mx;
+    __syncthreads();
+    for (int o = ML / 2; o > 0; o >>= 1) {
+        if (tid < o) red[tid] = fmaxf(red[tid], red[tid + o]);
+        __syncthreads();
+    }
+    mx = red[0];
+    __syncthreads();
+    float ls = 0.0f;
+    for (int s = tid; s < ns; s += ML) {
+        const float m = pr[s * PSTRIDE + ML];
+        const float wgt = m == -INFINITY ? 0.0f : fast_exp2(m - mx);
+        wsh[s] = wgt;
+        ls += pr[s * PSTRIDE + ML + 1] * wgt;
+    }
+    red[tid] = ls;
+    __syncthreads();
+    for (int o = ML / 2; o > 0; o >>= 1) {
+        if (tid < o) red[tid] += red[tid + o];
+        __syncthreads();
+    }
+    const float L = red[0];
+    float acc = 0.0f;
+#pragma unroll 8
+    for (int s = 0; s < ns; ++s) acc += pr[s * PSTRIDE + tid] * wsh[s];
+    store_o<QT>(u, row * ML + tid, L > 0.0f ? acc / L : 0.0f);
+}
+
+// q~ = k_b q_nope: qa [T][H][L + R] = [k_b[h] q[t][h][:nope] | q[t][h][nope:]]; a work-group a (row, head), a thread two
+// latent rows of k_b (kernels/llm/deepseek2/ds2.cpp:176-184)
+__global__ __launch_bounds__(256) void mla_absorb_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kb, float* __restrict__ qa,
+                                                         int64_t H) {
+    constexpr int NOPE = 128, R = 64;
+    __shared__ float qs[NOPE + R];
+    const int64_t th = blockIdx.x, h = th % H;
+    const int tid = threadIdx.x;
+    if (tid < NOPE + R) qs[tid] = q[th * (NOPE + R) + tid];
+    __syncthreads();
+    for (int r = tid; r < ML; r += 256) {
+        const uint4* wr = reinterpret_cast<const uint4*>(kb + ((size_t) h * ML + r) * NOPE);
+        float a = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NOPE / 8; ++c) {
+            const uint4 x = wr[c];
+            const uint32_t ww[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a += f16_to_f32((uint16_t) (ww[e >> 1] >> (16 * (e & 1)))) * qs[c * 8 + e];
+        }
+        qa[th * (ML + R) + r] = a;
+    }
+    if (tid < R) qa[th * (ML + R) + ML + tid] = qs[NOPE + tid];
+}
+
+// out [T][H][V] = v_b u: a work-group a (row, head), a wave a value row at a time (kernels/llm/deepseek2/ds2.cpp:237-255)
+__global__ __launch_bounds__(256) void mla_vb_kernel(const float* __restrict__ u, const uint16_t* __restrict__ vb, float* __restrict__ out,
+                                                     int64_t H) {
+    constexpr int V = 128;
+    __shared__ float us[ML];
+    const int64_t th = blockIdx.x, h = th % H;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    for (int i = tid; i < ML; i += 256) us[i] = u[th * ML + i];
+    __syncthreads();
+    for (int r = w; r < V; r += 4) {
+        const uint4 x = reinterpret_cast<const uint4*>(vb + ((size_t) h * V + r) * ML)[lane];
+        const uint32_t ww[4] = {x.x, x.y, x.z, x.w};
+        float a = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a += f16_to_f32((uint16_t) (ww[e >> 1] >> (16 * (e & 1)))) * us[lane * 8 + e];
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) a += __shfl_xor(a, o);
+        if (lane == 0) out[th * V + r] = a;
+    }
+}
+
+// ggml's rope_yarn angle of pair i0 (kernels/llm/deepseek2/ds2.cpp:15-34): the angle by repeated products, as it does
+__device__ float yarn_ramp(float low, float high, int i0) {
+    const float y = ((float) (i0 / 2) - low) / fmaxf(0.001f, high - low);
+    return 1.0f - fminf(1.0f, fmaxf(0.0f, y));
+}
+__device__ void yarn_cs(float pos, int i0, int n_dims, float freq_base, float freq_scale, float ext_factor, float mscale, float corr0, float corr1,
+                        float& c, float& s) {
+    const float theta_scale = powf(freq_base, -2.0f / (float) n_dims);
+    float theta_extrap = pos;
+    for (int k = 0; k < i0 / 2; ++k) theta_extrap *= theta_scale;
+    const float theta_interp = freq_scale * theta_extrap;
+    float theta = theta_interp;
+    if (ext_factor != 0.0f) {
+        const float ramp_mix = yarn_ramp(corr0, corr1, i0) * ext_factor;
+        theta = theta_interp * (1 - ramp_mix) + theta_extrap * ramp_mix;
+    }
+    c = cosf(theta) * mscale;
+    s = sinf(theta) * mscale;
+}
+
+// the latent cache's rows pos0..: [RMSnorm(kv[:L]) w | YaRN-rope(kv[L:L+R])] as half; a work-group a row
+__global__ __launch_bounds__(256) void ds2_kv_store_kernel(const float* __restrict__ kv, const float* __restrict__ wgt, float eps,
+                                                           uint16_t* __restrict__ cache, int64_t L, int64_t R, int64_t pos0, float freq_base,
+                                                           float freq_scale, float ext_factor, float mscale, float corr0, float corr1) {
+    __shared__ float red[256];
+    const int64_t t = blockIdx.x;
+    const int tid = threadIdx.x;
+    const float* xr = kv + t * (L + R);
+    float ss = 0.0f;
+    for (int64_t i = tid; i < L; i += 256) ss += xr[i] * xr[i];
+    red[tid] = ss;
+    __syncthreads();
+    for (int o = 128; o > 0; o >>= 1) {
+        if (tid < o) red[tid] += red[tid + o];
+        __syncthreads();
+    }
+    const float inv = 1.0f / sqrtf(red[0] / (float) L + eps);
+    uint16_t* o = cache + (pos0 + t) * (L + R);
+    for (int64_t i = tid; i < L; i += 256) o[i] = f32_to_f16(xr[i] * inv * wgt[i]);
+    for (int64_t i = tid; i < R / 2; i += 256) {
+        const int i0 = (int) (2 * i);
+        float c, s;
+        yarn_cs((float) (pos0 + t), i0, (int) R, freq_base, freq_scale, ext_factor, mscale, corr0, corr1, c, s);
+        const float x0 = xr[L + i0], x1 = xr[L + i0 + 1];
+        o[L + i0] = f32_to_f16(x0 * c - x1 * s);
+        o[L + i0 + 1] = f32_to_f16(x0 * s + x1 * c);
+    }
+}
+
+// GLM's q8 latent rows: a wave a row, a lane... 16 lanes a row, a lane a block of 32: the scale rounded to half BEFORE it
+// divides, clamp to +-127 (kernels/llm/glm5next/glm.cpp:1282-1299)
+__global__ __launch_bounds__(256) void to_q8row_kernel(const float* __restrict__ x, uint8_t* __restrict__ y, int64_t n) {
+    const int64_t gi = (int64_t) blockIdx.x * 256 + threadIdx.x, r = gi / 16;
+    const int b = (int) (gi % 16);
+    if (r >= n) return;
+    const float* xr = x + r * ML + b * 32;
+    float v[32], amax = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 32; e += 4) {
+        const float4 f = *reinterpret_cast<const float4*>(xr + e);
+        v[e] = f.x; v[e + 1] = f.y; v[e + 2] = f.z; v[e + 3] = f.w;
+    }
+#pragma unroll
+    for (int e = 0; e < 32; ++e) amax = fmaxf(amax, fabsf(v[e]));
+    const uint16_t dh = f32_to_f16(amax / 127.0f);
+    const float d = f16_to_f32(dh), inv = d > 0.0f ? 1.0f / d : 0.0f;
+    uint8_t* row = y + r * (ML / 32 * 2 + ML);
+    reinterpret_cast<uint16_t*>(row)[b] = dh;
+    uint32_t* qs = reinterpret_cast<uint32_t*>(row + 32 + b * 32);
+#pragma unroll
+    for (int e = 0; e < 32; e += 4) {
+        uint32_t wv = 0;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) wv |= (uint32_t) (uint8_t) (int8_t) fminf(127.0f, fmaxf(-127.0f, roundf(v[e + k] * inv))) << (8 * k);
+        qs[e / 4] = wv;
+    }
+}
+
+// ---- host side --------------------------------------------------------------------------------------------------------
+
+int64_t mla_target_wgs() {
+    static const int64_t v = [] {
+        const char* e = getenv("NS_MLA_WGS");
+        const int64_t x = e ? atoll(e) : 0;
+        return x > 0 ? x : 256;
+    }();
+    return v;
+}
+// cells a split: ~mla_target_wgs() work-groups over the pass, whole 32-cell tiles, at least 2 tiles
+int64_t mla_kbs(int64_t cells, int64_t groups) {
+    const int64_t t = mla_target_wgs(), want = (cells * groups + t - 1) / t;
+    return std::max<int64_t>(2 * MTILE, (want + MTILE - 1) / MTILE * MTILE);
+}
+
+int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const void* qa, const void* cache, void* u, int64_t T, int64_t H,
+               int64_t pos0, float scale, float* scratch, size_t scratch_floats) {
+    const std::string w(who);
+    if (T <= 0) return 0;
+    if (H <= 0 || pos0 < 0) return ns_fail(w + ": heads and a position");
+    if (T > 16) return ns_fail(w + ": 1..16 rows (decode widths)");
+    if (!qa || !cache || !u || !scratch) return ns_fail(w + ": a null buffer");
+    if (((uintptr_t) qa | (uintptr_t) cache | (uintptr_t) scratch) % 16) return ns_fail(w + ": buffers 16-byte aligned");
+    if (!(scale > 0.0f)) return ns_fail(w + ": a positive scale");
+    NS_HIP(hipSetDevice(g->dev));
+    const int64_t rows = T * H, nz = (rows + MROWS - 1) / MROWS, cells = pos0 + T;
+    int64_t kbs = mla_kbs(cells, nz), ns = (cells + kbs - 1) / kbs;
+    // a caller's scratch may be smaller than the rule asks (the library's own, for the reference-named entry points):
+    // fewer, longer splits then
+    while ((size_t) (rows * ns * PSTRIDE) > scratch_floats && ns > 1) {
+        kbs *= 2;
+        ns = (cells + kbs - 1) / kbs;
+    }
+    if ((size_t) (rows * ns * PSTRIDE) > scratch_floats) return ns_fail(w + ": scratch too small");
+    if (ns > 1024) return ns_fail(w + ": more cell splits than the merge holds");
+    MlaParams p{};
+    p.qa = qa;
+    p.qt = qt;
+    p.cache = (const uint8_t*) cache;
+    p.T = (int) T;
+    p.H = (int) H;
+    p.pos0 = pos0;
+    p.kbs = kbs;
+    p.ns = (int) ns;
+    p.sl2 = scale * 1.4426950408889634f;
+    p.part = scratch;
+    dim3 grid((unsigned) ns, (unsigned) nz);
+    if (ns_profile_mark(g, 0)) return -1;
+    if (q8) mla_decode_kernel<0, true><<<grid, MW * 64, 0, g->q>>>(p);
+    else if (R == 64) mla_decode_kernel<64, false><<<grid, MW * 64, 0, g->q>>>(p);
+    else mla_decode_kernel<0, false><<<grid, MW * 64, 0, g->q>>>(p);
+    NS_LAUNCHED("mla_decode");
+    if (ns_profile_mark(g, 1)) return -1;
+    if (ot == 0) mla_merge_kernel<0><<<(unsigned) rows, ML, 0, g->q>>>(scratch, (int) ns, u);
+    else mla_merge_kernel<1><<<(unsigned) rows, ML, 0, g->q>>>(scratch, (int) ns, u);
+    NS_LAUNCHED("mla_merge");
+    return ns_profile_mark(g, 2);
+}
+
+}  // namespace
+
+extern "C" {
+
+int64_t ns_mla_decode_latent_scratch(int64_t T, int64_t H, int64_t pos0) {
+    if (T <= 0 || H <= 0) return 0;
+    const int64_t rows = T * H, nz = (rows + MROWS - 1) / MROWS, cells = pos0 + T, kbs = mla_kbs(cells, nz);
+    return rows * ((cells + kbs - 1) / kbs) * PSTRIDE;
+}
+
+int ns_mla_decode_latent(ns_gpu* g, int qt, const void* qa, const uint16_t* cache, void* u, int64_t T, int64_t H, int64_t R, int64_t pos0,
+                         float scale, float* scratch) {
+    NS_TRY
+    if (T <= 0) return 0;
+    if (qt != 0 && qt != 1) return ns_fail("ns_mla_decode_latent: rows of type 0 (float32) or 1 (half)");
+    if (R != 0 && R != 64) return ns_fail("ns_mla_decode_latent: a rope part of 64 (DeepSeek's [512 | 64] rows) or none");
+    return mla_latent(g, "ns_mla_decode_latent", qt, qt, (int) R, false, qa, cache, u, T, H, pos0, scale, scratch,
+                      (size_t) ns_mla_decode_latent_scratch(T, H, pos0));
+    NS_CATCH
+}
+
+int ns_ds2_mla_decode(ns_gpu* g, const float* q, const uint16_t* kb, const uint16_t* vb, const uint16_t* cache, float* out, int64_t T, int64_t H,
+                      int64_t pos0, float scale) {
+    NS_TRY
+    if (T <= 0) return 0;
+    if (H <= 0 || pos0 < 0 || T > 16) return ns_fail("ns_ds2_mla_decode: 1..16 rows, heads and a position");
+    if (!q || !kb || !vb || !cache || !out) return ns_fail("ns_ds2_mla_decode: a null buffer");
+    // the library's own scratch (the reference's signature has none): the absorbed queries, u, then the partials
+    const size_t rows = (size_t) (T * H), qa_f = (rows * (ML + 64) + 3) / 4 * 4, u_f = rows * ML;
+    if (qa_f + u_f + rows * PSTRIDE > g->own_scratch_floats) return ns_fail("ns_ds2_mla_decode: the pass needs more scratch than the library keeps");
+    float* qa = g->own_scratch;
+    float* u = qa + qa_f;
+    float* part = u + u_f;
+    NS_HIP(hipSetDevice(g->dev));
+    mla_absorb_kernel<<<(unsigned) rows, 256, 0, g->q>>>(q, kb, qa, H);
+    NS_LAUNCHED("mla_absorb");
+    if (mla_latent(g, "ns_ds2_mla_decode", 0, 0, 64, false, qa, cache, u, T, H, pos0, scale, part, g->own_scratch_floats - qa_f - u_f)) return -1;
+    mla_vb_kernel<<<(unsigned) rows, 256, 0, g->q>>>(u, vb, out, H);
+    NS_LAUNCHED("mla_vb");
+    return 0;
+    NS_CATCH
+}
+
+int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint16_t* cache, int64_t T, int64_t L, int64_t R, int64_t pos0,
+                    float freq_base, float freq_scale, float ext_factor, float mscale, float corr0, float corr1) {
+    NS_TRY
+    if (T <= 0) return 0;
+    if (R % 2 != 0) return ns_fail("ns_ds2_kv_store: an even rotated width");
+    NS_HIP(hipSetDevice(g->dev));
+    ds2_kv_store_kernel<<<(unsigned) T, 256, 0, g->q>>>(kv, w, eps, cache, L, R, pos0, freq_base, freq_scale, ext_factor, mscale, corr0, corr1);
+    NS_LAUNCHED("ds2_kv_store");
+    return 0;
+    NS_CATCH
+}
+
+int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
+                      const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
+    NS_TRY
+    (void) K;
+    if (T <= 0) return 0;
+    if (L != 512) return ns_fail("ns_mla_attend_sel: latent width 512");
+    if (sel || sel_cnt) return ns_fail("ns_mla_attend_sel: the sparse cell selection is not built; pass sel = sel_cnt = NULL (dense)");
+    return mla_latent(g, "ns_mla_attend_sel", 0, 0, 0, false, qa, c, u, T, H, pos0, scale, g->own_scratch, g->own_scratch_floats);
+    NS_CATCH
+}
+
+int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
+                         const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
+    NS_TRY
+    (void) K;
+    if (T <= 0) return 0;
+    if (L != 512 || T > 8) return ns_fail("ns_mla_attend_sel_q8: latent width 512, at most 8 rows");
+    if (sel || sel_cnt) return ns_fail("ns_mla_attend_sel_q8: the sparse cell selection is not built; pass sel = sel_cnt = NULL (dense)");
+    return mla_latent(g, "ns_mla_attend_sel_q8", 0, 0, 0, true, qa, c, u, T, H, pos0, scale, g->own_scratch, g->own_scratch_floats);
+    NS_CATCH
+}
+
+int ns_to_q8row(ns_gpu* g, const float* x, void* y, int64_t n, int64_t L) {
+    NS_TRY
+    if (n <= 0) return 0;
+    if (L != 512) return ns_fail("ns_to_q8row: latent width 512");
+    NS_HIP(hipSetDevice(g->dev));
+    to_q8row_kernel<<<(unsigned) ((n * 16 + 255) / 256), 256, 0, g->q>>>(x, (uint8_t*) y, n);
+    NS_LAUNCHED("to_q8row");
+    return 0;
+    NS_CATCH
+}
+
+}  // extern "C"

@@ -7,7 +7,7 @@
 namespace {
 thread_local std::string g_err;
 constexpr size_t EV_RING = 1 << 16;
-constexpr size_t OWN_SCRATCH_FLOATS = (size_t) 4 << 20;   // 16 MiB
+constexpr size_t OWN_SCRATCH_FLOATS = (size_t) 16 << 20;   // 64 MiB
 
 int bad_index(int index, int n) { return ns_fail("no GPU " + std::to_string(index) + " (" + std::to_string(n) + " found)"); }
 

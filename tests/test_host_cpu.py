@@ -7,7 +7,7 @@ import re
 import pytest
 
 from nextsycl_amd import Error, library_path
-from nextsycl_amd.attn import ATTN_H, kv_row_bytes
+from nextsycl_amd.attn import ATTN_H, MLA_H, kv_row_bytes
 from nextsycl_amd.sys import NS_H
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -29,13 +29,14 @@ def _declared(header):
 
 
 def test_library_exports_every_declared_symbol(handle):
-    declared = _declared("ns.h") | _declared("ns_attn.h")
+    declared = _declared("ns.h") | _declared("ns_attn.h") | _declared("ns_mla.h")
     assert len(_declared("ns.h")) == 26                      # the reference's 26 (kernels/ns/ns.h:18-56)
     missing = [n for n in sorted(declared) if not hasattr(handle, n)]
     assert not missing, missing
     # and the host tables bind exactly the declared set
     assert set(NS_H) == _declared("ns.h")
     assert set(ATTN_H) == _declared("ns_attn.h")
+    assert set(MLA_H) == _declared("ns_mla.h")
 
 
 def test_pure_functions_without_a_gpu(handle):
@@ -54,6 +55,9 @@ def test_pure_functions_without_a_gpu(handle):
     p = handle.ns_mg_attn_prompt_supported
     p.restype, p.argtypes = C.c_int, [C.c_int64] * 4
     assert p(17, 64, 4, 128) == 1 and p(16, 64, 4, 128) == 0 and p(100, 64, 4, 256) == 0
+    m = handle.ns_mla_decode_latent_scratch
+    m.restype, m.argtypes = C.c_int64, [C.c_int64] * 3
+    assert m(1, 128, 32767) == 128 * 256 * 516 and m(0, 128, 5) == 0     # 256 splits of 128 cells, 512 + 4 floats a partial
     handle.ns_version.restype = C.c_char_p
     assert b"gfx950" in handle.ns_version()
     handle.ns_last_error.restype = C.c_char_p
