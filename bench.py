@@ -191,6 +191,8 @@ def main():
     ap.add_argument("--workload", default="prefill8k", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the decode-side workloads of the metric")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
+                    help="first run a plain copy kernel of this many MiB 5 times (the known-size kernel rocprofv3 traffic counters are scaled against)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (the path shards by key head or by context, see DESIGN.md)" % a.gpus,
@@ -205,6 +207,16 @@ def main():
         build()
     g = Gpu.open(0)
     ops = Ops(g)
+
+    if a.copy_probe:
+        from nextsycl_amd import DevBuf
+        n = a.copy_probe << 20
+        src, dst = DevBuf(g, n), DevBuf(g, n)
+        src.fill(0x5A)
+        for _ in range(5):
+            ops.copy_probe(dst, src, n)
+        g.sync()
+        del src, dst
 
     def run(name, steps, warmup):
         kind = WORKLOADS[name][0]

@@ -134,6 +134,9 @@ int ns_llm_minimaxm3_attend(ns_gpu* g, const float* q, const uint16_t* kc, const
  * after; ns_attn_profile_last waits for the last call's and returns the two kernels' device times in nanoseconds
  * (merge_ns 0 for a call without a merge). Off by default: the events add gaps between the launches */
 int ns_attn_profile(ns_gpu* g, int on);
+/* a plain device-to-device copy kernel (16 bytes a thread, reads `bytes`, writes `bytes`): the kernel of known size that
+ * rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled against. This library's own */
+int ns_attn_copy_probe(ns_gpu* g, void* dst, const void* src, size_t bytes);
 int ns_attn_profile_last(ns_gpu* g, double* main_ns, double* merge_ns);
 
 #ifdef __cplusplus

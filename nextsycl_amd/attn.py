@@ -56,6 +56,7 @@ ATTN_H = {
     "ns_mg_attn": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, i32, P, P]),
     "ns_llm_minimaxm3_attend": (i32, [P, P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
     "ns_attn_profile": (i32, [P, i32]),
+    "ns_attn_copy_probe": (i32, [P, P, P, C.c_size_t]),
     "ns_attn_profile_last": (i32, [P, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
 }
 
@@ -121,6 +122,11 @@ class Ops:
         a, b = C.c_double(), C.c_double()
         self.ok(self.k.attn_profile_last(self.raw(), C.byref(a), C.byref(b)), "profile_last")
         return a.value, b.value
+
+    def copy_probe(self, dst, src, nbytes):
+        _need(dst, nbytes, "copy_probe dst")
+        _need(src, nbytes, "copy_probe src")
+        self.ok(self.k.attn_copy_probe(self.raw(), dst.ptr, src.ptr, nbytes), "copy_probe")
 
     # ---- caches
     def cache_bytes(self, kt, Hkv, cap, D):

@@ -128,6 +128,12 @@ __global__ void fwht32_kernel(float* __restrict__ x, int64_t rows, int64_t nb, i
     for (int j = 0; j < 32; ++j) p[j] = v[j] * 0.17677669529663687f;
 }
 
+// a plain copy, 16 bytes a thread: the known-size kernel that hardware traffic counters are calibrated against
+__global__ void copy_probe_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t n16) {
+    const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n16) dst[i] = src[i];
+}
+
 inline unsigned blocks_for(int64_t n, int per) { return (unsigned) ((n + per - 1) / per); }
 
 }  // namespace
@@ -189,6 +195,17 @@ int ns_attn_kv_dequant(ns_gpu* g, int kt, const void* rows, int64_t n, int64_t D
     NS_HIP(hipSetDevice(g->dev));
     kv_dequant_kernel<<<blocks_for(n * D, 256), 256, 0, g->q>>>(kt, (const uint8_t*) rows, n, D, stride, out);
     NS_LAUNCHED("kv_dequant");
+    return 0;
+    NS_CATCH
+}
+
+int ns_attn_copy_probe(ns_gpu* g, void* dst, const void* src, size_t bytes) {
+    NS_TRY
+    if (bytes == 0) return 0;
+    if (bytes % 16 || ((uintptr_t) dst | (uintptr_t) src) % 16) return ns_fail("ns_attn_copy_probe: a multiple of 16 bytes, 16-byte aligned");
+    NS_HIP(hipSetDevice(g->dev));
+    copy_probe_kernel<<<blocks_for((int64_t) (bytes / 16), 256), 256, 0, g->q>>>((const uint4*) src, (uint4*) dst, (int64_t) (bytes / 16));
+    NS_LAUNCHED("copy_probe");
     return 0;
     NS_CATCH
 }
