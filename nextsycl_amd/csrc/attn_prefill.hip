@@ -4,16 +4,18 @@
 // Bound: MFMA. 4 D flops a visible (row, key) pair against 2 x 2 D bytes a key shared by every row that sees it:
 // thousands of flops a byte at prompt lengths.
 //
-// Work split: grid (row block, query head). A work-group of 4 waves owns ROWS = 128 consecutive query rows of one
-// query head (a wave 32 of them: two 16-row MFMA tiles) and streams the keys its rows see in 32-key tiles, heaviest
-// row blocks first (the last block sees the most keys). The G query heads of a key head run as neighbouring
-// work-groups, so their key tiles meet in L2. A tile's K and V rows are fetched by all 256 threads (16-byte chunks,
-// global -> registers one tile ahead -> LDS, two LDS buffers, one barrier a tile).
+// Work split: one work-group per (row block, query head). A work-group of 4 waves owns ROWS = 128 consecutive query rows
+// of one query head (a wave 32 of them: two 16-row MFMA tiles) and streams the keys its rows see in 64-key tiles,
+// heaviest row blocks first (the last block sees the most keys). The G query heads of a key head on one row block are
+// neighbours in the logical order and, through the XCD-aware mapping of work-group ids, share one L2. A tile's K and V
+// rows are fetched by all 256 threads (16-byte chunks): global -> registers two tiles ahead -> LDS one tile ahead, two
+// register sets, two LDS buffers, one barrier a tile.
 //
 // A wave's tile step, in the transposed orientation (a lane owns one query row of each row tile, so the row maximum,
 // the rescale and the normalisation never leave the lane):
 //   S^T[key][row] = K Q^T        K from LDS as the A operand (ds_read_b128, rows padded to 272 bytes), Q^T in registers
-//   base-2 online softmax in float32; only tiles crossing a row's causal or window edge are masked
+//   base-2 online softmax in float32 (scale folded into the exponent's fma; the accumulators rescaled only when a
+//   row's maximum moved); only 32-key halves crossing a row's causal or window edge are masked
 //   P^T -> 16 bit = the B operand of the second product as it stands
 //   O^T[d][row]  += V^T P^T      V^T from LDS through ds_read_b64_tr_b16 (rows padded to 288 bytes)
 //
@@ -30,7 +32,7 @@
 
 namespace {
 
-constexpr int PW = 4, ROWS = 128, KT_TILE = 32;
+constexpr int PW = 4, ROWS = 128, KT_TILE = 64;
 
 struct PrefillParams {
     const void* q;
@@ -46,20 +48,32 @@ struct PrefillParams {
     void* out;
 };
 
+// one thread's share of a 64-key tile on its way from global memory to LDS: 4 chunks of K, 4 of V
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+struct Staged {
+    u4v k[4], v[4];
+};
+
 template <int D, bool BF>
 __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillParams p) {
     static_assert(D == 128, "head size 128");
     constexpr int KB = D / 32, DT = D / 16;
     constexpr int KS = D * 2 + 16, VS = D * 2 + 32;             // bytes a staged key row / value row
     constexpr int KBUF = KT_TILE * KS, VBUF = KT_TILE * VS;
-    constexpr int CH = KT_TILE * D * 2 / 16 / (PW * 64);         // 16-byte chunks a thread fetches per tile and matrix (2)
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * (KBUF + VBUF)];
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // ---- which (row block, head) this work-group owns. Consecutive work-group ids go round the 8 XCDs (each with its
+    // own L2): undo that, so that neighbours in the logical order - the G query heads of one key head on one row block,
+    // which stream the same K / V tiles - share an L2. Logical order: heaviest row blocks first.
+    const int nwg = gridDim.x, pid = blockIdx.x;
+    const int xq = nwg / 8, xr = nwg % 8, xcd = pid % 8, xi = pid / 8;
+    const int logical = (xcd < xr ? xcd * (xq + 1) : xr * (xq + 1) + (xcd - xr) * xq) + xi;
     const int nblk = (p.T + ROWS - 1) / ROWS;
-    const int blk = nblk - 1 - (int) blockIdx.x;                 // heaviest first
-    const int hq = blockIdx.y, hk = hq / p.G;
+    const int hq = logical % p.Hq;                               // heads fastest: hq / G is the key head
+    const int blk = nblk - 1 - logical / p.Hq;
+    const int hk = hq / p.G;
     const int r0 = blk * ROWS;
     const int rl = std::min(r0 + ROWS, p.T) - 1;                  // the block's last row
     const int64_t kend = p.p0 + rl + 1;                           // keys [kbeg, kend) cover every row of the block
@@ -105,7 +119,7 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
             }
         }
     }
-    // the wave's own key range: its first row's first key to its last row's last (tiles outside are skipped)
+    // the wave's own key range: its first row's first key to its last row's last (32-key halves outside are skipped)
     const int wrow0 = r0 + w * 32, wrow1 = std::min(wrow0 + 31, p.T - 1);
     const int64_t w_end = wrow0 < p.T ? p.p0 + wrow1 + 1 : 0;
     const int64_t w_beg = p.win > 0 ? std::max<int64_t>(0, p.p0 + wrow0 + 1 - p.win) : 0;
@@ -113,6 +127,7 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
     const int64_t w_full_end = p.p0 + wrow0 + 1;
     const int64_t w_full_beg = p.win > 0 ? std::max<int64_t>(0, p.p0 + wrow1 + 1 - p.win) : 0;
 
+    // running maximum in raw score units (the scale x log2(e) is folded into the exponent's fma), running sum
     float m_r[2] = {-INFINITY, -INFINITY}, l_r[2] = {0.0f, 0.0f};
     f4v o[2][DT];
 #pragma unroll
@@ -123,17 +138,18 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
     const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
     const uint8_t* vbase = p.vc + (int64_t) hk * p.head_stride;
     const int64_t t0 = kbeg / KT_TILE, t1 = (kend + KT_TILE - 1) / KT_TILE;
+    const int nt = (int) (t1 - t0);
 
     // a thread's chunks of a tile: chunk c = tid + 256 i -> key c / 16, 16-byte piece c % 16. Keys outside the block's
-    // [kbeg, kend) are clamped into it (a valid row, masked). A wrapped ring's slot is position % cap: the first key's
-    // once, then offsets from it with at most two wraps (a pass's keys span less than two rings)
-    uint4 kst[CH], vst[CH];
+    // [kbeg, kend) are clamped into it (a valid row, masked; a tile past the last is fetched as the last row over and
+    // over and never read). A wrapped ring's slot is position % cap: the first key's once, then offsets from it with at
+    // most two wraps (a pass's keys span less than two rings)
     const int64_t kbeg_slot = p.wrap ? kbeg % p.cap : kbeg;
     const int kspan = (int) (kend - kbeg) - 1;
-    auto fetch = [&](int64_t ti) {
+    auto fetch = [&](Staged& st, int64_t ti) {
         const int rel0 = (int) (ti * KT_TILE - kbeg);
 #pragma unroll
-        for (int i = 0; i < CH; ++i) {
+        for (int i = 0; i < 4; ++i) {
             const int c = tid + PW * 64 * i, key = c >> 4, piece = c & 15;
             const int rel = std::min(std::max(rel0 + key, 0), kspan);
             int64_t slot = kbeg_slot + rel;
@@ -141,95 +157,120 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
                 slot = slot >= p.cap ? slot - p.cap : slot;
                 slot = slot >= p.cap ? slot - p.cap : slot;
             }
-            kst[i] = *reinterpret_cast<const uint4*>(kbase + slot * p.row_stride + piece * 16);
-            vst[i] = *reinterpret_cast<const uint4*>(vbase + slot * p.row_stride + piece * 16);
+            st.k[i] = *reinterpret_cast<const u4v*>(kbase + slot * p.row_stride + piece * 16);
+            st.v[i] = *reinterpret_cast<const u4v*>(vbase + slot * p.row_stride + piece * 16);
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](const Staged& st, int buf) {
         uint8_t* kb_ = lds + buf * (KBUF + VBUF);
         uint8_t* vb_ = kb_ + KBUF;
 #pragma unroll
-        for (int i = 0; i < CH; ++i) {
+        for (int i = 0; i < 4; ++i) {
             const int c = tid + PW * 64 * i, key = c >> 4, piece = c & 15;
-            *reinterpret_cast<uint4*>(kb_ + key * KS + piece * 16) = kst[i];
-            *reinterpret_cast<uint4*>(vb_ + key * VS + piece * 16) = vst[i];
+            *reinterpret_cast<u4v*>(kb_ + key * KS + piece * 16) = st.k[i];
+            *reinterpret_cast<u4v*>(vb_ + key * VS + piece * 16) = st.v[i];
         }
     };
 
-    if (t0 < t1) {
-        fetch(t0);
-        stash(0);
-    }
-    __syncthreads();
-    for (int64_t ti = t0; ti < t1; ++ti) {
-        const int buf = (int) ((ti - t0) & 1);
-        if (ti + 1 < t1) fetch(ti + 1);
-        const int64_t j0 = ti * KT_TILE;
-        if (j0 < w_end && j0 + KT_TILE > w_beg) {
-            const uint8_t* kl = lds + buf * (KBUF + VBUF);
-            uint8_t* vl = lds + buf * (KBUF + VBUF) + KBUF;
-            // ---- S^T = K Q^T
-            f4v s[2][2];
+    // one 32-key half of a staged tile against this wave's 32 rows
+    auto half = [&](const uint8_t* kl, uint8_t* vl, int64_t j0) {
+        // ---- S^T = K Q^T
+        f4v s[2][2];
 #pragma unroll
-            for (int kt2 = 0; kt2 < 2; ++kt2) {
-                s8v ka[KB];
+        for (int kt2 = 0; kt2 < 2; ++kt2) {
+            s8v ka[KB];
 #pragma unroll
-                for (int kb = 0; kb < KB; ++kb) ka[kb] = *reinterpret_cast<const s8v*>(kl + (kt2 * 16 + n) * KS + kb * 64 + g4 * 16);
-#pragma unroll
-                for (int rt = 0; rt < 2; ++rt) {
-                    f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                    for (int kb = 0; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
-                    s[rt][kt2] = acc;
-                }
-            }
-            // ---- softmax; a tile inside [w_full_beg, w_full_end) needs no mask
-            const bool masked = !(j0 >= w_full_beg && j0 + KT_TILE <= w_full_end);
-            s8v pb[2];
+            for (int kb = 0; kb < KB; ++kb) ka[kb] = *reinterpret_cast<const s8v*>(kl + (kt2 * 16 + n) * KS + kb * 64 + g4 * 16);
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
-                float x[8], mx = -INFINITY;
+                f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int kt2 = 0; kt2 < 2; ++kt2)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int64_t j = j0 + kt2 * 16 + g4 * 4 + i;
-                        float v = s[rt][kt2][i] * p.sl2;
-                        if (masked) v = (j >= lo_r[rt] && j <= hi_r[rt]) ? v : -INFINITY;
-                        x[kt2 * 4 + i] = v;
-                        mx = fmaxf(mx, v);
-                    }
-                mx = fmaxf(mx, __shfl_xor(mx, 16));
-                mx = fmaxf(mx, __shfl_xor(mx, 32));
-                const float mn = fmaxf(m_r[rt], mx);
-                const float c = mn == -INFINITY ? 1.0f : fast_exp2(m_r[rt] - mn);
-                float sum = 0.0f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float pv = x[e] == -INFINITY ? 0.0f : fast_exp2(x[e] - mn);
-                    sum += pv;
-                    pb[rt][e] = to16<BF>(pv);
-                }
-                sum += __shfl_xor(sum, 16);
-                sum += __shfl_xor(sum, 32);
-                m_r[rt] = mn;
-                l_r[rt] = l_r[rt] * c + sum;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
-            }
-            // ---- O^T += V^T P^T
-            const int kk = g4 * 4 + (n >> 2);
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                uint8_t* src = vl + kk * VS + (dt * 16 + 4 * (n & 3)) * 2;
-                const s4v lo = lds_read_tr16(src), hi = lds_read_tr16(src + 16 * VS);
-                const s8v va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#pragma unroll
-                for (int rt = 0; rt < 2; ++rt) o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
+                for (int kb = 0; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
+                s[rt][kt2] = acc;
             }
         }
-        if (ti + 1 < t1) stash(buf ^ 1);
+        // ---- softmax; a half inside [w_full_beg, w_full_end) needs no mask
+        const bool masked = !(j0 >= w_full_beg && j0 + 32 <= w_full_end);
+        s8v pb[2];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            float x[8];
+#pragma unroll
+            for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float v = s[rt][kt2][i];
+                    if (masked) {
+                        const int64_t j = j0 + kt2 * 16 + g4 * 4 + i;
+                        v = (j >= lo_r[rt] && j <= hi_r[rt]) ? v : -INFINITY;
+                    }
+                    x[kt2 * 4 + i] = v;
+                }
+            float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float mn = fmaxf(m_r[rt], mx);
+            // the accumulators are rescaled only when some row's maximum moved (rare after the first tiles)
+            if (__any(mn != m_r[rt])) {
+                const float c = mn == -INFINITY ? 1.0f : fast_exp2((m_r[rt] - mn) * p.sl2);
+                l_r[rt] *= c;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
+                m_r[rt] = mn;
+            }
+            const float nb = mn == -INFINITY ? 0.0f : -mn * p.sl2;
+            float sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float pv = fast_exp2(__builtin_fmaf(x[e], p.sl2, nb));   // x = -inf -> 0
+                sum += pv;
+                pb[rt][e] = to16<BF>(pv);
+            }
+            sum += __shfl_xor(sum, 16);
+            sum += __shfl_xor(sum, 32);
+            l_r[rt] += sum;
+        }
+        // ---- O^T += V^T P^T
+        const int kk = g4 * 4 + (n >> 2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            uint8_t* src = vl + kk * VS + (dt * 16 + 4 * (n & 3)) * 2;
+            const s4v lo = lds_read_tr16(src), hi = lds_read_tr16(src + 16 * VS);
+            const s8v va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
+        }
+    };
+    auto compute = [&](int buf, int64_t ti) {
+        const uint8_t* kl = lds + buf * (KBUF + VBUF);
+        uint8_t* vl = lds + buf * (KBUF + VBUF) + KBUF;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int64_t j0 = ti * KT_TILE + h * 32;
+            if (j0 < w_end && j0 + 32 > w_beg) half(kl + h * 32 * KS, vl + h * 32 * VS, j0);
+        }
+    };
+
+    // ---- the pipeline: tile k computed from LDS buffer k & 1 while tile k + 1 sits in registers (written to the other
+    // buffer at the iteration's end) and tile k + 2 is on its way from global memory. Fetches and stashes past the last
+    // tile are harmless repeats, so that no register array is conditionally defined
+    if (nt > 0) {
+        Staged sa, sb;
+        fetch(sa, t0);
+        fetch(sb, t0 + 1);
+        stash(sa, 0);
         __syncthreads();
+        for (int k = 0; k < nt; k += 2) {
+            fetch(sa, t0 + k + 2);
+            compute(0, t0 + k);
+            stash(sb, 1);
+            __syncthreads();
+            if (k + 1 >= nt) break;
+            fetch(sb, t0 + k + 3);
+            compute(1, t0 + k + 1);
+            stash(sa, 0);
+            __syncthreads();
+        }
     }
 
     // ---- out = O / l; a lane holds dims 16 dt + 4 g4 .. + 3 of its rows
@@ -271,7 +312,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     if (!q || !kc || !vc || !out) return ns_fail(w + ": a null buffer");
     if ((uintptr_t) q % 16 || qs % (qt == 0 ? 4 : 8) || (uintptr_t) out % 16) return ns_fail(w + ": query and output rows 16-byte aligned");
     if (((uintptr_t) kc | (uintptr_t) vc) % 16) return ns_fail(w + ": caches 16-byte aligned");
-    if (T > (int64_t) 1 << 30 || Hq > 65535) return ns_fail(w + ": too many rows or heads");
+    if (T > (int64_t) 1 << 30 || ((T + ROWS - 1) / ROWS) * Hq > (int64_t) 1 << 30) return ns_fail(w + ": too many rows or heads");
     NS_HIP(hipSetDevice(g->dev));
     const int64_t rb = 2 * D;
     PrefillParams p{};
@@ -291,7 +332,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     p.win = win;
     p.sl2 = (scale > 0.0f ? scale : 1.0f / sqrtf((float) D)) * 1.4426950408889634f;
     p.out = out;
-    dim3 grid((unsigned) ((T + ROWS - 1) / ROWS), (unsigned) Hq);
+    dim3 grid((unsigned) (((T + ROWS - 1) / ROWS) * Hq));
     if (ns_profile_mark(g, 0)) return -1;
     if (kt == 3) attn_prefill_kernel<128, true><<<grid, PW * 64, 0, g->q>>>(p);
     else attn_prefill_kernel<128, false><<<grid, PW * 64, 0, g->q>>>(p);
