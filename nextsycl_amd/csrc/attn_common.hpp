@@ -51,6 +51,16 @@ __device__ __forceinline__ s4v lds_read_tr16(void* lds_addr) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Reductions over the 4 lanes {n, n + 16, n + 32, n + 48} that hold one query row's scores
+__device__ __forceinline__ float rows_max(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16));
+    return fmaxf(v, __shfl_xor(v, 32));
+}
+__device__ __forceinline__ float rows_sum(float v) {
+    v += __shfl_xor(v, 16);
+    return v + __shfl_xor(v, 32);
+}
+
 // element i of a row of query / output type QT (0 float32, 1 half, 2 bfloat16)
 template <int QT>
 __device__ __forceinline__ float load_q(const void* p, int64_t i) {

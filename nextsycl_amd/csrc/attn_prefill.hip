@@ -29,6 +29,7 @@
 
 #include <algorithm>
 #include <cmath>
+#include <type_traits>
 
 namespace {
 
@@ -127,7 +128,9 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
     const int64_t w_full_end = p.p0 + wrow0 + 1;
     const int64_t w_full_beg = p.win > 0 ? std::max<int64_t>(0, p.p0 + wrow1 + 1 - p.win) : 0;
 
-    // running maximum in raw score units (the scale x log2(e) is folded into the exponent's fma), running sum
+    // running maximum in raw score units (the scale x log2(e) is folded into the exponent's fma), running sum of this
+    // lane's own weights
+    const float margin = 8.0f / p.sl2;
     float m_r[2] = {-INFINITY, -INFINITY}, l_r[2] = {0.0f, 0.0f};
     f4v o[2][DT];
 #pragma unroll
@@ -146,19 +149,22 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
     // most two wraps (a pass's keys span less than two rings)
     const int64_t kbeg_slot = p.wrap ? kbeg % p.cap : kbeg;
     const int kspan = (int) (kend - kbeg) - 1;
+    const int key0 = tid >> 4;                                    // chunk i of this thread: key key0 + 16 i, piece tid & 15
+    const uint8_t* kpiece = kbase + (tid & 15) * 16;
+    const uint8_t* vpiece = vbase + (tid & 15) * 16;
     auto fetch = [&](Staged& st, int64_t ti) {
-        const int rel0 = (int) (ti * KT_TILE - kbeg);
+        const int rel0 = (int) (ti * KT_TILE - kbeg) + key0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int c = tid + PW * 64 * i, key = c >> 4, piece = c & 15;
-            const int rel = std::min(std::max(rel0 + key, 0), kspan);
+            const int rel = std::min(std::max(rel0 + 16 * i, 0), kspan);
             int64_t slot = kbeg_slot + rel;
             if (p.wrap) {
                 slot = slot >= p.cap ? slot - p.cap : slot;
                 slot = slot >= p.cap ? slot - p.cap : slot;
             }
-            st.k[i] = *reinterpret_cast<const u4v*>(kbase + slot * p.row_stride + piece * 16);
-            st.v[i] = *reinterpret_cast<const u4v*>(vbase + slot * p.row_stride + piece * 16);
+            const int64_t off = slot * p.row_stride;
+            st.k[i] = *reinterpret_cast<const u4v*>(kpiece + off);
+            st.v[i] = *reinterpret_cast<const u4v*>(vpiece + off);
         }
     };
     auto stash = [&](const Staged& st, int buf) {
@@ -172,15 +178,22 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
         }
     };
 
-    // one 32-key half of a staged tile against this wave's 32 rows
-    auto half = [&](const uint8_t* kl, uint8_t* vl, int64_t j0) {
+    // one 32-key half of a staged tile against this wave's 32 rows. LDS is addressed with 32-bit offsets from the
+    // array's start (kl, vl: byte offsets); the mask is applied under a wave-uniform branch, so halves no row edge
+    // crosses - nearly all of them - pay for no comparison
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    lds_u8* const L = (lds_u8*) lds;
+    const uint32_t k_rd = (uint32_t) (n * KS + g4 * 16);                          // + kt2 * 16 * KS + kb * 64
+    const uint32_t v_rd = (uint32_t) ((g4 * 4 + (n >> 2)) * VS + (n & 3) * 8);    // + dt * 32 (+ 16 * VS)
+    auto half = [&](uint32_t kl, uint32_t vl, int64_t j0, bool masked) {
         // ---- S^T = K Q^T
         f4v s[2][2];
 #pragma unroll
         for (int kt2 = 0; kt2 < 2; ++kt2) {
             s8v ka[KB];
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb) ka[kb] = *reinterpret_cast<const s8v*>(kl + (kt2 * 16 + n) * KS + kb * 64 + g4 * 16);
+            for (int kb = 0; kb < KB; ++kb)
+                ka[kb] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + kl + k_rd + kt2 * 16 * KS + kb * 64);
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
                 f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -189,8 +202,7 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
                 s[rt][kt2] = acc;
             }
         }
-        // ---- softmax; a half inside [w_full_beg, w_full_end) needs no mask
-        const bool masked = !(j0 >= w_full_beg && j0 + 32 <= w_full_end);
+        // ---- softmax
         s8v pb[2];
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) {
@@ -198,27 +210,35 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
 #pragma unroll
             for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float v = s[rt][kt2][i];
-                    if (masked) {
-                        const int64_t j = j0 + kt2 * 16 + g4 * 4 + i;
-                        v = (j >= lo_r[rt] && j <= hi_r[rt]) ? v : -INFINITY;
-                    }
-                    x[kt2 * 4 + i] = v;
+                for (int i = 0; i < 4; ++i) x[kt2 * 4 + i] = s[rt][kt2][i];
+            if (masked) {
+                // keys lo .. hi of this half (relative, clamped into 0 .. 32 / -1 .. 31) are the row's: one unsigned
+                // compare a key
+                const int lo = (int) std::min<int64_t>(std::max<int64_t>(lo_r[rt] - j0, 0), 32);
+                const int hi = (int) std::min<int64_t>(std::max<int64_t>(hi_r[rt] - j0, -1), 31);
+                const unsigned span = (unsigned) (hi - lo);          // hi < lo: no key, and span wraps to huge...
+                const bool none = hi < lo;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int j = (e >> 2) * 16 + g4 * 4 + (e & 3);
+                    x[e] = (!none && (unsigned) (j - lo) <= span) ? x[e] : -INFINITY;
                 }
-            float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float mn = fmaxf(m_r[rt], mx);
-            // the accumulators are rescaled only when some row's maximum moved (rare after the first tiles)
-            if (__any(mn != m_r[rt])) {
+            }
+            // The running maximum m_r is moved - and the accumulators rescaled - only when some score of the wave
+            // outgrows it by more than 2^8 after scaling; otherwise the weights are taken against the maximum as it
+            // stands (they may then exceed 1, by at most 2^8: harmless in float32 sums and 16-bit operands, and the
+            // final division by l makes the result the same function of the inputs). The common path therefore has
+            // no cross-lane step at all: a lane checks its own 8 scores.
+            const float mxl = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+            if (__any(mxl > m_r[rt] + margin)) {
+                const float mn = fmaxf(m_r[rt], rows_max(mxl));
                 const float c = mn == -INFINITY ? 1.0f : fast_exp2((m_r[rt] - mn) * p.sl2);
                 l_r[rt] *= c;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
                 m_r[rt] = mn;
             }
-            const float nb = mn == -INFINITY ? 0.0f : -mn * p.sl2;
+            const float nb = m_r[rt] == -INFINITY ? 0.0f : -m_r[rt] * p.sl2;
             float sum = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -226,28 +246,26 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
                 sum += pv;
                 pb[rt][e] = to16<BF>(pv);
             }
-            sum += __shfl_xor(sum, 16);
-            sum += __shfl_xor(sum, 32);
-            l_r[rt] += sum;
+            l_r[rt] += sum;                                        // this lane's keys only: reduced over the row at the end
         }
         // ---- O^T += V^T P^T
-        const int kk = g4 * 4 + (n >> 2);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            uint8_t* src = vl + kk * VS + (dt * 16 + 4 * (n & 3)) * 2;
-            const s4v lo = lds_read_tr16(src), hi = lds_read_tr16(src + 16 * VS);
+            const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + vl + v_rd + dt * 32));
+            const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + vl + v_rd + dt * 32 + 16 * VS));
             const s8v va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
         }
     };
     auto compute = [&](int buf, int64_t ti) {
-        const uint8_t* kl = lds + buf * (KBUF + VBUF);
-        uint8_t* vl = lds + buf * (KBUF + VBUF) + KBUF;
+        const uint32_t kl = (uint32_t) (buf * (KBUF + VBUF)), vl = kl + KBUF;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             const int64_t j0 = ti * KT_TILE + h * 32;
-            if (j0 < w_end && j0 + 32 > w_beg) half(kl + h * 32 * KS, vl + h * 32 * VS, j0);
+            if (j0 < w_end && j0 + 32 > w_beg) {
+                half(kl + h * 32 * KS, vl + h * 32 * VS, j0, !(j0 >= w_full_beg && j0 + 32 <= w_full_end));
+            }
         }
     };
 
@@ -277,8 +295,9 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt) {
         const int row = r0 + w * 32 + rt * 16 + n;
+        const float lsum = rows_sum(l_r[rt]);                 // every lane takes part, dead rows too
         if (row >= p.T) continue;
-        const float inv = l_r[rt] > 0.0f ? 1.0f / l_r[rt] : 0.0f;
+        const float inv = lsum > 0.0f ? 1.0f / lsum : 0.0f;
         const int64_t at = ((int64_t) row * p.Hq + hq) * D + g4 * 4;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
