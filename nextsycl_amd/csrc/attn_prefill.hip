@@ -49,11 +49,8 @@ struct PrefillParams {
     void* out;
 };
 
-// one thread's share of a 64-key tile on its way from global memory to LDS: 4 chunks of K, 4 of V
+// a 16-byte chunk of a K or V row on its way from global memory to LDS (a plain vector type: arrays of it stay in registers)
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
-struct Staged {
-    u4v k[4], v[4];
-};
 
 template <int D, bool BF>
 __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillParams p) {
@@ -120,74 +117,89 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
             }
         }
     }
-    // the wave's own key range: its first row's first key to its last row's last (32-key halves outside are skipped)
+    const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
+    const uint8_t* vbase = p.vc + (int64_t) hk * p.head_stride;
+    const int64_t t0 = kbeg / KT_TILE, t1 = (kend + KT_TILE - 1) / KT_TILE;
+    const int nt = (int) (t1 - t0);
+    // From here on keys are counted from the first tile's first key (32-bit): tile k holds keys 64 k .. 64 k + 63, step
+    // s = 2 k + h its 32-key half h
+    const int64_t base = t0 * KT_TILE;
+    int lo32[2], hi32[2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        const bool live = r0 + w * 32 + rt * 16 + n < p.T;
+        lo32[rt] = live ? (int) (lo_r[rt] - base) : 1;
+        hi32[rt] = live ? (int) (hi_r[rt] - base) : 0;
+    }
+    // the wave's own steps: from its first row's first key to its last row's last; steps in between that no row's edge
+    // crosses need no mask
     const int wrow0 = r0 + w * 32, wrow1 = std::min(wrow0 + 31, p.T - 1);
-    const int64_t w_end = wrow0 < p.T ? p.p0 + wrow1 + 1 : 0;
-    const int64_t w_beg = p.win > 0 ? std::max<int64_t>(0, p.p0 + wrow0 + 1 - p.win) : 0;
-    // keys every row of the wave sees without a mask: [w_full_beg, w_full_end)
-    const int64_t w_full_end = p.p0 + wrow0 + 1;
-    const int64_t w_full_beg = p.win > 0 ? std::max<int64_t>(0, p.p0 + wrow1 + 1 - p.win) : 0;
+    const int w_full_end = (int) (p.p0 + wrow0 + 1 - base);
+    const int w_full_beg = p.win > 0 ? (int) (std::max<int64_t>(0, p.p0 + wrow1 + 1 - p.win) - base) : 0;
 
-    // running maximum in raw score units (the scale x log2(e) is folded into the exponent's fma), running sum of this
-    // lane's own weights
-    const float margin = 8.0f / p.sl2;
-    float m_r[2] = {-INFINITY, -INFINITY}, l_r[2] = {0.0f, 0.0f};
+    // Online softmax state, in base-2 exponent units (scores x scale x log2 e): nbr = minus the reference the weights
+    // are taken against, thr = how far a score may exceed it before the reference moves (-inf while the row has seen no
+    // key: the first one sets it), l_r = this lane's own share of the row's sum
+    float nbr[2] = {0.0f, 0.0f}, thr[2] = {-INFINITY, -INFINITY}, l_r[2] = {0.0f, 0.0f};
     f4v o[2][DT];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[rt][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
 
-    const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
-    const uint8_t* vbase = p.vc + (int64_t) hk * p.head_stride;
-    const int64_t t0 = kbeg / KT_TILE, t1 = (kend + KT_TILE - 1) / KT_TILE;
-    const int nt = (int) (t1 - t0);
-
-    // a thread's chunks of a tile: chunk c = tid + 256 i -> key c / 16, 16-byte piece c % 16. Keys outside the block's
-    // [kbeg, kend) are clamped into it (a valid row, masked; a tile past the last is fetched as the last row over and
-    // over and never read). A wrapped ring's slot is position % cap: the first key's once, then offsets from it with at
-    // most two wraps (a pass's keys span less than two rings)
+    // ---- global -> registers -> LDS. A thread's chunks of a tile: chunk c = tid + 256 i -> key c / 16, 16-byte piece
+    // c % 16. A tile wholly inside [kbeg, kend) of an unwrapped cache is read at a wave-uniform address plus a 32-bit
+    // lane offset; otherwise keys outside are clamped into the range (a valid row, masked; a tile past the last is
+    // fetched as the last row over and over and never used) and a wrapped ring's slot is position % cap: the first
+    // key's once, then offsets from it with at most two wraps (a pass's keys span less than two rings)
     const int64_t kbeg_slot = p.wrap ? kbeg % p.cap : kbeg;
     const int kspan = (int) (kend - kbeg) - 1;
+    const int kbeg32 = (int) (kbeg - base);
     const int key0 = tid >> 4;                                    // chunk i of this thread: key key0 + 16 i, piece tid & 15
-    const uint8_t* kpiece = kbase + (tid & 15) * 16;
-    const uint8_t* vpiece = vbase + (tid & 15) * 16;
-    auto fetch = [&](Staged& st, int64_t ti) {
-        const int rel0 = (int) (ti * KT_TILE - kbeg) + key0;
+    const uint32_t lane_off = (uint32_t) (key0 * p.row_stride) + (uint32_t) (tid & 15) * 16;
+    const int plain0 = kbeg32 > 0 ? 1 : 0, plain1 = p.wrap ? -1 : (int) ((kend - base) / KT_TILE) - 1;
+    auto fetch = [&](u4v (&st)[4], const uint8_t* cache, int krel) {
+        const uint8_t* sp = cache;
+        uint32_t off[4];
+        if (krel >= plain0 && krel <= plain1) {
+            sp += (base + (int64_t) krel * KT_TILE) * p.row_stride;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int rel = std::min(std::max(rel0 + 16 * i, 0), kspan);
-            int64_t slot = kbeg_slot + rel;
-            if (p.wrap) {
-                slot = slot >= p.cap ? slot - p.cap : slot;
-                slot = slot >= p.cap ? slot - p.cap : slot;
+            for (int i = 0; i < 4; ++i) off[i] = lane_off + (uint32_t) (i * 16 * p.row_stride);
+        } else {
+            const int rel0 = krel * KT_TILE - kbeg32 + key0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int rel = std::min(std::max(rel0 + 16 * i, 0), kspan);
+                int64_t slot = kbeg_slot + rel;
+                if (p.wrap) {
+                    slot = slot >= p.cap ? slot - p.cap : slot;
+                    slot = slot >= p.cap ? slot - p.cap : slot;
+                }
+                off[i] = (uint32_t) (slot * p.row_stride) + (uint32_t) (tid & 15) * 16;   // a head's cache spans less than 4 GiB
             }
-            const int64_t off = slot * p.row_stride;
-            st.k[i] = *reinterpret_cast<const u4v*>(kpiece + off);
-            st.v[i] = *reinterpret_cast<const u4v*>(vpiece + off);
         }
-    };
-    auto stash = [&](const Staged& st, int buf) {
-        uint8_t* kb_ = lds + buf * (KBUF + VBUF);
-        uint8_t* vb_ = kb_ + KBUF;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int c = tid + PW * 64 * i, key = c >> 4, piece = c & 15;
-            *reinterpret_cast<u4v*>(kb_ + key * KS + piece * 16) = st.k[i];
-            *reinterpret_cast<u4v*>(vb_ + key * VS + piece * 16) = st.v[i];
-        }
+        for (int i = 0; i < 4; ++i) st[i] = *reinterpret_cast<const u4v*>(sp + off[i]);
     };
-
-    // one 32-key half of a staged tile against this wave's 32 rows. LDS is addressed with 32-bit offsets from the
-    // array's start (kl, vl: byte offsets); the mask is applied under a wave-uniform branch, so halves no row edge
-    // crosses - nearly all of them - pay for no comparison
     typedef __attribute__((address_space(3))) uint8_t lds_u8;
     lds_u8* const L = (lds_u8*) lds;
+    // LDS map: K tiles at 0 and KBUF, V tiles at 2 KBUF and 2 KBUF + VBUF
+    constexpr uint32_t V0 = 2 * KBUF;
+    const uint32_t k_wr = (uint32_t) (key0 * KS + (tid & 15) * 16), v_wr = (uint32_t) (key0 * VS + (tid & 15) * 16);
+    auto stash_k = [&](const u4v (&st)[4], int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<__attribute__((address_space(3))) u4v*>(L + buf * KBUF + k_wr + i * 16 * KS) = st[i];
+    };
+    auto stash_v = [&](const u4v (&st)[4], int buf) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<__attribute__((address_space(3))) u4v*>(L + V0 + buf * VBUF + v_wr + i * 16 * VS) = st[i];
+    };
+
     const uint32_t k_rd = (uint32_t) (n * KS + g4 * 16);                          // + kt2 * 16 * KS + kb * 64
     const uint32_t v_rd = (uint32_t) ((g4 * 4 + (n >> 2)) * VS + (n & 3) * 8);    // + dt * 32 (+ 16 * VS)
-    auto half = [&](uint32_t kl, uint32_t vl, int64_t j0, bool masked) {
-        // ---- S^T = K Q^T
-        f4v s[2][2];
+    s8v pb[2] = {s8v{0, 0, 0, 0, 0, 0, 0, 0}, s8v{0, 0, 0, 0, 0, 0, 0, 0}};
+    // S^T of one 32-key half (LDS byte offset kl) against the wave's 32 rows
+    auto scores = [&](f4v (&s)[2][2], uint32_t kl) {
 #pragma unroll
         for (int kt2 = 0; kt2 < 2; ++kt2) {
             s8v ka[KB];
@@ -202,53 +214,9 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
                 s[rt][kt2] = acc;
             }
         }
-        // ---- softmax
-        s8v pb[2];
-#pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
-            float x[8];
-#pragma unroll
-            for (int kt2 = 0; kt2 < 2; ++kt2)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) x[kt2 * 4 + i] = s[rt][kt2][i];
-            if (masked) {
-                // keys lo .. hi of this half (relative, clamped into 0 .. 32 / -1 .. 31) are the row's: one unsigned
-                // compare a key
-                const int lo = (int) std::min<int64_t>(std::max<int64_t>(lo_r[rt] - j0, 0), 32);
-                const int hi = (int) std::min<int64_t>(std::max<int64_t>(hi_r[rt] - j0, -1), 31);
-                const unsigned span = (unsigned) (hi - lo);          // hi < lo: no key, and span wraps to huge...
-                const bool none = hi < lo;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int j = (e >> 2) * 16 + g4 * 4 + (e & 3);
-                    x[e] = (!none && (unsigned) (j - lo) <= span) ? x[e] : -INFINITY;
-                }
-            }
-            // The running maximum m_r is moved - and the accumulators rescaled - only when some score of the wave
-            // outgrows it by more than 2^8 after scaling; otherwise the weights are taken against the maximum as it
-            // stands (they may then exceed 1, by at most 2^8: harmless in float32 sums and 16-bit operands, and the
-            // final division by l makes the result the same function of the inputs). The common path therefore has
-            // no cross-lane step at all: a lane checks its own 8 scores.
-            const float mxl = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-            if (__any(mxl > m_r[rt] + margin)) {
-                const float mn = fmaxf(m_r[rt], rows_max(mxl));
-                const float c = mn == -INFINITY ? 1.0f : fast_exp2((m_r[rt] - mn) * p.sl2);
-                l_r[rt] *= c;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
-                m_r[rt] = mn;
-            }
-            const float nb = m_r[rt] == -INFINITY ? 0.0f : -m_r[rt] * p.sl2;
-            float sum = 0.0f;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float pv = fast_exp2(__builtin_fmaf(x[e], p.sl2, nb));   // x = -inf -> 0
-                sum += pv;
-                pb[rt][e] = to16<BF>(pv);
-            }
-            l_r[rt] += sum;                                        // this lane's keys only: reduced over the row at the end
-        }
-        // ---- O^T += V^T P^T
+    };
+    // O^T += V^T P^T of one 32-key half (LDS byte offset vl) with the weights in pb
+    auto weigh = [&](uint32_t vl) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + vl + v_rd + dt * 32));
@@ -258,37 +226,127 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
             for (int rt = 0; rt < 2; ++rt) o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
         }
     };
-    auto compute = [&](int buf, int64_t ti) {
-        const uint32_t kl = (uint32_t) (buf * (KBUF + VBUF)), vl = kl + KBUF;
+    // One step of the wave's software pipeline. Step s holds the scores of its own half in sc (computed a step earlier)
+    // and runs, as two straight-line blocks in which matrix and vector work are independent and overlap:
+    //   A: O^T += V^T P^T of step s - 1   ||   exponent arguments of step s against the reference as it stands, and
+    //      this lane's largest
+    //   (only if some row's score outgrew its reference by more than 2^8: move the references, rescale; the weights may
+    //    otherwise exceed 1, by at most 2^8: harmless in float32 sums and 16-bit operands, and the final division by
+    //    the row's sum makes the result the same function of the inputs)
+    //   B: S^T of step s + 1              ||   weights of step s = exp2(arguments), their sum, rounding to 16 bit
+    // The mask is applied under a wave-uniform branch: steps no row's causal or window edge crosses pay no comparison.
+    auto step = [&](f4v (&sc)[2][2], f4v (&sn)[2][2], uint32_t kl_next, uint32_t vl_prev, int j0, bool masked) {
+        float a[2][8], amax[2];
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const int64_t j0 = ti * KT_TILE + h * 32;
-            if (j0 < w_end && j0 + 32 > w_beg) {
-                half(kl + h * 32 * KS, vl + h * 32 * VS, j0, !(j0 >= w_full_beg && j0 + 32 <= w_full_end));
+        for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[rt][e] = sc[rt][e >> 2][e & 3];
+        if (masked) {
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                // keys lo .. hi of this half (relative, clamped into 0 .. 32 / -1 .. 31) are the row's: one unsigned
+                // compare a key (no key at all: lo = 64 puts every key below it)
+                const int lo_ = std::min(std::max(lo32[rt] - j0, 0), 32);
+                const int hi = std::min(std::max(hi32[rt] - j0, -1), 31);
+                const int lo = hi < lo_ ? 64 : lo_;
+                const unsigned span = hi < lo_ ? 0u : (unsigned) (hi - lo_);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const int j = (e >> 2) * 16 + g4 * 4 + (e & 3);
+                    a[rt][e] = (unsigned) (j - lo) <= span ? a[rt][e] : -INFINITY;
+                }
             }
         }
+        weigh(vl_prev);
+        bool grow = false;
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[rt][e] = __builtin_fmaf(a[rt][e], p.sl2, nbr[rt]);
+            amax[rt] = fmaxf(fmaxf(fmaxf(a[rt][0], a[rt][1]), fmaxf(a[rt][2], a[rt][3])), fmaxf(fmaxf(a[rt][4], a[rt][5]), fmaxf(a[rt][6], a[rt][7])));
+            grow |= amax[rt] > thr[rt];
+        }
+        if (__any(grow)) {
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                const float mx = rows_max(amax[rt]);
+                const bool fresh = thr[rt] < 0.0f;
+                const bool nokey = mx == -INFINITY;
+                const float delta = fresh ? (nokey ? 0.0f : mx) : fmaxf(mx, 0.0f);
+                const float c = fresh ? 1.0f : fast_exp2(-delta);
+                l_r[rt] *= c;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
+                nbr[rt] -= delta;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a[rt][e] -= delta;
+                thr[rt] = (fresh && nokey) ? -INFINITY : 8.0f;
+            }
+        }
+        scores(sn, kl_next);
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float pv = fast_exp2(a[rt][e]);                // -inf -> 0
+                sum += pv;
+                pb[rt][e] = to16<BF>(pv);
+            }
+            l_r[rt] += sum;
+        }
+        // the step's results are complete here, in program order: nothing of it drifts past the next barrier or branch
+        asm volatile("" : "+v"(pb[0]), "+v"(pb[1]), "+v"(l_r[0]), "+v"(l_r[1]));
     };
 
-    // ---- the pipeline: tile k computed from LDS buffer k & 1 while tile k + 1 sits in registers (written to the other
-    // buffer at the iteration's end) and tile k + 2 is on its way from global memory. Fetches and stashes past the last
-    // tile are harmless repeats, so that no register array is conditionally defined
+    // ---- the pipeline over tiles. K and V tiles have two LDS buffers each (tile k in buffer k & 1) and one register
+    // set each; one barrier a tile, between its two steps:
+    //   step 2k   : K(k+1) registers -> LDS, fetch K(k+2); A reads V(k-1) half 1, B reads K(k) half 1
+    //   barrier
+    //   step 2k+1 : V(k+1) registers -> LDS, fetch V(k+2); A reads V(k) half 0,   B reads K(k+1) half 0
+    // A wave runs steps sb - 1 .. se of its own (the one before its first computes nothing it keeps except the scores of
+    // the first; the one after its last adds the last step's product); all waves take part in the staging of every tile.
     if (nt > 0) {
-        Staged sa, sb;
-        fetch(sa, t0);
-        fetch(sb, t0 + 1);
-        stash(sa, 0);
-        __syncthreads();
-        for (int k = 0; k < nt; k += 2) {
-            fetch(sa, t0 + k + 2);
-            compute(0, t0 + k);
-            stash(sb, 1);
-            __syncthreads();
-            if (k + 1 >= nt) break;
-            fetch(sb, t0 + k + 3);
-            compute(1, t0 + k + 1);
-            stash(sa, 0);
-            __syncthreads();
+        u4v stk[4], stv[4];
+        f4v sA[2][2], sB[2][2];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+            for (int kt2 = 0; kt2 < 2; ++kt2) sA[rt][kt2] = sB[rt][kt2] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+        fetch(stk, kbase, 0);
+        fetch(stv, vbase, 0);
+        {   // the V buffer step 0 "adds" with zero weights must hold numbers
+            const u4v z = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<__attribute__((address_space(3))) u4v*>(L + V0 + VBUF + v_wr + i * 16 * VS) = z;
         }
+        stash_k(stk, 0);
+        stash_v(stv, 0);
+        fetch(stk, kbase, 1);
+        fetch(stv, vbase, 1);
+        __syncthreads();
+        scores(sA, 0);
+        for (int k = 0; k < nt; k += 2) {
+            // tile k: buffers 0
+            stash_k(stk, 1);
+            fetch(stk, kbase, k + 2);
+            step(sA, sB, 32 * KS, V0 + VBUF + 32 * VS, 64 * k, !(64 * k >= w_full_beg && 64 * k + 32 <= w_full_end));
+            __syncthreads();
+            stash_v(stv, 1);
+            fetch(stv, vbase, k + 2);
+            step(sB, sA, KBUF, V0, 64 * k + 32, !(64 * k + 32 >= w_full_beg && 64 * k + 64 <= w_full_end));
+            if (k + 1 >= nt) break;
+            // tile k + 1: buffers 1
+            stash_k(stk, 0);
+            fetch(stk, kbase, k + 3);
+            step(sA, sB, KBUF + 32 * KS, V0 + 32 * VS, 64 * k + 64, !(64 * k + 64 >= w_full_beg && 64 * k + 96 <= w_full_end));
+            __syncthreads();
+            stash_v(stv, 0);
+            fetch(stv, vbase, k + 3);
+            step(sB, sA, 0, V0 + VBUF, 64 * k + 96, !(64 * k + 96 >= w_full_beg && 64 * k + 128 <= w_full_end));
+        }
+        // the last step's product
+        weigh(V0 + (uint32_t) ((nt - 1) & 1) * VBUF + 32 * VS);
     }
 
     // ---- out = O / l; a lane holds dims 16 dt + 4 g4 .. + 3 of its rows
