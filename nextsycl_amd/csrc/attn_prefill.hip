@@ -63,15 +63,18 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     // ---- which (row block, head) this work-group owns. Consecutive work-group ids go round the 8 XCDs (each with its
-    // own L2): undo that, so that neighbours in the logical order - the G query heads of one key head on one row block,
-    // which stream the same K / V tiles - share an L2. Logical order: heaviest row blocks first.
-    const int nwg = gridDim.x, pid = blockIdx.x;
-    const int xq = nwg / 8, xr = nwg % 8, xcd = pid % 8, xi = pid / 8;
-    const int logical = (xcd < xr ? xcd * (xq + 1) : xr * (xq + 1) + (xcd - xr) * xq) + xi;
+    // own L2). The G query heads of one key head on one row block stream the same K / V tiles: they are one unit, and a
+    // unit's work-groups are consecutive on one XCD. Units are dealt to the XCDs round-robin in order of weight (the last
+    // row block sees the most keys), so every XCD gets the same mix of heavy and light units, heaviest first. The grid is
+    // padded to a multiple of 8 units; the work-groups of the padding leave at once.
+    const int pid = blockIdx.x, xcd = pid % 8, xi = pid / 8;
     const int nblk = (p.T + ROWS - 1) / ROWS;
-    const int hq = logical % p.Hq;                               // heads fastest: hq / G is the key head
-    const int blk = nblk - 1 - logical / p.Hq;
-    const int hk = hq / p.G;
+    const int Hkv = p.Hq / p.G;
+    const int unit = (xi / p.G) * 8 + xcd;
+    if (unit >= nblk * Hkv) return;
+    const int hk = unit % Hkv;
+    const int hq = hk * p.G + xi % p.G;
+    const int blk = nblk - 1 - unit / Hkv;
     const int r0 = blk * ROWS;
     const int rl = std::min(r0 + ROWS, p.T) - 1;                  // the block's last row
     const int64_t kend = p.p0 + rl + 1;                           // keys [kbeg, kend) cover every row of the block
@@ -389,7 +392,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     if (!q || !kc || !vc || !out) return ns_fail(w + ": a null buffer");
     if ((uintptr_t) q % 16 || qs % (qt == 0 ? 4 : 8) || (uintptr_t) out % 16) return ns_fail(w + ": query and output rows 16-byte aligned");
     if (((uintptr_t) kc | (uintptr_t) vc) % 16) return ns_fail(w + ": caches 16-byte aligned");
-    if (T > (int64_t) 1 << 30 || ((T + ROWS - 1) / ROWS) * Hq > (int64_t) 1 << 30) return ns_fail(w + ": too many rows or heads");
+    if (T > (int64_t) 1 << 30 || ((T + ROWS - 1) / ROWS + 1) * Hq > (int64_t) 1 << 30) return ns_fail(w + ": too many rows or heads");
     NS_HIP(hipSetDevice(g->dev));
     const int64_t rb = 2 * D;
     PrefillParams p{};
@@ -409,7 +412,8 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     p.win = win;
     p.sl2 = (scale > 0.0f ? scale : 1.0f / sqrtf((float) D)) * 1.4426950408889634f;
     p.out = out;
-    dim3 grid((unsigned) (((T + ROWS - 1) / ROWS) * Hq));
+    const int64_t units = ((T + ROWS - 1) / ROWS) * Hkv;               // (row block, key head); padded to the 8 XCDs
+    dim3 grid((unsigned) ((units + 7) / 8 * 8 * (Hq / Hkv)));
     if (ns_profile_mark(g, 0)) return -1;
     if (kt == 3) attn_prefill_kernel<128, true><<<grid, PW * 64, 0, g->q>>>(p);
     else attn_prefill_kernel<128, false><<<grid, PW * 64, 0, g->q>>>(p);
