@@ -260,6 +260,7 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
                 }
             }
         }
+        __builtin_amdgcn_s_setprio(1);
         weigh(vl_prev);
         bool grow = false;
 #pragma unroll
@@ -300,6 +301,7 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
         }
         // the step's results are complete here, in program order: nothing of it drifts past the next barrier or branch
         asm volatile("" : "+v"(pb[0]), "+v"(pb[1]), "+v"(l_r[0]), "+v"(l_r[1]));
+        __builtin_amdgcn_s_setprio(0);
     };
 
     // ---- the pipeline over tiles. K and V tiles have two LDS buffers each (tile k in buffer k & 1) and one register
