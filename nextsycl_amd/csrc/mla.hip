@@ -50,6 +50,8 @@ struct MlaParams {
     float* part;         // [T * H][ns][PSTRIDE]
 };
 
+typedef uint32_t u4v __attribute__((ext_vector_type(4)));   // a 16-byte chunk in flight (a plain vector: stays in registers)
+
 __device__ __forceinline__ int swz(int r) { return (((r >> 1) & 3) << 1) | ((r >> 3) & 1); }
 
 // R: rope features (64: DeepSeek's [512 | 64] rows; 0: GLM's latent-only rows); Q8: GLM's q8 rows
@@ -97,26 +99,32 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
             }
         }
     }
-    float m_r = -INFINITY, l_r = 0.0f;
+    float nbr = 0.0f, thr = -INFINITY, l_r = 0.0f;
+    const int hi_rel = (int) std::max<int64_t>(std::min<int64_t>(hi_r - jb, (int64_t) 1 << 30), -1);
     f4v o[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
 
     // ---- tile traffic: chunk id = tid + 512 i -> row id / CPR, piece id % CPR; cells past the split's end are clamped
     // to its last (a valid row; their scores are masked)
-    uint4 st[NLD];
+    u4v st[NLD];
     uint16_t stsc[Q8 ? NLD : 1];
-    auto fetch = [&](int64_t j0) {
+    // (a tile wholly inside the split is read at a wave-uniform address plus a 32-bit lane offset)
+    const uint8_t* const split_base = p.cache + jb * CROW;
+    const int last_rel = (int) (je - 1 - jb);
+    auto fetch = [&](int it_) {
+        const bool plain = (it_ + 1) * MTILE - 1 <= last_rel;
+        const uint8_t* sp = split_base + (plain ? (int64_t) it_ * MTILE * CROW : 0);
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             const int id = tid + MW * 64 * i, r = id / CPR, c = id % CPR;
             if (NCH % (MW * 64) != 0 && id >= NCH) continue;
-            const uint8_t* row = p.cache + std::min(j0 + r, je - 1) * CROW;
+            const uint32_t off = (uint32_t) ((plain ? r : std::min(it_ * MTILE + r, last_rel)) * (int) CROW);
             if constexpr (Q8) {
-                st[i] = *reinterpret_cast<const uint4*>(row + ML / 32 * 2 + c * 16);
-                stsc[i] = *reinterpret_cast<const uint16_t*>(row + 2 * (c / 2));
+                st[i] = *reinterpret_cast<const u4v*>(sp + off + ML / 32 * 2 + c * 16);
+                stsc[i] = *reinterpret_cast<const uint16_t*>(sp + off + 2 * (c / 2));
             } else {
-                st[i] = *reinterpret_cast<const uint4*>(row + c * 16);
+                st[i] = *reinterpret_cast<const u4v*>(sp + off + c * 16);
             }
         }
     };
@@ -130,7 +138,7 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
                 // 16 int8 x one half scale -> 16 halfs = chunks 2c, 2c + 1; value = half(scale) x q, one rounding to
                 // half (the reference widens half(scale) x q in float32: kernels/llm/glm5next/glm.cpp:1116-1124)
                 const _Float16 d = __builtin_bit_cast(_Float16, stsc[i]);
-                const uint32_t ww[4] = {st[i].x, st[i].y, st[i].z, st[i].w};
+                const uint32_t ww[4] = {st[i][0], st[i][1], st[i][2], st[i][3]};
                 s8v a, b;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
@@ -142,76 +150,89 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
                 *reinterpret_cast<s8v*>(base + r * RSTRIDE + ((2 * c) ^ swz(r)) * 16) = a;
                 *reinterpret_cast<s8v*>(base + r * RSTRIDE + ((2 * c + 1) ^ swz(r)) * 16) = b;
             } else {
-                *reinterpret_cast<uint4*>(base + r * RSTRIDE + (c ^ swz(r)) * 16) = st[i];
+                *reinterpret_cast<u4v*>(base + r * RSTRIDE + (c ^ swz(r)) * 16) = st[i];
             }
         }
     };
 
+    // LDS read addresses as a few lane bases plus compile-time offsets. The swizzle touches the low 3 bits of a chunk
+    // index only, so chunk (8 a + b) ^ g = 8 a + (b ^ g): one base a value of b, 128 bytes a step of a.
+    //   score operand: row ct 16 + n (g the same for both ct), chunk 4 kb + g4        -> b = 4 (kb & 1) + g4, a = kb >> 1
+    //   transposed read: row kk (+ 16: same g), chunk 2 dt + ((n & 3) >> 1), half n & 1 -> b = 2 (dt & 3) + .., a = dt >> 2
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    lds_u8* const L = (lds_u8*) lds;
+    const int kk = g4 * 4 + (n >> 2);
+    uint32_t s_rd[2], v_rd[4];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) s_rd[b] = (uint32_t) (n * RSTRIDE + (((b * 4 + g4) ^ swz(n)) * 16));
+#pragma unroll
+    for (int b = 0; b < 4; ++b) v_rd[b] = (uint32_t) (kk * RSTRIDE + (((b * 2 + ((n & 3) >> 1)) ^ swz(kk)) * 16) + (n & 1) * 8);
+
     const int64_t nt = jb < je ? (je - jb + MTILE - 1) / MTILE : 0;
     if (nt > 0) {
-        fetch(jb);
+        fetch(0);
         stash(0);
     }
     __syncthreads();
-    for (int64_t it = 0; it < nt; ++it) {
-        const int buf = (int) (it & 1);
-        const int64_t j0 = jb + it * MTILE;
-        if (it + 1 < nt) fetch(j0 + MTILE);
-        uint8_t* tile = lds + buf * TILEB;
+    for (int it = 0; it < (int) nt; ++it) {
+        const int buf = it & 1;
+        if (it + 1 < (int) nt) fetch(it + 1);
+        const uint32_t tile = (uint32_t) buf * TILEB;
         // ---- S^T = C Q^T
         f4v s[2];
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) {
-            const int r = ct * 16 + n;
             f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
-                const s8v a = *reinterpret_cast<const s8v*>(tile + r * RSTRIDE + ((kb * 4 + g4) ^ swz(r)) * 16);
+                const s8v a = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + tile + s_rd[kb & 1] + ct * 16 * RSTRIDE + (kb >> 1) * 128);
                 acc = mfma16<false>(a, qreg[kb], acc);
             }
             s[ct] = acc;
         }
-        // ---- softmax of this lane's row
+        // ---- softmax of this lane's row, in base-2 exponent units. The reference the weights are taken against (minus
+        // it: nbr) moves - and the 128 accumulators are rescaled - only when some score of the wave outgrows it by more
+        // than 2^8 (thr; -inf while the row has seen no cell: the first one sets it). Weights may otherwise exceed 1, by
+        // at most 2^8: harmless in float32 sums and half operands, and the partial's {O, m, l} stay consistent. The
+        // common path has no cross-lane step: l_r is this lane's own share of the row's sum.
         s8v pb;
         {
-            float x[8], mx = -INFINITY;
+            float a[8];
+            const int hi = hi_rel - it * MTILE;            // cells 0 .. hi of this tile are the row's
 #pragma unroll
-            for (int ct = 0; ct < 2; ++ct)
+            for (int e = 0; e < 8; ++e) {
+                const int j = (e >> 2) * 16 + g4 * 4 + (e & 3);
+                a[e] = j <= hi ? __builtin_fmaf(s[e >> 2][e & 3], p.sl2, nbr) : -INFINITY;
+            }
+            const float amax = fmaxf(fmaxf(fmaxf(a[0], a[1]), fmaxf(a[2], a[3])), fmaxf(fmaxf(a[4], a[5]), fmaxf(a[6], a[7])));
+            if (__any(amax > thr)) {
+                const float mx = rows_max(amax);
+                const bool fresh = thr < 0.0f, nokey = mx == -INFINITY;
+                const float delta = fresh ? (nokey ? 0.0f : mx) : fmaxf(mx, 0.0f);
+                const float c = fresh ? 1.0f : fast_exp2(-delta);
+                l_r *= c;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int64_t j = j0 + ct * 16 + g4 * 4 + i;
-                    const float v = j <= hi_r ? s[ct][i] * p.sl2 : -INFINITY;
-                    x[ct * 4 + i] = v;
-                    mx = fmaxf(mx, v);
-                }
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float mn = fmaxf(m_r, mx);
-            const float c = mn == -INFINITY ? 1.0f : fast_exp2(m_r - mn);
+                for (int dt = 0; dt < DT; ++dt) o[dt] *= c;
+                nbr -= delta;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) a[e] -= delta;
+                thr = (fresh && nokey) ? -INFINITY : 8.0f;
+            }
             float sum = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float pv = x[e] == -INFINITY ? 0.0f : fast_exp2(x[e] - mn);
+                const float pv = fast_exp2(a[e]);                   // -inf -> 0
                 sum += pv;
                 pb[e] = to16<false>(pv);
             }
-            sum += __shfl_xor(sum, 16);
-            sum += __shfl_xor(sum, 32);
-            m_r = mn;
-            l_r = l_r * c + sum;
-            // the 128 accumulators are rescaled only when some row's maximum moved
-            if (__any(c != 1.0f)) {
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) o[dt] *= c;
-            }
+            l_r += sum;
         }
         // ---- O^T += C^T P^T
-        const int kk = g4 * 4 + (n >> 2);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            const int c = (dt * 2 + ((n & 3) >> 1)) ^ swz(kk);    // swz(kk + 16) == swz(kk)
-            uint8_t* src = tile + kk * RSTRIDE + c * 16 + (n & 1) * 8;
-            const s4v lo = lds_read_tr16(src), hi = lds_read_tr16(src + 16 * RSTRIDE);
+            const uint32_t src = tile + v_rd[dt & 3] + (dt >> 2) * 128;
+            const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + src));
+            const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + src + 16 * RSTRIDE));
             const s8v va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             o[dt] = mfma16<false>(va, pb, o[dt]);
         }
@@ -220,13 +241,15 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
     }
 
     // ---- the split's partial, straight from the registers: a lane holds latents 16 dt + 4 g4 .. + 3 of its row
+    const float l_row = rows_sum(l_r);
+    const float m_r = thr < 0.0f ? -INFINITY : -nbr;
     if (live) {
         float* pr = p.part + ((int64_t) ri * p.ns + split) * PSTRIDE;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f4v*>(pr + dt * 16 + g4 * 4) = o[dt];
         if (g4 == 0) {
             pr[ML] = m_r;
-            pr[ML + 1] = l_r;
+            pr[ML + 1] = l_row;
         }
     }
 }
