@@ -107,38 +107,43 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
 
     // ---- tile traffic: chunk id = tid + 512 i -> row id / CPR, piece id % CPR; cells past the split's end are clamped
     // to its last (a valid row; their scores are masked)
-    u4v st[NLD];
-    uint16_t stsc[Q8 ? NLD : 1];
+    // A tile is staged in two phases (loads H1 and NLD - H1 of a thread) through one small register set, so that the
+    // registers a tile in flight takes stay few beside the 200 of the queries and accumulators.
+    constexpr int H1 = (NLD + 1) / 2;
+    u4v st[H1];
+    uint16_t stsc[Q8 ? H1 : 1];
     // (a tile wholly inside the split is read at a wave-uniform address plus a 32-bit lane offset)
     const uint8_t* const split_base = p.cache + jb * CROW;
     const int last_rel = (int) (je - 1 - jb);
-    auto fetch = [&](int it_) {
+    auto fetch = [&](int it_, int i0, int i1) {
         const bool plain = (it_ + 1) * MTILE - 1 <= last_rel;
         const uint8_t* sp = split_base + (plain ? (int64_t) it_ * MTILE * CROW : 0);
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
+            if (i < i0 || i >= i1) continue;
             const int id = tid + MW * 64 * i, r = id / CPR, c = id % CPR;
             if (NCH % (MW * 64) != 0 && id >= NCH) continue;
             const uint32_t off = (uint32_t) ((plain ? r : std::min(it_ * MTILE + r, last_rel)) * (int) CROW);
             if constexpr (Q8) {
-                st[i] = *reinterpret_cast<const u4v*>(sp + off + ML / 32 * 2 + c * 16);
-                stsc[i] = *reinterpret_cast<const uint16_t*>(sp + off + 2 * (c / 2));
+                st[i % H1] = *reinterpret_cast<const u4v*>(sp + off + ML / 32 * 2 + c * 16);
+                stsc[i % H1] = *reinterpret_cast<const uint16_t*>(sp + off + 2 * (c / 2));
             } else {
-                st[i] = *reinterpret_cast<const u4v*>(sp + off + c * 16);
+                st[i % H1] = *reinterpret_cast<const u4v*>(sp + off + c * 16);
             }
         }
     };
-    auto stash = [&](int buf) {
+    auto stash = [&](int buf, int i0, int i1) {
         uint8_t* base = lds + buf * TILEB;
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
+            if (i < i0 || i >= i1) continue;
             const int id = tid + MW * 64 * i, r = id / CPR, c = id % CPR;
             if (NCH % (MW * 64) != 0 && id >= NCH) continue;
             if constexpr (Q8) {
                 // 16 int8 x one half scale -> 16 halfs = chunks 2c, 2c + 1; value = half(scale) x q, one rounding to
                 // half (the reference widens half(scale) x q in float32: kernels/llm/glm5next/glm.cpp:1116-1124)
-                const _Float16 d = __builtin_bit_cast(_Float16, stsc[i]);
-                const uint32_t ww[4] = {st[i][0], st[i][1], st[i][2], st[i][3]};
+                const _Float16 d = __builtin_bit_cast(_Float16, stsc[i % H1]);
+                const uint32_t ww[4] = {st[i % H1][0], st[i % H1][1], st[i % H1][2], st[i % H1][3]};
                 s8v a, b;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
@@ -150,7 +155,7 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
                 *reinterpret_cast<s8v*>(base + r * RSTRIDE + ((2 * c) ^ swz(r)) * 16) = a;
                 *reinterpret_cast<s8v*>(base + r * RSTRIDE + ((2 * c + 1) ^ swz(r)) * 16) = b;
             } else {
-                *reinterpret_cast<u4v*>(base + r * RSTRIDE + (c ^ swz(r)) * 16) = st[i];
+                *reinterpret_cast<u4v*>(base + r * RSTRIDE + (c ^ swz(r)) * 16) = st[i % H1];
             }
         }
     };
@@ -170,13 +175,16 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
 
     const int64_t nt = jb < je ? (je - jb + MTILE - 1) / MTILE : 0;
     if (nt > 0) {
-        fetch(0);
-        stash(0);
+        fetch(0, 0, H1);
+        stash(0, 0, H1);
+        fetch(0, H1, NLD);
+        stash(0, H1, NLD);
     }
     __syncthreads();
     for (int it = 0; it < (int) nt; ++it) {
         const int buf = it & 1;
-        if (it + 1 < (int) nt) fetch(it + 1);
+        const bool more = it + 1 < (int) nt;
+        if (more) fetch(it + 1, 0, H1);
         const uint32_t tile = (uint32_t) buf * TILEB;
         // ---- S^T = C Q^T
         f4v s[2];
@@ -227,6 +235,10 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
             }
             l_r += sum;
         }
+        if (more) {
+            stash(buf ^ 1, 0, H1);
+            fetch(it + 1, H1, NLD);
+        }
         // ---- O^T += C^T P^T
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -236,7 +248,7 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
             const s8v va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             o[dt] = mfma16<false>(va, pb, o[dt]);
         }
-        if (it + 1 < nt) stash(buf ^ 1);
+        if (more) stash(buf ^ 1, H1, NLD);
         __syncthreads();
     }
 
