@@ -64,7 +64,15 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
     constexpr int CPR = Q8 ? ML / 16 : DK / 8;           // 16-byte loads a cache row
     constexpr int NCH = MTILE * CPR;                     // loads a tile
     constexpr int NLD = (NCH + MW * 64 - 1) / (MW * 64); // loads a thread per tile (the last may be idle)
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * TILEB];
+    // three tile buffers, three separate arrays: reads of one are then known not to touch a buffer a transfer is
+    // still writing
+    __shared__ __attribute__((aligned(16))) uint8_t lds0[TILEB];
+    __shared__ __attribute__((aligned(16))) uint8_t lds1[TILEB];
+    __shared__ __attribute__((aligned(16))) uint8_t lds2[TILEB];
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    lds_u8* const B0 = (lds_u8*) lds0;
+    lds_u8* const B1 = (lds_u8*) lds1;
+    lds_u8* const B2 = (lds_u8*) lds2;
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -132,8 +140,7 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
             }
         }
     };
-    auto stash = [&](int buf, int i0, int i1) {
-        uint8_t* base = lds + buf * TILEB;
+    auto stash = [&](lds_u8* base, int i0, int i1) {
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             if (i < i0 || i >= i1) continue;
@@ -152,10 +159,10 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
                     a[e] = __builtin_bit_cast(short, x0);
                     b[e] = __builtin_bit_cast(short, x1);
                 }
-                *reinterpret_cast<s8v*>(base + r * RSTRIDE + ((2 * c) ^ swz(r)) * 16) = a;
-                *reinterpret_cast<s8v*>(base + r * RSTRIDE + ((2 * c + 1) ^ swz(r)) * 16) = b;
+                *reinterpret_cast<__attribute__((address_space(3))) s8v*>(base + r * RSTRIDE + ((2 * c) ^ swz(r)) * 16) = a;
+                *reinterpret_cast<__attribute__((address_space(3))) s8v*>(base + r * RSTRIDE + ((2 * c + 1) ^ swz(r)) * 16) = b;
             } else {
-                *reinterpret_cast<u4v*>(base + r * RSTRIDE + (c ^ swz(r)) * 16) = st[i % H1];
+                *reinterpret_cast<__attribute__((address_space(3))) u4v*>(base + r * RSTRIDE + (c ^ swz(r)) * 16) = st[i % H1];
             }
         }
     };
@@ -164,8 +171,6 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
     // index only, so chunk (8 a + b) ^ g = 8 a + (b ^ g): one base a value of b, 128 bytes a step of a.
     //   score operand: row ct 16 + n (g the same for both ct), chunk 4 kb + g4        -> b = 4 (kb & 1) + g4, a = kb >> 1
     //   transposed read: row kk (+ 16: same g), chunk 2 dt + ((n & 3) >> 1), half n & 1 -> b = 2 (dt & 3) + .., a = dt >> 2
-    typedef __attribute__((address_space(3))) uint8_t lds_u8;
-    lds_u8* const L = (lds_u8*) lds;
     const int kk = g4 * 4 + (n >> 2);
     uint32_t s_rd[2], v_rd[4];
 #pragma unroll
@@ -173,19 +178,38 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
 #pragma unroll
     for (int b = 0; b < 4; ++b) v_rd[b] = (uint32_t) (kk * RSTRIDE + (((b * 2 + ((n & 3) >> 1)) ^ swz(kk)) * 16) + (n & 1) * 8);
 
-    const int64_t nt = jb < je ? (je - jb + MTILE - 1) / MTILE : 0;
-    if (nt > 0) {
-        fetch(0, 0, H1);
-        stash(0, 0, H1);
-        fetch(0, H1, NLD);
-        stash(0, H1, NLD);
-    }
-    __syncthreads();
-    for (int it = 0; it < (int) nt; ++it) {
-        const int buf = it & 1;
-        const bool more = it + 1 < (int) nt;
-        if (more) fetch(it + 1, 0, H1);
-        const uint32_t tile = (uint32_t) buf * TILEB;
+    // Half rows go global -> LDS directly (global_load_lds_dwordx4: no register in between, so a tile can be two tiles
+    // ahead of the math at no cost in registers). An instruction's 64 lanes fill 64 consecutive 16-byte units of the
+    // buffer, so the swizzle is applied on the source side: unit u = 72 r + x holds chunk x ^ g(r) of row r. A wave
+    // issues NDMA instructions a tile (units 512 i + 64 w + lane; the last 256 units are fetched twice, by waves w and
+    // w + 4, so that every wave has the same count in flight).
+    constexpr int NU = MTILE * 72, NDMA = (NU + MW * 64 - 1) / (MW * 64);
+    auto dma = [&](lds_u8* dst, int it_) {
+        const bool plain = (it_ + 1) * MTILE - 1 <= last_rel;
+        const uint8_t* sp = split_base + (plain ? (int64_t) it_ * MTILE * CROW : 0);
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) {
+            const int u0 = i * MW * 64 + w * 64 < NU ? i * MW * 64 + w * 64 : i * MW * 64 + (w & 3) * 64;
+            const int u = u0 + lane, r = u / 72, c = (u % 72) ^ swz(r);
+            const uint32_t off = (uint32_t) ((plain ? r : std::min(it_ * MTILE + r, last_rel)) * (int) CROW + c * 16);
+            if (CPR == 72 || c < CPR)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (sp + off),
+                                                 (__attribute__((address_space(3))) void*) (dst + u0 * 16), 16, 0, 0);
+        }
+    };
+
+    // One tile: rd holds it, nx1 / nx2 are the buffers of the next two. Half rows: tile it + 2 is requested before the
+    // math and tile it + 1 (requested a tile ago) is waited for after it - by every wave for its own transfers, then
+    // the barrier makes them everybody's. q8 rows: tile it + 1 is fetched, widened and written in two phases around
+    // the math.
+    const int nt = jb < je ? (int) ((je - jb + MTILE - 1) / MTILE) : 0;
+    auto step = [&](lds_u8* rd, lds_u8* nx1, lds_u8* nx2, int it) {
+        const bool more = it + 1 < nt;
+        if constexpr (Q8) {
+            if (more) fetch(it + 1, 0, H1);
+        } else {
+            if (it + 2 < nt) dma(nx2, it + 2);
+        }
         // ---- S^T = C Q^T
         f4v s[2];
 #pragma unroll
@@ -193,7 +217,7 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
             f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
-                const s8v a = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + tile + s_rd[kb & 1] + ct * 16 * RSTRIDE + (kb >> 1) * 128);
+                const s8v a = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(rd + s_rd[kb & 1] + ct * 16 * RSTRIDE + (kb >> 1) * 128);
                 acc = mfma16<false>(a, qreg[kb], acc);
             }
             s[ct] = acc;
@@ -206,7 +230,7 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
         s8v pb;
         {
             float a[8];
-            const int hi = hi_rel - it * MTILE;            // cells 0 .. hi of this tile are the row's
+            const int hi = hi_rel - it * MTILE;                    // cells 0 .. hi of this tile are the row's
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const int j = (e >> 2) * 16 + g4 * 4 + (e & 3);
@@ -235,21 +259,58 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
             }
             l_r += sum;
         }
-        if (more) {
-            stash(buf ^ 1, 0, H1);
-            fetch(it + 1, H1, NLD);
+        if constexpr (Q8) {
+            if (more) {
+                stash(nx1, 0, H1);
+                fetch(it + 1, H1, NLD);
+            }
         }
         // ---- O^T += C^T P^T
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            const uint32_t src = tile + v_rd[dt & 3] + (dt >> 2) * 128;
-            const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + src));
-            const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + src + 16 * RSTRIDE));
+            const lds_u8* src = rd + v_rd[dt & 3] + (dt >> 2) * 128;
+            const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) src);
+            const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (src + 16 * RSTRIDE));
             const s8v va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             o[dt] = mfma16<false>(va, pb, o[dt]);
         }
-        if (more) stash(buf ^ 1, H1, NLD);
+        if constexpr (Q8) {
+            if (more) stash(nx1, H1, NLD);
+            __syncthreads();
+        } else {
+            // this wave's transfers of tile it + 1 are done when at most tile it + 2's are still in flight; a bare
+            // barrier then (the fence of __syncthreads would wait for tile it + 2 as well)
+            if (it + 2 < nt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        }
+    };
+    if (nt > 0) {
+        if constexpr (Q8) {
+            fetch(0, 0, H1);
+            stash(B0, 0, H1);
+            fetch(0, H1, NLD);
+            stash(B0, H1, NLD);
+        } else {
+            dma(B0, 0);
+            if (nt > 1) dma(B1, 1);
+            if (nt > 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+    }
+    if constexpr (Q8) {
         __syncthreads();
+    } else {
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    }
+    for (int it = 0; it < nt; it += 3) {
+        step(B0, B1, B2, it);
+        if (it + 1 >= nt) break;
+        step(B1, B2, B0, it + 1);
+        if (it + 2 >= nt) break;
+        step(B2, B0, B1, it + 2);
     }
 
     // ---- the split's partial, straight from the registers: a lane holds latents 16 dt + 4 g4 .. + 3 of its row
