@@ -210,17 +210,34 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
         } else {
             if (it + 2 < nt) dma(nx2, it + 2);
         }
-        // ---- S^T = C Q^T
-        f4v s[2];
+        // ---- S^T = C Q^T: the two cell tiles' chains alternate, operands read a few steps ahead of their use
+        f4v s[2] = {f4v{0.0f, 0.0f, 0.0f, 0.0f}, f4v{0.0f, 0.0f, 0.0f, 0.0f}};
+        {
+            auto ld = [&](int kb, int ct) {
+                return *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(rd + s_rd[kb & 1] + ct * 16 * RSTRIDE + (kb >> 1) * 128);
+            };
+            constexpr int AHEAD = 1;                               // kb steps (two reads each) in flight
+            s8v fa[AHEAD + 1][2];
 #pragma unroll
-        for (int ct = 0; ct < 2; ++ct) {
-            f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (int kb = 0; kb < AHEAD; ++kb) {
+                fa[kb][0] = ld(kb, 0);
+                fa[kb][1] = ld(kb, 1);
+            }
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
-                const s8v a = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(rd + s_rd[kb & 1] + ct * 16 * RSTRIDE + (kb >> 1) * 128);
-                acc = mfma16<false>(a, qreg[kb], acc);
+                if (kb + AHEAD < KB) {
+                    fa[(kb + AHEAD) % (AHEAD + 1)][0] = ld(kb + AHEAD, 0);
+                    fa[(kb + AHEAD) % (AHEAD + 1)][1] = ld(kb + AHEAD, 1);
+                }
+                s[0] = mfma16<false>(fa[kb % (AHEAD + 1)][0], qreg[kb], s[0]);
+                s[1] = mfma16<false>(fa[kb % (AHEAD + 1)][1], qreg[kb], s[1]);
             }
-            s[ct] = acc;
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * AHEAD, 0);
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                if (kb + AHEAD < KB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            }
         }
         // ---- softmax of this lane's row, in base-2 exponent units. The reference the weights are taken against (minus
         // it: nbr) moves - and the 128 accumulators are rescaled - only when some score of the wave outgrows it by more
@@ -265,14 +282,29 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
                 fetch(it + 1, H1, NLD);
             }
         }
-        // ---- O^T += C^T P^T
+        // ---- O^T += C^T P^T, the transposed reads two steps ahead of their use
+        {
+            auto ldt = [&](int dt) {
+                const lds_u8* src = rd + v_rd[dt & 3] + (dt >> 2) * 128;
+                const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) src);
+                const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (src + 16 * RSTRIDE));
+                return s8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            };
+            constexpr int AHEAD = 2;
+            s8v va[AHEAD + 1];
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const lds_u8* src = rd + v_rd[dt & 3] + (dt >> 2) * 128;
-            const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) src);
-            const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (src + 16 * RSTRIDE));
-            const s8v va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-            o[dt] = mfma16<false>(va, pb, o[dt]);
+            for (int dt = 0; dt < AHEAD; ++dt) va[dt] = ldt(dt);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                if (dt + AHEAD < DT) va[(dt + AHEAD) % (AHEAD + 1)] = ldt(dt + AHEAD);
+                o[dt] = mfma16<false>(va[dt % (AHEAD + 1)], pb, o[dt]);
+            }
+            __builtin_amdgcn_sched_group_barrier(0x100, 2 * AHEAD, 0);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                if (dt + AHEAD < DT) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            }
         }
         if constexpr (Q8) {
             if (more) stash(nx1, H1, NLD);
