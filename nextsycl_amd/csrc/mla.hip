@@ -359,26 +359,29 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
     }
 }
 
-// the splits of a row merged: u = sum O_s 2^(m_s - M) / sum l_s 2^(m_s - M); a work-group of 512 threads a row
+// the splits of a row merged: u = sum O_s 2^(m_s - M) / sum l_s 2^(m_s - M). Two work-groups of 256 threads a row, 256
+// latents each: a thread sums 4 latents (one 16-byte load a split) over every fourth split, then the four phases are
+// added in a fixed order.
 template <int QT>
-__global__ __launch_bounds__(ML) void mla_merge_kernel(const float* __restrict__ part, int ns, void* __restrict__ u) {
+__global__ __launch_bounds__(256) void mla_merge_kernel(const float* __restrict__ part, int ns, void* __restrict__ u) {
     __shared__ float wsh[1024];
-    __shared__ float red[ML];
+    __shared__ float red[256];
+    __shared__ f4v ph[256];
     const int64_t row = blockIdx.x;
     const int tid = threadIdx.x;
     const float* pr = part + row * ns * PSTRIDE;
     float mx = -INFINITY;
-    for (int s = tid; s < ns; s += ML) mx = fmaxf(mx, pr[s * PSTRIDE + ML]);
+    for (int s = tid; s < ns; s += 256) mx = fmaxf(mx, pr[s * PSTRIDE + ML]);
     red[tid] = mx;
     __syncthreads();
-    for (int o = ML / 2; o > 0; o >>= 1) {
+    for (int o = 128; o > 0; o >>= 1) {
         if (tid < o) red[tid] = fmaxf(red[tid], red[tid + o]);
         __syncthreads();
     }
     mx = red[0];
     __syncthreads();
     float ls = 0.0f;
-    for (int s = tid; s < ns; s += ML) {
+    for (int s = tid; s < ns; s += 256) {
         const float m = pr[s * PSTRIDE + ML];
         const float wgt = m == -INFINITY ? 0.0f : fast_exp2(m - mx);
         wsh[s] = wgt;
@@ -386,15 +389,23 @@ __global__ __launch_bounds__(ML) void mla_merge_kernel(const float* __restrict__
     }
     red[tid] = ls;
     __syncthreads();
-    for (int o = ML / 2; o > 0; o >>= 1) {
+    for (int o = 128; o > 0; o >>= 1) {
         if (tid < o) red[tid] += red[tid + o];
         __syncthreads();
     }
     const float L = red[0];
-    float acc = 0.0f;
+    const int quad = tid & 63, phase = tid >> 6;
+    const int lat = blockIdx.y * 256 + quad * 4;
+    f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll 8
-    for (int s = 0; s < ns; ++s) acc += pr[s * PSTRIDE + tid] * wsh[s];
-    store_o<QT>(u, row * ML + tid, L > 0.0f ? acc / L : 0.0f);
+    for (int s = phase; s < ns; s += 4) acc += *reinterpret_cast<const f4v*>(pr + s * PSTRIDE + lat) * wsh[s];
+    ph[tid] = acc;
+    __syncthreads();
+    if (phase == 0) {
+        const f4v t = ((ph[quad] + ph[64 + quad]) + ph[128 + quad]) + ph[192 + quad];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) store_o<QT>(u, row * ML + lat + i, L > 0.0f ? t[i] / L : 0.0f);
+    }
 }
 
 // q~ = k_b q_nope: qa [T][H][L + R] = [k_b[h] q[t][h][:nope] | q[t][h][nope:]]; a work-group a (row, head), a thread two
@@ -575,8 +586,8 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     else mla_decode_kernel<0, false><<<grid, MW * 64, 0, g->q>>>(p);
     NS_LAUNCHED("mla_decode");
     if (ns_profile_mark(g, 1)) return -1;
-    if (ot == 0) mla_merge_kernel<0><<<(unsigned) rows, ML, 0, g->q>>>(scratch, (int) ns, u);
-    else mla_merge_kernel<1><<<(unsigned) rows, ML, 0, g->q>>>(scratch, (int) ns, u);
+    if (ot == 0) mla_merge_kernel<0><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
+    else mla_merge_kernel<1><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
     NS_LAUNCHED("mla_merge");
     return ns_profile_mark(g, 2);
 }
