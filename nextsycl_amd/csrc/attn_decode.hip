@@ -507,7 +507,7 @@ int64_t target_wgs() {
     static const int64_t v = [] {
         const char* e = getenv("NS_DEC_WGS");
         const int64_t x = e ? atoll(e) : 0;
-        return x > 0 ? x : 1024;
+        return x > 0 ? x : 512;
     }();
     return v;
 }
