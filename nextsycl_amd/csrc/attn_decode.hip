@@ -119,61 +119,6 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     const int64_t fmin = p.win > 0 ? std::max<int64_t>(0, p.p0 + 1 - p.win) : 0;
     const int64_t jb = std::max((p.sp0 + split) * p.kbs, fmin), je = std::min((p.sp0 + split + 1) * p.kbs, pass_end);
 
-    // ---- this lane's rows (one per row tile): their key ranges and Q^T operands
-    int64_t lo_r[RT], hi_r[RT];
-    s8v qreg[RT][KB];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-        const int ri = (z * RT + rt) * 16 + n;
-        const bool live = ri < rows;
-        const int t = live ? ri / p.G : 0, gq = live ? ri % p.G : 0;
-        const int64_t pos = p.p0 + t, first = p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0;
-        lo_r[rt] = live ? std::max(first, jb) : 1;
-        hi_r[rt] = live ? std::min(p.causal ? pos : pass_end - 1, je - 1) : 0;
-        // 8 consecutive features per k-block, vector loads all issued before any is used (rows are 16-byte aligned:
-        // checked on the host); a dead row reads row 0's and is zeroed
-        const int64_t qoff = (int64_t) t * p.qs + ((int64_t) hk * p.G + gq) * D + g4 * 8;
-        if (p.qt == 0) {
-            float4 raw[KB][2];
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) {
-                raw[kb][0] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.q) + qoff + kb * 32);
-                raw[kb][1] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.q) + qoff + kb * 32 + 4);
-            }
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) {
-                const float f[8] = {raw[kb][0].x, raw[kb][0].y, raw[kb][0].z, raw[kb][0].w, raw[kb][1].x, raw[kb][1].y, raw[kb][1].z, raw[kb][1].w};
-#pragma unroll
-                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = live ? to16<BF>(f[i]) : (short) 0;
-            }
-        } else {
-            uint4 raw[KB];
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) raw[kb] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.q) + qoff + kb * 32);
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) {
-                const uint32_t ww[4] = {raw[kb].x, raw[kb].y, raw[kb].z, raw[kb].w};
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const uint16_t b16 = (uint16_t) (ww[i >> 1] >> (16 * (i & 1)));
-                    // the same 16-bit type as the kernel's operands passes through; the other is converted
-                    const short v = (p.qt == 2) == BF ? (short) b16 : to16<BF>(p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16));
-                    qreg[rt][kb][i] = live ? v : (short) 0;
-                }
-            }
-        }
-    }
-
-    float m_r[RT], l_r[RT];
-    f4v o[RT][DT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-        m_r[rt] = -INFINITY;
-        l_r[rt] = 0.0f;
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) o[rt][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-
     const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
     const uint8_t* vbase = p.vc + (int64_t) hk * p.head_stride;
     uint8_t* stage = lds + w * STAGE;
@@ -230,6 +175,68 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             }
         }
     };
+
+    // ---- this wave's tiles: absolute tile index % 4 == w, over [jb, je). The first one is requested before anything
+    // else: nothing in it depends on the queries
+    const int64_t tb = jb / TILE, te = jb < je ? (je + TILE - 1) / TILE : tb;
+    int64_t ti = tb + ((w - (int) (tb % WAVES) + WAVES) % WAVES);
+    R ra, rb;
+    if (ti < te) load_tile(ra, ti, 0);
+
+    // ---- this lane's rows (one per row tile): their key ranges and Q^T operands
+    int64_t lo_r[RT], hi_r[RT];
+    s8v qreg[RT][KB];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int ri = (z * RT + rt) * 16 + n;
+        const bool live = ri < rows;
+        const int t = live ? ri / p.G : 0, gq = live ? ri % p.G : 0;
+        const int64_t pos = p.p0 + t, first = p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0;
+        lo_r[rt] = live ? std::max(first, jb) : 1;
+        hi_r[rt] = live ? std::min(p.causal ? pos : pass_end - 1, je - 1) : 0;
+        // 8 consecutive features per k-block, vector loads all issued before any is used (rows are 16-byte aligned:
+        // checked on the host); a dead row reads row 0's and is zeroed
+        const int64_t qoff = (int64_t) t * p.qs + ((int64_t) hk * p.G + gq) * D + g4 * 8;
+        if (p.qt == 0) {
+            float4 raw[KB][2];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                raw[kb][0] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.q) + qoff + kb * 32);
+                raw[kb][1] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.q) + qoff + kb * 32 + 4);
+            }
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const float f[8] = {raw[kb][0].x, raw[kb][0].y, raw[kb][0].z, raw[kb][0].w, raw[kb][1].x, raw[kb][1].y, raw[kb][1].z, raw[kb][1].w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = live ? to16<BF>(f[i]) : (short) 0;
+            }
+        } else {
+            uint4 raw[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) raw[kb] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.q) + qoff + kb * 32);
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                const uint32_t ww[4] = {raw[kb].x, raw[kb].y, raw[kb].z, raw[kb].w};
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint16_t b16 = (uint16_t) (ww[i >> 1] >> (16 * (i & 1)));
+                    // the same 16-bit type as the kernel's operands passes through; the other is converted
+                    const short v = (p.qt == 2) == BF ? (short) b16 : to16<BF>(p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16));
+                    qreg[rt][kb][i] = live ? v : (short) 0;
+                }
+            }
+        }
+    }
+
+    float m_r[RT], l_r[RT];
+    f4v o[RT][DT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        m_r[rt] = -INFINITY;
+        l_r[rt] = 0.0f;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[rt][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    }
 
     // MORE: how many tiles' loads were issued after this tile's (0 or 1) - what the DMA wait may leave in flight
     auto process_tile = [&](R& r, int64_t ti, int buf, auto more_c) {
@@ -369,30 +376,24 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         asm volatile("" ::: "memory");
     };
 
-    // ---- this wave's tiles: absolute tile index % 4 == w, over [jb, je). The steady state is its own loop so that
-    // every wait in it knows exactly which loads were issued after the ones it needs
-    if (jb < je) {
-        const int64_t tb = jb / TILE, te = (je + TILE - 1) / TILE;
-        int64_t ti = tb + ((w - (int) (tb % WAVES) + WAVES) % WAVES);
-        if (ti < te) {
-            R ra, rb;
-            const std::true_type more;
-            const std::false_type last;
-            load_tile(ra, ti, 0);
-            while (ti + 2 * WAVES < te) {
-                load_tile(rb, ti + WAVES, 1);
-                process_tile(ra, ti, 0, more);
-                load_tile(ra, ti + 2 * WAVES, 0);
-                process_tile(rb, ti + WAVES, 1, more);
-                ti += 2 * WAVES;
-            }
-            if (ti + WAVES < te) {
-                load_tile(rb, ti + WAVES, 1);
-                process_tile(ra, ti, 0, more);
-                process_tile(rb, ti + WAVES, 1, last);
-            } else {
-                process_tile(ra, ti, 0, last);
-            }
+    // ---- the wave's tiles. The steady state is its own loop so that every wait in it knows exactly which loads were
+    // issued after the ones it needs
+    if (ti < te) {
+        const std::true_type more;
+        const std::false_type last;
+        while (ti + 2 * WAVES < te) {
+            load_tile(rb, ti + WAVES, 1);
+            process_tile(ra, ti, 0, more);
+            load_tile(ra, ti + 2 * WAVES, 0);
+            process_tile(rb, ti + WAVES, 1, more);
+            ti += 2 * WAVES;
+        }
+        if (ti + WAVES < te) {
+            load_tile(rb, ti + WAVES, 1);
+            process_tile(ra, ti, 0, more);
+            process_tile(rb, ti + WAVES, 1, last);
+        } else {
+            process_tile(ra, ti, 0, last);
         }
     }
 
