@@ -354,24 +354,40 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
         weigh(V0 + (uint32_t) ((nt - 1) & 1) * VBUF + 32 * VS);
     }
 
-    // ---- out = O / l; a lane holds dims 16 dt + 4 g4 .. + 3 of its rows
+    // ---- out = O / l. A lane holds dims 16 dt + 4 g4 .. + 3 of its rows: the wave's 32 x D block goes through LDS (the
+    // tile buffers, free now) so that it leaves as whole rows, 16 bytes a lane and 4 (float32: 2) rows an instruction
+    __syncthreads();                                              // every wave is done with the tiles
+    {
+        const int esz = p.qt == 0 ? 4 : 2;
+        const uint32_t rowb = (uint32_t) (D * esz), rowp = rowb + 16;    // bytes a row, padded in LDS
+        const uint32_t ob = (uint32_t) w * 32 * (D * 4 + 16);
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-        const int row = r0 + w * 32 + rt * 16 + n;
-        const float lsum = rows_sum(l_r[rt]);                 // every lane takes part, dead rows too
-        if (row >= p.T) continue;
-        const float inv = lsum > 0.0f ? 1.0f / lsum : 0.0f;
-        const int64_t at = ((int64_t) row * p.Hq + hq) * D + g4 * 4;
+        for (int rt = 0; rt < 2; ++rt) {
+            const float lsum = rows_sum(l_r[rt]);
+            const float inv = lsum > 0.0f ? 1.0f / lsum : 0.0f;
+            const uint32_t at = ob + (uint32_t) (rt * 16 + n) * rowp + (uint32_t) (g4 * 4 * esz);
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const f4v v = o[rt][dt] * inv;
-            if (p.qt == 0) {
-                *reinterpret_cast<f4v*>(reinterpret_cast<float*>(p.out) + at + dt * 16) = v;
-            } else {
-                ushort4 h;
-                if (p.qt == 1) h = make_ushort4(f32_to_f16(v[0]), f32_to_f16(v[1]), f32_to_f16(v[2]), f32_to_f16(v[3]));
-                else h = make_ushort4(f32_to_bf16(v[0]), f32_to_bf16(v[1]), f32_to_bf16(v[2]), f32_to_bf16(v[3]));
-                *reinterpret_cast<ushort4*>(reinterpret_cast<uint16_t*>(p.out) + at + dt * 16) = h;
+            for (int dt = 0; dt < DT; ++dt) {
+                const f4v v = o[rt][dt] * inv;
+                if (p.qt == 0) {
+                    *reinterpret_cast<__attribute__((address_space(3))) f4v*>(L + at + dt * 64) = v;
+                } else {
+                    typedef uint16_t us4v __attribute__((ext_vector_type(4)));
+                    us4v h;
+                    if (p.qt == 1) h = us4v{f32_to_f16(v[0]), f32_to_f16(v[1]), f32_to_f16(v[2]), f32_to_f16(v[3])};
+                    else h = us4v{f32_to_bf16(v[0]), f32_to_bf16(v[1]), f32_to_bf16(v[2]), f32_to_bf16(v[3])};
+                    *reinterpret_cast<__attribute__((address_space(3))) us4v*>(L + at + dt * 32) = h;
+                }
+            }
+        }
+        // the wave reads back its own block only: no barrier, the LDS queue keeps a wave's accesses in order
+        const int ppr = (int) rowb / 16;                          // 16-byte pieces a row
+        uint8_t* const orow = reinterpret_cast<uint8_t*>(p.out) + (int64_t) hq * rowb;
+        for (int c = lane; c < 32 * ppr; c += 64) {
+            const int rl_ = c / ppr, piece = c % ppr, row = r0 + w * 32 + rl_;
+            if (row < p.T) {
+                const u4v x = *reinterpret_cast<const __attribute__((address_space(3))) u4v*>(L + ob + (uint32_t) rl_ * rowp + (uint32_t) piece * 16);
+                *reinterpret_cast<u4v*>(orow + (int64_t) row * p.Hq * rowb + piece * 16) = x;
             }
         }
     }
