@@ -73,12 +73,25 @@ MLA_H = {
 }
 
 
+# include/ns_pre.h
+PRE_H = {
+    "ns_q35_qk_norm_rope": (i32, [P, P, i64, i64, P, i64, i64, i64, i64, P, f32, i64, f32, i64]),
+    "ns_q35_qk_norm_rope_pos": (i32, [P, P, i64, i64, P, i64, i64, i64, i64, P, f32, i64, f32, P, i64, i64, i64]),
+    "ns_q35_rope": (i32, [P, P, i64, i64, P, i64, i64, i64, i64, i64, f32, i64]),
+    "ns_mg_qk_norm_rope": (i32, [P, P, i64, P, i64, i64, i64, i64, P, f32, i32, f32, i64]),
+    "ns_llm_minimaxm3_rope": (i32, [P, P, i64, i64, i64, i64, i64, i64, f32]),
+    "ns_mm3s_attn_post": (i32, [P, P, P, P, P, P, P, P, P, P, P, P, P, i64, i64, i64, i64, i64, i64, f32, f32]),
+    "ns_attn_pre_store": (i32, [P, i32, i32, i32, i32, P, i64, i64, P, i64, P, i64, i64, P, i64, P, P, f32, i64, f32, i64, i64, i64, i64, i64, i64,
+                                P, P]),
+}
+
+
 class Kernels:
     """Every attention entry point bound by name; a missing symbol fails the load."""
 
     def __init__(self, a=None):
         self.api = a or api()
-        for name, (res, args) in list(ATTN_H.items()) + list(MLA_H.items()):
+        for name, (res, args) in list(ATTN_H.items()) + list(MLA_H.items()) + list(PRE_H.items()):
             setattr(self, name[3:], self.api.symbol(name, res, args))
 
 
@@ -302,3 +315,56 @@ class Ops:
         _need(kc, (pos0 + T) * G * 128 * 2, "attend key cache")
         _need(vc, (pos0 + T) * G * 128 * 2, "attend value cache")
         self.ok(self.k.llm_minimaxm3_attend(self.raw(), q.ptr, kc.ptr, vc.ptr, None, 0, out.ptr, T, H, G, pos0, scale), "attend")
+
+    # ---- the step in front of attention: norm, rotary positions, store
+    def q35_qk_norm_rope(self, src, ss, hs, dst, ds, T, H, D, w, eps, n_rot, theta, p0, pos3=None, sections=(0, 0, 0)):
+        """ns_q35_qk_norm_rope (pos3 None) / ns_q35_qk_norm_rope_pos / ns_q35_rope (w None): float32 rows."""
+        _need(src, ((T - 1) * ss + (H - 1) * hs + D) * 4, "qk_norm_rope src")
+        _need(dst, ((T - 1) * ds + H * D) * 4, "qk_norm_rope dst")
+        if w is None:
+            return self.ok(self.k.q35_rope(self.raw(), src.ptr, ss, hs, dst.ptr, ds, T, H, D, n_rot, theta, p0), "q35_rope")
+        _need(w, D * 4, "qk_norm_rope weight")
+        if pos3 is None:
+            return self.ok(self.k.q35_qk_norm_rope(self.raw(), src.ptr, ss, hs, dst.ptr, ds, T, H, D, w.ptr, eps, n_rot, theta, p0), "q35_qk_norm_rope")
+        _need(pos3, T * 3 * 4, "qk_norm_rope positions")
+        self.ok(self.k.q35_qk_norm_rope_pos(self.raw(), src.ptr, ss, hs, dst.ptr, ds, T, H, D, w.ptr, eps, n_rot, theta, pos3.ptr, *sections),
+                "q35_qk_norm_rope_pos")
+
+    def mg_qk_norm_rope(self, x, xs, y, ys, T, H, D, w, eps, rope, theta, p0):
+        _need(x, ((T - 1) * xs + H * D) * 4, "mg_qk_norm_rope x")
+        _need(y, ((T - 1) * ys + H * D) * 4, "mg_qk_norm_rope y")
+        _need(w, D * 4, "mg_qk_norm_rope weight")
+        self.ok(self.k.mg_qk_norm_rope(self.raw(), x.ptr, xs, y.ptr, ys, T, H, D, w.ptr, eps, rope, theta, p0), "mg_qk_norm_rope")
+
+    def minimaxm3_rope(self, x, T, H, row, head, n_rot, pos0, base):
+        _need(x, ((T - 1) * row + H * head) * 4, "minimaxm3_rope x")
+        self.ok(self.k.llm_minimaxm3_rope(self.raw(), x.ptr, T, H, row, head, n_rot, pos0, base), "minimaxm3_rope")
+
+    def mm3s_attn_post(self, q, k, v, iq, ik, qn, kn, iqn, ikn, kc, vc, ic, H, G, IH, HD, n_rot, pos, base, eps):
+        """kc, vc, ic: (buffer, byte offset of the token's row). iq / ik / iqn / ikn / ic None when IH == 0."""
+        _need(q, H * HD * 4, "attn_post q")
+        _need(k, G * HD * 4, "attn_post k")
+        _need(v, G * HD * 4, "attn_post v")
+        _need(qn, HD * 4, "attn_post q weight")
+        _need(kn, HD * 4, "attn_post k weight")
+        for (b, off), n, what in ((kc, G * HD * 2, "kc"), (vc, G * HD * 2, "vc")) + (((ic, HD * 2, "ic"),) if IH > 0 else ()):
+            _need(b, off + n, "attn_post " + what)
+        if IH > 0:
+            _need(iq, IH * HD * 4, "attn_post iq")
+            _need(ik, HD * 4, "attn_post ik")
+        opt = lambda b: b.ptr if b is not None else None
+        self.ok(self.k.mm3s_attn_post(self.raw(), q.ptr, k.ptr, v.ptr, opt(iq), opt(ik), qn.ptr, kn.ptr, opt(iqn), opt(ikn), kc[0].ptr + kc[1],
+                                      vc[0].ptr + vc[1], (ic[0].ptr + ic[1]) if IH > 0 else None, H, G, IH, HD, n_rot, pos, base, eps), "mm3s_attn_post")
+
+    def pre_store(self, rope, qt, kt, ring, q, qss, qhs, qo, qos, k, kss, khs, v, vss, qw, kw, eps, n_rot, theta, T, Hq, Hkv, D, cap, p0, kc, vc):
+        """ns_attn_pre_store: q normed + rotated into qo, k normed + rotated + v written into the caches, one launch."""
+        _need(q, ((T - 1) * qss + (Hq - 1) * qhs + D) * 4, "pre_store q")
+        _need(qo, ((T - 1) * qos + Hq * D) * ELT[qt], "pre_store q out")
+        _need(k, ((T - 1) * kss + (Hkv - 1) * khs + D) * 4, "pre_store k")
+        _need(v, ((T - 1) * vss + Hkv * D) * 4, "pre_store v")
+        _need(qw, D * 4, "pre_store q weight")
+        _need(kw, D * 4, "pre_store k weight")
+        _need(kc, self.cache_bytes(kt, Hkv, cap, D), "pre_store kc")
+        _need(vc, self.cache_bytes(kt, Hkv, cap, D), "pre_store vc")
+        self.ok(self.k.attn_pre_store(self.raw(), rope, qt, kt, int(ring), q.ptr, qss, qhs, qo.ptr, qos, k.ptr, kss, khs, v.ptr, vss, qw.ptr, kw.ptr, eps,
+                                      n_rot, theta, T, Hq, Hkv, D, cap, p0, kc.ptr, vc.ptr), "pre_store")

@@ -22,6 +22,7 @@ COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-ta
 SOURCES = {
     "ns_hip.cpp": [],
     "kv_store.hip": ["-ffp-contract=off"],
+    "pre_attn.hip": ["-ffp-contract=off"],
     "attn_decode.hip": [],
     "attn_prefill.hip": [],
     "attn_api.cpp": [],

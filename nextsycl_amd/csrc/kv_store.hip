@@ -9,6 +9,7 @@
 #include "ns_internal.hpp"
 #include "ns_attn.h"
 #include "kv_formats.hpp"
+#include "kv_pack.hpp"
 
 namespace {
 
@@ -35,11 +36,7 @@ __global__ void kv_store16_kernel(const float* __restrict__ k, int64_t ks, const
     *reinterpret_cast<ushort4*>(vc + at) = vo;
 }
 
-// ---- q8_0 / q4_0 stores: 8 lanes a block of 32 values (a lane 4 consecutive floats), the block's largest magnitude
-// over the 8 lanes by xor-shuffles (max is exact in any order). q8_0: a lane writes its 4 int8 as one word. q4_0: the
-// block's signed extreme is the value of the largest magnitude, the FIRST of a tie - the lanes carry (magnitude,
-// index) and keep the lower index on equal magnitudes; byte j pairs value j with value j + 16, so a lane's 4 low
-// nibbles meet lane + 4's 4 high nibbles through a shuffle.
+// ---- q8_0 / q4_0 stores: 8 lanes a block of 32 values (a lane 4 consecutive floats); the packers are kv_pack.hpp's
 template <int KT>
 __global__ void kv_store_q_kernel(const float* __restrict__ k, int64_t ks, const float* __restrict__ v, int64_t vs, int64_t T, int64_t Hkv,
                                   int64_t D, int64_t cap, int64_t p0, uint8_t* __restrict__ kc, uint8_t* __restrict__ vc) {
@@ -60,43 +57,17 @@ __global__ void kv_store_q_kernel(const float* __restrict__ k, int64_t ks, const
     uint8_t* row = (isv ? vc : kc) + (h * cap + p0 + t) * rb;
     const float4 xv = *reinterpret_cast<const float4*>(x);
     const float xs[4] = {xv.x, xv.y, xv.z, xv.w};
+    float d;
     if (KT == 1) {
-        float amax = fmaxf(fmaxf(fabsf(xs[0]), fabsf(xs[1])), fmaxf(fabsf(xs[2]), fabsf(xs[3])));
-        amax = fmaxf(amax, __shfl_xor(amax, 1));
-        amax = fmaxf(amax, __shfl_xor(amax, 2));
-        amax = fmaxf(amax, __shfl_xor(amax, 4));
-        const float d = amax / 127.0f, id = d != 0.0f ? 1.0f / d : 0.0f;
-        uint32_t w = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) w |= (uint32_t) (uint8_t) (int8_t) roundf(xs[j] * id) << (8 * j);
+        const uint32_t w = q8_0_pack4(xs, d);
         if (live) {
             *reinterpret_cast<uint32_t*>(row + b * 32 + ln * 4) = w;
             if (ln == 0) *reinterpret_cast<uint16_t*>(row + D + 2 * b) = f32_to_f16(d);
         }
     } else {
-        float am = 0.0f, m = 0.0f;
-        int at = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (fabsf(xs[j]) > am) { am = fabsf(xs[j]); m = xs[j]; at = ln * 4 + j; }
-        if (am == 0.0f) at = 32;   // no value yet: loses every tie
-#pragma unroll
-        for (int o = 1; o < 8; o <<= 1) {
-            const float am2 = __shfl_xor(am, o), m2 = __shfl_xor(m, o);
-            const int at2 = __shfl_xor(at, o);
-            if (am2 > am || (am2 == am && at2 < at)) { am = am2; m = m2; at = at2; }
-        }
-        const float d = m / -8.0f, id = d != 0.0f ? 1.0f / d : 0.0f;
-        uint32_t nib = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            int qv = (int) (xs[j] * id + 8.5f);
-            qv = qv > 15 ? 15 : qv;
-            nib |= (uint32_t) qv << (8 * j);
-        }
-        const uint32_t hi = __shfl_xor(nib, 4);   // lanes 0..3 hold values 0..15 (low nibbles), 4..7 values 16..31
+        const uint32_t w = q4_0_pack4(xs, ln, d);
         if (live && ln < 4) {
-            *reinterpret_cast<uint32_t*>(row + b * 16 + ln * 4) = nib | (hi << 4);
+            *reinterpret_cast<uint32_t*>(row + b * 16 + ln * 4) = w;
             if (ln == 0) *reinterpret_cast<uint16_t*>(row + D / 2 + 2 * b) = f32_to_f16(d);
         }
     }

@@ -1,0 +1,331 @@
+// pre_attn.hip: what runs in front of attention on every token - q / k RMS norm, rotary positions, the KV store - for
+// gfx950: the reference's separate entry points and one fused launch (norm + rotate + store, k never written as
+// float32). Bound: HBM, negligible volume (a few KB a token); the point of the fused form is two launches fewer a layer.
+//
+// One wave a (row, head); a lane four consecutive features (D up to 256; more: a lane several groups of four). Every
+// load of a wave precedes its stores, so source and destination may be the same rows. The arithmetic of an output
+// feature is one function (rope_feature) whatever entry point asks for it, and the quantized rows are kv_pack.hpp's:
+// the fused launch gives bit for bit what the separate calls give. Compiled with -ffp-contract=off (the packers).
+//
+// Reference behaviour kept: kernels/llm/qwen35/q35.cpp:220-279,350-386 (rotate-half over the first n_rot, angle
+// pos * theta^(-2 k / n_rot); interleaved position sections), kernels/llm/museglimmer/mg.cpp:157-190 (adjacent pairs or
+// halves over all D), kernels/llm/minimaxm3/mm3.cpp:18-35 and silo/moe.cpp:460-501 (angle by repeated multiplication,
+// norm as 1 / sqrt).
+#include "ns_internal.hpp"
+#include "ns_pre.h"
+#include "kv_formats.hpp"
+#include "kv_pack.hpp"
+
+#include <cmath>
+
+namespace {
+
+enum { ROPE_NONE = 0, ROPE_Q35 = 1, ROPE_MG_PAIRS = 2, ROPE_MG_HALVES = 3, ROPE_MM3 = 4 };
+// where a group's rows go: float32 / half / bfloat16 rows [t * ds + h * D], or cache rows of form kt
+enum { DST_F32 = 0, DST_F16 = 1, DST_BF16 = 2, DST_CACHE = 8 };
+
+struct PreGroup {
+    int heads;                 // heads of this group in a row t
+    const float* src;
+    int64_t ss, hs;            // floats between rows / heads of src
+    const float* w;            // norm weight [D], or null: no norm
+    int rope;                  // rotate this group
+    void* dst;
+    int64_t ds;                // elements between dst rows (plain destinations)
+    int dt;                    // DST_*; DST_CACHE + kt for cache rows
+    void* dst2;                // a second, half copy of the result (minimaxm3's in-place rows also stored as half), or null
+    int64_t ds2;
+};
+
+struct PreParams {
+    PreGroup gr[5];
+    int ngr;
+    int T, D;
+    int mode, n_rot, inv_sqrt;        // inv_sqrt: 1 / sqrt(..) instead of rsqrt(..)
+    float theta, ts, eps;
+    int64_t p0;
+    const int32_t* pos3;              // [T][3] positions, or null
+    int s0, s1, s2;
+    int64_t cap;
+    int ring;
+};
+
+// output feature i of a head row: v(j) = x[j] * inv * w[j] (or x[j]), rotated as the mode says
+__device__ __forceinline__ float rope_feature(const PreParams& p, const float* x, const float* w, float inv, int i, int t, bool rot) {
+    auto v = [&](int j) { return w ? x[j] * inv * w[j] : x[j]; };
+    const float me = v(i);
+    if (!rot || p.mode == ROPE_NONE) return me;
+    const int D = p.D;
+    if (p.mode == ROPE_Q35) {
+        if (i >= p.n_rot) return me;
+        const int hr = p.n_rot / 2, k = i < hr ? i : i - hr;
+        float pos = (float) (p.p0 + t);
+        if (p.pos3) {
+            const int sect = p.s0 + p.s1 + p.s2, sec = k % sect;
+            const int c = (sec % 3 == 1 && sec < 3 * p.s1) ? 1 : (sec % 3 == 2 && sec < 3 * p.s2) ? 2 : 0;
+            pos = (float) p.pos3[t * 3 + c];
+        }
+        const float a = pos * powf(p.theta, -2.0f * (float) k / (float) p.n_rot);
+        const float c = cosf(a), sn = sinf(a);
+        const float other = v(i < hr ? i + hr : i - hr);
+        return i < hr ? me * c - other * sn : me * c + other * sn;
+    }
+    if (p.mode == ROPE_MG_PAIRS || p.mode == ROPE_MG_HALVES) {
+        const bool halves = p.mode == ROPE_MG_HALVES;
+        const int pr = halves ? (i < D / 2 ? i : i - D / 2) : i / 2;
+        const int i0 = halves ? pr : 2 * pr, i1 = halves ? pr + D / 2 : 2 * pr + 1;
+        const float a = (float) (p.p0 + t) * powf(p.theta, -2.0f * (float) pr / (float) D);
+        const float c = cosf(a), sn = sinf(a);
+        const float a0 = i == i0 ? me : v(i0), a1 = i == i1 ? me : v(i1);
+        return i == i0 ? a0 * c - a1 * sn : a0 * sn + a1 * c;
+    }
+    // ROPE_MM3
+    if (i >= p.n_rot) return me;
+    const int hr = p.n_rot / 2, k = i % hr;
+    float th = (float) (p.p0 + t);
+    for (int j = 0; j < k; ++j) th *= p.ts;
+    const float c = cosf(th), s = sinf(th);
+    const float them = v(i < hr ? i + hr : i - hr);
+    return i < hr ? me * c - them * s : them * s + me * c;
+}
+
+__global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
+    const int lane = threadIdx.x & 63;
+    const int64_t rowid = (int64_t) blockIdx.x * 4 + (threadIdx.x >> 6);
+    int per_t = 0;
+    for (int gi = 0; gi < p.ngr; ++gi) per_t += p.gr[gi].heads;
+    if (rowid >= (int64_t) p.T * per_t) return;            // whole waves leave: no shuffle below misses a lane
+    const int t = (int) (rowid / per_t);
+    int h = (int) (rowid % per_t), gi = 0;
+    while (h >= p.gr[gi].heads) h -= p.gr[gi++].heads;
+    const PreGroup& G = p.gr[gi];
+    const int D = p.D;
+    const float* x = G.src + (int64_t) t * G.ss + (int64_t) h * G.hs;
+    // ---- the row's scale
+    float inv = 1.0f;
+    if (G.w) {
+        float s = 0.0f;
+        for (int i = lane * 4; i < D; i += 256) {
+            const float4 a = *reinterpret_cast<const float4*>(x + i);
+            s += a.x * a.x;
+            s += a.y * a.y;
+            s += a.z * a.z;
+            s += a.w * a.w;
+        }
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) s += __shfl_xor(s, o);
+        const float ms = s / (float) D + p.eps;
+        inv = p.inv_sqrt ? 1.0f / sqrtf(ms) : rsqrtf(ms);
+    }
+    // ---- this lane's features, all computed (every load done) before anything is stored
+    constexpr int MAXG = 2;                                  // D up to 512
+    float y[MAXG][4];
+#pragma unroll
+    for (int c = 0; c < MAXG; ++c) {
+        const int i = lane * 4 + c * 256;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) y[c][j] = i < D ? rope_feature(p, x, G.w, inv, i + j, t, G.rope != 0) : 0.0f;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // loads above, stores below (source may be destination)
+#pragma unroll
+    for (int c = 0; c < MAXG; ++c) {
+        const int i = lane * 4 + c * 256;
+        if (c * 256 >= D) break;
+        const bool live = i < D;
+        if (G.dt < DST_CACHE) {
+            if (!live) continue;
+            const int64_t at = (int64_t) t * G.ds + (int64_t) h * D + i;
+            if (G.dt == DST_F32) {
+                *reinterpret_cast<float4*>(reinterpret_cast<float*>(G.dst) + at) = make_float4(y[c][0], y[c][1], y[c][2], y[c][3]);
+            } else {
+                ushort4 o;
+                if (G.dt == DST_F16) o = make_ushort4(f32_to_f16(y[c][0]), f32_to_f16(y[c][1]), f32_to_f16(y[c][2]), f32_to_f16(y[c][3]));
+                else o = make_ushort4(f32_to_bf16(y[c][0]), f32_to_bf16(y[c][1]), f32_to_bf16(y[c][2]), f32_to_bf16(y[c][3]));
+                *reinterpret_cast<ushort4*>(reinterpret_cast<uint16_t*>(G.dst) + at) = o;
+            }
+            if (G.dst2) {
+                const int64_t at2 = (int64_t) t * G.ds2 + (int64_t) h * D + i;
+                *reinterpret_cast<ushort4*>(reinterpret_cast<uint16_t*>(G.dst2) + at2) =
+                    make_ushort4(f32_to_f16(y[c][0]), f32_to_f16(y[c][1]), f32_to_f16(y[c][2]), f32_to_f16(y[c][3]));
+            }
+        } else {
+            const int kt = G.dt - DST_CACHE;
+            const int64_t slot = p.ring ? (p.p0 + t) % p.cap : p.p0 + t;
+            uint8_t* row = reinterpret_cast<uint8_t*>(G.dst) + ((int64_t) h * p.cap + slot) * kv_row_bytes(kt, D);
+            if (kt == 0 || kt == 3) {
+                if (!live) continue;
+                ushort4 o;
+                if (kt == 0) o = make_ushort4(f32_to_f16(y[c][0]), f32_to_f16(y[c][1]), f32_to_f16(y[c][2]), f32_to_f16(y[c][3]));
+                else o = make_ushort4(f32_to_bf16(y[c][0]), f32_to_bf16(y[c][1]), f32_to_bf16(y[c][2]), f32_to_bf16(y[c][3]));
+                *reinterpret_cast<ushort4*>(row + 2 * i) = o;
+            } else {
+                // 8 lanes a block of 32: every lane takes part in the shuffles (dead lanes carry zeros, store nothing)
+                const int b = i / 32, ln = lane & 7;
+                float d;
+                if (kt == 1) {
+                    const uint32_t wv = q8_0_pack4(y[c], d);
+                    if (live) {
+                        *reinterpret_cast<uint32_t*>(row + i) = wv;
+                        if (ln == 0) *reinterpret_cast<uint16_t*>(row + D + 2 * b) = f32_to_f16(d);
+                    }
+                } else {
+                    const uint32_t wv = q4_0_pack4(y[c], ln, d);
+                    if (live && ln < 4) {
+                        *reinterpret_cast<uint32_t*>(row + b * 16 + ln * 4) = wv;
+                        if (ln == 0) *reinterpret_cast<uint16_t*>(row + D / 2 + 2 * b) = f32_to_f16(d);
+                    }
+                }
+            }
+        }
+    }
+}
+
+int launch_pre(ns_gpu* g, const PreParams& p, const char* who) {
+    NS_HIP(hipSetDevice(g->dev));
+    int64_t rows = 0;
+    for (int i = 0; i < p.ngr; ++i) rows += (int64_t) p.T * p.gr[i].heads;
+    if (rows <= 0) return 0;
+    if ((rows + 3) / 4 > (int64_t) 1 << 31) return ns_fail(std::string(who) + ": too many rows");
+    pre_attn_kernel<<<(unsigned) ((rows + 3) / 4), 256, 0, g->q>>>(p);
+    NS_LAUNCHED(who);
+    return 0;
+}
+
+inline bool al16(const void* p) { return (uintptr_t) p % 16 == 0; }
+
+}  // namespace
+
+extern "C" {
+
+int ns_q35_qk_norm_rope_pos(ns_gpu* g, const float* src, int64_t ss, int64_t hs, float* dst, int64_t ds, int64_t T, int64_t H, int64_t D,
+                            const float* w, float eps, int64_t n_rot, float theta, const int32_t* pos, int64_t s0, int64_t s1, int64_t s2) {
+    NS_TRY
+    if (T <= 0) return 0;
+    if (D % 16 != 0 || D > 512 || n_rot > D || n_rot % 2 || n_rot < 0 || s0 + s1 + s2 <= 0)
+        return ns_fail("ns_q35_qk_norm_rope_pos: D a multiple of 16 up to 512, n_rot even and at most D, sections");
+    if (!src || !dst || !w || !pos) return ns_fail("ns_q35_qk_norm_rope_pos: a null buffer");
+    if (!al16(src) || !al16(dst) || ss % 4 || hs % 4 || ds % 4) return ns_fail("ns_q35_qk_norm_rope_pos: rows 16-byte aligned");
+    PreParams p{};
+    p.gr[0] = PreGroup{(int) H, src, ss, hs, w, 1, dst, ds, DST_F32, nullptr, 0};
+    p.ngr = 1;
+    p.T = (int) T; p.D = (int) D; p.mode = ROPE_Q35; p.n_rot = (int) n_rot; p.theta = theta; p.eps = eps;
+    p.pos3 = pos; p.s0 = (int) s0; p.s1 = (int) s1; p.s2 = (int) s2;
+    return launch_pre(g, p, "ns_q35_qk_norm_rope_pos");
+    NS_CATCH
+}
+
+int ns_q35_qk_norm_rope(ns_gpu* g, const float* src, int64_t ss, int64_t hs, float* dst, int64_t ds, int64_t T, int64_t H, int64_t D,
+                        const float* w, float eps, int64_t n_rot, float theta, int64_t p0) {
+    NS_TRY
+    if (T <= 0) return 0;
+    if (D % 16 != 0 || D > 512 || n_rot > D || n_rot % 2 || n_rot < 0) return ns_fail("ns_q35_qk_norm_rope: D a multiple of 16 up to 512, n_rot even and at most D");
+    if (!src || !dst || !w) return ns_fail("ns_q35_qk_norm_rope: a null buffer");
+    if (!al16(src) || !al16(dst) || ss % 4 || hs % 4 || ds % 4) return ns_fail("ns_q35_qk_norm_rope: rows 16-byte aligned");
+    PreParams p{};
+    p.gr[0] = PreGroup{(int) H, src, ss, hs, w, 1, dst, ds, DST_F32, nullptr, 0};
+    p.ngr = 1;
+    p.T = (int) T; p.D = (int) D; p.mode = ROPE_Q35; p.n_rot = (int) n_rot; p.theta = theta; p.eps = eps; p.p0 = p0;
+    return launch_pre(g, p, "ns_q35_qk_norm_rope");
+    NS_CATCH
+}
+
+int ns_q35_rope(ns_gpu* g, const float* src, int64_t ss, int64_t hs, float* dst, int64_t ds, int64_t T, int64_t H, int64_t D, int64_t n_rot,
+                float theta, int64_t p0) {
+    NS_TRY
+    if (T <= 0) return 0;
+    if (D % 16 != 0 || D > 512 || n_rot > D || n_rot % 2 || n_rot < 0) return ns_fail("ns_q35_rope: D a multiple of 16 up to 512, n_rot even and at most D");
+    if (!src || !dst) return ns_fail("ns_q35_rope: a null buffer");
+    if (!al16(src) || !al16(dst) || ss % 4 || hs % 4 || ds % 4) return ns_fail("ns_q35_rope: rows 16-byte aligned");
+    PreParams p{};
+    p.gr[0] = PreGroup{(int) H, src, ss, hs, nullptr, 1, dst, ds, DST_F32, nullptr, 0};
+    p.ngr = 1;
+    p.T = (int) T; p.D = (int) D; p.mode = ROPE_Q35; p.n_rot = (int) n_rot; p.theta = theta; p.p0 = p0;
+    return launch_pre(g, p, "ns_q35_rope");
+    NS_CATCH
+}
+
+int ns_mg_qk_norm_rope(ns_gpu* g, const float* x, int64_t xs, float* y, int64_t ys, int64_t T, int64_t H, int64_t D, const float* w, float eps,
+                       int rope, float theta, int64_t p0) {
+    NS_TRY
+    if (T <= 0) return 0;
+    if (D % 32 != 0 || D > 512) return ns_fail("ns_mg_qk_norm_rope: D a multiple of 32 up to 512");
+    if (rope < 0 || rope > 2) return ns_fail("ns_mg_qk_norm_rope: rope 0 (none), 1 (adjacent pairs) or 2 (halves)");
+    if (!x || !y || !w) return ns_fail("ns_mg_qk_norm_rope: a null buffer");
+    if (!al16(x) || !al16(y) || xs % 4 || ys % 4) return ns_fail("ns_mg_qk_norm_rope: rows 16-byte aligned");
+    PreParams p{};
+    p.gr[0] = PreGroup{(int) H, x, xs, D, w, rope != 0, y, ys, DST_F32, nullptr, 0};
+    p.ngr = 1;
+    p.T = (int) T; p.D = (int) D; p.mode = rope == 0 ? ROPE_NONE : rope == 1 ? ROPE_MG_PAIRS : ROPE_MG_HALVES; p.theta = theta; p.eps = eps; p.p0 = p0;
+    return launch_pre(g, p, "ns_mg_qk_norm_rope");
+    NS_CATCH
+}
+
+int ns_llm_minimaxm3_rope(ns_gpu* g, float* x, int64_t T, int64_t H, int64_t row, int64_t head, int64_t n_rot, int64_t pos0, float base) {
+    NS_TRY
+    if (n_rot <= 0 || n_rot % 2 || n_rot > head) return ns_fail("ns_llm_minimaxm3_rope: n_rot");
+    if (T <= 0 || H <= 0) return 0;
+    if (head % 4 || head > 512) return ns_fail("ns_llm_minimaxm3_rope: heads of a multiple of 4 up to 512 floats");
+    if (!x) return ns_fail("ns_llm_minimaxm3_rope: a null buffer");
+    if (!al16(x) || row % 4) return ns_fail("ns_llm_minimaxm3_rope: rows 16-byte aligned");
+    PreParams p{};
+    p.gr[0] = PreGroup{(int) H, x, row, head, nullptr, 1, x, row, DST_F32, nullptr, 0};
+    p.ngr = 1;
+    p.T = (int) T; p.D = (int) head; p.mode = ROPE_MM3; p.n_rot = (int) n_rot; p.ts = powf(base, -2.0f / (float) n_rot); p.p0 = pos0;
+    return launch_pre(g, p, "ns_llm_minimaxm3_rope");
+    NS_CATCH
+}
+
+int ns_mm3s_attn_post(ns_gpu* g, float* q, float* k, const float* v, float* iq, float* ik, const float* qn, const float* kn, const float* iqn,
+                      const float* ikn, uint16_t* kc, uint16_t* vc, uint16_t* ic, int64_t H, int64_t G, int64_t IH, int64_t HD, int64_t n_rot,
+                      int64_t pos, float base, float eps) {
+    NS_TRY
+    if (n_rot % 2 || n_rot > HD || n_rot < 0) return ns_fail("ns_mm3s_attn_post: n_rot");
+    if (HD % 4 || HD > 512 || H <= 0 || G <= 0 || IH < 0) return ns_fail("ns_mm3s_attn_post: heads of a multiple of 4 up to 512 floats");
+    if (!q || !k || !v || !qn || !kn || !kc || !vc || (IH > 0 && (!iq || !ik || !iqn || !ikn || !ic))) return ns_fail("ns_mm3s_attn_post: a null buffer");
+    if (!al16(q) || !al16(k) || !al16(v) || (IH > 0 && (!al16(iq) || !al16(ik))) || (uintptr_t) kc % 8 || (uintptr_t) vc % 8 || (IH > 0 && (uintptr_t) ic % 8))
+        return ns_fail("ns_mm3s_attn_post: rows 16-byte aligned (half rows 8)");
+    PreParams p{};
+    p.gr[0] = PreGroup{(int) H, q, 0, HD, qn, 1, q, 0, DST_F32, nullptr, 0};
+    p.gr[1] = PreGroup{(int) G, k, 0, HD, kn, 1, k, 0, DST_F32, kc, 0};
+    // v: no norm, no rotation; the float32 row is left as it is (written back to itself), the half copy is the store
+    p.gr[2] = PreGroup{(int) G, v, 0, HD, nullptr, 0, vc, 0, DST_F16, nullptr, 0};
+    p.ngr = 3;
+    if (IH > 0) {
+        p.gr[3] = PreGroup{(int) IH, iq, 0, HD, iqn, 1, iq, 0, DST_F32, nullptr, 0};
+        p.gr[4] = PreGroup{1, ik, 0, HD, ikn, 1, ik, 0, DST_F32, ic, 0};
+        p.ngr = 5;
+    }
+    p.T = 1; p.D = (int) HD; p.mode = n_rot > 0 ? ROPE_MM3 : ROPE_NONE; p.n_rot = (int) n_rot; p.ts = n_rot > 0 ? powf(base, -2.0f / (float) n_rot) : 1.0f;
+    p.eps = eps; p.p0 = pos; p.inv_sqrt = 1;
+    return launch_pre(g, p, "ns_mm3s_attn_post");
+    NS_CATCH
+}
+
+int ns_attn_pre_store(ns_gpu* g, int rope, int qt, int kt, int ring, const float* q, int64_t qss, int64_t qhs, void* qo, int64_t qos,
+                      const float* k, int64_t kss, int64_t khs, const float* v, int64_t vss, const float* qw, const float* kw, float eps,
+                      int64_t n_rot, float theta, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, void* kc, void* vc) {
+    NS_TRY
+    if (T <= 0) return 0;
+    if (D != 64 && D != 128 && D != 256) return ns_fail("ns_attn_pre_store: heads of 64, 128 or 256");
+    if (rope < 1 || rope > 3) return ns_fail("ns_attn_pre_store: rope 1 (rotate-half over n_rot), 2 (adjacent pairs) or 3 (halves)");
+    if (rope == 1 && (n_rot > D || n_rot % 2 || n_rot < 0)) return ns_fail("ns_attn_pre_store: n_rot even and at most D");
+    if (qt < 0 || qt > 2 || kt < 0 || kt > 3) return ns_fail("ns_attn_pre_store: rows of type 0..2, a cache form 0..3");
+    if (Hq <= 0 || Hkv <= 0 || cap <= 0 || p0 < 0) return ns_fail("ns_attn_pre_store: heads, a capacity and a position");
+    if (!ring && p0 + T > cap) return ns_fail("ns_attn_pre_store: past the cache's capacity");
+    if (ring && T > cap) return ns_fail("ns_attn_pre_store: more rows than the ring holds");
+    if (!q || !qo || !k || !v || !qw || !kw || !kc || !vc) return ns_fail("ns_attn_pre_store: a null buffer");
+    if (!al16(q) || !al16(k) || !al16(v) || qss % 4 || qhs % 4 || kss % 4 || khs % 4 || vss % 4 || (uintptr_t) qo % (qt == 0 ? 16 : 8) || qos % 4 ||
+        ((uintptr_t) kc | (uintptr_t) vc) % 8)
+        return ns_fail("ns_attn_pre_store: rows 16-byte aligned (16-bit rows and caches 8)");
+    PreParams p{};
+    p.gr[0] = PreGroup{(int) Hq, q, qss, qhs, qw, 1, qo, qos, qt, nullptr, 0};
+    p.gr[1] = PreGroup{(int) Hkv, k, kss, khs, kw, 1, kc, 0, DST_CACHE + kt, nullptr, 0};
+    p.gr[2] = PreGroup{(int) Hkv, v, vss, D, nullptr, 0, vc, 0, DST_CACHE + kt, nullptr, 0};
+    p.ngr = 3;
+    p.T = (int) T; p.D = (int) D; p.mode = rope == 1 ? ROPE_Q35 : rope == 2 ? ROPE_MG_PAIRS : ROPE_MG_HALVES; p.n_rot = (int) n_rot;
+    p.theta = theta; p.eps = eps; p.p0 = p0; p.cap = cap; p.ring = ring;
+    return launch_pre(g, p, "ns_attn_pre_store");
+    NS_CATCH
+}
+
+}  // extern "C"

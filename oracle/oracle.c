@@ -6,7 +6,8 @@
  *
  * Two kinds of functions live here:
  *   - "order" restatements: float32, the same operation order as the reference's exact (vector-unit) kernels
- *     (streams of keys, split/merge with exp) - orc_attn_exact, orc_mla_decode, orc_mm3_attend, orc_glm_mla_attend;
+ *     (streams of keys, split/merge with exp) - orc_attn_exact, orc_mla_decode, orc_mm3_attend, orc_glm_mla_attend - and
+ *     of the norm + rotary-position step in front of attention - orc_q35_norm_rope, orc_mg_norm_rope, orc_mm3_norm_rope_row;
  *   - float64 closed forms softmax(q k^T s + mask) v on the very same stored (f16 / q8_0 / q4_0 / bf16) values -
  *     orc_attn_f64, orc_mla_f64: the tolerance arm (max-abs 2e-3, relative L2 1e-3 for f16/bf16 outputs).
  * Integer/byte work (cache rows, q8_0 / q4_0 packing, dequant, split arithmetic) is restated exactly and compared
@@ -14,8 +15,9 @@
  *
  * What pins each function (see tests/test_oracle_*.py): closed forms evaluated independently in numpy float64,
  * hand-derived known answers for the quantizers (ggml's quantize_row_q8_0_ref / q4_0_ref rules), numpy.float16 for
- * the half conversions over every bit pattern, partition invariance of the split/merge, and brute force on tiny
- * shapes. The reference ships no golden vectors for this path.
+ * the half conversions over every bit pattern, partition invariance of the split/merge, brute force on tiny
+ * shapes, and for the rotary positions a float64 complex-rotation statement in numpy plus the rotation's invariants
+ * (position 0 is the identity, a pair's norm is kept, angles add). The reference ships no golden vectors for this path.
  *
  * Parity unpinned: none of the functions below.
  *
@@ -822,6 +824,122 @@ ORC_API void orc_glm_mla_attend(const float* qa, const uint8_t* cache, int q8, f
             free(s);
             free(c);
         }
+}
+
+/* ------------------------------------------------------------------------------------ norm + rotary positions */
+
+/* kernels/llm/qwen35/q35.cpp:220-254 (w != NULL: RMS norm first), :256-279 (w == NULL: ns_q35_rope), :350-386 (pos3 != NULL:
+ * each row at its own (t, h, w) positions, interleaved sections s0, s1, s2). Rotate-half over the first n_rot features:
+ * pair (i, i + n_rot / 2), angle pos * theta^(-2 k / n_rot), every product in float32. The reference sums the squares as 16
+ * lane sums (i = l, l + 16, ...) added by a group reduction; here the lane sums are added in lane order. */
+ORC_API int orc_q35_norm_rope(const float* src, int64_t ss, int64_t hs, float* dst, int64_t ds, int64_t T, int64_t H, int64_t D, const float* w,
+                              float eps, int64_t n_rot, float theta, int64_t p0, const int32_t* pos3, int64_t s0, int64_t s1, int64_t s2) {
+    if (D % 16 != 0 || n_rot > D || n_rot % 2 || (pos3 && s0 + s1 + s2 <= 0)) return -1;
+    const int64_t hr = n_rot / 2, sect = s0 + s1 + s2;
+    for (int64_t t = 0; t < T; ++t)
+        for (int64_t h = 0; h < H; ++h) {
+            const float* x = src + t * ss + h * hs;
+            float* y = dst + t * ds + h * D;
+            float inv = 1.0f;
+            if (w) {
+                float lane[16], s = 0.0f;
+                for (int l = 0; l < 16; ++l) {
+                    lane[l] = 0.0f;
+                    for (int64_t i = l; i < D; i += 16) lane[l] += x[i] * x[i];
+                }
+                for (int l = 0; l < 16; ++l) s += lane[l];
+                inv = 1.0f / sqrtf(s / (float) D + eps);
+            }
+            for (int64_t i = 0; i < D; ++i) {
+                const float v = w ? x[i] * inv * w[i] : x[i];
+                if (i < n_rot) {
+                    const int64_t k = i < hr ? i : i - hr;
+                    float pos = (float) (p0 + t);
+                    if (pos3) {
+                        const int64_t sec = k % sect;
+                        const int c = (sec % 3 == 1 && sec < 3 * s1) ? 1 : (sec % 3 == 2 && sec < 3 * s2) ? 2 : 0;
+                        pos = (float) pos3[t * 3 + c];
+                    }
+                    const float a = pos * powf(theta, -2.0f * (float) k / (float) n_rot);
+                    const float c = cosf(a), sn = sinf(a);
+                    const int64_t o = i < hr ? i + hr : i - hr;
+                    const float other = w ? x[o] * inv * w[o] : x[o];
+                    y[i] = i < hr ? v * c - other * sn : v * c + other * sn;
+                } else {
+                    y[i] = v;
+                }
+            }
+        }
+    return 0;
+}
+
+/* kernels/llm/museglimmer/mg.cpp:157-190: RMS norm, then rope 0 none, 1 adjacent pairs (2i, 2i + 1), 2 halves (i, i + D / 2)
+ * over all D, angle pos * theta^(-2 i / D). y may be x (a pair is read before it is written). */
+ORC_API int orc_mg_norm_rope(const float* x, int64_t xs, float* y, int64_t ys, int64_t T, int64_t H, int64_t D, const float* w, float eps, int rope,
+                             float theta, int64_t p0) {
+    if (D % 32 != 0) return -1;
+    for (int64_t t = 0; t < T; ++t)
+        for (int64_t h = 0; h < H; ++h) {
+            const float* xr = x + t * xs + h * D;
+            float* yr = y + t * ys + h * D;
+            float lane[16], s = 0.0f;
+            for (int l = 0; l < 16; ++l) {
+                lane[l] = 0.0f;
+                for (int64_t i = l; i < D; i += 16) lane[l] += xr[i] * xr[i];
+            }
+            for (int l = 0; l < 16; ++l) s += lane[l];
+            const float inv = 1.0f / sqrtf(s / (float) D + eps);
+            const float pos = (float) (p0 + t);
+            for (int64_t i = 0; i < D / 2; ++i) {
+                const int64_t i0 = rope == 2 ? i : 2 * i, i1 = rope == 2 ? i + D / 2 : 2 * i + 1;
+                const float a0 = xr[i0] * inv * w[i0], a1 = xr[i1] * inv * w[i1];
+                if (rope) {
+                    const float a = pos * powf(theta, -2.0f * (float) i / (float) D);
+                    const float c = cosf(a), sn = sinf(a);
+                    yr[i0] = a0 * c - a1 * sn;
+                    yr[i1] = a0 * sn + a1 * c;
+                } else {
+                    yr[i0] = a0;
+                    yr[i1] = a1;
+                }
+            }
+        }
+    return 0;
+}
+
+/* kernels/llm/minimaxm3/mm3.cpp:18-35 (w == NULL: in-place rotate-half, the angle of pair i = pos multiplied i times by
+ * base^(-2 / n_rot)) and silo/moe.cpp:477-497 (w != NULL: RMS norm as 1 / sqrt first; half != NULL: the result also stored
+ * as half; rot == 0 with w == NULL: a plain half store, the token's v rows). One head row of HD floats. */
+ORC_API int orc_mm3_norm_rope_row(float* p, const float* w, uint16_t* half, int rot, int64_t HD, int64_t n_rot, int64_t pos, float base, float eps) {
+    if (n_rot % 2 || n_rot > HD) return -1;
+    const int64_t hr = n_rot / 2;
+    const float ts = n_rot > 0 ? powf(base, -2.0f / (float) n_rot) : 1.0f;
+    float inv = 1.0f;
+    if (w) {
+        float sq = 0.0f;
+        for (int64_t i = 0; i < HD; ++i) sq += p[i] * p[i];
+        inv = 1.0f / sqrtf(sq / (float) HD + eps);
+    }
+    float* out = (float*) malloc((size_t) HD * sizeof(float));
+    for (int64_t i = 0; i < HD; ++i) {
+        const float me = w ? p[i] * inv * w[i] : p[i];
+        if (rot && i < n_rot) {
+            const int64_t k = i % hr, o = i < hr ? i + hr : i - hr;
+            float th = (float) pos;
+            for (int64_t j = 0; j < k; ++j) th *= ts;
+            const float c = cosf(th), s = sinf(th);
+            const float them = w ? p[o] * inv * w[o] : p[o];
+            out[i] = i < hr ? me * c - them * s : them * s + me * c;
+        } else {
+            out[i] = me;
+        }
+    }
+    for (int64_t i = 0; i < HD; ++i) {
+        if (w || rot) p[i] = out[i];
+        if (half) half[i] = orc_f2h(out[i]);
+    }
+    free(out);
+    return 0;
 }
 
 /* ------------------------------------------------------------------------------------------------ comparisons */

@@ -52,6 +52,9 @@ def lib():
             "orc_mla_vb": (None, [P, P, P, i64, i64, i64, i64]),
             "orc_mla_f64": (None, [P, P, P, i64, i64, i64, i64, i64, f64]),
             "orc_glm_mla_attend": (None, [P, P, C.c_int, P, i64, i64, i64, i64, f32]),
+            "orc_q35_norm_rope": (C.c_int, [P, i64, i64, P, i64, i64, i64, i64, P, f32, i64, f32, i64, P, i64, i64, i64]),
+            "orc_mg_norm_rope": (C.c_int, [P, i64, P, i64, i64, i64, i64, P, f32, C.c_int, f32, i64]),
+            "orc_mm3_norm_rope_row": (C.c_int, [P, P, P, C.c_int, i64, i64, i64, f32, f32]),
             "orc_compare": (None, [P, P, i64, P, P, P]),
             "orc_threads": (C.c_int, []),
         }
@@ -255,6 +258,39 @@ def glm_mla_attend(qa, cache, q8, T, H, L, pos0, scale):
 
 
 # ---- comparisons -------------------------------------------------------------------------------------------------
+# ---- norm + rotary positions ----------------------------------------------------------------------------------------
+def q35_norm_rope(x, T, H, D, w, eps, n_rot, theta, p0, pos3=None, sections=(0, 0, 0)):
+    """x [T][H][D] float32 -> RMS norm (w None: none) + rotate-half over the first n_rot (ns_q35_qk_norm_rope / _pos / ns_q35_rope)."""
+    x = _c(x, np.float32).reshape(T, H * D)
+    y = np.empty_like(x)
+    wp = _p(_c(w, np.float32)) if w is not None else None
+    pp = _p(_c(pos3, np.int32)) if pos3 is not None else None
+    rc = lib().orc_q35_norm_rope(_p(x), H * D, D, _p(y), H * D, T, H, D, wp, eps, n_rot, theta, p0, pp, *sections)
+    if rc:
+        raise ValueError("orc_q35_norm_rope: bad arguments")
+    return y
+
+
+def mg_norm_rope(x, T, H, D, w, eps, rope, theta, p0):
+    x = _c(x, np.float32).reshape(T, H * D)
+    y = np.empty_like(x)
+    rc = lib().orc_mg_norm_rope(_p(x), H * D, _p(y), H * D, T, H, D, _p(_c(w, np.float32)), eps, rope, theta, p0)
+    if rc:
+        raise ValueError("orc_mg_norm_rope: bad arguments")
+    return y
+
+
+def mm3_norm_rope_row(row, w, rot, n_rot, pos, base, eps, want_half=False):
+    """One head row: (new float32 row, half copy or None) of the MiniMax-M3 norm + rotate-half."""
+    row = np.array(row, np.float32)
+    half = np.empty(row.size, np.uint16) if want_half else None
+    wp = _p(_c(w, np.float32)) if w is not None else None
+    rc = lib().orc_mm3_norm_rope_row(_p(row), wp, _p(half) if want_half else None, int(rot), row.size, n_rot, pos, base, eps)
+    if rc:
+        raise ValueError("orc_mm3_norm_rope_row: bad arguments")
+    return row, half
+
+
 def compare(a, b):
     """(max-abs, relative L2, cosine) of a (float32) against b (float64) - the reference's `kernels` check's measures."""
     a = _c(a, np.float32).ravel()

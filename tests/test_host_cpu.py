@@ -7,7 +7,7 @@ import re
 import pytest
 
 from nextsycl_amd import Error, library_path
-from nextsycl_amd.attn import ATTN_H, MLA_H, kv_row_bytes
+from nextsycl_amd.attn import ATTN_H, MLA_H, PRE_H, kv_row_bytes
 from nextsycl_amd.sys import NS_H
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -29,7 +29,7 @@ def _declared(header):
 
 
 def test_library_exports_every_declared_symbol(handle):
-    declared = _declared("ns.h") | _declared("ns_attn.h") | _declared("ns_mla.h")
+    declared = _declared("ns.h") | _declared("ns_attn.h") | _declared("ns_mla.h") | _declared("ns_pre.h")
     assert len(_declared("ns.h")) == 26                      # the reference's 26 (kernels/ns/ns.h:18-56)
     missing = [n for n in sorted(declared) if not hasattr(handle, n)]
     assert not missing, missing
@@ -37,6 +37,7 @@ def test_library_exports_every_declared_symbol(handle):
     assert set(NS_H) == _declared("ns.h")
     assert set(ATTN_H) == _declared("ns_attn.h")
     assert set(MLA_H) == _declared("ns_mla.h")
+    assert set(PRE_H) == _declared("ns_pre.h")
 
 
 def test_pure_functions_without_a_gpu(handle):
