@@ -121,11 +121,20 @@ int ns_q35_attn(ns_gpu* g, const float* q, int64_t qs, const void* kc, const voi
 int64_t ns_mg_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win, int causal);
 int ns_mg_attn(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
                int64_t win, int causal, float* out, float* scratch);
-/* GQA over a position-major half cache [position][G][128], q [T][H][128], explicit scale; dense (sel must be NULL).
+/* GQA over a position-major half cache [position][G][128], q [T][H][128], explicit scale. sel NULL: dense; else
+ * sel [T][G][K] names K blocks of 128 keys a (row, key head) (-1: none), cut at the row's own position (a row is a launch).
  * Replaces: kernels/llm/minimaxm3/mm3.h:33-37 (mm3.cpp:118-190). Needs scratch: this library keeps
  * ns_attn_decode_scratch(T, H, G, 128, pos0, 0) floats per ns_gpu for it (allocated at ns_gpu_open, 64 MiB) */
 int ns_llm_minimaxm3_attend(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
                             int64_t H, int64_t G, int64_t pos0, float scale);
+
+/* kernels/llm/minimaxm3/mm3.h (indexer), mm3.cpp:59-116. The block indexer that fills `sel`: bs [T][G][nblk] = the largest
+ * iq [T][G][128] . ik_j over block b's keys j <= pos0 + t (ik half [pos][128]); -inf for a block wholly past the row,
+ * + 1e30 for the `local` most recent blocks. Then the K best blocks a (row, head) into sel [T][G][K], best first, the
+ * lowest index of equal scores, -1 once nothing finite is left; bs is consumed (picked scores become -inf). */
+int ns_llm_minimaxm3_idx_scores(ns_gpu* g, const float* iq, const uint16_t* ik, float* bs, int64_t T, int64_t G, int64_t nblk, int64_t pos0,
+                                int64_t local);
+int ns_llm_minimaxm3_idx_topk(ns_gpu* g, float* bs, int32_t* sel, int64_t T, int64_t G, int64_t nblk, int64_t K);
 
 /* ---- measurement ---------------------------------------------------------------------------------------------------- */
 

@@ -38,9 +38,10 @@ int ns_ds2_mla_decode(ns_gpu* g, const float* q, const uint16_t* kb, const uint1
 int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint16_t* cache, int64_t T, int64_t L, int64_t R, int64_t pos0,
                     float freq_base, float freq_scale, float ext_factor, float mscale, float corr0, float corr1);
 
-/* GLM-5.3's latent-only MLA over a half cache [n][512]: qa [T][H][512] float32 -> u [T][H][512] float32. Dense rows
- * only: sel and sel_cnt must be NULL (the sparse cell selection is not built). Replaces:
- * kernels/llm/glm5next/glm.h:65-66 (glm.cpp:1252-1264) */
+/* GLM-5.3's latent-only MLA over a half cache [n][512]: qa [T][H][512] float32 -> u [T][H][512] float32. sel_cnt NULL:
+ * every row sees every earlier cell. Else row t's cells are the pools sel[t K ..][0, sel_cnt[t]) of 4 cells each (cells
+ * 4 b .. 4 b + 3) followed by its incomplete pool 4 ((p + 1) / 4) .. p, p = pos0 + t; a negative sel_cnt[t] is a dense
+ * row. Replaces: kernels/llm/glm5next/glm.h:65-66 (glm.cpp:1062-1067,1095-1102,1252-1264) */
 int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                       const int32_t* sel, const int32_t* sel_cnt, int64_t K);
 /* the same over q8 latent rows, at most 8 rows. Replaces: kernels/llm/glm5next/glm.h:79-80 (glm.cpp:1267-1276) */

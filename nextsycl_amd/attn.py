@@ -55,6 +55,8 @@ ATTN_H = {
     "ns_mg_attn_scratch": (i64, [i64, i64, i64, i64, i64, i64, i32]),
     "ns_mg_attn": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, i32, P, P]),
     "ns_llm_minimaxm3_attend": (i32, [P, P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
+    "ns_llm_minimaxm3_idx_scores": (i32, [P, P, P, P, i64, i64, i64, i64, i64]),
+    "ns_llm_minimaxm3_idx_topk": (i32, [P, P, P, i64, i64, i64, i64]),
     "ns_attn_profile": (i32, [P, i32]),
     "ns_attn_copy_probe": (i32, [P, P, P, C.c_size_t]),
     "ns_attn_profile_last": (i32, [P, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
@@ -296,25 +298,43 @@ class Ops:
         self.ok(self.k.ds2_kv_store(self.raw(), kv.ptr, w.ptr, eps, cache.ptr, T, L, R, pos0, freq_base, freq_scale, ext_factor, mscale, corr0, corr1),
                 "kv_store")
 
-    def mla_attend(self, qa, c, u, T, H, L, pos0, scale, q8=False):
-        """GLM's latent-only MLA (dense): ns_mla_attend_sel / ns_mla_attend_sel_q8 with no selection."""
+    def mla_attend(self, qa, c, u, T, H, L, pos0, scale, q8=False, sel=None, sel_cnt=None, K=0):
+        """GLM's latent-only MLA: ns_mla_attend_sel / ns_mla_attend_sel_q8; sel [T][K] pools and sel_cnt [T], or dense."""
         _need(qa, T * H * L * 4, "mla_attend qa")
         _need(c, (pos0 + T) * ((L // 32 * 2 + L) if q8 else 2 * L), "mla_attend cache")
         _need(u, T * H * L * 4, "mla_attend u")
+        if sel_cnt is not None:
+            _need(sel, T * K * 4, "mla_attend pools")
+            _need(sel_cnt, T * 4, "mla_attend pool counts")
         f = self.k.mla_attend_sel_q8 if q8 else self.k.mla_attend_sel
-        self.ok(f(self.raw(), qa.ptr, c.ptr, u.ptr, T, H, L, pos0, scale, None, None, 0), "mla_attend")
+        opt = lambda b: b.ptr if b is not None else None
+        self.ok(f(self.raw(), qa.ptr, c.ptr, u.ptr, T, H, L, pos0, scale, opt(sel), opt(sel_cnt), K), "mla_attend")
 
     def to_q8row(self, x, y, n, L):
         _need(x, n * L * 4, "to_q8row x")
         _need(y, n * (L // 32 * 2 + L), "to_q8row y")
         self.ok(self.k.to_q8row(self.raw(), x.ptr, y.ptr, n, L), "to_q8row")
 
-    def minimaxm3_attend(self, q, kc, vc, out, T, H, G, pos0, scale):
+    def minimaxm3_attend(self, q, kc, vc, out, T, H, G, pos0, scale, sel=None, K=0):
         _need(q, T * H * 128 * 4, "attend q")
         _need(out, T * H * 128 * 4, "attend out")
         _need(kc, (pos0 + T) * G * 128 * 2, "attend key cache")
         _need(vc, (pos0 + T) * G * 128 * 2, "attend value cache")
-        self.ok(self.k.llm_minimaxm3_attend(self.raw(), q.ptr, kc.ptr, vc.ptr, None, 0, out.ptr, T, H, G, pos0, scale), "attend")
+        if sel is not None:
+            _need(sel, T * G * K * 4, "attend block lists")
+        self.ok(self.k.llm_minimaxm3_attend(self.raw(), q.ptr, kc.ptr, vc.ptr, sel.ptr if sel is not None else None, K, out.ptr, T, H, G, pos0, scale),
+                "attend")
+
+    def minimaxm3_idx_scores(self, iq, ik, bs, T, G, nblk, pos0, local):
+        _need(iq, T * G * 128 * 4, "idx_scores iq")
+        _need(ik, (pos0 + T) * 128 * 2, "idx_scores ik")
+        _need(bs, T * G * nblk * 4, "idx_scores scores")
+        self.ok(self.k.llm_minimaxm3_idx_scores(self.raw(), iq.ptr, ik.ptr, bs.ptr, T, G, nblk, pos0, local), "idx_scores")
+
+    def minimaxm3_idx_topk(self, bs, sel, T, G, nblk, K):
+        _need(bs, T * G * nblk * 4, "idx_topk scores")
+        _need(sel, T * G * K * 4, "idx_topk lists")
+        self.ok(self.k.llm_minimaxm3_idx_topk(self.raw(), bs.ptr, sel.ptr, T, G, nblk, K), "idx_topk")
 
     # ---- the step in front of attention: norm, rotary positions, store
     def q35_qk_norm_rope(self, src, ss, hs, dst, ds, T, H, D, w, eps, n_rot, theta, p0, pos3=None, sections=(0, 0, 0)):

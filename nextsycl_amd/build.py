@@ -24,6 +24,7 @@ SOURCES = {
     "kv_store.hip": ["-ffp-contract=off"],
     "pre_attn.hip": ["-ffp-contract=off"],
     "attn_decode.hip": [],
+    "indexer.hip": [],
     "attn_prefill.hip": [],
     "attn_api.cpp": [],
     "mla.hip": [],

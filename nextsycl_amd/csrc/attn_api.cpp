@@ -10,6 +10,8 @@ int ns_attn_decode_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
                        float* scratch);
 int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T,
                        int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out);
+int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K,
+                       float* out, int64_t T, int64_t Hq, int64_t Hkv, int64_t pos0, float scale, float* scratch, size_t scratch_floats);
 
 namespace {
 constexpr int64_t DECODE_ROWS = 16;   // passes up to this many rows take the decode kernel
@@ -73,11 +75,10 @@ int ns_mg_attn(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_
 
 int ns_llm_minimaxm3_attend(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
                             int64_t H, int64_t G, int64_t pos0, float scale) {
-    (void) K;
     if (T <= 0) return 0;
     if (G <= 0 || H % G) return ns_fail("ns_llm_minimaxm3_attend: heads");
-    if (sel) return ns_fail("ns_llm_minimaxm3_attend: block-sparse selection is not built; pass sel = NULL (dense)");
     if (!(scale > 0.0f)) return ns_fail("ns_llm_minimaxm3_attend: a positive scale");
+    if (sel) return ns_attn_decode_sel(g, "ns_llm_minimaxm3_attend", q, kc, vc, sel, K, out, T, H, G, pos0, scale, g->own_scratch, g->own_scratch_floats);
     const int64_t cap = pos0 + T;
     if (T <= DECODE_ROWS) {
         const int64_t need = ns_attn_decode_scratch(T, H, G, 128, pos0, 0);

@@ -59,6 +59,12 @@ struct DecodeParams {
     int ns;
     float sl2;                  // scale x log2(e)
     float* part;                // [T][Hq][ns][D + 2]
+    // block-sparse passes (one row a launch): the pass's keys are the listed blocks of 128 laid end to end - key j of
+    // the kernel's numbering is key sel[j / 128] * 128 + j % 128 of the cache (-1: no block), and keys past sel_pos
+    // are not the row's
+    const int32_t* sel;         // [Hkv][selK] block ids of this row, or null
+    int selK;
+    int64_t sel_pos;
 };
 
 template <int D, int KT>
@@ -122,6 +128,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
     const uint8_t* vbase = p.vc + (int64_t) hk * p.head_stride;
     uint8_t* stage = lds + w * STAGE;
+    const int32_t* selp = p.sel ? p.sel + (int64_t) hk * p.selK : nullptr;
 
     // a key's row offset: keys outside [jb, je) are clamped into it (their scores are masked, their values meet P = 0).
     // A wrapped ring's slot is position % cap: the split's first key's slot once, then offsets from it with at most two
@@ -139,11 +146,18 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     };
     // the tile's keys into registers (MFMA A layout) and its values on their way: DMA into LDS buffer `buf`, chunk
     // position cp of key kk holding the row's chunk cp ^ 2 (kk % 8); or raw into registers
+    // a listed block's tile: its 32 keys sit together in the cache (a block holds 4 tiles); no block: any valid rows
+    auto tile_off = [&](int64_t ti, int j0, int idx) -> int64_t {
+        if (!selp) return row_off(j0 + idx);
+        const int blk = selp[(ti * TILE) >> 7];
+        // (keys of a listed block past the row's position are masked: read the row's own key instead - the cache may end there)
+        return std::min<int64_t>((int64_t) (blk < 0 ? 0 : blk) * 128 + ((ti * TILE) & 127) + idx, p.sel_pos) * p.row_stride;
+    };
     auto load_tile = [&](R& r, int64_t ti, int buf) {
         const int j0 = (int) (ti * TILE - jb);                 // the tile's first key relative to the split's
 #pragma unroll
         for (int kt2 = 0; kt2 < 2; ++kt2) {
-            const uint8_t* kr = kbase + row_off(j0 + kt2 * 16 + n);
+            const uint8_t* kr = kbase + tile_off(ti, j0, kt2 * 16 + n);
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
                 if constexpr (DMA) {
@@ -163,7 +177,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
 #pragma unroll
         for (int i = 0; i < R::NLV; ++i) {
             const int kk = kr0 + R::KPI * i;
-            const uint8_t* vr = vbase + row_off(j0 + kk);
+            const uint8_t* vr = vbase + tile_off(ti, j0, kk);
             if constexpr (DMA) {
                 const int c = cp ^ (2 * (kk & 7));
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (vr + c * 16),
@@ -304,6 +318,12 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             }
         }
         // ---- online softmax a row (this lane: row n of each row tile, keys j0 + 16 kt2 + 4 g4 + i)
+        // (a listed block's keys count up to the row's own position; a hole in the list has none)
+        int64_t hi_tile = INT64_MAX;
+        if (selp) {
+            const int blk = selp[j0 >> 7];
+            hi_tile = blk < 0 ? -1 : (j0 & ~(int64_t) 127) + std::min<int64_t>(127, p.sel_pos - (int64_t) blk * 128);
+        }
         s8v pb[RT];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
@@ -313,7 +333,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int64_t j = j0 + kt2 * 16 + g4 * 4 + i;
-                    const float v = (j >= lo_r[rt] && j <= hi_r[rt]) ? s[rt][kt2][i] * p.sl2 : -INFINITY;
+                    const float v = (j >= lo_r[rt] && j <= std::min(hi_r[rt], hi_tile)) ? s[rt][kt2][i] * p.sl2 : -INFINITY;
                     x[kt2 * 4 + i] = v;
                     mx = fmaxf(mx, v);
                 }
@@ -633,6 +653,55 @@ int decode_checked(ns_gpu* g, const char* who, int qt, int kt, int pm, const voi
 }
 
 }  // namespace
+
+// Block-sparse decode over a position-major half cache [pos][Hkv][128] (MiniMax-M3: kernels/llm/minimaxm3/mm3.cpp:118-190
+// with sel != NULL): row t attends the K blocks of 128 keys sel[(t Hkv + hk) K ..] names (-1: none), cut at its own
+// position. Rows choose their own blocks, so a row is a launch (split over its K x 128 listed keys) and a merge.
+int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K,
+                       float* out, int64_t T, int64_t Hq, int64_t Hkv, int64_t pos0, float scale, float* scratch, size_t scratch_floats) {
+    NS_TRY
+    constexpr int D = 128;
+    const std::string w(who);
+    if (T <= 0) return 0;
+    if (Hkv <= 0 || Hq <= 0 || Hq % Hkv) return ns_fail(w + ": query heads a multiple of the key heads");
+    if (K < 0 || K > (int64_t) 1 << 20) return ns_fail(w + ": a block count");
+    if (!q || !kc || !vc || !out || !sel || !scratch) return ns_fail(w + ": a null buffer");
+    if ((uintptr_t) q % 16 || ((uintptr_t) kc | (uintptr_t) vc) % 16) return ns_fail(w + ": rows 16-byte aligned");
+    NS_HIP(hipSetDevice(g->dev));
+    if (K == 0) return ns_fill(g, out, 0, (size_t) (T * Hq * D) * sizeof(float));     // nothing listed: zeros (l = 0)
+    const int64_t keys = K * 128, kbs = dec_kbs(keys, Hkv), ns = (keys + kbs - 1) / kbs;
+    if ((size_t) (Hq * ns * (D + 2)) > scratch_floats) return ns_fail(w + ": the pass needs more scratch than the library keeps");
+    DecodeParams p{};
+    p.qt = 0;
+    p.qs = Hq * D;
+    p.kc = (const uint8_t*) kc;
+    p.vc = (const uint8_t*) vc;
+    p.head_stride = 2 * D;
+    p.row_stride = Hkv * 2 * D;
+    p.cap = keys;
+    p.wrap = 0;
+    p.T = 1;
+    p.Hq = (int) Hq;
+    p.G = (int) (Hq / Hkv);
+    p.causal = 1;
+    p.p0 = keys - 1;            // in the kernel's numbering the row sees every listed key; sel_pos cuts the real ones
+    p.win = 0;
+    p.kbs = kbs;
+    p.sp0 = 0;
+    p.ns = (int) ns;
+    p.sl2 = scale * 1.4426950408889634f;
+    p.part = scratch;
+    p.selK = (int) K;
+    for (int64_t t = 0; t < T; ++t) {
+        p.q = q + t * Hq * D;
+        p.sel = sel + t * Hkv * K;
+        p.sel_pos = pos0 + t;
+        if (launch_kt<D>(g, 0, p, p.G, dim3((unsigned) ns, (unsigned) Hkv))) return -1;
+        if (launch_merge<D, 0>(g, scratch, (int) ns, Hq, out + t * Hq * D)) return -1;
+    }
+    return 0;
+    NS_CATCH
+}
 
 // used by the exact-API routing in attn_api.cpp
 int ns_attn_decode_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T,

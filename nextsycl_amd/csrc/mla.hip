@@ -48,6 +48,12 @@ struct MlaParams {
     int ns;
     float sl2;
     float* part;         // [T * H][ns][PSTRIDE]
+    // a row's own cells (GLM's selection): sel_cnt[t] >= 0 -> the pools sel[t K ..][0, sel_cnt[t]) of 4 cells each, then
+    // the row's incomplete pool 4 ((p + 1) / 4) .. p; negative or no sel_cnt -> every earlier cell. With sel_cnt a row
+    // group holds one row t's heads only (per_t), and the kernel's cell numbering runs over the row's list
+    const int32_t* sel;
+    const int32_t* sel_cnt;
+    int K, per_t;
 };
 
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));   // a 16-byte chunk in flight (a plain vector: stays in registers)
@@ -78,14 +84,28 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int split = blockIdx.x, z = blockIdx.y;
     const int rows = p.T * p.H;
-    const int64_t n_all = p.pos0 + p.T;                                  // cells the pass's last row sees
+    // a row group: 128 consecutive (row, head) pairs of the pass, or (per_t) 128 heads of one row t
+    const int zpt = (p.H + MROWS - 1) / MROWS;
+    const int tz = p.per_t ? z / zpt : 0;
+    const int64_t pz = p.pos0 + tz;
+    const int64_t cnt = p.per_t && p.sel_cnt ? p.sel_cnt[tz] : -1;        // pools listed for row tz, or negative: dense
+    const int64_t tail0 = 4 * ((pz + 1) / 4);
+    // cells the group's last row sees (of its list, if it has one)
+    const int64_t n_all = !p.per_t ? p.pos0 + p.T : cnt < 0 ? pz + 1 : 4 * cnt + (pz + 1 - tail0);
     const int64_t jb = (int64_t) split * p.kbs, je = std::min(jb + p.kbs, n_all);
+    const int32_t* const selt = cnt >= 0 ? p.sel + (int64_t) tz * p.K : nullptr;
+    // cell i of the row's numbering -> the cache's cell
+    auto cell = [&](int64_t i) -> int64_t {
+        if (!selt) return i;
+        return i < 4 * cnt ? 4 * (int64_t) selt[i >> 2] + (i & 3) : tail0 + (i - 4 * cnt);
+    };
 
     // ---- this lane's row
-    const int ri = z * MROWS + w * 16 + n;
-    const bool live = ri < rows;
+    const int rin = (p.per_t ? z % zpt : z) * MROWS + w * 16 + n;        // within the pass, or within row tz's heads
+    const bool live = p.per_t ? rin < p.H : rin < rows;
+    const int ri = p.per_t ? tz * p.H + rin : rin;
     const int rr = live ? ri : rows - 1;
-    const int64_t hi_r = live ? std::min(p.pos0 + rr / p.H, je - 1) : -1;
+    const int64_t hi_r = !live ? -1 : p.per_t ? je - 1 : std::min(p.pos0 + rr / p.H, je - 1);
     s8v qreg[KB];
     {
         const int64_t qoff = (int64_t) rr * DK + g4 * 8;
@@ -124,14 +144,15 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
     const uint8_t* const split_base = p.cache + jb * CROW;
     const int last_rel = (int) (je - 1 - jb);
     auto fetch = [&](int it_, int i0, int i1) {
-        const bool plain = (it_ + 1) * MTILE - 1 <= last_rel;
-        const uint8_t* sp = split_base + (plain ? (int64_t) it_ * MTILE * CROW : 0);
+        const bool plain = !selt && (it_ + 1) * MTILE - 1 <= last_rel;
+        const uint8_t* sp = selt ? p.cache : split_base + (plain ? (int64_t) it_ * MTILE * CROW : 0);
 #pragma unroll
         for (int i = 0; i < NLD; ++i) {
             if (i < i0 || i >= i1) continue;
             const int id = tid + MW * 64 * i, r = id / CPR, c = id % CPR;
             if (NCH % (MW * 64) != 0 && id >= NCH) continue;
-            const uint32_t off = (uint32_t) ((plain ? r : std::min(it_ * MTILE + r, last_rel)) * (int) CROW);
+            const int rel = plain ? r : std::min(it_ * MTILE + r, last_rel);
+            const uint32_t off = (uint32_t) ((selt ? cell(jb + rel) : (int64_t) rel) * CROW);
             if constexpr (Q8) {
                 st[i % H1] = *reinterpret_cast<const u4v*>(sp + off + ML / 32 * 2 + c * 16);
                 stsc[i % H1] = *reinterpret_cast<const uint16_t*>(sp + off + 2 * (c / 2));
@@ -185,13 +206,14 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
     // w + 4, so that every wave has the same count in flight).
     constexpr int NU = MTILE * 72, NDMA = (NU + MW * 64 - 1) / (MW * 64);
     auto dma = [&](lds_u8* dst, int it_) {
-        const bool plain = (it_ + 1) * MTILE - 1 <= last_rel;
-        const uint8_t* sp = split_base + (plain ? (int64_t) it_ * MTILE * CROW : 0);
+        const bool plain = !selt && (it_ + 1) * MTILE - 1 <= last_rel;
+        const uint8_t* sp = selt ? p.cache : split_base + (plain ? (int64_t) it_ * MTILE * CROW : 0);
 #pragma unroll
         for (int i = 0; i < NDMA; ++i) {
             const int u0 = i * MW * 64 + w * 64 < NU ? i * MW * 64 + w * 64 : i * MW * 64 + (w & 3) * 64;
             const int u = u0 + lane, r = u / 72, c = (u % 72) ^ swz(r);
-            const uint32_t off = (uint32_t) ((plain ? r : std::min(it_ * MTILE + r, last_rel)) * (int) CROW + c * 16);
+            const int rel = plain ? r : std::min(it_ * MTILE + r, last_rel);
+            const uint32_t off = (uint32_t) ((selt ? cell(jb + rel) : (int64_t) rel) * CROW + c * 16);
             if (CPR == 72 || c < CPR)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (sp + off),
                                                  (__attribute__((address_space(3))) void*) (dst + u0 * 16), 16, 0, 0);
@@ -549,7 +571,8 @@ int64_t mla_kbs(int64_t cells, int64_t groups) {
 }
 
 int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const void* qa, const void* cache, void* u, int64_t T, int64_t H,
-               int64_t pos0, float scale, float* scratch, size_t scratch_floats) {
+               int64_t pos0, float scale, float* scratch, size_t scratch_floats, const int32_t* sel = nullptr, const int32_t* sel_cnt = nullptr,
+               int64_t K = 0) {
     const std::string w(who);
     if (T <= 0) return 0;
     if (H <= 0 || pos0 < 0) return ns_fail(w + ": heads and a position");
@@ -558,8 +581,17 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     if (((uintptr_t) qa | (uintptr_t) cache | (uintptr_t) scratch) % 16) return ns_fail(w + ": buffers 16-byte aligned");
     if (!(scale > 0.0f)) return ns_fail(w + ": a positive scale");
     NS_HIP(hipSetDevice(g->dev));
-    const int64_t rows = T * H, nz = (rows + MROWS - 1) / MROWS, cells = pos0 + T;
-    int64_t kbs = mla_kbs(cells, nz), ns = (cells + kbs - 1) / kbs;
+    // With a selection (sel_cnt on the device) a row group holds one row's heads; a row's cell count is only known there:
+    // at most 4 K + 3 listed cells, or every earlier cell where its count is negative. Splits are sized for the listed
+    // form and enough of them cover a dense row.
+    const bool per_t = sel_cnt != nullptr;
+    if (per_t && (!sel || K < 0 || K > (int64_t) 1 << 24)) return ns_fail(w + ": a selection has cell pools and their count");
+    if ((pos0 + T) * (int64_t) (q8 ? 544 : (512 + R) * 2) >= (int64_t) 1 << 32 && per_t) return ns_fail(w + ": a selection over a cache past 4 GiB");
+    const int64_t rows = T * H, nz = per_t ? T * ((H + MROWS - 1) / MROWS) : (rows + MROWS - 1) / MROWS;
+    const int64_t listed = 4 * K + 3, cells = per_t ? std::max(pos0 + T, listed) : pos0 + T;
+    int64_t kbs = mla_kbs(per_t ? listed : cells, nz);
+    if (per_t) kbs = std::max(kbs, ((cells + 1023) / 1024 + MTILE - 1) / MTILE * MTILE);
+    int64_t ns = (cells + kbs - 1) / kbs;
     // a caller's scratch may be smaller than the rule asks (the library's own, for the reference-named entry points):
     // fewer, longer splits then
     while ((size_t) (rows * ns * PSTRIDE) > scratch_floats && ns > 1) {
@@ -579,6 +611,10 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     p.ns = (int) ns;
     p.sl2 = scale * 1.4426950408889634f;
     p.part = scratch;
+    p.sel = sel;
+    p.sel_cnt = sel_cnt;
+    p.K = (int) K;
+    p.per_t = per_t;
     dim3 grid((unsigned) ns, (unsigned) nz);
     if (ns_profile_mark(g, 0)) return -1;
     if (q8) mla_decode_kernel<0, true><<<grid, MW * 64, 0, g->q>>>(p);
@@ -650,22 +686,18 @@ int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint1
 int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                       const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
     NS_TRY
-    (void) K;
     if (T <= 0) return 0;
     if (L != 512) return ns_fail("ns_mla_attend_sel: latent width 512");
-    if (sel || sel_cnt) return ns_fail("ns_mla_attend_sel: the sparse cell selection is not built; pass sel = sel_cnt = NULL (dense)");
-    return mla_latent(g, "ns_mla_attend_sel", 0, 0, 0, false, qa, c, u, T, H, pos0, scale, g->own_scratch, g->own_scratch_floats);
+    return mla_latent(g, "ns_mla_attend_sel", 0, 0, 0, false, qa, c, u, T, H, pos0, scale, g->own_scratch, g->own_scratch_floats, sel, sel_cnt, K);
     NS_CATCH
 }
 
 int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                          const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
     NS_TRY
-    (void) K;
     if (T <= 0) return 0;
     if (L != 512 || T > 8) return ns_fail("ns_mla_attend_sel_q8: latent width 512, at most 8 rows");
-    if (sel || sel_cnt) return ns_fail("ns_mla_attend_sel_q8: the sparse cell selection is not built; pass sel = sel_cnt = NULL (dense)");
-    return mla_latent(g, "ns_mla_attend_sel_q8", 0, 0, 0, true, qa, c, u, T, H, pos0, scale, g->own_scratch, g->own_scratch_floats);
+    return mla_latent(g, "ns_mla_attend_sel_q8", 0, 0, 0, true, qa, c, u, T, H, pos0, scale, g->own_scratch, g->own_scratch_floats, sel, sel_cnt, K);
     NS_CATCH
 }
 

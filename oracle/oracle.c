@@ -561,48 +561,110 @@ ORC_API int orc_attn_flash_model(const float* q, int64_t qs, const uint8_t* kc, 
 }
 
 /* MiniMax-M3's exact GQA over a position-major half cache [pos][G][128], explicit scale, chunks of 2048 keys with a
- * chunk-wide maximum, the values summed in key order - kernels/llm/minimaxm3/mm3.cpp:118-190 (dense: sel == NULL) */
-ORC_API int orc_mm3_attend(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int64_t T, int64_t H, int64_t G, int64_t pos0,
-                           float scale) {
+ * chunk-wide maximum, the values summed in key order - kernels/llm/minimaxm3/mm3.cpp:118-190. sel == NULL: dense
+ * (keys 0 .. pos); else sel [T][G][K] names K blocks of 128 keys a (row, key head) (-1: none), the keys of a listed block
+ * past the row's position dropped (:143-157). */
+ORC_API int orc_mm3_attend_sel(const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
+                               int64_t H, int64_t G, int64_t pos0, float scale) {
     enum { BLK = 128, CHK = 2048 };
     if (G <= 0 || H % G) return -1;
     const int64_t per = H / G;
 #pragma omp parallel for collapse(2) schedule(dynamic)
     for (int64_t t = 0; t < T; ++t)
         for (int64_t hq = 0; hq < H; ++hq) {
-            const int64_t gi = hq / per, pos = pos0 + t, total = pos + 1;
+            const int64_t gi = hq / per, pos = pos0 + t, total = sel ? K * BLK : pos + 1;
             const float* qr = q + (t * H + hq) * BLK;
             float sc[CHK], acc[BLK], m = -INFINITY, l = 0.0f;
+            int64_t jj[CHK];
             for (int d = 0; d < BLK; ++d) acc[d] = 0.0f;
             for (int64_t c0 = 0; c0 < total; c0 += CHK) {
                 const int n = (int) imin(CHK, total - c0);
                 float cm = -INFINITY;
                 for (int i = 0; i < n; ++i) {
-                    const uint16_t* kr = kc + ((c0 + i) * G + gi) * BLK;
-                    float a = 0.0f;
-                    for (int d = 0; d < BLK; ++d) a += qr[d] * orc_h2f(kr[d]);
-                    sc[i] = a * scale;
-                    cm = fmaxf(cm, sc[i]);
+                    const int64_t idx = c0 + i;
+                    int64_t j = idx;
+                    if (sel) {
+                        const int32_t b = sel[(t * G + gi) * K + idx / BLK];
+                        j = b < 0 ? -1 : (int64_t) b * BLK + idx % BLK;
+                    }
+                    float sv = -INFINITY;
+                    if (j >= 0 && j <= pos) {
+                        const uint16_t* kr = kc + (j * G + gi) * BLK;
+                        float a = 0.0f;
+                        for (int d = 0; d < BLK; ++d) a += qr[d] * orc_h2f(kr[d]);
+                        sv = a * scale;
+                    } else {
+                        j = -1;
+                    }
+                    sc[i] = sv;
+                    jj[i] = j;
+                    cm = fmaxf(cm, sv);
                 }
                 const float nm = fmaxf(m, cm), corr = m == -INFINITY ? 0.0f : expf(m - nm);
                 /* the device sums each of 128 lanes' weights i, i + 128, ... and then reduces; any order is float32
                  * reassociation */
                 float ls = 0.0f;
-                for (int i = 0; i < n; ++i) {
-                    sc[i] = expf(sc[i] - nm);
-                    ls += sc[i];
-                }
+                if (nm > -INFINITY)
+                    for (int i = 0; i < n; ++i) {
+                        sc[i] = sc[i] == -INFINITY ? 0.0f : expf(sc[i] - nm);
+                        ls += sc[i];
+                    }
                 l = l * corr + ls;
                 for (int d = 0; d < BLK; ++d) acc[d] *= corr;
-                for (int i = 0; i < n; ++i) {
-                    const uint16_t* vr = vc + ((c0 + i) * G + gi) * BLK;
-                    for (int d = 0; d < BLK; ++d) acc[d] += sc[i] * orc_h2f(vr[d]);
-                }
+                if (nm > -INFINITY)
+                    for (int i = 0; i < n; ++i) {
+                        if (jj[i] < 0) continue;
+                        const uint16_t* vr = vc + (jj[i] * G + gi) * BLK;
+                        for (int d = 0; d < BLK; ++d) acc[d] += sc[i] * orc_h2f(vr[d]);
+                    }
                 m = nm;
             }
             for (int d = 0; d < BLK; ++d) out[(t * H + hq) * BLK + d] = l > 0.0f ? acc[d] / l : 0.0f;
         }
     return 0;
+}
+ORC_API int orc_mm3_attend(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int64_t T, int64_t H, int64_t G, int64_t pos0,
+                           float scale) {
+    return orc_mm3_attend_sel(q, kc, vc, NULL, 0, out, T, H, G, pos0, scale);
+}
+
+/* MiniMax-M3's block indexer - kernels/llm/minimaxm3/mm3.cpp:59-116. Scores: bs [T][G][nblk] = the largest iq . ik_j over a
+ * block's keys j <= pos (ik half [pos][128]); -inf for a block wholly past the row; + 1e30 for the `local` most recent
+ * blocks (b + local > pos / 128), which therefore always win. */
+ORC_API void orc_mm3_idx_scores(const float* iq, const uint16_t* ik, float* bs, int64_t T, int64_t G, int64_t nblk, int64_t pos0, int64_t local) {
+    enum { BLK = 128 };
+    for (int64_t t = 0; t < T; ++t)
+        for (int64_t gi = 0; gi < G; ++gi)
+            for (int64_t b = 0; b < nblk; ++b) {
+                const int64_t pos = pos0 + t;
+                const float* qv = iq + (t * G + gi) * BLK;
+                float m = -INFINITY;
+                for (int64_t j = b * BLK; j < (b + 1) * BLK && j <= pos; ++j) {
+                    float sv = 0.0f;
+                    for (int d = 0; d < BLK; ++d) sv += qv[d] * orc_h2f(ik[j * BLK + d]);
+                    m = fmaxf(m, sv);
+                }
+                if (b * BLK > pos) m = -INFINITY;
+                else if (b + local > pos / BLK) m = m + 1e30f;
+                bs[(t * G + gi) * nblk + b] = m;
+            }
+}
+/* Top K blocks a row, best first, the lowest index of equal scores; -1 once nothing finite is left. The scores picked
+ * are overwritten with -inf, as the device does (:91-116). */
+ORC_API void orc_mm3_idx_topk(float* bs, int32_t* sel, int64_t T, int64_t G, int64_t nblk, int64_t K) {
+    for (int64_t row = 0; row < T * G; ++row) {
+        float* sc = bs + row * nblk;
+        for (int64_t k = 0; k < K; ++k) {
+            float best = -INFINITY;
+            for (int64_t b = 0; b < nblk; ++b) best = fmaxf(best, sc[b]);
+            int32_t at = -1;
+            if (best > -INFINITY)
+                for (int64_t b = 0; b < nblk; ++b)
+                    if (sc[b] == best) { at = (int32_t) b; break; }
+            sel[row * K + k] = at;
+            if (at >= 0) sc[at] = -INFINITY;
+        }
+    }
 }
 
 /* ------------------------------------------------------------------------------------------------ MLA */
@@ -786,20 +848,24 @@ ORC_API void orc_mla_f64(const float* qa, const uint16_t* cache, double* u, int6
 
 /* GLM-5.3's latent-only MLA, two passes: every score (qa . c_i) scale, their maximum, then w_i = exp(d_i - mx),
  * u = sum w_i c_i / sum w_i - kernels/llm/glm5next/glm.cpp:1129-1183. q8 != 0: rows [L/32 half scales][L int8], value
- * h2f(d_b) q. Dense cells 0..pos0 + t. */
-ORC_API void orc_glm_mla_attend(const float* qa, const uint8_t* cache, int q8, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0,
-                                float scale) {
+ * h2f(d_b) q. */
+ORC_API void orc_glm_mla_attend_sel(const float* qa, const uint8_t* cache, int q8, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0,
+                                    float scale, const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
     const int64_t nb = L / 32, rb = q8 ? nb * 2 + L : 2 * L;
 #pragma omp parallel for collapse(2) schedule(dynamic)
     for (int64_t t = 0; t < T; ++t)
         for (int64_t h = 0; h < H; ++h) {
             const float* qv = qa + (t * H + h) * L;
-            const int64_t n = pos0 + t + 1;
-            float* s = (float*) malloc(sizeof(float) * (size_t) n);
+            /* a row's cells: every earlier one (sel_cnt NULL or negative), or the pools sel[t][0, sel_cnt[t]) of 4 cells
+             * each and the row's incomplete pool 4 ((p + 1) / 4) .. p - kernels/llm/glm5next/glm.cpp:1062-1067,1095-1102 */
+            const int64_t p = pos0 + t, ns = sel_cnt ? sel_cnt[t] : -1, tail0 = 4 * ((p + 1) / 4);
+            const int64_t n = ns < 0 ? p + 1 : 4 * ns + (p + 1 - tail0);
+#define ORC_CELL(i) (ns < 0 ? (i) : (i) < 4 * ns ? 4 * (int64_t) sel[t * K + (i) / 4] + (i) % 4 : tail0 + ((i) - 4 * ns))
+            float* s = (float*) malloc(sizeof(float) * (size_t) (n > 0 ? n : 1));
             float* c = (float*) malloc(sizeof(float) * (size_t) L);
             float mx = -INFINITY;
             for (int64_t i = 0; i < n; ++i) {
-                const uint8_t* row = cache + i * rb;
+                const uint8_t* row = cache + ORC_CELL(i) * rb;
                 float a = 0.0f;
                 for (int64_t f = 0; f < L; ++f) {
                     const float cv = q8 ? orc_h2f(ld16(row + 2 * (f / 32))) * (float) (int8_t) row[nb * 2 + f] : orc_h2f(ld16(row + 2 * f));
@@ -812,7 +878,7 @@ ORC_API void orc_glm_mla_attend(const float* qa, const uint8_t* cache, int q8, f
             for (int64_t f = 0; f < L; ++f) o[f] = 0.0f;
             float tot = 0.0f;
             for (int64_t i = 0; i < n; ++i) {
-                const uint8_t* row = cache + i * rb;
+                const uint8_t* row = cache + ORC_CELL(i) * rb;
                 const float w = expf(s[i] - mx);
                 tot += w;
                 for (int64_t f = 0; f < L; ++f) {
@@ -820,10 +886,15 @@ ORC_API void orc_glm_mla_attend(const float* qa, const uint8_t* cache, int q8, f
                     o[f] += w * c[f];
                 }
             }
+#undef ORC_CELL
             for (int64_t f = 0; f < L; ++f) o[f] = tot > 0.0f ? o[f] / tot : 0.0f;
             free(s);
             free(c);
         }
+}
+ORC_API void orc_glm_mla_attend(const float* qa, const uint8_t* cache, int q8, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0,
+                                float scale) {
+    orc_glm_mla_attend_sel(qa, cache, q8, u, T, H, L, pos0, scale, NULL, NULL, 0);
 }
 
 /* ------------------------------------------------------------------------------------ norm + rotary positions */

@@ -46,6 +46,10 @@ def lib():
             "orc_attn_f64": (C.c_int, [P, i64, P, P, C.c_int, C.c_int, i64, i64, i64, i64, i64, i64, i64, C.c_int, f64, P]),
             "orc_attn_flash_model": (C.c_int, [P, i64, P, P, C.c_int, C.c_int, i64, i64, i64, i64, i64, i64, i64, i64, P]),
             "orc_mm3_attend": (C.c_int, [P, P, P, P, i64, i64, i64, i64, f32]),
+            "orc_mm3_attend_sel": (C.c_int, [P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
+            "orc_mm3_idx_scores": (None, [P, P, P, i64, i64, i64, i64, i64]),
+            "orc_mm3_idx_topk": (None, [P, P, i64, i64, i64, i64]),
+            "orc_glm_mla_attend_sel": (None, [P, P, C.c_int, P, i64, i64, i64, i64, f32, P, P, i64]),
             "orc_ds2_kv_store": (C.c_int, [P, P, f32, P, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32]),
             "orc_mla_absorb": (None, [P, P, P, i64, i64, i64, i64, i64]),
             "orc_mla_decode_u": (None, [P, P, P, i64, i64, i64, i64, i64, f32]),
@@ -203,13 +207,30 @@ def attn_flash_model(q, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=0, kbs=0, pm=Fal
     return out
 
 
-def mm3_attend(q, kc, vc, T, H, G, pos0, scale):
+def mm3_attend(q, kc, vc, T, H, G, pos0, scale, sel=None, K=0):
     q = _c(q, np.float32)
     out = np.empty((T, H * 128), np.float32)
-    rc = lib().orc_mm3_attend(_p(q), _p(kc), _p(vc), _p(out), T, H, G, pos0, float(scale))
+    sp = _p(_c(sel, np.int32)) if sel is not None else None
+    rc = lib().orc_mm3_attend_sel(_p(q), _p(kc), _p(vc), sp, K, _p(out), T, H, G, pos0, float(scale))
     if rc:
         raise ValueError("orc_mm3_attend: bad arguments")
     return out
+
+
+def mm3_idx_scores(iq, ik, T, G, nblk, pos0, local):
+    iq, ik = _c(iq, np.float32), _c(ik, np.uint16)
+    bs = np.empty((T, G, nblk), np.float32)
+    lib().orc_mm3_idx_scores(_p(iq), _p(ik), _p(bs), T, G, nblk, pos0, local)
+    return bs
+
+
+def mm3_idx_topk(bs, K):
+    """(sel [T][G][K], the scores as the selection leaves them)."""
+    bs = np.array(bs, np.float32)
+    T, G, nblk = bs.shape
+    sel = np.empty((T, G, K), np.int32)
+    lib().orc_mm3_idx_topk(_p(bs), _p(sel), T, G, nblk, K)
+    return sel, bs
 
 
 # ---- MLA ---------------------------------------------------------------------------------------------------------
@@ -246,6 +267,13 @@ def mla_f64(qa, cache, T, H, pos0, scale, L=512, R=64):
     qa, cache = _c(qa, np.float32), _c(cache, np.uint16)
     u = np.empty((T, H, L), np.float64)
     lib().orc_mla_f64(_p(qa), _p(cache), _p(u), T, H, L, R, pos0, float(scale))
+    return u
+
+
+def glm_mla_attend_sel(qa, cache, q8, T, H, L, pos0, scale, sel, sel_cnt, K):
+    qa = _c(qa, np.float32)
+    u = np.empty((T, H * L), np.float32)
+    lib().orc_glm_mla_attend_sel(_p(qa), _p(cache), int(q8), _p(u), T, H, L, pos0, float(scale), _p(_c(sel, np.int32)), _p(_c(sel_cnt, np.int32)), K)
     return u
 
 

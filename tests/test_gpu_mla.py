@@ -120,5 +120,6 @@ def test_glm_latent_only_and_q8_rows(ops):
     ops.mla_attend(DevBuf.of(g, qa), yb, u, T, H, L, pos0, 0.04, q8=True)
     ref = orc.glm_mla_attend(qa, want_rows, True, T, H, L, pos0, 0.04)
     _close(u.read(np.float32).reshape(T, H, L), ref.astype(np.float64), "GLM q8 latent MLA vs the reference-order restatement")
-    assert ops.k.mla_attend_sel(g.raw, u.ptr, u.ptr, u.ptr, 1, 1, 512, 0, 1.0, u.ptr, None, 4) == -1
-    assert "not built" in ops.k.api.error()
+    # pool counts without pools are rejected (pools without counts are a dense pass, as in the reference)
+    assert ops.k.mla_attend_sel(g.raw, u.ptr, u.ptr, u.ptr, 1, 1, 512, 0, 1.0, None, u.ptr, 4) == -1
+    assert "selection" in ops.k.api.error()

@@ -1,0 +1,95 @@
+"""Sparse selection on the GPU: MiniMax-M3's block lists and indexer, GLM's cell pools - against the oracle (pinned in
+tests/test_oracle_sparse.py). Attention within max-abs 2e-3 / relative L2 1e-3 of the oracle's float32 result; the
+selection itself (comparisons only) bit for bit."""
+import numpy as np
+import pytest
+
+from nextsycl_amd import DevBuf
+from oracle import orc
+
+pytestmark = pytest.mark.gpu
+
+
+def close(got, want):
+    err = np.abs(got - want).max()
+    rel = np.linalg.norm((got - want).ravel()) / max(np.linalg.norm(want.ravel()), 1e-30)
+    assert err <= 2e-3 and rel <= 1e-3, (err, rel)
+
+
+@pytest.mark.parametrize("T,H,G,pos0,K", [(1, 8, 2, 2000, 6), (3, 64, 4, 5000, 16), (2, 16, 1, 300, 4)])
+def test_minimaxm3_block_lists(ops, T, H, G, pos0, K):
+    g = ops.gpu
+    n = pos0 + T
+    nblk = (n + 127) // 128
+    q = orc.randn(41, (T, H * 128))
+    kc, _ = orc.randn_f16(42, (n, G, 128)); vc, _ = orc.randn_f16(43, (n, G, 128))
+    rng = np.random.default_rng(5)
+    sel = np.stack([np.stack([rng.permutation(nblk)[:K] if K <= nblk else np.r_[rng.permutation(nblk), [-1] * (K - nblk)] for _ in range(G)])
+                    for _ in range(T)]).astype(np.int32)
+    sel[0, 0, 1] = -1                                   # a hole
+    sel[-1, -1, 0] = nblk - 1                           # the block the row's own position cuts
+    scale = 0.0884
+    out = DevBuf(g, T * H * 128 * 4); out.fill(0xFF)
+    ops.minimaxm3_attend(DevBuf.of(g, q), DevBuf.of(g, kc), DevBuf.of(g, vc), out, T, H, G, pos0, scale, sel=DevBuf.of(g, sel), K=K)
+    want = orc.mm3_attend(q, kc, vc, T, H, G, pos0, scale, sel=sel, K=K)
+    close(out.read(np.float32).reshape(T, H * 128), want)
+    # every block listed in order = the dense pass
+    allb = np.tile(np.arange(nblk, dtype=np.int32), (T, G, 1))
+    out2 = DevBuf(g, T * H * 128 * 4)
+    ops.minimaxm3_attend(DevBuf.of(g, q), DevBuf.of(g, kc), DevBuf.of(g, vc), out2, T, H, G, pos0, scale, sel=DevBuf.of(g, allb), K=nblk)
+    close(out2.read(np.float32).reshape(T, H * 128), orc.mm3_attend(q, kc, vc, T, H, G, pos0, scale))
+    # nothing listed: zeros
+    none = np.full((T, G, 2), -1, np.int32)
+    ops.minimaxm3_attend(DevBuf.of(g, q), DevBuf.of(g, kc), DevBuf.of(g, vc), out2, T, H, G, pos0, scale, sel=DevBuf.of(g, none), K=2)
+    assert not out2.read(np.float32).any()
+
+
+def test_minimaxm3_indexer(ops):
+    g = ops.gpu
+    T, G, pos0, local, K = 3, 2, 3000, 2, 8
+    n = pos0 + T
+    nblk = (n + 127) // 128 + 1                         # one block wholly past the rows
+    iq = orc.randn(44, (T, G, 128)); ik, _ = orc.randn_f16(45, (n, 128))
+    bs = DevBuf(g, T * G * nblk * 4)
+    ops.minimaxm3_idx_scores(DevBuf.of(g, iq), DevBuf.of(g, ik), bs, T, G, nblk, pos0, local)
+    got = bs.read(np.float32).reshape(T, G, nblk)
+    want = orc.mm3_idx_scores(iq, ik, T, G, nblk, pos0, local)
+    fin = np.isfinite(want) & (want < 1e29)
+    assert np.array_equal(np.isneginf(got), np.isneginf(want)) and np.array_equal(got > 1e29, want > 1e29)
+    assert np.abs(got[fin] - want[fin]).max() < 1e-4
+    # selection on the GPU's own scores against the oracle's selection on the same scores: bit for bit
+    sel = DevBuf(g, T * G * K * 4)
+    ops.minimaxm3_idx_topk(bs, sel, T, G, nblk, K)
+    want_sel, want_left = orc.mm3_idx_topk(got, K)
+    assert np.array_equal(sel.read(np.int32).reshape(T, G, K), want_sel)
+    assert np.array_equal(bs.read(np.float32).reshape(T, G, nblk).view(np.uint32), want_left.view(np.uint32))
+    # ties and exhaustion
+    sc = np.array([[[1.0, 7.0, 7.0, -np.inf, 3.0, 7.0]]], np.float32)
+    b2, s2 = DevBuf.of(g, sc), DevBuf(g, 6 * 4)
+    ops.minimaxm3_idx_topk(b2, s2, 1, 1, 6, 6)
+    assert s2.read(np.int32).tolist() == [1, 2, 5, 4, 0, -1]
+
+
+@pytest.mark.parametrize("q8", [False, True])
+@pytest.mark.parametrize("T,H,pos0,K", [(1, 128, 5000, 64), (3, 64, 2500, 512), (2, 160, 900, 16)])
+def test_glm_cell_pools(ops, q8, T, H, pos0, K):
+    g = ops.gpu
+    L, scale = 512, 0.044
+    n = pos0 + T
+    qa = orc.randn(46, (T, H * L), 0.3)
+    x = orc.randn(47, (n, L))
+    if q8:
+        rows = orc.glm_to_q8row(x, L)
+    else:
+        rows = orc.f2h(x).view(np.uint8).reshape(n, 2 * L)
+    rng = np.random.default_rng(7)
+    npool = (pos0 + 1) // 4
+    sel = np.stack([rng.permutation(npool)[:K] if K <= npool else np.r_[rng.permutation(npool), [0] * (K - npool)] for _ in range(T)]).astype(np.int32)
+    cnt = np.array([min(K, npool)] + [K // 3, -1][:T - 1], np.int32)          # a full list, a short one, a dense row
+    u = DevBuf(g, T * H * L * 4); u.fill(0xFF)
+    ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, scale, q8=q8, sel=DevBuf.of(g, sel), sel_cnt=DevBuf.of(g, cnt), K=K)
+    want = orc.glm_mla_attend_sel(qa, rows, q8, T, H, L, pos0, scale, sel, cnt, K)
+    close(u.read(np.float32).reshape(T, H * L), want)
+    # no counts: the dense pass, as before
+    ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, scale, q8=q8)
+    close(u.read(np.float32).reshape(T, H * L), orc.glm_mla_attend(qa, rows, q8, T, H, L, pos0, scale).reshape(T, H * L))
