@@ -21,11 +21,13 @@ extern "C" {
 
 // ---- prompt form ------------------------------------------------------------------------------------------------------
 
-int ns_mg_attn_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) { return T > DECODE_ROWS && D == 128 && Hkv > 0 && Hq > 0 && Hq % Hkv == 0; }
+int ns_mg_attn_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) {
+    return T > DECODE_ROWS && (D == 128 || D == 256) && Hkv > 0 && Hq > 0 && Hq % Hkv == 0;
+}
 
 int ns_mg_attn_prompt(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap,
                       int64_t p0, int64_t win, float* out) {
-    if (!ns_mg_attn_prompt_supported(T, Hq, Hkv, D)) return ns_fail("ns_mg_attn_prompt: more than 16 rows, heads of 128, query heads a multiple of the key heads");
+    if (!ns_mg_attn_prompt_supported(T, Hq, Hkv, D)) return ns_fail("ns_mg_attn_prompt: more than 16 rows, heads of 128 or 256, query heads a multiple of the key heads");
     return ns_attn_prompt_any(g, "ns_mg_attn_prompt", 0, 0, 0, q, Hq * D, kc, vc, T, Hq, Hkv, D, cap, p0, win, 0.0f, out);
 }
 
@@ -33,14 +35,14 @@ int ns_q35_attn_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) 
 
 int ns_q35_attn_prompt(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
                        int64_t cap, int64_t p0, float* out) {
-    if (!ns_q35_attn_prompt_supported(T, Hq, Hkv, D)) return ns_fail("ns_q35_attn_prompt: more than 16 rows, heads of 128, query heads a multiple of the key heads");
+    if (!ns_q35_attn_prompt_supported(T, Hq, Hkv, D)) return ns_fail("ns_q35_attn_prompt: more than 16 rows, heads of 128 or 256, query heads a multiple of the key heads");
     return ns_attn_prompt_any(g, "ns_q35_attn_prompt", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, 0.0f, out);
 }
 
 int ns_q35_attn_prompt_kv(ns_gpu* g, int kt, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv,
                           int64_t D, int64_t cap, int64_t p0, float* out) {
-    if (!ns_q35_attn_prompt_supported(T, Hq, Hkv, D)) return ns_fail("ns_q35_attn_prompt_kv: more than 16 rows, heads of 128, query heads a multiple of the key heads");
-    if (kt != 0) return ns_fail("ns_q35_attn_prompt_kv: the prompt kernel reads a half cache (form 0); quantized forms take the decode kernel");
+    if (!ns_q35_attn_prompt_supported(T, Hq, Hkv, D)) return ns_fail("ns_q35_attn_prompt_kv: more than 16 rows, heads of 128 or 256, query heads a multiple of the key heads");
+    if (kt < 0 || kt > 2) return ns_fail("ns_q35_attn_prompt_kv: a cache form 0 (half), 1 (q8_0) or 2 (q4_0)");
     return ns_attn_prompt_any(g, "ns_q35_attn_prompt_kv", 0, kt, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, 0.0f, out);
 }
 

@@ -82,24 +82,6 @@ struct TileRegs {
     uint16_t vsc[DMA ? 1 : NLV];
 };
 
-// 4 int8 in a word -> 4 halfs x scale; each product is exact in float32, so one rounding to half (what the reference
-// stages: half((float) q * (float) d))
-__device__ __forceinline__ void dq8x4(uint32_t w, _Float16 d, short* o) {
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        const _Float16 h = (_Float16) (short) (int8_t) (w >> (8 * b)) * d;
-        o[b] = __builtin_bit_cast(short, h);
-    }
-}
-// 4 nibbles (bits sh .. sh + 3 of each byte) -> 4 halfs: (nibble - 8) x scale
-__device__ __forceinline__ void dq4x4(uint32_t w, int sh, _Float16 d, short* o) {
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        const _Float16 h = (_Float16) (short) ((int) ((w >> (8 * b + sh)) & 15u) - 8) * d;
-        o[b] = __builtin_bit_cast(short, h);
-    }
-}
-
 template <int D, int RT, int KT>
 __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kernel(const DecodeParams p) {
     constexpr bool BF = KT == 3;

@@ -33,7 +33,8 @@
 
 namespace {
 
-constexpr int PW = 4, ROWS = 128, KT_TILE = 64;
+constexpr int PW = 4, KT_TILE = 64;
+constexpr int rows_of(int D) { return D == 128 ? 128 : 64; }   // query rows a work-group
 
 struct PrefillParams {
     const void* q;
@@ -52,9 +53,12 @@ struct PrefillParams {
 // a 16-byte chunk of a K or V row on its way from global memory to LDS (a plain vector type: arrays of it stay in registers)
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
 
-template <int D, bool BF>
-__global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillParams p) {
-    static_assert(D == 128, "head size 128");
+template <int D, bool BF, int KT>
+__global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel(const PrefillParams p) {
+    static_assert(D == 128 || D == 256, "head size 128 or 256");
+    static_assert(KT == 0 || !BF, "quantized rows are widened to half");
+    // a wave owns RT row tiles of 16: 32 rows at D = 128; 16 at D = 256, whose accumulators are twice as wide
+    constexpr int RT = D == 128 ? 2 : 1, WROWS = RT * 16, ROWS = PW * WROWS;
     constexpr int KB = D / 32, DT = D / 16;
     constexpr int KS = D * 2 + 16, VS = D * 2 + 32;             // bytes a staged key row / value row
     constexpr int KBUF = KT_TILE * KS, VBUF = KT_TILE * VS;
@@ -81,11 +85,11 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
     const int64_t kbeg = p.win > 0 ? std::max<int64_t>(0, p.p0 + r0 + 1 - p.win) : 0;
 
     // ---- this lane's two rows: positions, key ranges, Q^T operands
-    int64_t lo_r[2], hi_r[2];
-    s8v qreg[2][KB];
+    int64_t lo_r[RT], hi_r[RT];
+    s8v qreg[RT][KB];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-        const int row = r0 + w * 32 + rt * 16 + n;
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = r0 + w * WROWS + rt * 16 + n;
         const bool live = row < p.T;
         const int rr = live ? row : p.T - 1;
         const int64_t pos = p.p0 + rr;
@@ -127,82 +131,132 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
     // From here on keys are counted from the first tile's first key (32-bit): tile k holds keys 64 k .. 64 k + 63, step
     // s = 2 k + h its 32-key half h
     const int64_t base = t0 * KT_TILE;
-    int lo32[2], hi32[2];
+    int lo32[RT], hi32[RT];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-        const bool live = r0 + w * 32 + rt * 16 + n < p.T;
+    for (int rt = 0; rt < RT; ++rt) {
+        const bool live = r0 + w * WROWS + rt * 16 + n < p.T;
         lo32[rt] = live ? (int) (lo_r[rt] - base) : 1;
         hi32[rt] = live ? (int) (hi_r[rt] - base) : 0;
     }
     // the wave's own steps: from its first row's first key to its last row's last; steps in between that no row's edge
     // crosses need no mask
-    const int wrow0 = r0 + w * 32, wrow1 = std::min(wrow0 + 31, p.T - 1);
+    const int wrow0 = r0 + w * WROWS, wrow1 = std::min(wrow0 + WROWS - 1, p.T - 1);
     const int w_full_end = (int) (p.p0 + wrow0 + 1 - base);
     const int w_full_beg = p.win > 0 ? (int) (std::max<int64_t>(0, p.p0 + wrow1 + 1 - p.win) - base) : 0;
 
     // Online softmax state, in base-2 exponent units (scores x scale x log2 e): nbr = minus the reference the weights
     // are taken against, thr = how far a score may exceed it before the reference moves (-inf while the row has seen no
     // key: the first one sets it), l_r = this lane's own share of the row's sum
-    float nbr[2] = {0.0f, 0.0f}, thr[2] = {-INFINITY, -INFINITY}, l_r[2] = {0.0f, 0.0f};
-    f4v o[2][DT];
+    float nbr[RT], thr[RT], l_r[RT];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
+    for (int rt = 0; rt < RT; ++rt) {
+        nbr[rt] = 0.0f;
+        thr[rt] = -INFINITY;
+        l_r[rt] = 0.0f;
+    }
+    f4v o[RT][DT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[rt][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
 
-    // ---- global -> registers -> LDS. A thread's chunks of a tile: chunk c = tid + 256 i -> key c / 16, 16-byte piece
-    // c % 16. A tile wholly inside [kbeg, kend) of an unwrapped cache is read at a wave-uniform address plus a 32-bit
-    // lane offset; otherwise keys outside are clamped into the range (a valid row, masked; a tile past the last is
-    // fetched as the last row over and over and never used) and a wrapped ring's slot is position % cap: the first
+    // ---- global -> registers -> LDS. A cache row is fetched in 16-byte raw chunks: 16-bit rows D / 8 of them, each one
+    // LDS piece; q8_0 rows D / 16 (16 int8 -> 2 pieces of 8 halfs, the block's half scale fetched beside it); q4_0 rows
+    // D / 32 (one block: 32 nibbles -> 4 pieces). A thread's chunks of a tile: chunk c = tid + 256 i -> key c / CPR, raw
+    // chunk c % CPR. A tile wholly inside [kbeg, kend) of an unwrapped cache is read at a wave-uniform address plus a
+    // 32-bit lane offset; otherwise keys outside are clamped into the range (a valid row, masked; a tile past the last
+    // is fetched as the last row over and over and never used) and a wrapped ring's slot is position % cap: the first
     // key's once, then offsets from it with at most two wraps (a pass's keys span less than two rings)
+    constexpr int CPR = KT == 0 ? D / 8 : KT == 1 ? D / 16 : D / 32;             // raw chunks a row
+    constexpr int NST = KT_TILE * CPR / (PW * 64);                                // raw chunks a thread per tile
+    constexpr int KPI = PW * 64 / CPR;                                            // keys between a thread's chunks
+    constexpr int PPC = KT == 0 ? 1 : KT == 1 ? 2 : 4;                            // LDS pieces a raw chunk
+    static_assert(NST >= 1 && NST * PW * 64 == KT_TILE * CPR, "whole chunks a thread");
+    struct Stage {
+        u4v raw[NST];
+        uint16_t sc[KT == 0 ? 1 : NST];
+    };
     const int64_t kbeg_slot = p.wrap ? kbeg % p.cap : kbeg;
     const int kspan = (int) (kend - kbeg) - 1;
     const int kbeg32 = (int) (kbeg - base);
-    const int key0 = tid >> 4;                                    // chunk i of this thread: key key0 + 16 i, piece tid & 15
-    const uint32_t lane_off = (uint32_t) (key0 * p.row_stride) + (uint32_t) (tid & 15) * 16;
+    const int key0 = tid / CPR, rc = tid % CPR;                   // chunk i of this thread: key key0 + KPI i, raw chunk rc
+    const uint32_t lane_off = (uint32_t) (key0 * p.row_stride) + (uint32_t) rc * 16;
+    // where a chunk's scale sits in its row: q8_0 a half a block of 32 behind D values, q4_0 behind D / 2 bytes
+    // (as a distance from the chunk itself)
+    const uint32_t sc_rel = (KT == 1 ? (uint32_t) (D + 2 * (rc / 2)) : (uint32_t) (D / 2 + 2 * rc)) - (uint32_t) rc * 16;
     const int plain0 = kbeg32 > 0 ? 1 : 0, plain1 = p.wrap ? -1 : (int) ((kend - base) / KT_TILE) - 1;
-    auto fetch = [&](u4v (&st)[4], const uint8_t* cache, int krel) {
+    auto fetch = [&](Stage& st, const uint8_t* cache, int krel) {
         const uint8_t* sp = cache;
-        uint32_t off[4];
+        uint32_t off[NST];                                        // of the raw chunk
         if (krel >= plain0 && krel <= plain1) {
             sp += (base + (int64_t) krel * KT_TILE) * p.row_stride;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) off[i] = lane_off + (uint32_t) (i * 16 * p.row_stride);
+            for (int i = 0; i < NST; ++i) off[i] = lane_off + (uint32_t) (i * KPI * p.row_stride);
         } else {
             const int rel0 = krel * KT_TILE - kbeg32 + key0;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int rel = std::min(std::max(rel0 + 16 * i, 0), kspan);
+            for (int i = 0; i < NST; ++i) {
+                const int rel = std::min(std::max(rel0 + KPI * i, 0), kspan);
                 int64_t slot = kbeg_slot + rel;
                 if (p.wrap) {
                     slot = slot >= p.cap ? slot - p.cap : slot;
                     slot = slot >= p.cap ? slot - p.cap : slot;
                 }
-                off[i] = (uint32_t) (slot * p.row_stride) + (uint32_t) (tid & 15) * 16;   // a head's cache spans less than 4 GiB
+                off[i] = (uint32_t) (slot * p.row_stride) + (uint32_t) rc * 16;   // a head's cache spans less than 4 GiB
             }
         }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) st[i] = *reinterpret_cast<const u4v*>(sp + off[i]);
+        for (int i = 0; i < NST; ++i) {
+            st.raw[i] = *reinterpret_cast<const u4v*>(sp + off[i]);
+            if constexpr (KT != 0) st.sc[i] = *reinterpret_cast<const uint16_t*>(sp + off[i] + sc_rel);
+        }
     };
     typedef __attribute__((address_space(3))) uint8_t lds_u8;
     lds_u8* const L = (lds_u8*) lds;
-    // LDS map: K tiles at 0 and KBUF, V tiles at 2 KBUF and 2 KBUF + VBUF
+    // LDS map: K tiles at 0 and KBUF, V tiles at 2 KBUF and 2 KBUF + VBUF; rows of D halfs (+ padding) whatever the cache
     constexpr uint32_t V0 = 2 * KBUF;
-    const uint32_t k_wr = (uint32_t) (key0 * KS + (tid & 15) * 16), v_wr = (uint32_t) (key0 * VS + (tid & 15) * 16);
-    auto stash_k = [&](const u4v (&st)[4], int buf) {
+    // a raw chunk's pieces written at row stride RS from byte offset at (quantized rows widened: one rounding to half of
+    // (float) q x (float) scale, what the reference stages - qwen35/silo/attn.cpp:56-76)
+    const uint32_t k_wr = (uint32_t) (key0 * KS + rc * 16 * PPC), v_wr = (uint32_t) (key0 * VS + rc * 16 * PPC);
+    auto put = [&](const Stage& st, uint32_t at0, int RS) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<__attribute__((address_space(3))) u4v*>(L + buf * KBUF + k_wr + i * 16 * KS) = st[i];
-    };
-    auto stash_v = [&](const u4v (&st)[4], int buf) {
+        for (int i = 0; i < NST; ++i) {
+            const uint32_t at = at0 + (uint32_t) (i * KPI * RS);
+            if constexpr (KT == 0) {
+                *reinterpret_cast<__attribute__((address_space(3))) u4v*>(L + at) = st.raw[i];
+            } else {
+                const _Float16 d = __builtin_bit_cast(_Float16, st.sc[i]);
+                short tmp[8 * PPC];
+                if constexpr (KT == 1) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<__attribute__((address_space(3))) u4v*>(L + V0 + buf * VBUF + v_wr + i * 16 * VS) = st[i];
+                    for (int q = 0; q < 4; ++q) dq8x4(st.raw[i][q], d, tmp + 4 * q);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        dq4x4(st.raw[i][q], 0, d, tmp + 4 * q);            // values 0 .. 15: the low nibbles
+                        dq4x4(st.raw[i][q], 4, d, tmp + 16 + 4 * q);       // values 16 .. 31: the high nibbles
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < PPC; ++q) {
+                    s8v v8;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) v8[e] = tmp[q * 8 + e];
+                    *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at + q * 16) = v8;
+                }
+            }
+        }
     };
+    auto stash_k = [&](const Stage& st, int buf) { put(st, (uint32_t) (buf * KBUF) + k_wr, KS); };
+    auto stash_v = [&](const Stage& st, int buf) { put(st, V0 + (uint32_t) (buf * VBUF) + v_wr, VS); };
 
     const uint32_t k_rd = (uint32_t) (n * KS + g4 * 16);                          // + kt2 * 16 * KS + kb * 64
     const uint32_t v_rd = (uint32_t) ((g4 * 4 + (n >> 2)) * VS + (n & 3) * 8);    // + dt * 32 (+ 16 * VS)
-    s8v pb[2] = {s8v{0, 0, 0, 0, 0, 0, 0, 0}, s8v{0, 0, 0, 0, 0, 0, 0, 0}};
+    s8v pb[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) pb[rt] = s8v{0, 0, 0, 0, 0, 0, 0, 0};
     // S^T of one 32-key half (LDS byte offset kl) against the wave's 32 rows
-    auto scores = [&](f4v (&s)[2][2], uint32_t kl) {
+    auto scores = [&](f4v (&s)[RT][2], uint32_t kl) {
 #pragma unroll
         for (int kt2 = 0; kt2 < 2; ++kt2) {
             s8v ka[KB];
@@ -210,7 +264,7 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
             for (int kb = 0; kb < KB; ++kb)
                 ka[kb] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + kl + k_rd + kt2 * 16 * KS + kb * 64);
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) {
+            for (int rt = 0; rt < RT; ++rt) {
                 f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int kb = 0; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
@@ -226,7 +280,7 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
             const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + vl + v_rd + dt * 32 + 16 * VS));
             const s8v va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
+            for (int rt = 0; rt < RT; ++rt) o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
         }
     };
     // One step of the wave's software pipeline. Step s holds the scores of its own half in sc (computed a step earlier)
@@ -238,15 +292,15 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
     //    the row's sum makes the result the same function of the inputs)
     //   B: S^T of step s + 1              ||   weights of step s = exp2(arguments), their sum, rounding to 16 bit
     // The mask is applied under a wave-uniform branch: steps no row's causal or window edge crosses pay no comparison.
-    auto step = [&](f4v (&sc)[2][2], f4v (&sn)[2][2], uint32_t kl_next, uint32_t vl_prev, int j0, bool masked) {
-        float a[2][8], amax[2];
+    auto step = [&](f4v (&sc)[RT][2], f4v (&sn)[RT][2], uint32_t kl_next, uint32_t vl_prev, int j0, bool masked) {
+        float a[RT][8], amax[RT];
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt)
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int e = 0; e < 8; ++e) a[rt][e] = sc[rt][e >> 2][e & 3];
         if (masked) {
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) {
+            for (int rt = 0; rt < RT; ++rt) {
                 // keys lo .. hi of this half (relative, clamped into 0 .. 32 / -1 .. 31) are the row's: one unsigned
                 // compare a key (no key at all: lo = 64 puts every key below it)
                 const int lo_ = std::min(std::max(lo32[rt] - j0, 0), 32);
@@ -264,7 +318,7 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
         weigh(vl_prev);
         bool grow = false;
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
+        for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) a[rt][e] = __builtin_fmaf(a[rt][e], p.sl2, nbr[rt]);
             amax[rt] = fmaxf(fmaxf(fmaxf(a[rt][0], a[rt][1]), fmaxf(a[rt][2], a[rt][3])), fmaxf(fmaxf(a[rt][4], a[rt][5]), fmaxf(a[rt][6], a[rt][7])));
@@ -272,7 +326,7 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
         }
         if (__any(grow)) {
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) {
+            for (int rt = 0; rt < RT; ++rt) {
                 const float mx = rows_max(amax[rt]);
                 const bool fresh = thr[rt] < 0.0f;
                 const bool nokey = mx == -INFINITY;
@@ -289,7 +343,7 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
         }
         scores(sn, kl_next);
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
+        for (int rt = 0; rt < RT; ++rt) {
             float sum = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -300,7 +354,8 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
             l_r[rt] += sum;
         }
         // the step's results are complete here, in program order: nothing of it drifts past the next barrier or branch
-        asm volatile("" : "+v"(pb[0]), "+v"(pb[1]), "+v"(l_r[0]), "+v"(l_r[1]));
+        if constexpr (RT == 2) asm volatile("" : "+v"(pb[0]), "+v"(pb[1]), "+v"(l_r[0]), "+v"(l_r[1]));
+        else asm volatile("" : "+v"(pb[0]), "+v"(l_r[0]));
         __builtin_amdgcn_s_setprio(0);
     };
 
@@ -312,18 +367,18 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
     // A wave runs steps sb - 1 .. se of its own (the one before its first computes nothing it keeps except the scores of
     // the first; the one after its last adds the last step's product); all waves take part in the staging of every tile.
     if (nt > 0) {
-        u4v stk[4], stv[4];
-        f4v sA[2][2], sB[2][2];
+        Stage stk, stv;
+        f4v sA[RT][2], sB[RT][2];
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt)
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int kt2 = 0; kt2 < 2; ++kt2) sA[rt][kt2] = sB[rt][kt2] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
         fetch(stk, kbase, 0);
         fetch(stv, vbase, 0);
         {   // the V buffer step 0 "adds" with zero weights must hold numbers
             const u4v z = {0u, 0u, 0u, 0u};
-#pragma unroll
-            for (int i = 0; i < 4; ++i) *reinterpret_cast<__attribute__((address_space(3))) u4v*>(L + V0 + VBUF + v_wr + i * 16 * VS) = z;
+            for (uint32_t at = (uint32_t) tid * 16; at < (uint32_t) VBUF; at += PW * 64 * 16)
+                *reinterpret_cast<__attribute__((address_space(3))) u4v*>(L + V0 + VBUF + at) = z;
         }
         stash_k(stk, 0);
         stash_v(stv, 0);
@@ -360,9 +415,9 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
     {
         const int esz = p.qt == 0 ? 4 : 2;
         const uint32_t rowb = (uint32_t) (D * esz), rowp = rowb + 16;    // bytes a row, padded in LDS
-        const uint32_t ob = (uint32_t) w * 32 * (D * 4 + 16);
+        const uint32_t ob = (uint32_t) w * WROWS * (D * 4 + 16);
 #pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
+        for (int rt = 0; rt < RT; ++rt) {
             const float lsum = rows_sum(l_r[rt]);
             const float inv = lsum > 0.0f ? 1.0f / lsum : 0.0f;
             const uint32_t at = ob + (uint32_t) (rt * 16 + n) * rowp + (uint32_t) (g4 * 4 * esz);
@@ -383,14 +438,25 @@ __global__ __launch_bounds__(PW * 64, 2) void attn_prefill_kernel(const PrefillP
         // the wave reads back its own block only: no barrier, the LDS queue keeps a wave's accesses in order
         const int ppr = (int) rowb / 16;                          // 16-byte pieces a row
         uint8_t* const orow = reinterpret_cast<uint8_t*>(p.out) + (int64_t) hq * rowb;
-        for (int c = lane; c < 32 * ppr; c += 64) {
-            const int rl_ = c / ppr, piece = c % ppr, row = r0 + w * 32 + rl_;
+        for (int c = lane; c < WROWS * ppr; c += 64) {
+            const int rl_ = c / ppr, piece = c % ppr, row = r0 + w * WROWS + rl_;
             if (row < p.T) {
                 const u4v x = *reinterpret_cast<const __attribute__((address_space(3))) u4v*>(L + ob + (uint32_t) rl_ * rowp + (uint32_t) piece * 16);
                 *reinterpret_cast<u4v*>(orow + (int64_t) row * p.Hq * rowb + piece * 16) = x;
             }
         }
     }
+}
+
+template <int D>
+int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
+    switch (kt) {
+        case 0: attn_prefill_kernel<D, false, 0><<<grid, PW * 64, 0, g->q>>>(p); break;
+        case 3: attn_prefill_kernel<D, true, 0><<<grid, PW * 64, 0, g->q>>>(p); break;
+        case 1: attn_prefill_kernel<D, false, 1><<<grid, PW * 64, 0, g->q>>>(p); break;
+        default: attn_prefill_kernel<D, false, 2><<<grid, PW * 64, 0, g->q>>>(p); break;
+    }
+    return 0;
 }
 
 }  // namespace
@@ -400,19 +466,24 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     NS_TRY
     const std::string w(who);
     if (T <= 0) return 0;
-    if (D != 128) return ns_fail(w + ": heads of 128");
+    if (D != 128 && D != 256) return ns_fail(w + ": heads of 128 or 256");
     if (Hkv <= 0 || Hq <= 0 || Hq % Hkv) return ns_fail(w + ": query heads a multiple of the key heads");
-    if (kt != 0 && kt != 3) return ns_fail(w + ": a cache form 0 (half) or 3 (bfloat16)");
+    if (kt < 0 || kt > 3) return ns_fail(w + ": a cache form 0 (half), 1 (q8_0), 2 (q4_0) or 3 (bfloat16)");
     if (qt < 0 || qt > 2) return ns_fail(w + ": rows of type 0 (float32), 1 (half) or 2 (bfloat16)");
     if (p0 < 0 || cap <= 0) return ns_fail(w + ": a position and a capacity");
     const int64_t need = pm ? p0 + T : (win > 0 ? std::min(p0 + T, win + T - 1) : p0 + T);
     if (need > cap) return ns_fail(w + (win > 0 ? ": the cache's ring is shorter than the window and the pass" : ": past the cache's capacity"));
     if (!q || !kc || !vc || !out) return ns_fail(w + ": a null buffer");
     if ((uintptr_t) q % 16 || qs % (qt == 0 ? 4 : 8) || (uintptr_t) out % 16) return ns_fail(w + ": query and output rows 16-byte aligned");
+    const int64_t rb = kv_row_bytes(kt, D);
+    // rows are fetched in 16-byte chunks, so a row's size must keep that alignment: every 16-bit row does, q8_0 / q4_0
+    // rows do at D = 256 (272 / 144 bytes; the reference's quantized prompt form is D = 256 only), not at D = 128 (136 / 72)
     if (((uintptr_t) kc | (uintptr_t) vc) % 16) return ns_fail(w + ": caches 16-byte aligned");
+    if (rb % 16) return ns_fail(w + ": quantized cache rows with heads of 256 (shorter passes and other heads take the decode kernel)");
+    const int64_t ROWS = rows_of((int) D);
     if (T > (int64_t) 1 << 30 || ((T + ROWS - 1) / ROWS + 1) * Hq > (int64_t) 1 << 30) return ns_fail(w + ": too many rows or heads");
+    if ((pm ? cap * Hkv : cap) * rb >= (int64_t) 1 << 32) return ns_fail(w + ": a key head's cache spans 4 GiB or more");
     NS_HIP(hipSetDevice(g->dev));
-    const int64_t rb = 2 * D;
     PrefillParams p{};
     p.q = q;
     p.qt = qt;
@@ -433,8 +504,8 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     const int64_t units = ((T + ROWS - 1) / ROWS) * Hkv;               // (row block, key head); padded to the 8 XCDs
     dim3 grid((unsigned) ((units + 7) / 8 * 8 * (Hq / Hkv)));
     if (ns_profile_mark(g, 0)) return -1;
-    if (kt == 3) attn_prefill_kernel<128, true><<<grid, PW * 64, 0, g->q>>>(p);
-    else attn_prefill_kernel<128, false><<<grid, PW * 64, 0, g->q>>>(p);
+    if (D == 128) launch_prefill<128>(g, kt, p, grid);
+    else launch_prefill<256>(g, kt, p, grid);
     NS_LAUNCHED("attn_prefill");
     return ns_profile_mark(g, 1);
     NS_CATCH

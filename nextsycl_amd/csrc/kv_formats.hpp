@@ -32,3 +32,21 @@ __device__ __forceinline__ float kv_value_f32(const uint8_t* row, int kt, int D,
     const uint8_t w = row[b * 16 + (j & 15)];
     return (float) ((int) (j < 16 ? w & 15 : w >> 4) - 8) * f16_to_f32(*reinterpret_cast<const uint16_t*>(row + D / 2 + 2 * b));
 }
+
+// 4 int8 in a word -> 4 halfs x scale; each product is exact in float32, so one rounding to half (what the reference
+// stages: half((float) q * (float) d))
+__device__ __forceinline__ void dq8x4(uint32_t w, _Float16 d, short* o) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const _Float16 h = (_Float16) (short) (int8_t) (w >> (8 * b)) * d;
+        o[b] = __builtin_bit_cast(short, h);
+    }
+}
+// 4 nibbles (bits sh .. sh + 3 of each byte) -> 4 halfs: (nibble - 8) x scale
+__device__ __forceinline__ void dq4x4(uint32_t w, int sh, _Float16 d, short* o) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+        const _Float16 h = (_Float16) (short) ((int) ((w >> (8 * b + sh)) & 15u) - 8) * d;
+        o[b] = __builtin_bit_cast(short, h);
+    }
+}

@@ -94,6 +94,45 @@ def test_reference_named_prompt_entry_points(ops):
     ob.fill(0)
     ops.q35_attn(qb, Hq * D, bufs[0], bufs[1], T, Hq, Hkv, D, cap, p0, ob, None)
     assert np.array_equal(ob.read(np.float32).reshape(T, -1), want)
+    # quantized rows at heads of 128 are not 16-byte rows: rejected with the reason (the reference's form is D = 256)
     assert k.q35_attn_prompt_kv(g.raw, 1, qb.ptr, Hq * D, bufs[0].ptr, bufs[1].ptr, T, Hq, Hkv, D, cap, p0, ob.ptr) == -1
-    assert k.attn_prompt_t(g.raw, 0, 0, 0, qb.ptr, Hq * D, bufs[0].ptr, bufs[1].ptr, T, Hq, Hkv, 256, cap, p0, 0, 0.0, ob.ptr) == -1
-    assert "heads of 128" in k.api.error()
+    assert "heads of 256" in k.api.error()
+    assert k.attn_prompt_t(g.raw, 0, 0, 0, qb.ptr, Hq * D, bufs[0].ptr, bufs[1].ptr, T, Hq, Hkv, 64, cap, p0, 0, 0.0, ob.ptr) == -1
+    assert "heads of 128 or 256" in k.api.error()
+
+
+WIDE = [
+    # T, Hq, Hkv, p0, win, kt, qt        heads of 256 (Qwen3.5's), every cache form of the reference's prompt kernel
+    (17, 6, 1, 0, 0, 0, F32),
+    (200, 12, 2, 333, 0, 0, F32),        # G 6, a later chunk
+    (130, 4, 2, 0, 0, 3, BF16),
+    (190, 12, 2, 100, 0, 1, F32),        # q8_0 rows (272 bytes)
+    (150, 6, 1, 60, 0, 2, F16),          # q4_0 rows (144 bytes)
+    (100, 4, 1, 700, 128, 1, F32),       # q8_0 under a window
+]
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,p0,win,kt,qt", WIDE)
+def test_prefill_heads_of_256_and_quantized_rows(ops, T, Hq, Hkv, p0, win, kt, qt):
+    D = 256
+    cap = p0 + T + 3
+    kc, vc = make_kv(kt, Hkv, D, cap, p0 + T)
+    qd, qf = make_q(qt, T, Hq, D)
+    got, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got, ref, qt, "prefill, heads of 256", kt=kt)
+
+
+def test_q35_prompt_kv_entry_point(ops):
+    """ns_q35_attn_prompt_kv as the engine calls it (llm/qwen35/src/engine.rs:1598-1617): float32 rows, D = 256, Hq = 6 Hkv."""
+    T, Hq, Hkv, D, p0 = 90, 12, 2, 256, 40
+    cap = p0 + T
+    g = ops.gpu
+    qd, qf = make_q(F32, T, Hq, D)
+    for kt in (0, 1, 2):
+        kc, vc = make_kv(kt, Hkv, D, cap, cap)
+        ob = DevBuf(g, T * Hq * D * 4); ob.fill(0xFF)
+        qb, kb, vb = DevBuf.of(g, qd), DevBuf.of(g, kc), DevBuf.of(g, vc)        # held: a buffer is freed with its object
+        rc = ops.k.q35_attn_prompt_kv(g.raw, kt, qb.ptr, Hq * D, kb.ptr, vb.ptr, T, Hq, Hkv, D, cap, p0, ob.ptr)
+        assert rc == 0, ops.k.api.error()
+        check_close(ob.read(np.float32).reshape(T, -1), orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0), F32, "ns_q35_attn_prompt_kv kt %d" % kt)
