@@ -55,7 +55,7 @@ def test_pure_functions_without_a_gpu(handle):
     assert s(1, 12, 2, 256) == 1 and s(8, 32, 8, 128) == 1 and s(17, 32, 8, 128) == 0 and s(1, 12, 5, 128) == 0 and s(1, 12, 2, 96) == 0
     p = handle.ns_mg_attn_prompt_supported
     p.restype, p.argtypes = C.c_int, [C.c_int64] * 4
-    assert p(17, 64, 4, 128) == 1 and p(16, 64, 4, 128) == 0 and p(100, 64, 4, 256) == 0
+    assert p(17, 64, 4, 128) == 1 and p(16, 64, 4, 128) == 0 and p(100, 64, 4, 256) == 1 and p(100, 64, 4, 64) == 0
     m = handle.ns_mla_decode_latent_scratch
     m.restype, m.argtypes = C.c_int64, [C.c_int64] * 3
     assert m(1, 128, 32767) == 128 * 256 * 516 and m(0, 128, 5) == 0     # 256 splits of 128 cells, 512 + 4 floats a partial
