@@ -36,7 +36,9 @@
 namespace {
 
 constexpr int MW = 8, MTILE = 32, MROWS = 128, ML = 512;
-constexpr int PSTRIDE = ML + 4;   // floats a partial: O[512], m, l, 2 of padding (rows stay 16-byte aligned)
+// a split's partial of a row: u_s[512] = O_s / l_s as halfs (the split's own normalized result: bounded by the cache's
+// values, so half holds it; a quarter of the float32 form's bytes go to m and l), then m (log2 units), l, 2 of padding
+constexpr int PSTRIDE = ML / 2 + 4;   // in floats: 1040 bytes, rows stay 16-byte aligned
 
 struct MlaParams {
     const void* qa;      // [T][H][L + R] absorbed queries
@@ -47,7 +49,7 @@ struct MlaParams {
     int64_t kbs;         // cells a split
     int ns;
     float sl2;
-    float* part;         // [T * H][ns][PSTRIDE]
+    float* part;         // [T * H][ns][PSTRIDE]: {half u_s[512], float m, l, -, -}
     // a row's own cells (GLM's selection): sel_cnt[t] >= 0 -> the pools sel[t K ..][0, sel_cnt[t]) of 4 cells each, then
     // the row's incomplete pool 4 ((p + 1) / 4) .. p; negative or no sel_cnt -> every earlier cell. With sel_cnt a row
     // group holds one row t's heads only (per_t), and the kernel's cell numbering runs over the row's list
@@ -367,22 +369,47 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
         step(B2, B0, B1, it + 2);
     }
 
-    // ---- the split's partial, straight from the registers: a lane holds latents 16 dt + 4 g4 .. + 3 of its row
+    // ---- the split's partial {u_s = O / l as halfs, m, l}. A lane holds latents 16 dt + 4 g4 .. + 3 of its row: the
+    // wave's 16 x 512 block goes through LDS (the tile buffers, free now: the loop ended on a barrier with every transfer
+    // landed), half of the latents at a time, so that it leaves as 512-byte runs of a row
     const float l_row = rows_sum(l_r);
     const float m_r = thr < 0.0f ? -INFINITY : -nbr;
-    if (live) {
-        float* pr = p.part + ((int64_t) ri * p.ns + split) * PSTRIDE;
+    const float inv_l = l_row > 0.0f ? 1.0f / l_row : 0.0f;
+    {
+        constexpr int OROW = 256 * 2 + 16;                        // bytes a staged row of 256 halfs, padded
+        lds_u8* const ob = (w < 4 ? B0 : B1) + (w & 3) * 16 * OROW;   // 4 waves x 8,448 bytes in each of the first two buffers
+        static_assert(4 * 16 * OROW <= TILEB, "the staging fits a tile buffer");
+        typedef _Float16 h4v __attribute__((ext_vector_type(4)));
+        float* const prow = p.part + (int64_t) split * PSTRIDE;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f4v*>(pr + dt * 16 + g4 * 4) = o[dt];
-        if (g4 == 0) {
-            pr[ML] = m_r;
-            pr[ML + 1] = l_row;
+        for (int hp = 0; hp < 2; ++hp) {
+#pragma unroll
+            for (int d2 = 0; d2 < DT / 2; ++d2) {
+                const f4v v = o[hp * (DT / 2) + d2] * inv_l;
+                const h4v h = {(_Float16) v[0], (_Float16) v[1], (_Float16) v[2], (_Float16) v[3]};
+                *reinterpret_cast<__attribute__((address_space(3))) h4v*>(ob + n * OROW + (d2 * 16 + g4 * 4) * 2) = h;
+            }
+            // the wave reads back its own rows only: no barrier (the LDS queue keeps a wave's accesses in order)
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const int id = c * 64 + lane, r = id >> 5, piece = id & 31;      // 32 pieces of 16 bytes a row's half
+                const int rg = (p.per_t ? z % zpt : z) * MROWS + w * 16 + r;
+                const bool ok = p.per_t ? rg < p.H : rg < rows;
+                const int64_t rrow = p.per_t ? (int64_t) tz * p.H + rg : rg;
+                const u4v x = *reinterpret_cast<const __attribute__((address_space(3))) u4v*>(ob + r * OROW + piece * 16);
+                if (ok) *reinterpret_cast<u4v*>(reinterpret_cast<uint8_t*>(prow + rrow * p.ns * PSTRIDE) + hp * 512 + piece * 16) = x;
+            }
+        }
+        if (live && g4 == 0) {
+            float* pr = prow + (int64_t) ri * p.ns * PSTRIDE;
+            pr[ML / 2] = m_r;
+            pr[ML / 2 + 1] = l_row;
         }
     }
 }
 
-// the splits of a row merged: u = sum O_s 2^(m_s - M) / sum l_s 2^(m_s - M). Two work-groups of 256 threads a row, 256
-// latents each: a thread sums 4 latents (one 16-byte load a split) over every fourth split, then the four phases are
+// the splits of a row merged: u = sum_s u_s w_s / sum_s w_s, w_s = l_s 2^(m_s - M). Two work-groups of 256 threads a row,
+// 256 latents each: a thread sums 4 latents (one 8-byte load a split) over every fourth split, then the four phases are
 // added in a fixed order.
 template <int QT>
 __global__ __launch_bounds__(256) void mla_merge_kernel(const float* __restrict__ part, int ns, void* __restrict__ u) {
@@ -393,7 +420,7 @@ __global__ __launch_bounds__(256) void mla_merge_kernel(const float* __restrict_
     const int tid = threadIdx.x;
     const float* pr = part + row * ns * PSTRIDE;
     float mx = -INFINITY;
-    for (int s = tid; s < ns; s += 256) mx = fmaxf(mx, pr[s * PSTRIDE + ML]);
+    for (int s = tid; s < ns; s += 256) mx = fmaxf(mx, pr[s * PSTRIDE + ML / 2]);
     red[tid] = mx;
     __syncthreads();
     for (int o = 128; o > 0; o >>= 1) {
@@ -404,10 +431,10 @@ __global__ __launch_bounds__(256) void mla_merge_kernel(const float* __restrict_
     __syncthreads();
     float ls = 0.0f;
     for (int s = tid; s < ns; s += 256) {
-        const float m = pr[s * PSTRIDE + ML];
-        const float wgt = m == -INFINITY ? 0.0f : fast_exp2(m - mx);
+        const float m = pr[s * PSTRIDE + ML / 2];
+        const float wgt = m == -INFINITY ? 0.0f : pr[s * PSTRIDE + ML / 2 + 1] * fast_exp2(m - mx);
         wsh[s] = wgt;
-        ls += pr[s * PSTRIDE + ML + 1] * wgt;
+        ls += wgt;
     }
     red[tid] = ls;
     __syncthreads();
@@ -418,9 +445,13 @@ __global__ __launch_bounds__(256) void mla_merge_kernel(const float* __restrict_
     const float L = red[0];
     const int quad = tid & 63, phase = tid >> 6;
     const int lat = blockIdx.y * 256 + quad * 4;
+    typedef _Float16 h4v __attribute__((ext_vector_type(4)));
     f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll 8
-    for (int s = phase; s < ns; s += 4) acc += *reinterpret_cast<const f4v*>(pr + s * PSTRIDE + lat) * wsh[s];
+    for (int s = phase; s < ns; s += 4) {
+        const h4v h = *reinterpret_cast<const h4v*>(reinterpret_cast<const _Float16*>(pr + s * PSTRIDE) + lat);
+        acc += f4v{(float) h[0], (float) h[1], (float) h[2], (float) h[3]} * wsh[s];
+    }
     ph[tid] = acc;
     __syncthreads();
     if (phase == 0) {
