@@ -92,12 +92,12 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     constexpr int RS = DMA ? D * 2 : D * 2 + 32;
     constexpr int VTILE = TILE * RS;
     constexpr int STAGE = DMA ? 2 * VTILE : VTILE;
-    constexpr int OROW = D + 4;                                    // floats a row of the merge buffer
+    constexpr int OROW = D + 4;                                    // floats a row of a wave's merge buffer
     constexpr int MERGE = RT * 16 * OROW * 4;
-    constexpr int LDS_MAIN = WAVES * STAGE > MERGE ? WAVES * STAGE : MERGE;
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_MAIN];
+    // a wave's own region: its value stage while it streams, its (O, m, l) for the merge afterwards
+    constexpr int WREG = ((STAGE > MERGE ? STAGE : MERGE) + 1023) / 1024 * 1024;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[WAVES * WREG];
     __shared__ float ml[WAVES][RT * 16][2];
-    __shared__ float ML[RT * 16][2];
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // the wave's index, known uniform to the compiler
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
 
     const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
     const uint8_t* vbase = p.vc + (int64_t) hk * p.head_stride;
-    uint8_t* stage = lds + w * STAGE;
+    uint8_t* stage = lds + w * WREG;
     const int32_t* selp = p.sel ? p.sel + (int64_t) hk * p.selK : nullptr;
 
     // a key's row offset: keys outside [jb, je) are clamped into it (their scores are masked, their values meet P = 0).
@@ -399,55 +399,42 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         }
     }
 
-    // ---- the 4 waves' partials merged in wave order, then written as the split's partial
-    if (g4 == 0)
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-            ml[w][rt * 16 + n][0] = m_r[rt];
-            ml[w][rt * 16 + n][1] = l_r[rt];
-        }
-    __syncthreads();
+    // ---- the 4 waves' (O, m, l) merged in wave order and written as the split's partial. Each wave parks its live rows
+    // in its own region (free: every read of its stage has returned), one barrier, then a thread a (row, 4 features)
+    const int live_rows = std::min(RT * 16, rows - z * RT * 16);
+    float* ow = reinterpret_cast<float*>(stage);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        const int row = rt * 16 + n;
+        if (rt * 16 + n < live_rows) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<f4v*>(ow + (rt * 16 + n) * OROW + dt * 16 + g4 * 4) = o[rt][dt];
+            if (g4 == 0) {
+                ml[w][rt * 16 + n][0] = m_r[rt];
+                ml[w][rt * 16 + n][1] = l_r[rt];
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < live_rows * (D / 4); idx += WAVES * 64) {
+        const int row = idx / (D / 4), c = idx % (D / 4), ri = z * RT * 16 + row;
+        const int t = ri / p.G, gq = ri % p.G;
         float M = -INFINITY;
 #pragma unroll
         for (int k = 0; k < WAVES; ++k) M = fmaxf(M, ml[k][row][0]);
         float L = 0.0f;
+        f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int k = 0; k < WAVES; ++k) L += ml[k][row][0] == -INFINITY ? 0.0f : ml[k][row][1] * fast_exp2(ml[k][row][0] - M);
-        const float f = m_r[rt] == -INFINITY ? 0.0f : fast_exp2(m_r[rt] - M);
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= f;
-        if (w == 0 && g4 == 0) {
-            ML[row][0] = M;
-            ML[row][1] = L;
+        for (int k = 0; k < WAVES; ++k) {
+            const float f = ml[k][row][0] == -INFINITY ? 0.0f : fast_exp2(ml[k][row][0] - M);
+            L += ml[k][row][1] * f;
+            const f4v ok = *reinterpret_cast<const f4v*>(reinterpret_cast<const float*>(lds + k * WREG) + row * OROW + c * 4);
+            acc = k == 0 ? ok * f : acc + ok * f;
         }
-    }
-    float* obuf = reinterpret_cast<float*>(lds);
-    for (int k = 0; k < WAVES; ++k) {
-        if (w == k) {
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    f4v* dst = reinterpret_cast<f4v*>(obuf + (rt * 16 + n) * OROW + dt * 16 + g4 * 4);
-                    if (k == 0) *dst = o[rt][dt];
-                    else *dst = *dst + o[rt][dt];
-                }
-        }
-        __syncthreads();
-    }
-    const int live_rows = std::min(RT * 16, rows - z * RT * 16);
-    for (int idx = tid; idx < live_rows * D; idx += WAVES * 64) {
-        const int row = idx / D, d = idx % D, ri = z * RT * 16 + row;
-        const int t = ri / p.G, gq = ri % p.G;
+        // partial rows are D + 2 floats: 8-byte aligned
         float* pr = p.part + (((int64_t) t * p.Hq + hk * p.G + gq) * p.ns + split) * (D + 2);
-        pr[d] = obuf[row * OROW + d];
-        if (d == 0) {
-            pr[D] = ML[row][0];
-            pr[D + 1] = ML[row][1];
-        }
+        *reinterpret_cast<float2*>(pr + c * 4) = float2{acc[0], acc[1]};
+        *reinterpret_cast<float2*>(pr + c * 4 + 2) = float2{acc[2], acc[3]};
+        if (c == 0) *reinterpret_cast<float2*>(pr + D) = float2{M, L};
     }
 }
 
@@ -615,6 +602,7 @@ int decode_checked(ns_gpu* g, const char* who, int qt, int kt, int pm, const voi
     const int64_t need = pm ? p0 + T : (win > 0 ? std::min(p0 + T, win + T - 1) : p0 + T);
     if (need > cap) return ns_fail(w + (win > 0 ? ": the cache's ring is shorter than the window and the pass" : ": past the cache's capacity"));
     if (!scratch) return ns_fail(w + ": no scratch");
+    if ((uintptr_t) scratch % 8) return ns_fail(w + ": scratch 8-byte aligned");
     if (!q || !kc || !vc || !out) return ns_fail(w + ": a null buffer");
     if ((uintptr_t) q % 16 || qs % (qt == 0 ? 4 : 8)) return ns_fail(w + ": query rows 16-byte aligned");
     if (((uintptr_t) kc | (uintptr_t) vc) % 16 && (kt == 0 || kt == 3)) return ns_fail(w + ": caches 16-byte aligned");
