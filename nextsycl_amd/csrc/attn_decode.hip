@@ -82,6 +82,80 @@ struct TileRegs {
     uint16_t vsc[DMA ? 1 : NLV];
 };
 
+// The splits of a (row, head) merged by one wave: out = sum_s O_s w_s / sum_s l_s w_s, w_s = 2^(m_s - M). A lane owns
+// D / 64 features in 8-byte pieces and adds the splits in ascending order (fused multiply-adds), so the result does not
+// depend on how many empty splits a pass appends to a row's own (their weight is 0). The first splits' values are
+// requested before the weights exist; wsh: ns rounded up to 16 (at least 32) floats of the wave's own LDS.
+constexpr int MERGE_MAX_NS = 2048;
+
+template <int D>
+__device__ __forceinline__ void merge_row_wave(const float* __restrict__ pr, int ns, int qt, void* __restrict__ out, int64_t oidx, int lane,
+                                               float* wsh) {
+    constexpr int C = D / 128, PS = D + 2, PF = 32, B = 16;
+    float2 x[PF][C];
+#pragma unroll
+    for (int i = 0; i < PF; ++i)
+#pragma unroll
+        for (int c = 0; c < C; ++c) x[i][c] = *reinterpret_cast<const float2*>(pr + (int64_t) std::min(i, ns - 1) * PS + 2 * (lane + 64 * c));
+    float mx = -INFINITY;
+    for (int s = lane; s < ns; s += 64) mx = fmaxf(mx, pr[(int64_t) s * PS + D]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    float ls = 0.0f;
+    const int nsp = (ns + B - 1) / B * B, nsf = nsp < PF ? PF : nsp;
+    for (int s = lane; s < nsf; s += 64) {
+        float wgt = 0.0f;
+        if (s < ns) {
+            const float2 mlv = *reinterpret_cast<const float2*>(pr + (int64_t) s * PS + D);
+            wgt = mlv.x == -INFINITY ? 0.0f : fast_exp2(mlv.x - mx);
+            ls = fmaf(mlv.y, wgt, ls);
+        }
+        wsh[s] = wgt;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ls += __shfl_xor(ls, o);
+    // the wave's own lanes wrote wsh: LDS operations of a wave complete in order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    float2 acc[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) acc[c] = float2{0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+        const float wgt = wsh[i];
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            acc[c].x = fmaf(x[i][c].x, wgt, acc[c].x);
+            acc[c].y = fmaf(x[i][c].y, wgt, acc[c].y);
+        }
+    }
+    for (int s0 = PF; s0 < nsp; s0 += B) {
+        float2 y[B][C];
+#pragma unroll
+        for (int i = 0; i < B; ++i)
+#pragma unroll
+            for (int c = 0; c < C; ++c) y[i][c] = *reinterpret_cast<const float2*>(pr + (int64_t) std::min(s0 + i, ns - 1) * PS + 2 * (lane + 64 * c));
+#pragma unroll
+        for (int i = 0; i < B; ++i) {
+            const float wgt = wsh[s0 + i];
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                acc[c].x = fmaf(y[i][c].x, wgt, acc[c].x);
+                acc[c].y = fmaf(y[i][c].y, wgt, acc[c].y);
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const int64_t i = oidx + 2 * (lane + 64 * c);
+        const float a = ls > 0.0f ? acc[c].x / ls : 0.0f, b = ls > 0.0f ? acc[c].y / ls : 0.0f;
+        if (qt == 0) *reinterpret_cast<float2*>(reinterpret_cast<float*>(out) + i) = float2{a, b};
+        else if (qt == 1) *reinterpret_cast<uint32_t*>(reinterpret_cast<uint16_t*>(out) + i) = (uint32_t) (uint16_t) to16<false>(a) | (uint32_t) (uint16_t) to16<false>(b) << 16;
+        else *reinterpret_cast<uint32_t*>(reinterpret_cast<uint16_t*>(out) + i) = (uint32_t) (uint16_t) to16<true>(a) | (uint32_t) (uint16_t) to16<true>(b) << 16;
+    }
+}
+
 template <int D, int RT, int KT>
 __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kernel(const DecodeParams p) {
     constexpr bool BF = KT == 3;
@@ -438,56 +512,12 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     }
 }
 
-// The splits of a (row, head) merged: out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M). A work-group of 512 threads per
-// (row, head): the splits' maxima and weights first (a thread a split), then 512 / D groups of D threads each take every
-// (512 / D)-th split's values, and the groups' sums are added pairwise. Every sum runs over a fixed shape (slots past the
-// last split hold zeros), so the result does not depend on how many empty splits a pass appends to a row's own.
-constexpr int MERGE_T = 512, MERGE_MAX_NS = 2048;
-
-__device__ __forceinline__ float block_reduce(float v, float* red, int tid, bool is_max) {
-    red[tid] = v;
-    __syncthreads();
-#pragma unroll
-    for (int o = MERGE_T / 2; o > 0; o >>= 1) {
-        if (tid < o) red[tid] = is_max ? fmaxf(red[tid], red[tid + o]) : red[tid] + red[tid + o];
-        __syncthreads();
-    }
-    const float r = red[0];
-    __syncthreads();
-    return r;
-}
-
-template <int D, int QT>
-__global__ __launch_bounds__(MERGE_T) void attn_merge_kernel(const float* __restrict__ part, int ns, void* __restrict__ out) {
-    constexpr int GROUPS = MERGE_T / D;
+// The merge launch: a wave a (row, head), a work-group each so that the rows' loads spread over the device.
+template <int D>
+__global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ part, int ns, int qt, void* __restrict__ out) {
     __shared__ float wsh[MERGE_MAX_NS];
-    __shared__ float red[MERGE_T];
     const int64_t rh = blockIdx.x;
-    const int tid = threadIdx.x;
-    const float* pr = part + rh * ns * (D + 2);
-    float mx = -INFINITY;
-    for (int s = tid; s < ns; s += MERGE_T) mx = fmaxf(mx, pr[s * (D + 2) + D]);
-    mx = block_reduce(mx, red, tid, true);
-    float ls = 0.0f;
-    for (int s = tid; s < ns; s += MERGE_T) {
-        const float m = pr[s * (D + 2) + D];
-        const float wgt = m == -INFINITY ? 0.0f : fast_exp2(m - mx);
-        wsh[s] = wgt;
-        ls += pr[s * (D + 2) + D + 1] * wgt;
-    }
-    const float L = block_reduce(ls, red, tid, false);   // its barriers also publish wsh
-    const int grp = tid / D, d = tid % D;
-    float acc = 0.0f;
-#pragma unroll 8
-    for (int s = grp; s < ns; s += GROUPS) acc += pr[s * (D + 2) + d] * wsh[s];
-    red[tid] = acc;
-    __syncthreads();
-    if (grp == 0) {
-        float A;
-        if constexpr (GROUPS == 4) A = (red[d] + red[D + d]) + (red[2 * D + d] + red[3 * D + d]);
-        else A = red[d] + red[D + d];
-        store_o<QT>(out, rh * D + d, L > 0.0f ? A / L : 0.0f);
-    }
+    merge_row_wave<D>(part + rh * ns * (D + 2), ns, qt, out, rh * D, threadIdx.x, wsh);
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------------
@@ -530,10 +560,10 @@ int launch_kt(ns_gpu* g, int kt, const DecodeParams& p, int rows, dim3 grid_xy) 
     }
 }
 
-template <int D, int QT>
-int launch_merge(ns_gpu* g, const float* part, int ns, int64_t rh, void* out) {
+template <int D>
+int launch_merge(ns_gpu* g, const float* part, int ns, int qt, int64_t rh, void* out) {
     if (ns > MERGE_MAX_NS) return ns_fail("ns_attn_decode: more key splits than the merge holds");
-    attn_merge_kernel<D, QT><<<(unsigned) rh, MERGE_T, 0, g->q>>>(part, ns, out);
+    attn_merge_kernel<D><<<(unsigned) rh, 64, 0, g->q>>>(part, ns, qt, out);
     NS_LAUNCHED("attn_merge");
     return 0;
 }
@@ -579,7 +609,7 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
         if (ns_profile_mark(g, 0)) return -1;
         if (launch_kt<D>(g, kt, c, (int) (nr * c.G), dim3((unsigned) ns, (unsigned) Hkv))) return -1;
         if (ns_profile_mark(g, 1)) return -1;
-        if (launch_merge<D, QT>(g, c.part, (int) ns, nr * Hq, (uint8_t*) out + r0 * Hq * D * esz)) return -1;
+        if (launch_merge<D>(g, c.part, (int) ns, QT, nr * Hq, (uint8_t*) out + r0 * Hq * D * esz)) return -1;
         return ns_profile_mark(g, 2);
     };
     if (same) return launch(0, T, kb_of(0));
@@ -667,7 +697,7 @@ int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_
         p.sel = sel + t * Hkv * K;
         p.sel_pos = pos0 + t;
         if (launch_kt<D>(g, 0, p, p.G, dim3((unsigned) ns, (unsigned) Hkv))) return -1;
-        if (launch_merge<D, 0>(g, scratch, (int) ns, Hq, out + t * Hq * D)) return -1;
+        if (launch_merge<D>(g, scratch, (int) ns, 0, Hq, out + t * Hq * D)) return -1;
     }
     return 0;
     NS_CATCH
