@@ -82,80 +82,6 @@ struct TileRegs {
     uint16_t vsc[DMA ? 1 : NLV];
 };
 
-// The splits of a (row, head) merged by one wave: out = sum_s O_s w_s / sum_s l_s w_s, w_s = 2^(m_s - M). A lane owns
-// D / 64 features in 8-byte pieces and adds the splits in ascending order (fused multiply-adds), so the result does not
-// depend on how many empty splits a pass appends to a row's own (their weight is 0). The first splits' values are
-// requested before the weights exist; wsh: ns rounded up to 16 (at least 32) floats of the wave's own LDS.
-constexpr int MERGE_MAX_NS = 2048;
-
-template <int D>
-__device__ __forceinline__ void merge_row_wave(const float* __restrict__ pr, int ns, int qt, void* __restrict__ out, int64_t oidx, int lane,
-                                               float* wsh) {
-    constexpr int C = D / 128, PS = D + 2, PF = 32, B = 16;
-    float2 x[PF][C];
-#pragma unroll
-    for (int i = 0; i < PF; ++i)
-#pragma unroll
-        for (int c = 0; c < C; ++c) x[i][c] = *reinterpret_cast<const float2*>(pr + (int64_t) std::min(i, ns - 1) * PS + 2 * (lane + 64 * c));
-    float mx = -INFINITY;
-    for (int s = lane; s < ns; s += 64) mx = fmaxf(mx, pr[(int64_t) s * PS + D]);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-    float ls = 0.0f;
-    const int nsp = (ns + B - 1) / B * B, nsf = nsp < PF ? PF : nsp;
-    for (int s = lane; s < nsf; s += 64) {
-        float wgt = 0.0f;
-        if (s < ns) {
-            const float2 mlv = *reinterpret_cast<const float2*>(pr + (int64_t) s * PS + D);
-            wgt = mlv.x == -INFINITY ? 0.0f : fast_exp2(mlv.x - mx);
-            ls = fmaf(mlv.y, wgt, ls);
-        }
-        wsh[s] = wgt;
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) ls += __shfl_xor(ls, o);
-    // the wave's own lanes wrote wsh: LDS operations of a wave complete in order
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    float2 acc[C];
-#pragma unroll
-    for (int c = 0; c < C; ++c) acc[c] = float2{0.0f, 0.0f};
-#pragma unroll
-    for (int i = 0; i < PF; ++i) {
-        const float wgt = wsh[i];
-#pragma unroll
-        for (int c = 0; c < C; ++c) {
-            acc[c].x = fmaf(x[i][c].x, wgt, acc[c].x);
-            acc[c].y = fmaf(x[i][c].y, wgt, acc[c].y);
-        }
-    }
-    for (int s0 = PF; s0 < nsp; s0 += B) {
-        float2 y[B][C];
-#pragma unroll
-        for (int i = 0; i < B; ++i)
-#pragma unroll
-            for (int c = 0; c < C; ++c) y[i][c] = *reinterpret_cast<const float2*>(pr + (int64_t) std::min(s0 + i, ns - 1) * PS + 2 * (lane + 64 * c));
-#pragma unroll
-        for (int i = 0; i < B; ++i) {
-            const float wgt = wsh[s0 + i];
-#pragma unroll
-            for (int c = 0; c < C; ++c) {
-                acc[c].x = fmaf(y[i][c].x, wgt, acc[c].x);
-                acc[c].y = fmaf(y[i][c].y, wgt, acc[c].y);
-            }
-        }
-    }
-#pragma unroll
-    for (int c = 0; c < C; ++c) {
-        const int64_t i = oidx + 2 * (lane + 64 * c);
-        const float a = ls > 0.0f ? acc[c].x / ls : 0.0f, b = ls > 0.0f ? acc[c].y / ls : 0.0f;
-        if (qt == 0) *reinterpret_cast<float2*>(reinterpret_cast<float*>(out) + i) = float2{a, b};
-        else if (qt == 1) *reinterpret_cast<uint32_t*>(reinterpret_cast<uint16_t*>(out) + i) = (uint32_t) (uint16_t) to16<false>(a) | (uint32_t) (uint16_t) to16<false>(b) << 16;
-        else *reinterpret_cast<uint32_t*>(reinterpret_cast<uint16_t*>(out) + i) = (uint32_t) (uint16_t) to16<true>(a) | (uint32_t) (uint16_t) to16<true>(b) << 16;
-    }
-}
-
 template <int D, int RT, int KT>
 __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kernel(const DecodeParams p) {
     constexpr bool BF = KT == 3;
@@ -512,12 +438,93 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     }
 }
 
-// The merge launch: a wave a (row, head), a work-group each so that the rows' loads spread over the device.
+// The splits of a (row, head) merged by a work-group of 4 waves: out = sum_s O_s w_s / sum_s l_s w_s, w_s = 2^(m_s - M).
+// Wave k adds the splits s = k, k + 4, ... in ascending order (fused multiply-adds; a lane owns D / 64 features in 8-byte
+// pieces) and the four sums are added as (0 + 1) + (2 + 3): a fixed shape, so the result does not depend on how many
+// empty splits a pass appends to a row's own (their weight is 0). Every wave works out all the weights itself (no
+// barrier before the sums), and its first 32 splits' values are requested before the weights exist.
+constexpr int MERGE_MAX_NS = 2048, MERGE_W = 4;
+
 template <int D>
-__global__ __launch_bounds__(64) void attn_merge_kernel(const float* __restrict__ part, int ns, int qt, void* __restrict__ out) {
-    __shared__ float wsh[MERGE_MAX_NS];
+__global__ __launch_bounds__(MERGE_W * 64) void attn_merge_kernel(const float* __restrict__ part, int ns, int qt, void* __restrict__ out) {
+    constexpr int C = D / 128, PS = D + 2, PF = 32, B = 16;
+    __shared__ float wsh[MERGE_W][MERGE_MAX_NS + MERGE_W * PF];
+    __shared__ float2 sums[MERGE_W][C][64];
+    const int lane = threadIdx.x & 63, k = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t rh = blockIdx.x;
-    merge_row_wave<D>(part + rh * ns * (D + 2), ns, qt, out, rh * D, threadIdx.x, wsh);
+    const float* pr = part + rh * ns * PS;
+    float2 x[PF][C];
+#pragma unroll
+    for (int j = 0; j < PF; ++j)
+#pragma unroll
+        for (int c = 0; c < C; ++c) x[j][c] = *reinterpret_cast<const float2*>(pr + (int64_t) std::min(k + MERGE_W * j, ns - 1) * PS + 2 * (lane + 64 * c));
+    float mx = -INFINITY;
+    for (int s = lane; s < ns; s += 64) mx = fmaxf(mx, pr[(int64_t) s * PS + D]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    // this wave's splits: nk of them, walked in batches of B after the first PF (slots past the last hold weight 0)
+    const int nk = ns > k ? (ns - k + MERGE_W - 1) / MERGE_W : 0;
+    const int njp = std::max(PF, (nk + B - 1) / B * B), nsz = MERGE_W * njp;
+    float* wk = wsh[k];
+    float ls = 0.0f;
+    for (int s = lane; s < nsz; s += 64) {
+        float wgt = 0.0f;
+        if (s < ns) {
+            const float2 mlv = *reinterpret_cast<const float2*>(pr + (int64_t) s * PS + D);
+            wgt = mlv.x == -INFINITY ? 0.0f : fast_exp2(mlv.x - mx);
+            ls = fmaf(mlv.y, wgt, ls);
+        }
+        wk[s] = wgt;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ls += __shfl_xor(ls, o);
+    // wk was written by this wave's own lanes: a wave's LDS operations complete in order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    float2 acc[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) acc[c] = float2{0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+        const float wgt = wk[k + MERGE_W * j];
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            acc[c].x = fmaf(x[j][c].x, wgt, acc[c].x);
+            acc[c].y = fmaf(x[j][c].y, wgt, acc[c].y);
+        }
+    }
+    for (int j0 = PF; j0 < njp; j0 += B) {
+        float2 y[B][C];
+#pragma unroll
+        for (int j = 0; j < B; ++j)
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+                y[j][c] = *reinterpret_cast<const float2*>(pr + (int64_t) std::min(k + MERGE_W * (j0 + j), ns - 1) * PS + 2 * (lane + 64 * c));
+#pragma unroll
+        for (int j = 0; j < B; ++j) {
+            const float wgt = wk[k + MERGE_W * (j0 + j)];
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                acc[c].x = fmaf(y[j][c].x, wgt, acc[c].x);
+                acc[c].y = fmaf(y[j][c].y, wgt, acc[c].y);
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c) sums[k][c][lane] = acc[c];
+    __syncthreads();
+    if (k != 0) return;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+        const float2 s0 = sums[0][c][lane], s1 = sums[1][c][lane], s2 = sums[2][c][lane], s3 = sums[3][c][lane];
+        const float ax = (s0.x + s1.x) + (s2.x + s3.x), ay = (s0.y + s1.y) + (s2.y + s3.y);
+        const float a = ls > 0.0f ? ax / ls : 0.0f, b = ls > 0.0f ? ay / ls : 0.0f;
+        const int64_t i = rh * D + 2 * (lane + 64 * c);
+        if (qt == 0) *reinterpret_cast<float2*>(reinterpret_cast<float*>(out) + i) = float2{a, b};
+        else if (qt == 1) *reinterpret_cast<uint32_t*>(reinterpret_cast<uint16_t*>(out) + i) = (uint32_t) (uint16_t) to16<false>(a) | (uint32_t) (uint16_t) to16<false>(b) << 16;
+        else *reinterpret_cast<uint32_t*>(reinterpret_cast<uint16_t*>(out) + i) = (uint32_t) (uint16_t) to16<true>(a) | (uint32_t) (uint16_t) to16<true>(b) << 16;
+    }
 }
 
 // ---- host side ----------------------------------------------------------------------------------------------------
@@ -563,7 +570,7 @@ int launch_kt(ns_gpu* g, int kt, const DecodeParams& p, int rows, dim3 grid_xy) 
 template <int D>
 int launch_merge(ns_gpu* g, const float* part, int ns, int qt, int64_t rh, void* out) {
     if (ns > MERGE_MAX_NS) return ns_fail("ns_attn_decode: more key splits than the merge holds");
-    attn_merge_kernel<D><<<(unsigned) rh, 64, 0, g->q>>>(part, ns, qt, out);
+    attn_merge_kernel<D><<<(unsigned) rh, MERGE_W * 64, 0, g->q>>>(part, ns, qt, out);
     NS_LAUNCHED("attn_merge");
     return 0;
 }
