@@ -42,6 +42,9 @@ namespace {
 
 constexpr int WAVES = 4, TILE = 32;
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+// Keys and values are read once a pass: their loads carry the non-temporal hint (the cache-policy bit of the direct
+// global -> LDS load; __builtin_nontemporal_load elsewhere), which measured ~10 % more HBM bandwidth on streaming reads
+constexpr int NT_AUX = 2;
 
 struct DecodeParams {
     const void* q;
@@ -75,7 +78,6 @@ struct TileRegs {
     static constexpr int CPR = KT == 1 ? D / 16 : KT == 2 ? D / 32 : D / 8;   // 16-byte chunks a value row
     static constexpr int KPI = 64 / CPR;                                 // keys a wave covers per V load
     static constexpr int NLV = TILE / KPI;                               // V loads a lane per tile
-    u4v k4[2][DMA ? KB : 1];                                             // 16-bit rows: 8 features per (key tile, k-block)
     uint32_t k[2][DMA ? 1 : KB][KW];                                     // quantized rows: 8 int8 / 8 nibbles
     uint16_t ksc[2][DMA ? 1 : KB];
     uint4 v[DMA ? 1 : NLV];                                              // quantized forms only
@@ -88,7 +90,8 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     using R = TileRegs<D, KT>;
     constexpr bool DMA = R::DMA;
     constexpr int KB = R::KB, DT = D / 16;
-    // a wave's value stage: DMA: two unpadded swizzled tiles [32][2 D bytes]; else one padded tile (rows + 32 bytes)
+    // a wave's stage: DMA: a key tile and a value tile, unpadded and swizzled, [32][2 D bytes] each; else one padded
+    // value tile (rows + 32 bytes)
     constexpr int RS = DMA ? D * 2 : D * 2 + 32;
     constexpr int VTILE = TILE * RS;
     constexpr int STAGE = DMA ? 2 * VTILE : VTILE;
@@ -135,16 +138,30 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         // (keys of a listed block past the row's position are masked: read the row's own key instead - the cache may end there)
         return std::min<int64_t>((int64_t) (blk < 0 ? 0 : blk) * 128 + ((ti * TILE) & 127) + idx, p.sel_pos) * p.row_stride;
     };
-    auto load_tile = [&](R& r, int64_t ti, int buf) {
+    // 16-bit rows: a tile's keys (which = 0) or values (1) on their way global -> LDS, 1 KiB a load: position cp of key kk
+    // holds the row's 16-byte chunk cp ^ (kk % 16) (keys: the operand reads of 16 keys' same chunk meet no bank
+    // conflict) or cp ^ 2 (kk % 8) (values: the transposing reads)
+    auto dma_tile = [&](int64_t ti, int which) {
         const int j0 = (int) (ti * TILE - jb);                 // the tile's first key relative to the split's
+        const int cp = lane % R::CPR, kr0 = lane / R::CPR;
+#pragma unroll
+        for (int i = 0; i < R::NLV; ++i) {
+            const int kk = kr0 + R::KPI * i;
+            const uint8_t* row = (which ? vbase : kbase) + tile_off(ti, j0, kk);
+            const int c = which ? cp ^ (2 * (kk & 7)) : cp ^ (kk & 15);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (row + c * 16),
+                                             (__attribute__((address_space(3))) void*) (stage + which * VTILE + i * 1024), 16, 0, NT_AUX);
+        }
+    };
+    // quantized rows: the tile's keys (MFMA A layout) and values raw into registers
+    auto load_tile = [&](R& r, int64_t ti) {
+        const int j0 = (int) (ti * TILE - jb);
 #pragma unroll
         for (int kt2 = 0; kt2 < 2; ++kt2) {
             const uint8_t* kr = kbase + tile_off(ti, j0, kt2 * 16 + n);
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
-                if constexpr (DMA) {
-                    r.k4[kt2][kb] = *reinterpret_cast<const u4v*>(kr + kb * 64 + g4 * 16);
-                } else if constexpr (KT == 1) {
+                if constexpr (KT == 1) {
                     const uint2 x = *reinterpret_cast<const uint2*>(kr + kb * 32 + g4 * 8);
                     r.k[kt2][kb][0] = x.x; r.k[kt2][kb][1] = x.y;
                     r.ksc[kt2][kb] = *reinterpret_cast<const uint16_t*>(kr + D + 2 * kb);
@@ -158,17 +175,10 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         const int cp = lane % R::CPR, kr0 = lane / R::CPR;
 #pragma unroll
         for (int i = 0; i < R::NLV; ++i) {
-            const int kk = kr0 + R::KPI * i;
-            const uint8_t* vr = vbase + tile_off(ti, j0, kk);
-            if constexpr (DMA) {
-                const int c = cp ^ (2 * (kk & 7));
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (vr + c * 16),
-                                                 (__attribute__((address_space(3))) void*) (stage + buf * VTILE + i * 1024), 16, 0, 0);
-            } else {
-                r.v[i] = *reinterpret_cast<const uint4*>(vr + cp * 16);
-                if constexpr (KT == 1) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D + 2 * (cp / 2));
-                if constexpr (KT == 2) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D / 2 + 2 * cp);
-            }
+            const uint8_t* vr = vbase + tile_off(ti, j0, kr0 + R::KPI * i);
+            r.v[i] = *reinterpret_cast<const uint4*>(vr + cp * 16);
+            if constexpr (KT == 1) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D + 2 * (cp / 2));
+            if constexpr (KT == 2) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D / 2 + 2 * cp);
         }
     };
 
@@ -177,7 +187,18 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     const int64_t tb = jb / TILE, te = jb < je ? (je + TILE - 1) / TILE : tb;
     int64_t ti = tb + ((w - (int) (tb % WAVES) + WAVES) % WAVES);
     R ra, rb;
-    if (ti < te) load_tile(ra, ti, 0);
+    if (ti < te) {
+        if constexpr (DMA) {
+            dma_tile(ti, 0);
+            dma_tile(ti, 1);
+        } else {
+            load_tile(ra, ti);
+        }
+    }
+    // where this lane reads its key operands in the key tile: key n (and 16 + n), chunk 4 kb + g4 at its swizzled position
+    uint32_t k_rd[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) k_rd[kb] = (uint32_t) (uintptr_t) (stage + n * RS + (((kb * 4 + g4) ^ n) * 16));
 
     // ---- this lane's rows (one per row tile): their key ranges and Q^T operands
     int64_t lo_r[RT], hi_r[RT];
@@ -234,10 +255,33 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         for (int dt = 0; dt < DT; ++dt) o[rt][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
     }
 
-    // MORE: how many tiles' loads were issued after this tile's (0 or 1) - what the DMA wait may leave in flight
-    auto process_tile = [&](R& r, int64_t ti, int buf, auto more_c) {
+    // 16-bit rows: loads complete in the order they were issued - ... K(i), V(i), K(i + 1), V(i + 1) ... - so a wait
+    // that leaves one tile's NLV loads outstanding has seen everything older. MORE: the wave has a tile after this one
+    // (at ti + WAVES), whose keys are requested as soon as this tile's have been read out of the key buffer and whose
+    // values as soon as this tile's have been read out of the value buffer.
+    auto process_tile = [&](R& r, int64_t ti, auto more_c) {
         constexpr bool more = decltype(more_c)::value;
         const int64_t j0 = ti * TILE;
+        s8v kall[2][KB];
+        if constexpr (DMA) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R::NLV) : "memory");           // V(i) may be out; K(i) is in
+#pragma unroll
+            for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+                    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kall[kt2][kb]) : "v"(k_rd[kb]), "n"(kt2 * 16 * RS));
+            // (every register the reads fill is named, so that no use of one moves above the wait)
+#pragma unroll
+            for (int kt2 = 0; kt2 < 2; ++kt2) {
+                if constexpr (KB == 4)
+                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kall[kt2][0]), "+v"(kall[kt2][1]), "+v"(kall[kt2][2]), "+v"(kall[kt2][3])::"memory");
+                else
+                    asm volatile("s_waitcnt lgkmcnt(0)"
+                                 : "+v"(kall[kt2][0]), "+v"(kall[kt2][1]), "+v"(kall[kt2][2]), "+v"(kall[kt2][3]), "+v"(kall[kt2][4]),
+                                   "+v"(kall[kt2][5]), "+v"(kall[kt2][6]), "+v"(kall[kt2][7])::"memory");
+            }
+            if constexpr (more) dma_tile(ti + WAVES, 0);
+        }
         if constexpr (!DMA) {
             // ---- the value tile dequantized into this wave's LDS stage, [key][D] halfs
             const int c = lane % R::CPR, kr0 = lane / R::CPR;
@@ -275,7 +319,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
                 if constexpr (DMA) {
-                    ka[kb] = __builtin_bit_cast(s8v, r.k4[kt2][kb]);
+                    ka[kb] = kall[kt2][kb];
                 } else {
                     const _Float16 d = __builtin_bit_cast(_Float16, r.ksc[kt2][kb]);
                     short tmp[8];
@@ -342,7 +386,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         // too) before any LDS read it can see. DMA: this tile's loads are older than the next tile's 2 KB + NLV
         // (issued after them, in order), so waiting until only those remain makes the tile visible
         if constexpr (DMA) {
-            if constexpr (more) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * KB + R::NLV) : "memory");
+            if constexpr (more) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R::NLV) : "memory");     // K(i + 1) may be out
             else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         } else {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -358,7 +402,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                 uint32_t src;
                 if constexpr (DMA) {
                     const int c = (dt * 2 + ((n & 3) >> 1)) ^ (2 * (kk & 7));
-                    src = (uint32_t) (uintptr_t) (stage + buf * VTILE + kk * RS + c * 16 + (n & 1) * 8);
+                    src = (uint32_t) (uintptr_t) (stage + VTILE + kk * RS + c * 16 + (n & 1) * 8);
                 } else {
                     src = (uint32_t) (uintptr_t) (stage + kk * RS + (dt * 16 + 4 * (n & 3)) * 2);
                 }
@@ -376,26 +420,31 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         }
         // every read of the stage has returned: it is free for the next loads
         asm volatile("" ::: "memory");
+        if constexpr (DMA && more) dma_tile(ti + WAVES, 1);
     };
 
-    // ---- the wave's tiles. The steady state is its own loop so that every wait in it knows exactly which loads were
-    // issued after the ones it needs
+    // ---- the wave's tiles. Quantized rows alternate two register sets, the next tile's loads issued before this one's math
     if (ti < te) {
         const std::true_type more;
         const std::false_type last;
-        while (ti + 2 * WAVES < te) {
-            load_tile(rb, ti + WAVES, 1);
-            process_tile(ra, ti, 0, more);
-            load_tile(ra, ti + 2 * WAVES, 0);
-            process_tile(rb, ti + WAVES, 1, more);
-            ti += 2 * WAVES;
-        }
-        if (ti + WAVES < te) {
-            load_tile(rb, ti + WAVES, 1);
-            process_tile(ra, ti, 0, more);
-            process_tile(rb, ti + WAVES, 1, last);
+        if constexpr (DMA) {
+            for (; ti + WAVES < te; ti += WAVES) process_tile(ra, ti, more);
+            process_tile(ra, ti, last);
         } else {
-            process_tile(ra, ti, 0, last);
+            while (ti + 2 * WAVES < te) {
+                load_tile(rb, ti + WAVES);
+                process_tile(ra, ti, more);
+                load_tile(ra, ti + 2 * WAVES);
+                process_tile(rb, ti + WAVES, more);
+                ti += 2 * WAVES;
+            }
+            if (ti + WAVES < te) {
+                load_tile(rb, ti + WAVES);
+                process_tile(ra, ti, more);
+                process_tile(rb, ti + WAVES, last);
+            } else {
+                process_tile(ra, ti, last);
+            }
         }
     }
 
