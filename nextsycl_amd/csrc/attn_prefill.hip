@@ -60,7 +60,9 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
     // a wave owns RT row tiles of 16: 32 rows at D = 128; 16 at D = 256, whose accumulators are twice as wide
     constexpr int RT = D == 128 ? 2 : 1, WROWS = RT * 16, ROWS = PW * WROWS;
     constexpr int KB = D / 32, DT = D / 16;
-    constexpr int KS = D * 2 + 16, VS = D * 2 + 32;             // bytes a staged key row / value row
+    // bytes a staged key row / value row: rows 32 bytes apart modulo 256, so that the 16-byte operand reads of 16 keys (and
+    // the transposing reads of the values) meet no bank conflict - 16 bytes apart the key reads would, two ways
+    constexpr int KS = D * 2 + 32, VS = D * 2 + 32;
     constexpr int KBUF = KT_TILE * KS, VBUF = KT_TILE * VS;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * (KBUF + VBUF)];
 
@@ -84,7 +86,8 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
     const int64_t kend = p.p0 + rl + 1;                           // keys [kbeg, kend) cover every row of the block
     const int64_t kbeg = p.win > 0 ? std::max<int64_t>(0, p.p0 + r0 + 1 - p.win) : 0;
 
-    // ---- this lane's two rows: positions, key ranges, Q^T operands
+    // ---- this lane's two rows: positions, key ranges, Q^T operands. The queries carry the softmax scale (x log2 e) into
+    // the 16-bit operand, so that the score product comes out in exponent units and needs no multiplication a score
     int64_t lo_r[RT], hi_r[RT];
     s8v qreg[RT][KB];
 #pragma unroll
@@ -107,7 +110,7 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
             for (int kb = 0; kb < KB; ++kb) {
                 const float f[8] = {raw[kb][0].x, raw[kb][0].y, raw[kb][0].z, raw[kb][0].w, raw[kb][1].x, raw[kb][1].y, raw[kb][1].z, raw[kb][1].w};
 #pragma unroll
-                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = to16<BF>(f[i]);
+                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = to16<BF>(f[i] * p.sl2);
             }
         } else {
             uint4 raw[KB];
@@ -119,7 +122,7 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const uint16_t b16 = (uint16_t) (ww[i >> 1] >> (16 * (i & 1)));
-                    qreg[rt][kb][i] = (p.qt == 2) == BF ? (short) b16 : to16<BF>(p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16));
+                    qreg[rt][kb][i] = to16<BF>((p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16)) * p.sl2);
                 }
             }
         }
@@ -147,10 +150,13 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
     // Online softmax state, in base-2 exponent units (scores x scale x log2 e): nbr = minus the reference the weights
     // are taken against, thr = how far a score may exceed it before the reference moves (-inf while the row has seen no
     // key: the first one sets it), l_r = this lane's own share of the row's sum
+    // (nb4: nbr in all four slots of an accumulator, the value the score products start from)
     float nbr[RT], thr[RT], l_r[RT];
+    f4v nb4[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         nbr[rt] = 0.0f;
+        nb4[rt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
         thr[rt] = -INFINITY;
         l_r[rt] = 0.0f;
     }
@@ -255,7 +261,8 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
     s8v pb[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) pb[rt] = s8v{0, 0, 0, 0, 0, 0, 0, 0};
-    // S^T of one 32-key half (LDS byte offset kl) against the wave's 32 rows
+    // S^T of one 32-key half (LDS byte offset kl) against the wave's 32 rows, in exponent units and counted from the
+    // row's reference: the accumulators start at nbr
     auto scores = [&](f4v (&s)[RT][2], uint32_t kl) {
 #pragma unroll
         for (int kt2 = 0; kt2 < 2; ++kt2) {
@@ -265,9 +272,9 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
                 ka[kb] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + kl + k_rd + kt2 * 16 * KS + kb * 64);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+                f4v acc = mfma16<BF>(ka[0], qreg[rt][0], nb4[rt]);
 #pragma unroll
-                for (int kb = 0; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
+                for (int kb = 1; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
                 s[rt][kt2] = acc;
             }
         }
@@ -319,9 +326,7 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
         bool grow = false;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) a[rt][e] = __builtin_fmaf(a[rt][e], p.sl2, nbr[rt]);
-            amax[rt] = fmaxf(fmaxf(fmaxf(a[rt][0], a[rt][1]), fmaxf(a[rt][2], a[rt][3])), fmaxf(fmaxf(a[rt][4], a[rt][5]), fmaxf(a[rt][6], a[rt][7])));
+            amax[rt] = fmaxf(fmaxf(fmaxf(fmaxf(fmaxf(fmaxf(fmaxf(a[rt][0], a[rt][1]), a[rt][2]), a[rt][3]), a[rt][4]), a[rt][5]), a[rt][6]), a[rt][7]);
             grow |= amax[rt] > thr[rt];
         }
         if (__any(grow)) {
@@ -336,6 +341,7 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
                 nbr[rt] -= delta;
+                nb4[rt] = f4v{nbr[rt], nbr[rt], nbr[rt], nbr[rt]};
 #pragma unroll
                 for (int e = 0; e < 8; ++e) a[rt][e] -= delta;
                 thr[rt] = (fresh && nokey) ? -INFINITY : 8.0f;
