@@ -9,9 +9,10 @@
 // Work split: grid (cell split, row group). A work-group of 8 waves owns 128 (row, head) pairs - one decode row's 128
 // heads - a wave 16 of them (one 16-row MFMA tile: 72 registers of queries, 128 of accumulators), and a split of the
 // cells in 32-cell tiles. A tile is fetched by all 512 threads (16-byte chunks, global -> registers one tile ahead ->
-// LDS, two LDS buffers, one barrier a tile; GLM's q8 rows are widened to half on the way) and shared by the 8 waves. LDS rows are 72 chunks; chunk c of row r sits at
-// position c ^ g(r), g(r) = 2 ((r >> 1) & 3) | ((r >> 3) & 1), which spreads both access patterns over the banks: 16
-// rows x 16 bytes of one column (the score product's operand) and 8 rows x 32 bytes (the transposing read).
+// LDS, two LDS buffers, one barrier a tile; GLM's q8 rows are widened to half on the way) and shared by the 8 waves. LDS
+// rows are 74 chunks of 16 bytes (72 of data, 2 of padding): rows 32 bytes apart modulo 256 spread both access patterns
+// over the banks - 16 rows x 16 bytes of one column (the score product's operand) and 8 rows x 32 bytes (the
+// transposing read); both measured at the full LDS rate, where rows a multiple of 128 bytes apart halve the first.
 //
 // A wave's tile step (transposed orientation: a lane owns one row of each row tile):
 //   S^T[cell][row] = C Q^T          A = cache rows from LDS (ds_read_b128), B = absorbed queries, in registers
@@ -60,13 +61,11 @@ struct MlaParams {
 
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));   // a 16-byte chunk in flight (a plain vector: stays in registers)
 
-__device__ __forceinline__ int swz(int r) { return (((r >> 1) & 3) << 1) | ((r >> 3) & 1); }
-
 // R: rope features (64: DeepSeek's [512 | 64] rows; 0: GLM's latent-only rows); Q8: GLM's q8 rows
 template <int R, bool Q8>
 __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams p) {
     constexpr int DK = ML + R, KB = DK / 32, DT = ML / 16;
-    constexpr int RSTRIDE = 72 * 16;                     // bytes a staged row (72 chunks, whatever DK)
+    constexpr int RCH = 74, RSTRIDE = RCH * 16;          // chunks / bytes a staged row (whatever DK)
     constexpr int TILEB = MTILE * RSTRIDE;
     constexpr int64_t CROW = Q8 ? ML / 32 * 2 + ML : DK * 2;   // bytes a cache row
     constexpr int CPR = Q8 ? ML / 16 : DK / 8;           // 16-byte loads a cache row
@@ -182,43 +181,43 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
                     a[e] = __builtin_bit_cast(short, x0);
                     b[e] = __builtin_bit_cast(short, x1);
                 }
-                *reinterpret_cast<__attribute__((address_space(3))) s8v*>(base + r * RSTRIDE + ((2 * c) ^ swz(r)) * 16) = a;
-                *reinterpret_cast<__attribute__((address_space(3))) s8v*>(base + r * RSTRIDE + ((2 * c + 1) ^ swz(r)) * 16) = b;
+                *reinterpret_cast<__attribute__((address_space(3))) s8v*>(base + r * RSTRIDE + (2 * c) * 16) = a;
+                *reinterpret_cast<__attribute__((address_space(3))) s8v*>(base + r * RSTRIDE + (2 * c + 1) * 16) = b;
             } else {
-                *reinterpret_cast<__attribute__((address_space(3))) u4v*>(base + r * RSTRIDE + (c ^ swz(r)) * 16) = st[i % H1];
+                *reinterpret_cast<__attribute__((address_space(3))) u4v*>(base + r * RSTRIDE + c * 16) = st[i % H1];
             }
         }
     };
 
-    // LDS read addresses as a few lane bases plus compile-time offsets. The swizzle touches the low 3 bits of a chunk
-    // index only, so chunk (8 a + b) ^ g = 8 a + (b ^ g): one base a value of b, 128 bytes a step of a.
+    // LDS read addresses as a few lane bases plus compile-time offsets: chunk 8 a + b -> one base a value of b, 128 bytes a
+    // step of a.
     //   score operand: row ct 16 + n (g the same for both ct), chunk 4 kb + g4        -> b = 4 (kb & 1) + g4, a = kb >> 1
     //   transposed read: row kk (+ 16: same g), chunk 2 dt + ((n & 3) >> 1), half n & 1 -> b = 2 (dt & 3) + .., a = dt >> 2
     const int kk = g4 * 4 + (n >> 2);
     uint32_t s_rd[2], v_rd[4];
 #pragma unroll
-    for (int b = 0; b < 2; ++b) s_rd[b] = (uint32_t) (n * RSTRIDE + (((b * 4 + g4) ^ swz(n)) * 16));
+    for (int b = 0; b < 2; ++b) s_rd[b] = (uint32_t) (n * RSTRIDE + (b * 4 + g4) * 16);
 #pragma unroll
-    for (int b = 0; b < 4; ++b) v_rd[b] = (uint32_t) (kk * RSTRIDE + (((b * 2 + ((n & 3) >> 1)) ^ swz(kk)) * 16) + (n & 1) * 8);
+    for (int b = 0; b < 4; ++b) v_rd[b] = (uint32_t) (kk * RSTRIDE + (b * 2 + ((n & 3) >> 1)) * 16 + (n & 1) * 8);
 
     // Half rows go global -> LDS directly (global_load_lds_dwordx4: no register in between, so a tile can be two tiles
     // ahead of the math at no cost in registers). An instruction's 64 lanes fill 64 consecutive 16-byte units of the
-    // buffer, so the swizzle is applied on the source side: unit u = 72 r + x holds chunk x ^ g(r) of row r. A wave
-    // issues NDMA instructions a tile (units 512 i + 64 w + lane; the last 256 units are fetched twice, by waves w and
-    // w + 4, so that every wave has the same count in flight).
-    constexpr int NU = MTILE * 72, NDMA = (NU + MW * 64 - 1) / (MW * 64);
+    // buffer: unit u = 74 r + x holds chunk x of row r (the two units of padding fetch the row's last chunk again). A wave
+    // issues NDMA instructions a tile (units 512 i + 64 w + lane; in the last round the waves past the tile's end fetch units
+    // of waves 1 .. 3 again, so that every wave has the same count in flight).
+    constexpr int NU = MTILE * RCH, NDMA = (NU + MW * 64 - 1) / (MW * 64);
+    static_assert(NU % 64 == 0, "whole instructions a tile");
     auto dma = [&](lds_u8* dst, int it_) {
         const bool plain = !selt && (it_ + 1) * MTILE - 1 <= last_rel;
         const uint8_t* sp = selt ? p.cache : split_base + (plain ? (int64_t) it_ * MTILE * CROW : 0);
 #pragma unroll
         for (int i = 0; i < NDMA; ++i) {
             const int u0 = i * MW * 64 + w * 64 < NU ? i * MW * 64 + w * 64 : i * MW * 64 + (w & 3) * 64;
-            const int u = u0 + lane, r = u / 72, c = (u % 72) ^ swz(r);
+            const int u = u0 + lane, r = u / RCH, c = std::min(u % RCH, CPR - 1);
             const int rel = plain ? r : std::min(it_ * MTILE + r, last_rel);
             const uint32_t off = (uint32_t) ((selt ? cell(jb + rel) : (int64_t) rel) * CROW + c * 16);
-            if (CPR == 72 || c < CPR)
-                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (sp + off),
-                                                 (__attribute__((address_space(3))) void*) (dst + u0 * 16), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (sp + off),
+                                             (__attribute__((address_space(3))) void*) (dst + u0 * 16), 16, 0, 0);
         }
     };
 
