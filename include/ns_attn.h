@@ -70,10 +70,10 @@ int ns_q35_fwht32(ns_gpu* g, float* x, int64_t rows, int64_t n, int64_t stride);
 /* Typed decode: rows q [T][Hq*D] (element type qt, rows qs elements apart) at positions p0.. against caches of form kt;
  * pm 0 head-major [Hkv][cap][row] (slot = position % cap), 1 position-major [position][Hkv][row]; window win (<= 0:
  * all earlier keys); scale <= 0: 1/sqrt(D). out [T][Hq*D] of type qt. The keys are cut at absolute multiples of the
- * split size into ~1024 work-groups, every row of the pass riding on each key tile (a key is read once for all T x G
+ * split size into ~512 work-groups, every row of the pass riding on each key tile (a key is read once for all T x G
  * rows of its key head); partials (values, max in log2 units, sum) [T][Hq][ns][D + 2] go through `scratch`
- * (ns_attn_decode_scratch floats) and are merged by a second kernel. A row's result does not depend on which other
- * rows share its pass, bit for bit. D 128 or 256, T 1..16 */
+ * (ns_attn_decode_scratch floats, 8-byte aligned) and are merged by a second kernel. A row's result does not depend on
+ * which other rows share its pass, bit for bit. D 128 or 256, T 1..16 */
 int64_t ns_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win);
 int ns_attn_decode_t(ns_gpu* g, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq,
                      int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out, float* scratch);
