@@ -79,9 +79,9 @@ struct TileRegs {
     static constexpr int KPI = 64 / CPR;                                 // keys a wave covers per V load
     static constexpr int NLV = TILE / KPI;                               // V loads a lane per tile
     uint32_t k[2][DMA ? 1 : KB][KW];                                     // quantized rows: 8 int8 / 8 nibbles
-    uint16_t ksc[2][DMA ? 1 : KB];
+    uint32_t ksc[2][DMA ? 1 : KB];                                       // a block's half scale (in the low 16 bits)
     uint4 v[DMA ? 1 : NLV];                                              // quantized forms only
-    uint16_t vsc[DMA ? 1 : NLV];
+    uint32_t vsc[DMA ? 1 : NLV];
 };
 
 template <int D, int RT, int KT>
@@ -202,6 +202,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
 
     // ---- this lane's rows (one per row tile): their key ranges and Q^T operands
     int64_t lo_r[RT], hi_r[RT];
+    bool live_r[RT];
     s8v qreg[RT][KB];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
@@ -209,6 +210,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         const bool live = ri < rows;
         const int t = live ? ri / p.G : 0, gq = live ? ri % p.G : 0;
         const int64_t pos = p.p0 + t, first = p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0;
+        live_r[rt] = live;
         lo_r[rt] = live ? std::max(first, jb) : 1;
         hi_r[rt] = live ? std::min(p.causal ? pos : pass_end - 1, je - 1) : 0;
         // 8 consecutive features per k-block, vector loads all issued before any is used (rows are 16-byte aligned:
@@ -288,15 +290,10 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
 #pragma unroll
             for (int i = 0; i < R::NLV; ++i) {
                 uint8_t* dst = stage + (kr0 + R::KPI * i) * RS;
-                const _Float16 d = __builtin_bit_cast(_Float16, r.vsc[i]);
+                const _Float16 d = __builtin_bit_cast(_Float16, (uint16_t) r.vsc[i]);
                 if constexpr (KT == 1) {
-                    short tmp[16];
-                    dq8x4(r.v[i].x, d, tmp); dq8x4(r.v[i].y, d, tmp + 4); dq8x4(r.v[i].z, d, tmp + 8); dq8x4(r.v[i].w, d, tmp + 12);
-                    s8v a, b;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) { a[e] = tmp[e]; b[e] = tmp[8 + e]; }
-                    *reinterpret_cast<s8v*>(dst + c * 32) = a;
-                    *reinterpret_cast<s8v*>(dst + c * 32 + 16) = b;
+                    *reinterpret_cast<s8v*>(dst + c * 32) = dq8x8(r.v[i].x, r.v[i].y, d);
+                    *reinterpret_cast<s8v*>(dst + c * 32 + 16) = dq8x8(r.v[i].z, r.v[i].w, d);
                 } else {
                     short tmp[32];
                     dq4x4(r.v[i].x, 0, d, tmp); dq4x4(r.v[i].y, 0, d, tmp + 4); dq4x4(r.v[i].z, 0, d, tmp + 8); dq4x4(r.v[i].w, 0, d, tmp + 12);
@@ -321,18 +318,17 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                 if constexpr (DMA) {
                     ka[kb] = kall[kt2][kb];
                 } else {
-                    const _Float16 d = __builtin_bit_cast(_Float16, r.ksc[kt2][kb]);
-                    short tmp[8];
+                    const _Float16 d = __builtin_bit_cast(_Float16, (uint16_t) r.ksc[kt2][kb]);
                     if constexpr (KT == 1) {
-                        dq8x4(r.k[kt2][kb][0], d, tmp);
-                        dq8x4(r.k[kt2][kb][1], d, tmp + 4);
+                        ka[kb] = dq8x8(r.k[kt2][kb][0], r.k[kt2][kb][1], d);
                     } else {
+                        short tmp[8];
                         const int sh = g4 >= 2 ? 4 : 0;
                         dq4x4(r.k[kt2][kb][0], sh, d, tmp);
                         dq4x4(r.k[kt2][kb][1], sh, d, tmp + 4);
-                    }
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) ka[kb][e] = tmp[e];
+                        for (int e = 0; e < 8; ++e) ka[kb][e] = tmp[e];
+                    }
                 }
             }
 #pragma unroll
@@ -350,6 +346,20 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             const int blk = selp[j0 >> 7];
             hi_tile = blk < 0 ? -1 : (j0 & ~(int64_t) 127) + std::min<int64_t>(127, p.sel_pos - (int64_t) blk * 128);
         }
+        // a row's keys inside this tile: lo .. lo + span of 0 .. 31 (none: lo = 64 puts every key below it). Tiles that no
+        // live row's edge crosses - all but the first and last of a pass - take no comparison at all
+        int lo_t[RT];
+        unsigned span_t[RT];
+        bool edge = false;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const int lo_ = (int) std::min<int64_t>(std::max<int64_t>(lo_r[rt] - j0, 0), 32);
+            const int hi = (int) std::min<int64_t>(std::max<int64_t>(std::min(hi_r[rt], hi_tile) - j0, -1), 31);
+            lo_t[rt] = hi < lo_ ? 64 : lo_;
+            span_t[rt] = hi < lo_ ? 0u : (unsigned) (hi - lo_);
+            edge |= live_r[rt] && (lo_ > 0 || hi < 31);                   // (a dead row may keep its zero scores)
+        }
+        const bool masked = __any(edge);
         s8v pb[RT];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
@@ -358,8 +368,8 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const int64_t j = j0 + kt2 * 16 + g4 * 4 + i;
-                    const float v = (j >= lo_r[rt] && j <= std::min(hi_r[rt], hi_tile)) ? s[rt][kt2][i] * p.sl2 : -INFINITY;
+                    float v = s[rt][kt2][i] * p.sl2;
+                    if (masked) v = (unsigned) (kt2 * 16 + g4 * 4 + i - lo_t[rt]) <= span_t[rt] ? v : -INFINITY;
                     x[kt2 * 4 + i] = v;
                     mx = fmaxf(mx, v);
                 }

@@ -232,23 +232,23 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
                 *reinterpret_cast<__attribute__((address_space(3))) u4v*>(L + at) = st.raw[i];
             } else {
                 const _Float16 d = __builtin_bit_cast(_Float16, st.sc[i]);
-                short tmp[8 * PPC];
                 if constexpr (KT == 1) {
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) dq8x4(st.raw[i][q], d, tmp + 4 * q);
+                    *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at) = dq8x8(st.raw[i][0], st.raw[i][1], d);
+                    *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at + 16) = dq8x8(st.raw[i][2], st.raw[i][3], d);
                 } else {
+                    short tmp[8 * PPC];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         dq4x4(st.raw[i][q], 0, d, tmp + 4 * q);            // values 0 .. 15: the low nibbles
                         dq4x4(st.raw[i][q], 4, d, tmp + 16 + 4 * q);       // values 16 .. 31: the high nibbles
                     }
-                }
 #pragma unroll
-                for (int q = 0; q < PPC; ++q) {
-                    s8v v8;
+                    for (int q = 0; q < PPC; ++q) {
+                        s8v v8;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) v8[e] = tmp[q * 8 + e];
-                    *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at + q * 16) = v8;
+                        for (int e = 0; e < 8; ++e) v8[e] = tmp[q * 8 + e];
+                        *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at + q * 16) = v8;
+                    }
                 }
             }
         }

@@ -33,14 +33,21 @@ __device__ __forceinline__ float kv_value_f32(const uint8_t* row, int kt, int D,
     return (float) ((int) (j < 16 ? w & 15 : w >> 4) - 8) * f16_to_f32(*reinterpret_cast<const uint16_t*>(row + D / 2 + 2 * b));
 }
 
-// 4 int8 in a word -> 4 halfs x scale; each product is exact in float32, so one rounding to half (what the reference
-// stages: half((float) q * (float) d))
-__device__ __forceinline__ void dq8x4(uint32_t w, _Float16 d, short* o) {
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        const _Float16 h = (_Float16) (short) (int8_t) (w >> (8 * b)) * d;
-        o[b] = __builtin_bit_cast(short, h);
-    }
+// 8 int8 in two words -> 8 halfs x scale, as an MFMA operand / LDS piece. Each product is exact in float32, so one
+// rounding to half (what the reference stages: half((float) q * (float) d)). Two values an instruction: a byte b of
+// q + 128 under the exponent byte 0x64 is the half 1024 + b exactly, minus 1152 is q exactly, and the half product q x d
+// rounds once.
+__device__ __forceinline__ uint32_t dq8x2(uint32_t x, uint32_t sel, _Float16 d) {
+    typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+    const h2v off = {(_Float16) -1152.0f, (_Float16) -1152.0f}, dd = {d, d};
+    return __builtin_bit_cast(uint32_t, (__builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x, sel)) + off) * dd);
+}
+typedef short dq_s8v __attribute__((ext_vector_type(8)));   // (the attention kernels' s8v)
+__device__ __forceinline__ dq_s8v dq8x8(uint32_t w0, uint32_t w1, _Float16 d) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
+    const u4 r = {dq8x2(x0, 0x04010400u, d), dq8x2(x0, 0x04030402u, d), dq8x2(x1, 0x04010400u, d), dq8x2(x1, 0x04030402u, d)};
+    return __builtin_bit_cast(dq_s8v, r);
 }
 // 4 nibbles (bits sh .. sh + 3 of each byte) -> 4 halfs: (nibble - 8) x scale
 __device__ __forceinline__ void dq4x4(uint32_t w, int sh, _Float16 d, short* o) {
