@@ -295,16 +295,11 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                     *reinterpret_cast<s8v*>(dst + c * 32) = dq8x8(r.v[i].x, r.v[i].y, d);
                     *reinterpret_cast<s8v*>(dst + c * 32 + 16) = dq8x8(r.v[i].z, r.v[i].w, d);
                 } else {
-                    short tmp[32];
-                    dq4x4(r.v[i].x, 0, d, tmp); dq4x4(r.v[i].y, 0, d, tmp + 4); dq4x4(r.v[i].z, 0, d, tmp + 8); dq4x4(r.v[i].w, 0, d, tmp + 12);
-                    dq4x4(r.v[i].x, 4, d, tmp + 16); dq4x4(r.v[i].y, 4, d, tmp + 20); dq4x4(r.v[i].z, 4, d, tmp + 24); dq4x4(r.v[i].w, 4, d, tmp + 28);
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; ++q4) {
-                        s8v a;
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) a[e] = tmp[q4 * 8 + e];
-                        *reinterpret_cast<s8v*>(dst + c * 64 + q4 * 16) = a;
-                    }
+                    // values 0 .. 15: the low nibbles of the 16 bytes, 16 .. 31: the high ones
+                    *reinterpret_cast<s8v*>(dst + c * 64) = dq4x8(r.v[i].x, r.v[i].y, 0, d);
+                    *reinterpret_cast<s8v*>(dst + c * 64 + 16) = dq4x8(r.v[i].z, r.v[i].w, 0, d);
+                    *reinterpret_cast<s8v*>(dst + c * 64 + 32) = dq4x8(r.v[i].x, r.v[i].y, 4, d);
+                    *reinterpret_cast<s8v*>(dst + c * 64 + 48) = dq4x8(r.v[i].z, r.v[i].w, 4, d);
                 }
             }
         }
@@ -322,12 +317,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                     if constexpr (KT == 1) {
                         ka[kb] = dq8x8(r.k[kt2][kb][0], r.k[kt2][kb][1], d);
                     } else {
-                        short tmp[8];
-                        const int sh = g4 >= 2 ? 4 : 0;
-                        dq4x4(r.k[kt2][kb][0], sh, d, tmp);
-                        dq4x4(r.k[kt2][kb][1], sh, d, tmp + 4);
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) ka[kb][e] = tmp[e];
+                        ka[kb] = dq4x8(r.k[kt2][kb][0], r.k[kt2][kb][1], g4 >= 2 ? 4 : 0, d);
                     }
                 }
             }
@@ -608,10 +598,16 @@ inline int64_t row_first(int64_t pos, int64_t win) { return win > 0 ? std::max<i
 // rows than 32 re-read the keys once per chunk)
 template <int D, int KT>
 int launch_rt(ns_gpu* g, const DecodeParams& p, int rows, dim3 grid_xy) {
-    const int RT = rows <= 16 ? 1 : 2;
+    // (quantized rows of 256: two row tiles and the staging registers do not fit the register file - one tile a chunk)
+    constexpr bool ONE = D == 256 && (KT == 1 || KT == 2);
+    const int RT = rows <= 16 || ONE ? 1 : 2;
     dim3 grid(grid_xy.x, grid_xy.y, (unsigned) ((rows + RT * 16 - 1) / (RT * 16)));
-    if (RT == 1) attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(p);
-    else attn_decode_kernel<D, 2, KT><<<grid, WAVES * 64, 0, g->q>>>(p);
+    if constexpr (ONE) {
+        attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(p);
+    } else {
+        if (RT == 1) attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(p);
+        else attn_decode_kernel<D, 2, KT><<<grid, WAVES * 64, 0, g->q>>>(p);
+    }
     NS_LAUNCHED("attn_decode");
     return 0;
 }

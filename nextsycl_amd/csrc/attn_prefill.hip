@@ -236,19 +236,11 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
                     *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at) = dq8x8(st.raw[i][0], st.raw[i][1], d);
                     *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at + 16) = dq8x8(st.raw[i][2], st.raw[i][3], d);
                 } else {
-                    short tmp[8 * PPC];
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        dq4x4(st.raw[i][q], 0, d, tmp + 4 * q);            // values 0 .. 15: the low nibbles
-                        dq4x4(st.raw[i][q], 4, d, tmp + 16 + 4 * q);       // values 16 .. 31: the high nibbles
-                    }
-#pragma unroll
-                    for (int q = 0; q < PPC; ++q) {
-                        s8v v8;
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) v8[e] = tmp[q * 8 + e];
-                        *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at + q * 16) = v8;
-                    }
+                    // values 0 .. 15: the low nibbles of the 16 bytes, 16 .. 31: the high ones
+                    *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at) = dq4x8(st.raw[i][0], st.raw[i][1], 0, d);
+                    *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at + 16) = dq4x8(st.raw[i][2], st.raw[i][3], 0, d);
+                    *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at + 32) = dq4x8(st.raw[i][0], st.raw[i][1], 4, d);
+                    *reinterpret_cast<__attribute__((address_space(3))) s8v*>(L + at + 48) = dq4x8(st.raw[i][2], st.raw[i][3], 4, d);
                 }
             }
         }

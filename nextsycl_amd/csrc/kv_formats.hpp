@@ -49,11 +49,16 @@ __device__ __forceinline__ dq_s8v dq8x8(uint32_t w0, uint32_t w1, _Float16 d) {
     const u4 r = {dq8x2(x0, 0x04010400u, d), dq8x2(x0, 0x04030402u, d), dq8x2(x1, 0x04010400u, d), dq8x2(x1, 0x04030402u, d)};
     return __builtin_bit_cast(dq_s8v, r);
 }
-// 4 nibbles (bits sh .. sh + 3 of each byte) -> 4 halfs: (nibble - 8) x scale
-__device__ __forceinline__ void dq4x4(uint32_t w, int sh, _Float16 d, short* o) {
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-        const _Float16 h = (_Float16) (short) ((int) ((w >> (8 * b + sh)) & 15u) - 8) * d;
-        o[b] = __builtin_bit_cast(short, h);
-    }
+// 8 nibbles (bits sh .. sh + 3 of each byte of two words) -> 8 halfs (nibble - 8) x scale: the same two-a-time form,
+// a nibble under the exponent byte being 1024 + nibble and 1032 taken off
+__device__ __forceinline__ uint32_t dq4x2(uint32_t x, uint32_t sel, _Float16 d) {
+    typedef _Float16 h2v __attribute__((ext_vector_type(2)));
+    const h2v off = {(_Float16) -1032.0f, (_Float16) -1032.0f}, dd = {d, d};
+    return __builtin_bit_cast(uint32_t, (__builtin_bit_cast(h2v, __builtin_amdgcn_perm(0x64646464u, x, sel)) + off) * dd);
+}
+__device__ __forceinline__ dq_s8v dq4x8(uint32_t w0, uint32_t w1, int sh, _Float16 d) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const uint32_t x0 = (w0 >> sh) & 0x0f0f0f0fu, x1 = (w1 >> sh) & 0x0f0f0f0fu;
+    const u4 r = {dq4x2(x0, 0x04010400u, d), dq4x2(x0, 0x04030402u, d), dq4x2(x1, 0x04010400u, d), dq4x2(x1, 0x04030402u, d)};
+    return __builtin_bit_cast(dq_s8v, r);
 }

@@ -26,6 +26,8 @@ SMALL = [
     (1, 12, 2, 256, 1500, 0, 0, F32),      # qwen35's head size, G 6
     (2, 12, 2, 256, 900, 0, 1, F32),       # ... with a q8_0 cache
     (2, 8, 2, 256, 700, 0, 2, F32),        # ... with a q4_0 cache
+    (4, 12, 2, 256, 800, 0, 1, F32),       # ... q8_0 and 24 rows a key head: chunks of one row tile
+    (4, 16, 2, 128, 1200, 0, 1, F16),      # q8_0, 32 rows a key head: two row tiles
     (1, 8, 2, 128, 5000, 1024, 0, F32),    # a window
     (5, 8, 2, 128, 130, 100, 0, F32),      # a window shorter than a split
 ]
