@@ -42,6 +42,7 @@ namespace {
 
 constexpr int WAVES = 4, TILE = 32;
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u4a8 __attribute__((ext_vector_type(4), aligned(8)));   // 16 bytes at an 8-byte aligned address
 // Keys and values are read once a pass: their loads carry the non-temporal hint (the cache-policy bit of the direct
 // global -> LDS load; __builtin_nontemporal_load elsewhere), which measured ~10 % more HBM bandwidth on streaming reads
 constexpr int NT_AUX = 2;
@@ -162,9 +163,15 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
                 if constexpr (KT == 1) {
-                    const uint2 x = *reinterpret_cast<const uint2*>(kr + kb * 32 + g4 * 8);
-                    r.k[kt2][kb][0] = x.x; r.k[kt2][kb][1] = x.y;
-                    r.ksc[kt2][kb] = *reinterpret_cast<const uint16_t*>(kr + D + 2 * kb);
+                    // 16 bytes a lane and pair of k-blocks (rows are 8-byte aligned): k-block 2 j + h, lane group g4, slot e
+                    // stands for feature 64 j + 16 g4 + 8 h + e - the queries are loaded in the same order - and both
+                    // k-blocks of a pair lie in the scale block 2 j + g4 / 2
+                    if (kb % 2 == 0) {
+                        const u4a8 x = *reinterpret_cast<const u4a8*>(kr + kb * 32 + g4 * 16);
+                        r.k[kt2][kb][0] = x[0]; r.k[kt2][kb][1] = x[1];
+                        r.k[kt2][kb + 1][0] = x[2]; r.k[kt2][kb + 1][1] = x[3];
+                        r.ksc[kt2][kb] = r.ksc[kt2][kb + 1] = *reinterpret_cast<const uint16_t*>(kr + D + 2 * (kb + g4 / 2));
+                    }
                 } else {
                     const uint2 x = *reinterpret_cast<const uint2*>(kr + kb * 16 + (g4 & 1) * 8);
                     r.k[kt2][kb][0] = x.x; r.k[kt2][kb][1] = x.y;
@@ -215,13 +222,15 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         hi_r[rt] = live ? std::min(p.causal ? pos : pass_end - 1, je - 1) : 0;
         // 8 consecutive features per k-block, vector loads all issued before any is used (rows are 16-byte aligned:
         // checked on the host); a dead row reads row 0's and is zeroed
-        const int64_t qoff = (int64_t) t * p.qs + ((int64_t) hk * p.G + gq) * D + g4 * 8;
+        // feature order of the k-blocks: plain (k-block kb, lane group g4: features 32 kb + 8 g4 ..), q8_0 keys: see load_tile
+        auto foff = [&](int kb) { return KT == 1 ? 64 * (kb / 2) + 16 * g4 + 8 * (kb % 2) : 32 * kb + 8 * g4; };
+        const int64_t qoff = (int64_t) t * p.qs + ((int64_t) hk * p.G + gq) * D;
         if (p.qt == 0) {
             float4 raw[KB][2];
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
-                raw[kb][0] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.q) + qoff + kb * 32);
-                raw[kb][1] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.q) + qoff + kb * 32 + 4);
+                raw[kb][0] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.q) + qoff + foff(kb));
+                raw[kb][1] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p.q) + qoff + foff(kb) + 4);
             }
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
@@ -232,7 +241,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         } else {
             uint4 raw[KB];
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb) raw[kb] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.q) + qoff + kb * 32);
+            for (int kb = 0; kb < KB; ++kb) raw[kb] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.q) + qoff + foff(kb));
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
                 const uint32_t ww[4] = {raw[kb].x, raw[kb].y, raw[kb].z, raw[kb].w};
