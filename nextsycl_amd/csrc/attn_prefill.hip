@@ -4,16 +4,16 @@
 // Bound: MFMA. 4 D flops a visible (row, key) pair against 2 x 2 D bytes a key shared by every row that sees it:
 // thousands of flops a byte at prompt lengths.
 //
-// Work split: one work-group per (row block, query head). A work-group of 4 waves owns ROWS = 128 consecutive query rows
+// Work split: one work-group per (row block, query head). A work-group of 8 waves owns ROWS = 256 consecutive query rows
 // of one query head (a wave 32 of them: two 16-row MFMA tiles) and streams the keys its rows see in 64-key tiles,
 // heaviest row blocks first (the last block sees the most keys). The G query heads of a key head on one row block are
 // neighbours in the logical order and, through the XCD-aware mapping of work-group ids, share one L2. A tile's K and V
-// rows are fetched by all 256 threads (16-byte chunks): global -> registers two tiles ahead -> LDS one tile ahead, two
+// rows are fetched by all 512 threads (16-byte chunks): global -> registers two tiles ahead -> LDS one tile ahead, two
 // register sets, two LDS buffers, one barrier a tile.
 //
 // A wave's tile step, in the transposed orientation (a lane owns one query row of each row tile, so the row maximum,
 // the rescale and the normalisation never leave the lane):
-//   S^T[key][row] = K Q^T        K from LDS as the A operand (ds_read_b128, rows padded to 272 bytes), Q^T in registers
+//   S^T[key][row] = K Q^T        K from LDS as the A operand (ds_read_b128, rows padded to 288 bytes), Q^T in registers
 //   base-2 online softmax in float32 (scale folded into the exponent's fma; the accumulators rescaled only when a
 //   row's maximum moved); only 32-key halves crossing a row's causal or window edge are masked
 //   P^T -> 16 bit = the B operand of the second product as it stands
@@ -29,12 +29,16 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <type_traits>
 
 namespace {
 
-constexpr int PW = 4, KT_TILE = 64;
-constexpr int rows_of(int D) { return D == 128 ? 128 : 64; }   // query rows a work-group
+constexpr int KT_TILE = 64;
+// waves a work-group (PW): at D = 128 a wave owns 32 rows and a work-group 8 waves = 256 rows when that still leaves two
+// work-groups for every CU - a tile staged for 256 rows costs half the fetches and LDS writes a row, and two work-groups
+// of 4 waves on a CU were measured to run no faster than one of 8 - else 4 waves = 128 rows; at D = 256 4 waves of 16 rows
+constexpr int rows_of(int D, int PW) { return PW * (D == 128 ? 32 : 16); }   // query rows a work-group
 
 struct PrefillParams {
     const void* q;
@@ -53,8 +57,8 @@ struct PrefillParams {
 // a 16-byte chunk of a K or V row on its way from global memory to LDS (a plain vector type: arrays of it stay in registers)
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
 
-template <int D, bool BF, int KT>
-__global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel(const PrefillParams p) {
+template <int D, bool BF, int KT, int PW>
+__global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_prefill_kernel(const PrefillParams p) {
     static_assert(D == 128 || D == 256, "head size 128 or 256");
     static_assert(KT == 0 || !BF, "quantized rows are widened to half");
     // a wave owns RT row tiles of 16: 32 rows at D = 128; 16 at D = 256, whose accumulators are twice as wide
@@ -413,12 +417,14 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
     {
         const int esz = p.qt == 0 ? 4 : 2;
         const uint32_t rowb = (uint32_t) (D * esz), rowp = rowb + 16;    // bytes a row, padded in LDS
-        const uint32_t ob = (uint32_t) w * WROWS * (D * 4 + 16);
+        const uint32_t ob = (uint32_t) w * 16 * (D * 4 + 16);       // a wave's own region: one row tile at a time
+        const int ppr = (int) rowb / 16;                          // 16-byte pieces a row
+        uint8_t* const orow = reinterpret_cast<uint8_t*>(p.out) + (int64_t) hq * rowb;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             const float lsum = rows_sum(l_r[rt]);
             const float inv = lsum > 0.0f ? 1.0f / lsum : 0.0f;
-            const uint32_t at = ob + (uint32_t) (rt * 16 + n) * rowp + (uint32_t) (g4 * 4 * esz);
+            const uint32_t at = ob + (uint32_t) n * rowp + (uint32_t) (g4 * 4 * esz);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 const f4v v = o[rt][dt] * inv;
@@ -432,27 +438,31 @@ __global__ __launch_bounds__(PW * 64, D == 128 ? 2 : 1) void attn_prefill_kernel
                     *reinterpret_cast<__attribute__((address_space(3))) us4v*>(L + at + dt * 32) = h;
                 }
             }
-        }
-        // the wave reads back its own block only: no barrier, the LDS queue keeps a wave's accesses in order
-        const int ppr = (int) rowb / 16;                          // 16-byte pieces a row
-        uint8_t* const orow = reinterpret_cast<uint8_t*>(p.out) + (int64_t) hq * rowb;
-        for (int c = lane; c < WROWS * ppr; c += 64) {
-            const int rl_ = c / ppr, piece = c % ppr, row = r0 + w * WROWS + rl_;
-            if (row < p.T) {
-                const u4v x = *reinterpret_cast<const __attribute__((address_space(3))) u4v*>(L + ob + (uint32_t) rl_ * rowp + (uint32_t) piece * 16);
-                *reinterpret_cast<u4v*>(orow + (int64_t) row * p.Hq * rowb + piece * 16) = x;
+            // the wave reads back its own block only: no barrier, the LDS queue keeps a wave's accesses in order
+            for (int c = lane; c < 16 * ppr; c += 64) {
+                const int rl_ = c / ppr, piece = c % ppr, row = r0 + w * WROWS + rt * 16 + rl_;
+                if (row < p.T) {
+                    const u4v x = *reinterpret_cast<const __attribute__((address_space(3))) u4v*>(L + ob + (uint32_t) rl_ * rowp + (uint32_t) piece * 16);
+                    *reinterpret_cast<u4v*>(orow + (int64_t) row * p.Hq * rowb + piece * 16) = x;
+                }
             }
         }
     }
 }
 
-template <int D>
+template <int D, int PW>
 int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
-    switch (kt) {
-        case 0: attn_prefill_kernel<D, false, 0><<<grid, PW * 64, 0, g->q>>>(p); break;
-        case 3: attn_prefill_kernel<D, true, 0><<<grid, PW * 64, 0, g->q>>>(p); break;
-        case 1: attn_prefill_kernel<D, false, 1><<<grid, PW * 64, 0, g->q>>>(p); break;
-        default: attn_prefill_kernel<D, false, 2><<<grid, PW * 64, 0, g->q>>>(p); break;
+    constexpr int TH = PW * 64;
+    if (kt == 0) {
+        attn_prefill_kernel<D, false, 0, PW><<<grid, TH, 0, g->q>>>(p);
+    } else if (kt == 3) {
+        attn_prefill_kernel<D, true, 0, PW><<<grid, TH, 0, g->q>>>(p);
+    } else if constexpr (D == 256) {
+        // (quantized rows are a multiple of 16 bytes at D = 256 only: the caller has checked)
+        if (kt == 1) attn_prefill_kernel<D, false, 1, PW><<<grid, TH, 0, g->q>>>(p);
+        else attn_prefill_kernel<D, false, 2, PW><<<grid, TH, 0, g->q>>>(p);
+    } else {
+        return ns_fail("ns_attn_prompt: internal: quantized rows at this head size");
     }
     return 0;
 }
@@ -478,7 +488,11 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // rows do at D = 256 (272 / 144 bytes; the reference's quantized prompt form is D = 256 only), not at D = 128 (136 / 72)
     if (((uintptr_t) kc | (uintptr_t) vc) % 16) return ns_fail(w + ": caches 16-byte aligned");
     if (rb % 16) return ns_fail(w + ": quantized cache rows with heads of 256 (shorter passes and other heads take the decode kernel)");
-    const int64_t ROWS = rows_of((int) D);
+    // (512 work-groups of 256 rows: two for each of the chip's 256 CUs; NS_PREFILL_WAVES = 4 or 8 overrides: tuning, tests)
+    int PWs = D == 128 && ((T + 255) / 256) * Hq >= 512 ? 8 : 4;
+    if (const char* e = getenv("NS_PREFILL_WAVES"))
+        if (D == 128 && (atoi(e) == 4 || atoi(e) == 8)) PWs = atoi(e);
+    const int64_t ROWS = rows_of((int) D, PWs);
     if (T > (int64_t) 1 << 30 || ((T + ROWS - 1) / ROWS + 1) * Hq > (int64_t) 1 << 30) return ns_fail(w + ": too many rows or heads");
     if ((pm ? cap * Hkv : cap) * rb >= (int64_t) 1 << 32) return ns_fail(w + ": a key head's cache spans 4 GiB or more");
     NS_HIP(hipSetDevice(g->dev));
@@ -502,8 +516,8 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     const int64_t units = ((T + ROWS - 1) / ROWS) * Hkv;               // (row block, key head); padded to the 8 XCDs
     dim3 grid((unsigned) ((units + 7) / 8 * 8 * (Hq / Hkv)));
     if (ns_profile_mark(g, 0)) return -1;
-    if (D == 128) launch_prefill<128>(g, kt, p, grid);
-    else launch_prefill<256>(g, kt, p, grid);
+    if ((D == 256 ? launch_prefill<256, 4>(g, kt, p, grid) : PWs == 8 ? launch_prefill<128, 8>(g, kt, p, grid) : launch_prefill<128, 4>(g, kt, p, grid)) != 0)
+        return -1;
     NS_LAUNCHED("attn_prefill");
     return ns_profile_mark(g, 1);
     NS_CATCH

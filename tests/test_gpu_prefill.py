@@ -34,6 +34,23 @@ def test_prefill_small(ops, T, Hq, Hkv, p0, win, kt, qt):
     check_close(got, ref, qt, "prefill vs float64 closed form", kt=kt)
 
 
+@pytest.mark.parametrize("T,Hq,Hkv,p0,win,kt,qt", [(700, 10, 2, 300, 0, 3, BF16), (513, 4, 1, 0, 400, 0, F32)])
+def test_prefill_work_groups_of_8_waves(ops, monkeypatch, T, Hq, Hkv, p0, win, kt, qt):
+    """Long passes run work-groups of 8 waves (256-row blocks), short ones of 4: the same rows, keys and order of a wave's
+    arithmetic, so the two agree bit for bit; forced here on a shape the oracle finishes in seconds."""
+    D = 128
+    cap = p0 + T + 5
+    kc, vc = make_kv(kt, Hkv, D, cap, p0 + T)
+    qd, qf = make_q(qt, T, Hq, D)
+    monkeypatch.setenv("NS_PREFILL_WAVES", "8")
+    got8, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    monkeypatch.setenv("NS_PREFILL_WAVES", "4")
+    got4, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got8, ref, qt, "prefill (8 waves) vs float64 closed form", kt=kt)
+    assert np.array_equal(got8, got4)
+
+
 def test_prefill_ring(ops):
     T, Hq, Hkv, D, cap, win, p0 = 150, 4, 2, 128, 512, 300, 900
     k = orc.randn(11, (p0 + T, Hkv * D))
