@@ -8,8 +8,9 @@
 //
 // Work split: grid (cell split, row group). A work-group of 8 waves owns 128 (row, head) pairs - one decode row's 128
 // heads - a wave 16 of them (one 16-row MFMA tile: 72 registers of queries, 128 of accumulators), and a split of the
-// cells in 32-cell tiles. A tile is fetched by all 512 threads (16-byte chunks, global -> registers one tile ahead ->
-// LDS, two LDS buffers, one barrier a tile; GLM's q8 rows are widened to half on the way) and shared by the 8 waves. LDS
+// cells in 32-cell tiles; short passes of at most 128 rows run 4 waves = 64 pairs a work-group (mla_waves). Half rows go
+// global -> LDS directly two tiles ahead into three LDS buffers, one barrier a tile; GLM's q8 rows are fetched through
+// registers and widened to half on the way. The tile is shared by the work-group's waves. LDS
 // rows are 74 chunks of 16 bytes (72 of data, 2 of padding): rows 32 bytes apart modulo 256 spread both access patterns
 // over the banks - 16 rows x 16 bytes of one column (the score product's operand) and 8 rows x 32 bytes (the
 // transposing read); both measured at the full LDS rate, where rows a multiple of 128 bytes apart halve the first.
@@ -36,7 +37,12 @@
 
 namespace {
 
-constexpr int MW = 8, MTILE = 32, MROWS = 128, ML = 512;
+constexpr int MTILE = 32, ML = 512;
+// waves a work-group (16 rows each): 8 = 128-row groups; 4 = 64-row groups where a group (the pass's rows, or one row's
+// heads under a selection) has at most 128 rows and the pass at most 40960 cells - a decode step of 128 heads then runs
+// two groups over half as many cell splits: half the query loads and half the partials, which outweighs a tile loop
+// twice as long up to about that length (measured: 40.6 against 43.6 us at 32768 cells, 56.9 against 52.6 at 65536)
+constexpr int mla_waves(int64_t group_rows, int64_t cells) { return group_rows <= 128 && cells <= 40960 ? 4 : 8; }
 // a split's partial of a row: u_s[512] = O_s / l_s as halfs (the split's own normalized result: bounded by the cache's
 // values, so half holds it; a quarter of the float32 form's bytes go to m and l), then m (log2 units), l, 2 of padding
 constexpr int PSTRIDE = ML / 2 + 4;   // in floats: 1040 bytes, rows stay 16-byte aligned
@@ -62,8 +68,9 @@ struct MlaParams {
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));   // a 16-byte chunk in flight (a plain vector: stays in registers)
 
 // R: rope features (64: DeepSeek's [512 | 64] rows; 0: GLM's latent-only rows); Q8: GLM's q8 rows
-template <int R, bool Q8>
+template <int R, bool Q8, int MW>
 __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams p) {
+    constexpr int MROWS = MW * 16;
     constexpr int DK = ML + R, KB = DK / 32, DT = ML / 16;
     constexpr int RCH = 74, RSTRIDE = RCH * 16;          // chunks / bytes a staged row (whatever DK)
     constexpr int TILEB = MTILE * RSTRIDE;
@@ -203,8 +210,8 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
     // Half rows go global -> LDS directly (global_load_lds_dwordx4: no register in between, so a tile can be two tiles
     // ahead of the math at no cost in registers). An instruction's 64 lanes fill 64 consecutive 16-byte units of the
     // buffer: unit u = 74 r + x holds chunk x of row r (the two units of padding fetch the row's last chunk again). A wave
-    // issues NDMA instructions a tile (units 512 i + 64 w + lane; in the last round the waves past the tile's end fetch units
-    // of waves 1 .. 3 again, so that every wave has the same count in flight).
+    // issues NDMA instructions a tile (units 64 (MW i + w) + lane; in the last round the waves past the tile's end fetch its
+    // last 64 units again, so that every wave has the same count in flight).
     constexpr int NU = MTILE * RCH, NDMA = (NU + MW * 64 - 1) / (MW * 64);
     static_assert(NU % 64 == 0, "whole instructions a tile");
     auto dma = [&](lds_u8* dst, int it_) {
@@ -212,7 +219,7 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
         const uint8_t* sp = selt ? p.cache : split_base + (plain ? (int64_t) it_ * MTILE * CROW : 0);
 #pragma unroll
         for (int i = 0; i < NDMA; ++i) {
-            const int u0 = i * MW * 64 + w * 64 < NU ? i * MW * 64 + w * 64 : i * MW * 64 + (w & 3) * 64;
+            const int u0 = std::min(i * MW * 64 + w * 64, NU - 64);
             const int u = u0 + lane, r = u / RCH, c = std::min(u % RCH, CPR - 1);
             const int rel = plain ? r : std::min(it_ * MTILE + r, last_rel);
             const uint32_t off = (uint32_t) ((selt ? cell(jb + rel) : (int64_t) rel) * CROW + c * 16);
@@ -617,7 +624,9 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     const bool per_t = sel_cnt != nullptr;
     if (per_t && (!sel || K < 0 || K > (int64_t) 1 << 24)) return ns_fail(w + ": a selection has cell pools and their count");
     if ((pos0 + T) * (int64_t) (q8 ? 544 : (512 + R) * 2) >= (int64_t) 1 << 32 && per_t) return ns_fail(w + ": a selection over a cache past 4 GiB");
-    const int64_t rows = T * H, nz = per_t ? T * ((H + MROWS - 1) / MROWS) : (rows + MROWS - 1) / MROWS;
+    const int64_t rows = T * H;
+    const int MW = mla_waves(per_t ? H : rows, pos0 + T), MROWS = MW * 16;
+    const int64_t nz = per_t ? T * ((H + MROWS - 1) / MROWS) : (rows + MROWS - 1) / MROWS;
     const int64_t listed = 4 * K + 3, cells = per_t ? std::max(pos0 + T, listed) : pos0 + T;
     int64_t kbs = mla_kbs(per_t ? listed : cells, nz);
     if (per_t) kbs = std::max(kbs, ((cells + 1023) / 1024 + MTILE - 1) / MTILE * MTILE);
@@ -647,9 +656,15 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     p.per_t = per_t;
     dim3 grid((unsigned) ns, (unsigned) nz);
     if (ns_profile_mark(g, 0)) return -1;
-    if (q8) mla_decode_kernel<0, true><<<grid, MW * 64, 0, g->q>>>(p);
-    else if (R == 64) mla_decode_kernel<64, false><<<grid, MW * 64, 0, g->q>>>(p);
-    else mla_decode_kernel<0, false><<<grid, MW * 64, 0, g->q>>>(p);
+    if (MW == 4) {
+        if (q8) mla_decode_kernel<0, true, 4><<<grid, 256, 0, g->q>>>(p);
+        else if (R == 64) mla_decode_kernel<64, false, 4><<<grid, 256, 0, g->q>>>(p);
+        else mla_decode_kernel<0, false, 4><<<grid, 256, 0, g->q>>>(p);
+    } else {
+        if (q8) mla_decode_kernel<0, true, 8><<<grid, 512, 0, g->q>>>(p);
+        else if (R == 64) mla_decode_kernel<64, false, 8><<<grid, 512, 0, g->q>>>(p);
+        else mla_decode_kernel<0, false, 8><<<grid, 512, 0, g->q>>>(p);
+    }
     NS_LAUNCHED("mla_decode");
     if (ns_profile_mark(g, 1)) return -1;
     if (ot == 0) mla_merge_kernel<0><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
@@ -664,7 +679,7 @@ extern "C" {
 
 int64_t ns_mla_decode_latent_scratch(int64_t T, int64_t H, int64_t pos0) {
     if (T <= 0 || H <= 0) return 0;
-    const int64_t rows = T * H, nz = (rows + MROWS - 1) / MROWS, cells = pos0 + T, kbs = mla_kbs(cells, nz);
+    const int64_t rows = T * H, cells = pos0 + T, MROWS = mla_waves(rows, cells) * 16, nz = (rows + MROWS - 1) / MROWS, kbs = mla_kbs(cells, nz);
     return rows * ((cells + kbs - 1) / kbs) * PSTRIDE;
 }
 

@@ -58,7 +58,8 @@ def test_pure_functions_without_a_gpu(handle):
     assert p(17, 64, 4, 128) == 1 and p(16, 64, 4, 128) == 0 and p(100, 64, 4, 256) == 1 and p(100, 64, 4, 64) == 0
     m = handle.ns_mla_decode_latent_scratch
     m.restype, m.argtypes = C.c_int64, [C.c_int64] * 3
-    assert m(1, 128, 32767) == 128 * 256 * 260 and m(0, 128, 5) == 0     # 256 splits of 128 cells; a partial: 512 halfs + m, l (+ 2)
+    assert m(1, 128, 32767) == 128 * 128 * 260 and m(0, 128, 5) == 0     # two 64-row groups x 128 splits of 256 cells; a partial: 512 halfs + m, l (+ 2)
+    assert m(2, 128, 32766) == 256 * 128 * 260                           # two 128-row groups x 128 splits
     handle.ns_version.restype = C.c_char_p
     assert b"gfx950" in handle.ns_version()
     handle.ns_last_error.restype = C.c_char_p
