@@ -69,7 +69,7 @@ typedef uint32_t u4v __attribute__((ext_vector_type(4)));   // a 16-byte chunk i
 
 // R: rope features (64: DeepSeek's [512 | 64] rows; 0: GLM's latent-only rows); Q8: GLM's q8 rows
 template <int R, bool Q8, int MW>
-__global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams p) {
+__global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(const MlaParams p) {
     constexpr int MROWS = MW * 16;
     constexpr int DK = ML + R, KB = DK / 32, DT = ML / 16;
     constexpr int RCH = 74, RSTRIDE = RCH * 16;          // chunks / bytes a staged row (whatever DK)
@@ -246,7 +246,7 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
             auto ld = [&](int kb, int ct) {
                 return *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(rd + s_rd[kb & 1] + ct * 16 * RSTRIDE + (kb >> 1) * 128);
             };
-            constexpr int AHEAD = 1;                               // kb steps (two reads each) in flight
+            constexpr int AHEAD = MW == 4 ? 3 : 1;                 // kb steps (two reads each) in flight
             s8v fa[AHEAD + 1][2];
 #pragma unroll
             for (int kb = 0; kb < AHEAD; ++kb) {
@@ -320,7 +320,7 @@ __global__ __launch_bounds__(MW * 64, 2) void mla_decode_kernel(const MlaParams 
                 const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (src + 16 * RSTRIDE));
                 return s8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             };
-            constexpr int AHEAD = 2;
+            constexpr int AHEAD = MW == 4 ? 6 : 2;
             s8v va[AHEAD + 1];
 #pragma unroll
             for (int dt = 0; dt < AHEAD; ++dt) va[dt] = ldt(dt);
