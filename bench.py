@@ -127,12 +127,15 @@ def timed(w, steps, warmup):
     g.sync()
     ms = (time.perf_counter() - t0) * 1e3 / steps
     # the dominant kernel alone: HIP events on the library's compute stream around each launch (a pass of its own:
-    # the events open gaps between the launches that the throughput pass must not see)
+    # the events open gaps between the launches that the throughput pass must not see). Steps run back to back in short
+    # runs and the last step of each run is read, so the kernel is timed on a busy stream like the one above - a
+    # launch bracketed on an idle stream reads several microseconds long
     w.ops.profile(True)
     main = merge = 0.0
     n = max(3, min(steps, 20))
     for _ in range(n):
-        w.step()
+        for _ in range(6):
+            w.step()
         a, b = w.ops.profile_last()
         main += a
         merge += b
