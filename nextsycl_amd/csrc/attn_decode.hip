@@ -142,8 +142,31 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // 16-bit rows: a tile's keys (which = 0) or values (1) on their way global -> LDS, 1 KiB a load: position cp of key kk
     // holds the row's 16-byte chunk cp ^ (kk % 16) (keys: the operand reads of 16 keys' same chunk meet no bank
     // conflict) or cp ^ 2 (kk % 8) (values: the transposing reads)
+    // (a tile wholly inside the split of an unwrapped, unlisted cache - all but a pass's last - is read at a wave-uniform
+    // address plus per-lane offsets worked out once: FAST, where the registers allow)
+    constexpr bool FAST = DMA && D == 128;
+    uint32_t koff[FAST ? R::NLV : 1], voff[FAST ? R::NLV : 1];
+    if constexpr (FAST) {
+        const int cp = lane % R::CPR, kr0 = lane / R::CPR;
+#pragma unroll
+        for (int i = 0; i < R::NLV; ++i) {
+            const int kk = kr0 + R::KPI * i;
+            koff[i] = (uint32_t) (kk * p.row_stride) + (uint32_t) ((cp ^ (kk & 15)) * 16);
+            voff[i] = (uint32_t) (kk * p.row_stride) + (uint32_t) ((cp ^ (2 * (kk & 7))) * 16);
+        }
+    }
     auto dma_tile = [&](int64_t ti, int which) {
         const int j0 = (int) (ti * TILE - jb);                 // the tile's first key relative to the split's
+        if constexpr (FAST) {
+            if (!selp && !p.wrap && j0 >= 0 && j0 + TILE - 1 <= span) {
+                const uint8_t* base = (which ? vbase : kbase) + (jb_slot + j0) * p.row_stride;
+#pragma unroll
+                for (int i = 0; i < R::NLV; ++i)
+                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (base + (which ? voff[i] : koff[i])),
+                                                     (__attribute__((address_space(3))) void*) (stage + which * VTILE + i * 1024), 16, 0, NT_AUX);
+                return;
+            }
+        }
         const int cp = lane % R::CPR, kr0 = lane / R::CPR;
 #pragma unroll
         for (int i = 0; i < R::NLV; ++i) {
