@@ -63,6 +63,7 @@ struct MlaParams {
     const int32_t* sel;
     const int32_t* sel_cnt;
     int K, per_t;
+    int nz;              // row groups
 };
 
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));   // a 16-byte chunk in flight (a plain vector: stays in registers)
@@ -90,7 +91,12 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int split = blockIdx.x, z = blockIdx.y;
+    // Work-group ids go round the 8 XCDs (each with its own L2). The row groups of one cell split read the same tiles:
+    // they get consecutive ids on one XCD, so that they run side by side and a tile comes from memory once. The grid is
+    // padded to 8 splits a round; the padding's work-groups leave at once.
+    const int xcd = blockIdx.x % 8, xj = blockIdx.x / 8;
+    const int z = xj % p.nz, split = (xj / p.nz) * 8 + xcd;
+    if (split >= p.ns) return;
     const int rows = p.T * p.H;
     // a row group: 128 consecutive (row, head) pairs of the pass, or (per_t) 128 heads of one row t
     const int zpt = (p.H + MROWS - 1) / MROWS;
@@ -654,7 +660,8 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     p.sel_cnt = sel_cnt;
     p.K = (int) K;
     p.per_t = per_t;
-    dim3 grid((unsigned) ns, (unsigned) nz);
+    p.nz = (int) nz;
+    dim3 grid((unsigned) ((ns + 7) / 8 * 8 * nz));
     if (ns_profile_mark(g, 0)) return -1;
     if (MW == 4) {
         if (q8) mla_decode_kernel<0, true, 4><<<grid, 256, 0, g->q>>>(p);
