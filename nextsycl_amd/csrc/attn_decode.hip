@@ -178,11 +178,12 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         }
     };
     // quantized rows: the tile's keys (MFMA A layout) and values raw into registers
-    auto load_tile = [&](R& r, int64_t ti) {
-        const int j0 = (int) (ti * TILE - jb);
+    // (interior tiles of an unwrapped, unlisted cache: a wave-uniform tile address plus a lane's row offset, worked out once)
+    const uint32_t qk_lane = (uint32_t) (n * p.row_stride), qv_lane = (uint32_t) ((lane / R::CPR) * p.row_stride);
+    auto load_rows = [&](R& r, auto krow, auto vrow) {
 #pragma unroll
         for (int kt2 = 0; kt2 < 2; ++kt2) {
-            const uint8_t* kr = kbase + tile_off(ti, j0, kt2 * 16 + n);
+            const uint8_t* kr = krow(kt2);
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
                 if constexpr (KT == 1) {
@@ -202,13 +203,24 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                 }
             }
         }
-        const int cp = lane % R::CPR, kr0 = lane / R::CPR;
+        const int cp = lane % R::CPR;
 #pragma unroll
         for (int i = 0; i < R::NLV; ++i) {
-            const uint8_t* vr = vbase + tile_off(ti, j0, kr0 + R::KPI * i);
+            const uint8_t* vr = vrow(i);
             r.v[i] = *reinterpret_cast<const uint4*>(vr + cp * 16);
             if constexpr (KT == 1) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D + 2 * (cp / 2));
             if constexpr (KT == 2) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D / 2 + 2 * cp);
+        }
+    };
+    auto load_tile = [&](R& r, int64_t ti) {
+        const int j0 = (int) (ti * TILE - jb);
+        if (!selp && !p.wrap && j0 >= 0 && j0 + TILE - 1 <= span) {
+            const uint8_t* kt0 = kbase + (jb_slot + j0) * p.row_stride;
+            const uint8_t* vt0 = vbase + (jb_slot + j0) * p.row_stride;
+            load_rows(r, [&](int kt2) { return kt0 + kt2 * 16 * p.row_stride + qk_lane; }, [&](int i) { return vt0 + R::KPI * i * p.row_stride + qv_lane; });
+        } else {
+            const int kr0 = lane / R::CPR;
+            load_rows(r, [&](int kt2) { return kbase + tile_off(ti, j0, kt2 * 16 + n); }, [&](int i) { return vbase + tile_off(ti, j0, kr0 + R::KPI * i); });
         }
     };
 
