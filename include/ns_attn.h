@@ -61,6 +61,14 @@ int ns_attn_kv_store(ns_gpu* g, int kt, int ring, const float* k, int64_t ks, co
 /* n cache rows of form kt (`stride` bytes apart) widened to float32 [n][D] exactly as the attention kernels read them
  * into float32 (kernels/llm/qwen35/q35.cpp:19-25): the check of the byte formats. This library's own */
 int ns_attn_kv_dequant(ns_gpu* g, int kt, const void* rows, int64_t n, int64_t D, int64_t stride, float* out);
+/* The rows of positions [from, to) of every head moved between two caches of `row_bytes`-byte rows, head-major
+ * [heads][cap][row]: position p sits in slot (p - base) % cap of each. A ring is base 0, cap its slots; position
+ * order (a checkpoint's buffer) is base `from`, cap to - from. to - from may not pass either capacity. One launch for
+ * every head; queued like every call. Replaces the host loops of one or two copies a head in the engines' save /
+ * restore / copy_session (llm/museglimmer/src/engine.rs:1334-1346,1475-1528, llm/qwen35/src/engine.rs:2977-3011):
+ * the reference has no kernel for it */
+int ns_attn_kv_rows_copy(ns_gpu* g, const void* src, int64_t scap, int64_t sbase, void* dst, int64_t dcap, int64_t dbase, int64_t heads,
+                         int64_t row_bytes, int64_t from, int64_t to);
 /* normalized 32-point Walsh-Hadamard transform of each block of 32 in place (a quantized cache's optional rotation).
  * Replaces: kernels/llm/qwen35/q35.h:43-45 (q35.cpp:328-348) */
 int ns_q35_fwht32(ns_gpu* g, float* x, int64_t rows, int64_t n, int64_t stride);

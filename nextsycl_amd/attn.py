@@ -34,6 +34,7 @@ ATTN_H = {
     "ns_mg_kv_store": (i32, [P, P, P, i64, i64, i64, i64, i64, P, P]),
     "ns_attn_kv_store": (i32, [P, i32, i32, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]),
     "ns_attn_kv_dequant": (i32, [P, i32, P, i64, i64, i64, P]),
+    "ns_attn_kv_rows_copy": (i32, [P, P, i64, i64, P, i64, i64, i64, i64, i64, i64]),
     "ns_q35_fwht32": (i32, [P, P, i64, i64, i64]),
     "ns_attn_decode_scratch": (i64, [i64, i64, i64, i64, i64, i64]),
     "ns_attn_decode_t": (i32, [P, i32, i32, i32, P, i64, P, P, i64, i64, i64, i64, i64, i64, i64, f32, P, P]),
@@ -185,6 +186,12 @@ class Ops:
         _need(rows, n * rb, "kv_dequant rows")
         _need(out, n * D * 4, "kv_dequant out")
         self.ok(self.k.attn_kv_dequant(self.raw(), kt, rows.ptr, n, D, rb, out.ptr), "kv_dequant")
+
+    def kv_rows_copy(self, src, scap, sbase, dst, dcap, dbase, heads, row_bytes, pos_from, pos_to):
+        """Positions [pos_from, pos_to) of every head from one cache geometry into another (slot = (p - base) % cap)."""
+        _need(src, heads * scap * row_bytes, "kv_rows_copy source")
+        _need(dst, heads * dcap * row_bytes, "kv_rows_copy destination")
+        self.ok(self.k.attn_kv_rows_copy(self.raw(), src.ptr, scap, sbase, dst.ptr, dcap, dbase, heads, row_bytes, pos_from, pos_to), "kv_rows_copy")
 
     def fwht32(self, x, rows, n, stride):
         if rows > 0:

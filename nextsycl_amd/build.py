@@ -22,6 +22,7 @@ COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-ta
 SOURCES = {
     "ns_hip.cpp": [],
     "kv_store.hip": ["-ffp-contract=off"],
+    "kv_rows.hip": [],
     "pre_attn.hip": ["-ffp-contract=off"],
     "attn_decode.hip": [],
     "indexer.hip": [],

@@ -319,6 +319,74 @@ def mm3_norm_rope_row(row, w, rot, n_rot, pos, base, eps, want_half=False):
     return row, half
 
 
+# ---- checkpoints: the engines' host loops over a ring cache's runs, restated in numpy (byte moves only)
+def ring_kept(w, pos):
+    """llm/museglimmer/src/engine.rs:1358-1361."""
+    return max(pos - (w - 1), 0) if w > 0 else 0
+
+
+def ring_save(cache, heads, cap, row, w, pos):
+    """One cache's checkpoint buffer: [heads][kept .. pos)[row] bytes out of a ring [heads][cap][row] (slot = p % cap),
+    read as the engine does - runs that end at the ring's last slot (llm/museglimmer/src/engine.rs:1479-1494)."""
+    cache = np.ascontiguousarray(cache).view(np.uint8).reshape(-1)
+    first = ring_kept(w, pos)
+    n = pos - first
+    b = np.zeros(heads * n * row, np.uint8)
+    for h in range(heads):
+        p = first
+        while p < pos:
+            si = p % cap
+            run = min(pos - p, cap - si)
+            at = (h * n + p - first) * row
+            src = (h * cap + si) * row
+            b[at:at + run * row] = cache[src:src + run * row]
+            p += run
+    return b
+
+
+def ring_restore(cache, b, heads, cap, row, w, pos):
+    """`ring_save`'s buffer written back into a ring in place (llm/museglimmer/src/engine.rs:1509-1523)."""
+    cache = cache.view(np.uint8).reshape(-1)
+    first = ring_kept(w, pos)
+    n = pos - first
+    if b.size != heads * n * row:
+        raise ValueError("a checkpoint of another shape")
+    for h in range(heads):
+        p = first
+        while p < pos:
+            si = p % cap
+            run = min(pos - p, cap - si)
+            at = (h * n + p - first) * row
+            dst = (h * cap + si) * row
+            cache[dst:dst + run * row] = b[at:at + run * row]
+            p += run
+
+
+def ring_copy(dst, dcap, src, scap, heads, row, first, to):
+    """Positions [first, to) of one ring into another of other capacity, in place (llm/museglimmer/src/engine.rs:1334-1346)."""
+    dst = dst.view(np.uint8).reshape(-1)
+    src = np.ascontiguousarray(src).view(np.uint8).reshape(-1)
+    for h in range(heads):
+        p = first
+        while p < to:
+            si, di = p % scap, p % dcap
+            run = min(to - p, scap - si, dcap - di)
+            d0, s0 = (h * dcap + di) * row, (h * scap + si) * row
+            dst[d0:d0 + run * row] = src[s0:s0 + run * row]
+            p += run
+
+
+def checkpoint_file(magic, pos, bufs):
+    """The engines' checkpoint file: magic, u64 position, u64 count, then u64 length + bytes a buffer, little-endian
+    (llm/museglimmer/src/engine.rs:230-240)."""
+    out = bytearray(magic)
+    out += int(pos).to_bytes(8, "little") + len(bufs).to_bytes(8, "little")
+    for b in bufs:
+        b = np.ascontiguousarray(b).view(np.uint8).reshape(-1)
+        out += int(b.size).to_bytes(8, "little") + b.tobytes()
+    return bytes(out)
+
+
 def compare(a, b):
     """(max-abs, relative L2, cosine) of a (float32) against b (float64) - the reference's `kernels` check's measures."""
     a = _c(a, np.float32).ravel()
