@@ -115,12 +115,23 @@ class Workload:
             o.decode(self.qt, self.kt, self.q, self.Hq * self.D, kc, vc, self.T, self.Hq, self.Hkv, self.D, self.kv, self.p0, self.out, self.scratch)
 
 
+SETTLE_MS = 100.0
+
+
 def timed(w, steps, warmup):
     """(ms per step over exactly `steps` steps, average device ns of the dominant kernel, of the merge kernel)."""
     g = w.ops.gpu
+    # untimed: the W warmup steps, and then more of the same until the GPU has been under load for SETTLE_MS - an idle
+    # MI355X takes tens of milliseconds of work to reach its steady clocks (the first MFMA-bound launches after a pause
+    # run 15 - 30 % long), and the figure wanted is the sustained one
     for _ in range(warmup):
         w.step()
     g.sync()
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+        for _ in range(8):
+            w.step()
+        g.sync()
     t0 = time.perf_counter()
     for _ in range(steps):
         w.step()
@@ -255,7 +266,8 @@ def main():
         "dtype": {0: "f32", 1: "f16", 2: "bf16"}[w.qt] if w.kt in (0, 3) else "q8_0/f16",
         "data": "synthetic (seeded xorshift64* + Box-Muller N(0,1))",
         "config": {"workload": w.desc, "name": a.workload, "rows": w.T, "q_heads": w.Hq, "kv_heads": w.Hkv, "head_dim": w.D, "kv_len": w.kv,
-                   "kv_form": {0: "f16", 1: "q8_0", 2: "q4_0", 3: "bf16"}[w.kt], "flops_per_step": w.flops, "bytes_per_step": w.bytes},
+                   "kv_form": {0: "f16", 1: "q8_0", 2: "q4_0", 3: "bf16"}[w.kt], "flops_per_step": w.flops, "bytes_per_step": w.bytes,
+                   "untimed_settle_ms": SETTLE_MS},
         "tokens_per_s": round(w.T / (ms * 1e-3), 1),
         "roofline": roofline(w, main_ns),
     }
