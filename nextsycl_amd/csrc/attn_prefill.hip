@@ -478,7 +478,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     if (Hkv <= 0 || Hq <= 0 || Hq % Hkv) return ns_fail(w + ": query heads a multiple of the key heads");
     if (kt < 0 || kt > 3) return ns_fail(w + ": a cache form 0 (half), 1 (q8_0), 2 (q4_0) or 3 (bfloat16)");
     if (qt < 0 || qt > 2) return ns_fail(w + ": rows of type 0 (float32), 1 (half) or 2 (bfloat16)");
-    if (p0 < 0 || cap <= 0) return ns_fail(w + ": a position and a capacity");
+    if (p0 < 0 || cap <= 0 || win < 0) return ns_fail(w + ": a position, a capacity and a window of 0 or more");
     const int64_t need = pm ? p0 + T : (win > 0 ? std::min(p0 + T, win + T - 1) : p0 + T);
     if (need > cap) return ns_fail(w + (win > 0 ? ": the cache's ring is shorter than the window and the pass" : ": past the cache's capacity"));
     if (!q || !kc || !vc || !out) return ns_fail(w + ": a null buffer");
