@@ -221,7 +221,7 @@ def main():
                     help="first run a plain copy kernel of this many MiB 5 times (the known-size kernel rocprofv3 traffic counters are scaled against)")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on one GPU; --gpus %d is not supported (the path shards by key head or by context, see DESIGN.md)" % a.gpus,
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (the path would shard by key head, or by context with a merge of partials across GPUs)" % a.gpus,
               file=sys.stderr)
         sys.exit(2)
 
