@@ -51,14 +51,33 @@ __device__ __forceinline__ s4v lds_read_tr16(void* lds_addr) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Reductions over the 4 lanes {n, n + 16, n + 32, n + 48} that hold one query row's scores
+// Reductions over the 4 lanes {n, n + 16, n + 32, n + 48} that hold one query row's scores. The partner's value comes
+// by v_permlane16_swap / v_permlane32_swap (vector instructions: given two copies of v they return, in every lane, the
+// values of the even and the odd 16-lane row of its pair / of the lower and the upper half of the wave), not through LDS
+// as a general shuffle does: no LDS round trip to wait for in the softmax's dependency chain. Same operands, same sums.
+__device__ __forceinline__ void pair16(float v, float& a, float& b) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, v);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    a = __builtin_bit_cast(float, (uint32_t) r[0]);
+    b = __builtin_bit_cast(float, (uint32_t) r[1]);
+}
+__device__ __forceinline__ void pair32(float v, float& a, float& b) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, v);
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    a = __builtin_bit_cast(float, (uint32_t) r[0]);
+    b = __builtin_bit_cast(float, (uint32_t) r[1]);
+}
 __device__ __forceinline__ float rows_max(float v) {
-    v = fmaxf(v, __shfl_xor(v, 16));
-    return fmaxf(v, __shfl_xor(v, 32));
+    float a, b;
+    pair16(v, a, b);
+    pair32(fmaxf(a, b), a, b);
+    return fmaxf(a, b);
 }
 __device__ __forceinline__ float rows_sum(float v) {
-    v += __shfl_xor(v, 16);
-    return v + __shfl_xor(v, 32);
+    float a, b;
+    pair16(v, a, b);
+    pair32(a + b, a, b);
+    return a + b;
 }
 
 // element i of a row of query / output type QT (0 float32, 1 half, 2 bfloat16)

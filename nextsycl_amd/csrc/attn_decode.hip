@@ -243,7 +243,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     for (int kb = 0; kb < KB; ++kb) k_rd[kb] = (uint32_t) (uintptr_t) (stage + n * RS + (((kb * 4 + g4) ^ n) * 16));
 
     // ---- this lane's rows (one per row tile): their key ranges and Q^T operands
-    int64_t lo_r[RT], hi_r[RT];
+    int lo_r[RT], hi_r[RT];     // the row's first and last key in this split, relative to the split's first (none: 1, 0)
     bool live_r[RT];
     s8v qreg[RT][KB];
 #pragma unroll
@@ -253,8 +253,10 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         const int t = live ? ri / p.G : 0, gq = live ? ri % p.G : 0;
         const int64_t pos = p.p0 + t, first = p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0;
         live_r[rt] = live;
-        lo_r[rt] = live ? std::max(first, jb) : 1;
-        hi_r[rt] = live ? std::min(p.causal ? pos : pass_end - 1, je - 1) : 0;
+        // (a row whose last key lies before the split keeps an empty range; the differences fit 32 bits: a split's keys do)
+        const int64_t hi64 = std::min(p.causal ? pos : pass_end - 1, je - 1);
+        lo_r[rt] = live && hi64 >= jb ? (int) (std::max(first, jb) - jb) : 1;
+        hi_r[rt] = live && hi64 >= jb ? (int) (hi64 - jb) : 0;
         // 8 consecutive features per k-block, vector loads all issued before any is used (rows are 16-byte aligned:
         // checked on the host); a dead row reads row 0's and is zeroed
         // feature order of the k-blocks: plain (k-block kb, lane group g4: features 32 kb + 8 g4 ..), q8_0 keys: see load_tile
@@ -374,56 +376,67 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             }
         }
         // ---- online softmax a row (this lane: row n of each row tile, keys j0 + 16 kt2 + 4 g4 + i)
-        // (a listed block's keys count up to the row's own position; a hole in the list has none)
-        int64_t hi_tile = INT64_MAX;
+        // a row's keys inside this tile: lo .. lo + span of 0 .. 31 (none: lo = 64 puts every key below it), in 32-bit
+        // arithmetic relative to the split's first key. Tiles that no live row's edge crosses - all but the first and last
+        // of a pass - take no comparison at all (a wave-uniform branch)
+        const int j0r = (int) (j0 - jb);
+        int hi_tile = INT32_MAX;
         if (selp) {
+            // (a listed block's keys count up to the row's own position; a hole in the list has none)
             const int blk = selp[j0 >> 7];
-            hi_tile = blk < 0 ? -1 : (j0 & ~(int64_t) 127) + std::min<int64_t>(127, p.sel_pos - (int64_t) blk * 128);
+            hi_tile = blk < 0 ? j0r - 1 : (int) ((j0 & ~(int64_t) 127) - jb + std::min<int64_t>(127, p.sel_pos - (int64_t) blk * 128));
         }
-        // a row's keys inside this tile: lo .. lo + span of 0 .. 31 (none: lo = 64 puts every key below it). Tiles that no
-        // live row's edge crosses - all but the first and last of a pass - take no comparison at all
         int lo_t[RT];
         unsigned span_t[RT];
         bool edge = false;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-            const int lo_ = (int) std::min<int64_t>(std::max<int64_t>(lo_r[rt] - j0, 0), 32);
-            const int hi = (int) std::min<int64_t>(std::max<int64_t>(std::min(hi_r[rt], hi_tile) - j0, -1), 31);
+            const int lo_ = std::min(std::max(lo_r[rt] - j0r, 0), 32);
+            const int hi = std::min(std::max(std::min(hi_r[rt], hi_tile) - j0r, -1), 31);
             lo_t[rt] = hi < lo_ ? 64 : lo_;
             span_t[rt] = hi < lo_ ? 0u : (unsigned) (hi - lo_);
             edge |= live_r[rt] && (lo_ > 0 || hi < 31);                   // (a dead row may keep its zero scores)
         }
-        const bool masked = __any(edge);
+        float x[RT][8];
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[rt][e] = s[rt][e >> 2][e & 3];
+        if (__any(edge)) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    x[rt][e] = (unsigned) ((e >> 2) * 16 + g4 * 4 + (e & 3) - lo_t[rt]) <= span_t[rt] ? x[rt][e] : -INFINITY;
+        }
+        // the scale rides in the exponent's fused multiply-add: weights 2^(x sl2 - m), m the running maximum of x sl2
+        // (0 in its place while a row has seen no key: its weights are 2^(-inf) = 0 either way)
         s8v pb[RT];
+        float cs[RT];
+        bool shrink = false;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-            float x[8], mx = -INFINITY;
-#pragma unroll
-            for (int kt2 = 0; kt2 < 2; ++kt2)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float v = s[rt][kt2][i] * p.sl2;
-                    if (masked) v = (unsigned) (kt2 * 16 + g4 * 4 + i - lo_t[rt]) <= span_t[rt] ? v : -INFINITY;
-                    x[kt2 * 4 + i] = v;
-                    mx = fmaxf(mx, v);
-                }
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float mn = fmaxf(m_r[rt], mx);
-            const float c = mn == -INFINITY ? 1.0f : fast_exp2(m_r[rt] - mn);
+            const float mx = rows_max(fmaxf(fmaxf(fmaxf(x[rt][0], x[rt][1]), fmaxf(x[rt][2], x[rt][3])), fmaxf(fmaxf(x[rt][4], x[rt][5]), fmaxf(x[rt][6], x[rt][7]))));
+            const float mn = fmaxf(m_r[rt], mx * p.sl2);
+            const float ms = mn == -INFINITY ? 0.0f : mn;
+            cs[rt] = fast_exp2(m_r[rt] - ms);
+            shrink |= m_r[rt] != mn;
             float sum = 0.0f;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float pv = x[e] == -INFINITY ? 0.0f : fast_exp2(x[e] - mn);
+                const float pv = fast_exp2(fmaf(x[rt][e], p.sl2, -ms));
                 sum += pv;
                 pb[rt][e] = to16<BF>(pv);
             }
-            sum += __shfl_xor(sum, 16);
-            sum += __shfl_xor(sum, 32);
             m_r[rt] = mn;
-            l_r[rt] = l_r[rt] * c + sum;
+            l_r[rt] = l_r[rt] * cs[rt] + rows_sum(sum);
+        }
+        // the running output shrinks only when some row's maximum moved (rare once a pass is under way): wave-uniform
+        if (__any(shrink)) {
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= cs[rt];
         }
         // ---- O^T += V^T P^T: the value tile read back transposed. The reads and their waits are written in assembly:
         // the compiler's own tracking of LDS writes by DMA would wait for EVERY outstanding load here (the next tile's
