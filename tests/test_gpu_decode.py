@@ -48,6 +48,34 @@ def test_decode_small(ops, T, Hq, Hkv, D, p0, win, kt, qt):
         assert mx <= 2e-3 and rel <= 1e-3 + (2.0 ** -9 if qt == BF16 else 0)
 
 
+def _random_cases(n, seed):
+    """Seeded shapes over everything the kernel branches on: rows and groups (one or two row tiles, chunks), head size,
+    cache form, context from inside one tile to many splits, windows shorter and longer than a split."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        D = int(rng.choice([128, 128, 256]))
+        kt = int(rng.choice([0, 0, 1, 2, 3]))
+        Hkv = int(rng.integers(1, 4))
+        G = int(rng.choice([1, 2, 3, 4, 8, 16]))
+        T = int(rng.choice([1, 1, 2, 3, 5, 8, 16]))
+        p0 = int(rng.choice([rng.integers(0, 70), rng.integers(70, 700), rng.integers(700, 6000)]))
+        win = int(rng.choice([0, 0, rng.integers(1, 64), rng.integers(64, 2000)]))
+        qt = BF16 if kt == 3 else int(rng.choice([F32, F16]))
+        out.append((T, Hkv * G, Hkv, D, p0, win, kt, qt))
+    return out
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0,win,kt,qt", _random_cases(48, 20240607))
+def test_decode_seeded_shapes(ops, T, Hq, Hkv, D, p0, win, kt, qt):
+    cap = p0 + T + 3
+    kc, vc = make_kv(kt, Hkv, D, cap, p0 + T, cfg=p0 % 7)
+    qd, qf = make_q(qt, T, Hq, D, cfg=T)
+    got, _ = gpu_decode(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got, ref, qt, "decode vs float64 closed form", kt=kt)
+
+
 def test_decode_ring_wrap(ops):
     """A ring cache that has wrapped: slot = position % cap, window inside the ring."""
     T, Hq, Hkv, D, cap, win = 3, 8, 2, 128, 512, 400

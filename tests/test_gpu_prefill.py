@@ -34,6 +34,34 @@ def test_prefill_small(ops, T, Hq, Hkv, p0, win, kt, qt):
     check_close(got, ref, qt, "prefill vs float64 closed form", kt=kt)
 
 
+def _random_cases(n, seed):
+    """Seeded shapes over what the kernel branches on: rows around the block sizes, groups, head size (256 also over
+    quantized caches), a context before the pass, windows shorter and longer than a tile and than the pass."""
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        D = int(rng.choice([128, 128, 256]))
+        kt = int(rng.choice([0, 3, 1, 2])) if D == 256 else int(rng.choice([0, 3]))
+        Hkv = int(rng.integers(1, 3))
+        G = int(rng.choice([1, 2, 4, 5, 8]))
+        T = int(rng.choice([rng.integers(17, 70), rng.integers(70, 300), rng.integers(300, 600)]))
+        p0 = int(rng.choice([0, rng.integers(1, 100), rng.integers(100, 900)]))
+        win = int(rng.choice([0, 0, rng.integers(1, 64), rng.integers(64, 700)]))
+        qt = BF16 if kt == 3 else int(rng.choice([F32, F16]))
+        out.append((T, Hkv * G, Hkv, D, p0, win, kt, qt))
+    return out
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0,win,kt,qt", _random_cases(32, 20240608))
+def test_prefill_seeded_shapes(ops, T, Hq, Hkv, D, p0, win, kt, qt):
+    cap = p0 + T + 5
+    kc, vc = make_kv(kt, Hkv, D, cap, p0 + T, cfg=T % 5)
+    qd, qf = make_q(qt, T, Hq, D, cfg=p0 % 3)
+    got, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got, ref, qt, "prefill vs float64 closed form", kt=kt)
+
+
 @pytest.mark.parametrize("T,Hq,Hkv,p0,win,kt,qt", [(700, 10, 2, 300, 0, 3, BF16), (513, 4, 1, 0, 400, 0, F32)])
 def test_prefill_work_groups_of_8_waves(ops, monkeypatch, T, Hq, Hkv, p0, win, kt, qt):
     """Long passes run work-groups of 8 waves (256-row blocks), short ones of 4: the same rows, keys and order of a wave's
