@@ -44,6 +44,29 @@ def test_latent_decode_small(ops, T, H, R, pos0, qt):
         _close(orc.mla_decode_u(qf, cache, T, H, pos0, scale), ref, "the restatement itself")
 
 
+def _random_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(n):
+        T = int(rng.choice([1, 1, 2, 4, 7, 16]))
+        H = int(rng.choice([1, 8, 16, 20, 64, 128]))
+        R = int(rng.choice([64, 64, 0]))
+        pos0 = int(rng.choice([rng.integers(0, 40), rng.integers(40, 600), rng.integers(600, 5000)]))
+        out.append((T, H, R, pos0, int(rng.choice([F32, F16]))))
+    return out
+
+
+@pytest.mark.parametrize("T,H,R,pos0,qt", _random_cases(24, 20240609))
+def test_latent_decode_seeded_shapes(ops, T, H, R, pos0, qt):
+    n = pos0 + T
+    cache = orc.f2h(orc.randn(5 + pos0 % 3, (n, 512 + R), 0.5))
+    qa = orc.randn(6 + T, (T, H, 512 + R))
+    scale = 1.0 / np.sqrt(192.0)
+    qd, qf = (qa, qa) if qt == F32 else (orc.f2h(qa), orc.h2f(orc.f2h(qa)))
+    got = _latent(ops, qt, qd, cache, T, H, R, pos0, scale)
+    _close(got, orc.mla_f64(qf, cache, T, H, pos0, scale, 512, R), "latent decode vs float64 closed form")
+
+
 def test_config4_mla_decode_32k(ops):
     """BASELINE configs[3]: 128 heads, 512 latent + 64 rope, latent cache f16 ~N(0, 0.5), absorbed q of 576 a head,
     KV length 32768, scale 1/sqrt(192); output the 512-d latent a head, f16."""
