@@ -121,7 +121,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // wraps (a pass's keys span less than two rings). 32-bit arithmetic relative to the split's first key.
     const int64_t jb_slot = p.wrap && jb < je ? jb % p.cap : jb;
     const int span = (int) (je - jb) - 1;
-    auto row_off = [&](int rel) -> int64_t {
+    auto row_off = [&](int rel) __attribute__((always_inline)) -> int64_t {
         const int rc = std::min(std::max(rel, 0), span);
         int64_t slot = jb_slot + rc;
         if (p.wrap) {
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // the tile's keys into registers (MFMA A layout) and its values on their way: DMA into LDS buffer `buf`, chunk
     // position cp of key kk holding the row's chunk cp ^ 2 (kk % 8); or raw into registers
     // a listed block's tile: its 32 keys sit together in the cache (a block holds 4 tiles); no block: any valid rows
-    auto tile_off = [&](int64_t ti, int j0, int idx) -> int64_t {
+    auto tile_off = [&](int64_t ti, int j0, int idx) __attribute__((always_inline)) -> int64_t {
         if (!selp) return row_off(j0 + idx);
         const int blk = selp[(ti * TILE) >> 7];
         // (keys of a listed block past the row's position are masked: read the row's own key instead - the cache may end there)
@@ -143,10 +143,16 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // holds the row's 16-byte chunk cp ^ (kk % 16) (keys: the operand reads of 16 keys' same chunk meet no bank
     // conflict) or cp ^ 2 (kk % 8) (values: the transposing reads)
     // (a tile wholly inside the split of an unwrapped, unlisted cache - all but a pass's last - is read at a wave-uniform
-    // address plus per-lane offsets worked out once: FAST, where the registers allow)
-    constexpr bool FAST = DMA && D == 128;
-    uint32_t koff[FAST ? R::NLV : 1], voff[FAST ? R::NLV : 1];
-    if constexpr (FAST) {
+    // address plus a 32-bit lane offset: FAST. Rows of 128: the 8 offsets of a stream are worked out once and kept. Rows of
+    // 256 - 16 loads a stream, two keys a load - have no registers for that: key kk = kr0 + 2 i is i double-rows on from
+    // the tile's base (wave-uniform) plus the lane's own row kr0, and its swizzle splits the same way, since 2 i is even
+    // and kr0 one bit: cp ^ (kk % 16) = (cp ^ kr0) ^ (2 i % 16), cp ^ 2 (kk % 8) = (cp ^ 2 kr0) ^ (4 i % 16) - an
+    // exclusive-or with a constant and a shift-add a load)
+    constexpr bool FAST = DMA;
+    constexpr bool FAST_KEPT = DMA && R::NLV <= 8;
+    uint32_t koff[FAST_KEPT ? R::NLV : 1], voff[FAST_KEPT ? R::NLV : 1];
+    uint32_t lane_row = 0, cpk = 0, cpv = 0;
+    if constexpr (FAST_KEPT) {
         const int cp = lane % R::CPR, kr0 = lane / R::CPR;
 #pragma unroll
         for (int i = 0; i < R::NLV; ++i) {
@@ -154,16 +160,29 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             koff[i] = (uint32_t) (kk * p.row_stride) + (uint32_t) ((cp ^ (kk & 15)) * 16);
             voff[i] = (uint32_t) (kk * p.row_stride) + (uint32_t) ((cp ^ (2 * (kk & 7))) * 16);
         }
+    } else if constexpr (FAST) {
+        static_assert(!FAST || FAST_KEPT || R::KPI == 2, "the split of the swizzle assumes two keys a load");
+        const uint32_t cp = lane % R::CPR, kr0 = lane / R::CPR;
+        lane_row = kr0 * (uint32_t) p.row_stride;
+        cpk = cp ^ kr0;
+        cpv = cp ^ (2 * kr0);
     }
-    auto dma_tile = [&](int64_t ti, int which) {
+    auto dma_tile = [&](int64_t ti, int which) __attribute__((always_inline)) {
         const int j0 = (int) (ti * TILE - jb);                 // the tile's first key relative to the split's
         if constexpr (FAST) {
             if (!selp && !p.wrap && j0 >= 0 && j0 + TILE - 1 <= span) {
                 const uint8_t* base = (which ? vbase : kbase) + (jb_slot + j0) * p.row_stride;
 #pragma unroll
-                for (int i = 0; i < R::NLV; ++i)
-                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (base + (which ? voff[i] : koff[i])),
-                                                     (__attribute__((address_space(3))) void*) (stage + which * VTILE + i * 1024), 16, 0, NT_AUX);
+                for (int i = 0; i < R::NLV; ++i) {
+                    if constexpr (FAST_KEPT) {
+                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (base + (which ? voff[i] : koff[i])),
+                                                         (__attribute__((address_space(3))) void*) (stage + which * VTILE + i * 1024), 16, 0, NT_AUX);
+                    } else {
+                        const uint32_t off = lane_row + ((which ? cpv ^ (uint32_t) ((2 * R::KPI * i) & 14) : cpk ^ (uint32_t) ((R::KPI * i) & 15)) << 4);
+                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (base + (int64_t) (R::KPI * i) * p.row_stride + off),
+                                                         (__attribute__((address_space(3))) void*) (stage + which * VTILE + i * 1024), 16, 0, NT_AUX);
+                    }
+                }
                 return;
             }
         }
@@ -180,7 +199,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // quantized rows: the tile's keys (MFMA A layout) and values raw into registers
     // (interior tiles of an unwrapped, unlisted cache: a wave-uniform tile address plus a lane's row offset, worked out once)
     const uint32_t qk_lane = (uint32_t) (n * p.row_stride), qv_lane = (uint32_t) ((lane / R::CPR) * p.row_stride);
-    auto load_rows = [&](R& r, auto krow, auto vrow) {
+    auto load_rows = [&](R& r, auto krow, auto vrow) __attribute__((always_inline)) {
 #pragma unroll
         for (int kt2 = 0; kt2 < 2; ++kt2) {
             const uint8_t* kr = krow(kt2);
@@ -212,7 +231,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             if constexpr (KT == 2) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D / 2 + 2 * cp);
         }
     };
-    auto load_tile = [&](R& r, int64_t ti) {
+    auto load_tile = [&](R& r, int64_t ti) __attribute__((always_inline)) {
         const int j0 = (int) (ti * TILE - jb);
         if (!selp && !p.wrap && j0 >= 0 && j0 + TILE - 1 <= span) {
             const uint8_t* kt0 = kbase + (jb_slot + j0) * p.row_stride;
@@ -307,29 +326,9 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // that leaves one tile's NLV loads outstanding has seen everything older. MORE: the wave has a tile after this one
     // (at ti + WAVES), whose keys are requested as soon as this tile's have been read out of the key buffer and whose
     // values as soon as this tile's have been read out of the value buffer.
-    auto process_tile = [&](R& r, int64_t ti, auto more_c) {
+    auto process_tile = [&](R& r, int64_t ti, auto more_c) __attribute__((always_inline)) {
         constexpr bool more = decltype(more_c)::value;
         const int64_t j0 = ti * TILE;
-        s8v kall[2][KB];
-        if constexpr (DMA) {
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R::NLV) : "memory");           // V(i) may be out; K(i) is in
-#pragma unroll
-            for (int kt2 = 0; kt2 < 2; ++kt2)
-#pragma unroll
-                for (int kb = 0; kb < KB; ++kb)
-                    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kall[kt2][kb]) : "v"(k_rd[kb]), "n"(kt2 * 16 * RS));
-            // (every register the reads fill is named, so that no use of one moves above the wait)
-#pragma unroll
-            for (int kt2 = 0; kt2 < 2; ++kt2) {
-                if constexpr (KB == 4)
-                    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kall[kt2][0]), "+v"(kall[kt2][1]), "+v"(kall[kt2][2]), "+v"(kall[kt2][3])::"memory");
-                else
-                    asm volatile("s_waitcnt lgkmcnt(0)"
-                                 : "+v"(kall[kt2][0]), "+v"(kall[kt2][1]), "+v"(kall[kt2][2]), "+v"(kall[kt2][3]), "+v"(kall[kt2][4]),
-                                   "+v"(kall[kt2][5]), "+v"(kall[kt2][6]), "+v"(kall[kt2][7])::"memory");
-            }
-            if constexpr (more) dma_tile(ti + WAVES, 0);
-        }
         if constexpr (!DMA) {
             // ---- the value tile dequantized into this wave's LDS stage, [key][D] halfs
             const int c = lane % R::CPR, kr0 = lane / R::CPR;
@@ -349,16 +348,50 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                 }
             }
         }
-        // ---- S^T = K Q^T for both 16-key tiles and every row tile
+        // ---- S^T = K Q^T for both 16-key tiles and every row tile. 16-bit rows: the key operands come out of the key
+        // buffer - both 16-key halves at once at D = 128, a half at a time at D = 256 (32 registers instead of 64) - and
+        // the next tile's keys are requested as soon as the last of them has been read
         f4v s[RT][2];
+        if constexpr (DMA) {
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R::NLV) : "memory");           // V(i) may be out; K(i) is in
+            constexpr int KH = D == 128 ? 2 : 1;
 #pragma unroll
-        for (int kt2 = 0; kt2 < 2; ++kt2) {
-            s8v ka[KB];
+            for (int h0 = 0; h0 < 2; h0 += KH) {
+                s8v kall[KH][KB];
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb) {
-                if constexpr (DMA) {
-                    ka[kb] = kall[kt2][kb];
-                } else {
+                for (int kt2 = 0; kt2 < KH; ++kt2)
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb)
+                        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(kall[kt2][kb]) : "v"(k_rd[kb]), "n"((h0 + kt2) * 16 * RS));
+                // (every register the reads fill is named, so that no use of one moves above the wait)
+#pragma unroll
+                for (int kt2 = 0; kt2 < KH; ++kt2) {
+                    if constexpr (KB == 4)
+                        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(kall[kt2][0]), "+v"(kall[kt2][1]), "+v"(kall[kt2][2]), "+v"(kall[kt2][3])::"memory");
+                    else
+                        asm volatile("s_waitcnt lgkmcnt(0)"
+                                     : "+v"(kall[kt2][0]), "+v"(kall[kt2][1]), "+v"(kall[kt2][2]), "+v"(kall[kt2][3]), "+v"(kall[kt2][4]),
+                                       "+v"(kall[kt2][5]), "+v"(kall[kt2][6]), "+v"(kall[kt2][7])::"memory");
+                }
+                if constexpr (more) {
+                    if (h0 + KH == 2) dma_tile(ti + WAVES, 0);
+                }
+#pragma unroll
+                for (int kt2 = 0; kt2 < KH; ++kt2)
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt) {
+                        f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                        for (int kb = 0; kb < KB; ++kb) acc = mfma16<BF>(kall[kt2][kb], qreg[rt][kb], acc);
+                        s[rt][h0 + kt2] = acc;
+                    }
+            }
+        } else {
+#pragma unroll
+            for (int kt2 = 0; kt2 < 2; ++kt2) {
+                s8v ka[KB];
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
                     const _Float16 d = __builtin_bit_cast(_Float16, (uint16_t) r.ksc[kt2][kb]);
                     if constexpr (KT == 1) {
                         ka[kb] = dq8x8(r.k[kt2][kb][0], r.k[kt2][kb][1], d);
@@ -366,13 +399,13 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                         ka[kb] = dq4x8(r.k[kt2][kb][0], r.k[kt2][kb][1], g4 >= 2 ? 4 : 0, d);
                     }
                 }
-            }
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) {
-                f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+                for (int rt = 0; rt < RT; ++rt) {
+                    f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int kb = 0; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
-                s[rt][kt2] = acc;
+                    for (int kb = 0; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
+                    s[rt][kt2] = acc;
+                }
             }
         }
         // ---- online softmax a row (this lane: row n of each row tile, keys j0 + 16 kt2 + 4 g4 + i)
@@ -449,9 +482,9 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         }
         const int kk = g4 * 4 + (n >> 2);                      // the key row this lane's address names (and + 16)
-        constexpr int HALF = DT / 2;
+        constexpr int HALF = D == 128 ? DT / 2 : DT / 4;       // column tiles whose reads are in flight together
 #pragma unroll
-        for (int h2 = 0; h2 < 2; ++h2) {
+        for (int h2 = 0; h2 < DT / HALF; ++h2) {
             s4v lo[HALF], hi[HALF];
 #pragma unroll
             for (int d2 = 0; d2 < HALF; ++d2) {
