@@ -62,11 +62,12 @@ def test_prefill_seeded_shapes(ops, T, Hq, Hkv, D, p0, win, kt, qt):
     check_close(got, ref, qt, "prefill vs float64 closed form", kt=kt)
 
 
-@pytest.mark.parametrize("T,Hq,Hkv,p0,win,kt,qt", [(700, 10, 2, 300, 0, 3, BF16), (513, 4, 1, 0, 400, 0, F32)])
-def test_prefill_work_groups_of_8_waves(ops, monkeypatch, T, Hq, Hkv, p0, win, kt, qt):
-    """Long passes run work-groups of 8 waves (256-row blocks), short ones of 4: the same rows, keys and order of a wave's
-    arithmetic, so the two agree bit for bit; forced here on a shape the oracle finishes in seconds."""
-    D = 128
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0,win,kt,qt", [(700, 10, 2, 128, 300, 0, 3, BF16), (513, 4, 1, 128, 0, 400, 0, F32),
+                                                     (300, 8, 2, 256, 100, 0, 3, BF16), (260, 4, 1, 256, 0, 200, 0, F32)])
+def test_prefill_work_groups_of_8_waves(ops, monkeypatch, T, Hq, Hkv, D, p0, win, kt, qt):
+    """Long passes run work-groups of 8 waves (blocks of 256 rows; 128 at head size 256), short ones of 4: the same rows,
+    keys and order of a wave's arithmetic, so the two agree bit for bit; forced here on shapes the oracle finishes in
+    seconds."""
     cap = p0 + T + 5
     kc, vc = make_kv(kt, Hkv, D, cap, p0 + T)
     qd, qf = make_q(qt, T, Hq, D)
