@@ -668,18 +668,20 @@ __global__ __launch_bounds__(MERGE_W * 64) void attn_merge_kernel(const float* _
 
 // ---- host side ----------------------------------------------------------------------------------------------------
 
-// work-groups the key splits aim for (key heads x splits); NS_DEC_WGS overrides (tuning)
-int64_t target_wgs() {
+// work-groups the key splits aim for (key heads x splits): two a CU at head size 128, one at 256 (its LDS footprint admits
+// one a CU; 256 against 512 measured 17.6 against 23.2 us at 32K keys, and half the partials to merge); NS_DEC_WGS
+// overrides (tuning)
+int64_t target_wgs(int64_t D) {
     static const int64_t v = [] {
         const char* e = getenv("NS_DEC_WGS");
         const int64_t x = e ? atoll(e) : 0;
-        return x > 0 ? x : 512;
+        return x > 0 ? x : 0;
     }();
-    return v;
+    return v > 0 ? v : D == 256 ? 256 : 512;
 }
 // keys a split for a row that sees `keys` keys: a multiple of 128 (4 waves x 32-key tiles)
-int64_t dec_kbs(int64_t keys, int64_t Hkv) {
-    const int64_t t = target_wgs(), want = (keys * Hkv + t - 1) / t;
+int64_t dec_kbs(int64_t keys, int64_t Hkv, int64_t D) {
+    const int64_t t = target_wgs(D), want = (keys * Hkv + t - 1) / t;
     return std::max<int64_t>(128, (want + 127) / 128 * 128);
 }
 inline int64_t row_first(int64_t pos, int64_t win) { return win > 0 ? std::max<int64_t>(0, pos - win + 1) : 0; }
@@ -741,7 +743,7 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
     const int64_t last = p0 + T - 1;
     auto kb_of = [&](int64_t r) {
         const int64_t pos = causal ? p0 + r : last;
-        return dec_kbs(pos + 1 - row_first(p0 + r, win), Hkv);
+        return dec_kbs(pos + 1 - row_first(p0 + r, win), Hkv, D);
     };
     bool same = true;
     for (int64_t r = 1; r < T; ++r) same = same && kb_of(r) == kb_of(0);
@@ -822,7 +824,7 @@ int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_
     if ((uintptr_t) q % 16 || ((uintptr_t) kc | (uintptr_t) vc) % 16) return ns_fail(w + ": rows 16-byte aligned");
     NS_HIP(hipSetDevice(g->dev));
     if (K == 0) return ns_fill(g, out, 0, (size_t) (T * Hq * D) * sizeof(float));     // nothing listed: zeros (l = 0)
-    const int64_t keys = K * 128, kbs = dec_kbs(keys, Hkv), ns = (keys + kbs - 1) / kbs;
+    const int64_t keys = K * 128, kbs = dec_kbs(keys, Hkv, D), ns = (keys + kbs - 1) / kbs;
     if ((size_t) (Hq * ns * (D + 2)) > scratch_floats) return ns_fail(w + ": the pass needs more scratch than the library keeps");
     DecodeParams p{};
     p.qt = 0;
@@ -870,14 +872,14 @@ int64_t ns_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, in
     int64_t ns = 1;
     // a row launched alone: its own split size over its own keys
     for (int64_t r = 0; r < T; ++r) {
-        const int64_t pos = p0 + r, first = row_first(pos, win), kb = dec_kbs(pos + 1 - first, Hkv);
+        const int64_t pos = p0 + r, first = row_first(pos, win), kb = dec_kbs(pos + 1 - first, Hkv, D);
         ns = std::max(ns, pos / kb - first / kb + 1);
     }
     // the pass in one launch: from its first row's first key to its last row's last; causal or not, the last row's
     // key count bounds every row's
     const int64_t f0 = row_first(p0, win), last = p0 + T - 1;
     for (int64_t r = 0; r < T; ++r) {
-        const int64_t kb = dec_kbs(last + 1 - row_first(p0 + r, win), Hkv), kb2 = dec_kbs(p0 + r + 1 - row_first(p0 + r, win), Hkv);
+        const int64_t kb = dec_kbs(last + 1 - row_first(p0 + r, win), Hkv, D), kb2 = dec_kbs(p0 + r + 1 - row_first(p0 + r, win), Hkv, D);
         ns = std::max(ns, last / kb - f0 / kb + 1);
         ns = std::max(ns, last / kb2 - f0 / kb2 + 1);
     }
