@@ -80,6 +80,32 @@ __device__ __forceinline__ float rows_sum(float v) {
     return a + b;
 }
 
+// Reductions over all 64 lanes without LDS: lane pairs inside a row of 16 through DPP (quad permutes, then the mirror
+// of 8 and of 16 lanes, which pair the two halves as well as an exclusive-or would), rows through the permlane swaps.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+    return (uint32_t) __builtin_amdgcn_update_dpp(0, (int) v, CTRL, 0xF, 0xF, true);
+}
+template <typename F>
+__device__ __forceinline__ uint32_t wave_reduce_u32(uint32_t v, F f) {
+    v = f(v, dpp_u32<0xB1>(v));        // quad_perm [1, 0, 3, 2]
+    v = f(v, dpp_u32<0x4E>(v));        // quad_perm [2, 3, 0, 1]
+    v = f(v, dpp_u32<0x141>(v));       // row_half_mirror
+    v = f(v, dpp_u32<0x140>(v));       // row_mirror
+    auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    v = f((uint32_t) r[0], (uint32_t) r[1]);
+    r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return f((uint32_t) r[0], (uint32_t) r[1]);
+}
+__device__ __forceinline__ float wave_max(float v) {
+    return __builtin_bit_cast(float, wave_reduce_u32(__builtin_bit_cast(uint32_t, v), [](uint32_t a, uint32_t b) {
+        return __builtin_bit_cast(uint32_t, fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b)));
+    }));
+}
+__device__ __forceinline__ int wave_min(int v) {
+    return (int) wave_reduce_u32((uint32_t) v, [](uint32_t a, uint32_t b) { return (uint32_t) min((int) a, (int) b); });
+}
+
 // element i of a row of query / output type QT (0 float32, 1 half, 2 bfloat16)
 template <int QT>
 __device__ __forceinline__ float load_q(const void* p, int64_t i) {

@@ -8,47 +8,61 @@
 #include "ns_internal.hpp"
 #include "ns_attn.h"
 #include "kv_formats.hpp"
+#include "attn_common.hpp"
 
+#include <algorithm>
 #include <cmath>
 
 namespace {
 
 constexpr int BLK = 128;
 
-// one work-group of 128 threads a (row, head, block): a thread a key, the dot product in feature order
-__global__ __launch_bounds__(BLK) void idx_scores_kernel(const float* __restrict__ iq, const uint16_t* __restrict__ ik, float* __restrict__ bs, int64_t G,
-                                                         int64_t nblk, int64_t pos0, int64_t local) {
-    __shared__ float qs[BLK];
-    __shared__ float red[2];
-    const int64_t grp = blockIdx.x;
+// one work-group of 128 threads a block of 128 keys: a thread holds its key's row (read once, whatever the number of
+// rows and heads) and takes its dot product - in feature order - with every (row, head) query in turn; the block's best
+// a query is reduced over the two waves
+constexpr int QCH = 16;     // queries staged in LDS at a time
+
+__global__ __launch_bounds__(BLK) void idx_scores_kernel(const float* __restrict__ iq, const uint16_t* __restrict__ ik, float* __restrict__ bs, int64_t TG,
+                                                         int64_t G, int64_t nblk, int64_t pos0, int64_t local) {
+    __shared__ float qs[QCH][BLK];
+    __shared__ float red[QCH][2];
+    const int64_t b = blockIdx.x;
     const int lid = threadIdx.x;
-    const int64_t b = grp % nblk, tg = grp / nblk, t = tg / G;
-    const int64_t pos = pos0 + t;
-    qs[lid] = iq[tg * BLK + lid];
-    __syncthreads();
-    float v = -INFINITY;
-    const int64_t j = b * BLK + lid;
-    if (j <= pos) {
-        const uint4* kr = reinterpret_cast<const uint4*>(ik + j * BLK);
-        float s = 0.0f;
-#pragma unroll 4
+    const int64_t j = b * BLK + lid, last = pos0 + (TG - 1) / G;      // the pass's last row sees the most keys
+    float kf[BLK];              // the key's row widened once: 128 registers
+    {
+        uint4 row[BLK / 8];
+        const uint4* kr = reinterpret_cast<const uint4*>(ik + std::min(j, last) * BLK);
+#pragma unroll
+        for (int c = 0; c < BLK / 8; ++c) row[c] = kr[c];
+#pragma unroll
         for (int c = 0; c < BLK / 8; ++c) {
-            const uint4 x = kr[c];
-            const uint32_t ww[4] = {x.x, x.y, x.z, x.w};
+            const uint32_t ww[4] = {row[c].x, row[c].y, row[c].z, row[c].w};
 #pragma unroll
-            for (int e = 0; e < 8; ++e) s += qs[c * 8 + e] * f16_to_f32((uint16_t) (ww[e >> 1] >> (16 * (e & 1))));
+            for (int e = 0; e < 8; ++e) kf[c * 8 + e] = f16_to_f32((uint16_t) (ww[e >> 1] >> (16 * (e & 1))));
         }
-        v = s;
     }
+    for (int64_t q0 = 0; q0 < TG; q0 += QCH) {
+        const int nq = (int) std::min<int64_t>(QCH, TG - q0);
+        __syncthreads();
+        for (int i = 0; i < nq; ++i) qs[i][lid] = iq[(q0 + i) * BLK + lid];
+        __syncthreads();
+        for (int i = 0; i < nq; ++i) {
+            const int64_t pos = pos0 + (q0 + i) / G;
+            float s = 0.0f;
 #pragma unroll
-    for (int o = 1; o < 64; o <<= 1) v = fmaxf(v, __shfl_xor(v, o));
-    if ((lid & 63) == 0) red[lid >> 6] = v;
-    __syncthreads();
-    if (lid == 0) {
-        float m = fmaxf(red[0], red[1]);
-        if (b * BLK > pos) m = -INFINITY;
-        else if (b + local > pos / BLK) m = m + 1e30f;
-        bs[grp] = m;
+            for (int d = 0; d < BLK; ++d) s += qs[i][d] * kf[d];
+            const float v = wave_max(j <= pos ? s : -INFINITY);
+            if ((lid & 63) == 0) red[i][lid >> 6] = v;
+        }
+        __syncthreads();
+        if (lid < nq) {
+            const int64_t pos = pos0 + (q0 + lid) / G;
+            float m = fmaxf(red[lid][0], red[lid][1]);
+            if (b * BLK > pos) m = -INFINITY;
+            else if (b + local > pos / BLK) m = m + 1e30f;
+            bs[(q0 + lid) * nblk + b] = m;
+        }
     }
 }
 
@@ -77,6 +91,40 @@ __global__ __launch_bounds__(64) void idx_topk_kernel(float* __restrict__ bs, in
     }
 }
 
+// the same selection with the row's scores held in registers (VPL a lane: rows of up to 64 VPL blocks): a round is a
+// few compares and two wave reductions instead of two passes over the row in memory and a fence. The chosen blocks'
+// scores are overwritten with -inf in memory too, as the kernel above leaves them.
+template <int VPL>
+__global__ __launch_bounds__(64) void idx_topk_reg_kernel(float* __restrict__ bs, int32_t* __restrict__ sel, int nblk, int K) {
+    const int64_t row = blockIdx.x;
+    const int lane = threadIdx.x;
+    float* s = bs + row * nblk;
+    float v[VPL];
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) v[j] = lane + 64 * j < nblk ? s[lane + 64 * j] : -INFINITY;
+    for (int k = 0; k < K; ++k) {
+        float best = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) best = fmaxf(best, v[j]);
+        best = wave_max(best);
+        int at = 0x7fffffff;
+        if (best > -INFINITY) {
+#pragma unroll
+            for (int j = VPL - 1; j >= 0; --j) at = v[j] == best ? lane + 64 * j : at;     // this lane's lowest index of it
+        }
+        at = wave_min(at);
+        if (best > -INFINITY) {
+#pragma unroll
+            for (int j = 0; j < VPL; ++j)
+                if (lane + 64 * j == at) {
+                    v[j] = -INFINITY;
+                    s[at] = -INFINITY;
+                }
+        }
+        if (lane == 0) sel[row * K + k] = best > -INFINITY ? at : -1;
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -88,7 +136,7 @@ int ns_llm_minimaxm3_idx_scores(ns_gpu* g, const float* iq, const uint16_t* ik, 
     if ((uintptr_t) ik % 16) return ns_fail("ns_llm_minimaxm3_idx_scores: key rows 16-byte aligned");
     if (T * G * nblk > (int64_t) 1 << 31) return ns_fail("ns_llm_minimaxm3_idx_scores: too many blocks");
     NS_HIP(hipSetDevice(g->dev));
-    idx_scores_kernel<<<(unsigned) (T * G * nblk), BLK, 0, g->q>>>(iq, ik, bs, G, nblk, pos0, local);
+    idx_scores_kernel<<<(unsigned) nblk, BLK, 0, g->q>>>(iq, ik, bs, T * G, G, nblk, pos0, local);
     NS_LAUNCHED("idx_scores");
     return 0;
     NS_CATCH
@@ -100,7 +148,12 @@ int ns_llm_minimaxm3_idx_topk(ns_gpu* g, float* bs, int32_t* sel, int64_t T, int
     if (nblk < 0) return ns_fail("ns_llm_minimaxm3_idx_topk: a block count");
     if (!bs || !sel) return ns_fail("ns_llm_minimaxm3_idx_topk: a null buffer");
     NS_HIP(hipSetDevice(g->dev));
-    idx_topk_kernel<<<(unsigned) (T * G), 64, 0, g->q>>>(bs, sel, nblk, K);
+    const unsigned rows = (unsigned) (T * G);
+    if (K > (int64_t) 1 << 30) return ns_fail("ns_llm_minimaxm3_idx_topk: a list length");
+    if (nblk <= 64 * 8) idx_topk_reg_kernel<8><<<rows, 64, 0, g->q>>>(bs, sel, (int) nblk, (int) K);
+    else if (nblk <= 64 * 32) idx_topk_reg_kernel<32><<<rows, 64, 0, g->q>>>(bs, sel, (int) nblk, (int) K);
+    else if (nblk <= 64 * 128) idx_topk_reg_kernel<128><<<rows, 64, 0, g->q>>>(bs, sel, (int) nblk, (int) K);
+    else idx_topk_kernel<<<rows, 64, 0, g->q>>>(bs, sel, nblk, K);
     NS_LAUNCHED("idx_topk");
     return 0;
     NS_CATCH

@@ -70,6 +70,24 @@ def test_minimaxm3_indexer(ops):
     assert s2.read(np.int32).tolist() == [1, 2, 5, 4, 0, -1]
 
 
+@pytest.mark.parametrize("nblk,K", [(5, 8), (512, 16), (513, 16), (2048, 40), (2049, 3), (8192, 16), (8193, 5), (70, 70)])
+def test_minimaxm3_topk_row_lengths(ops, nblk, K):
+    """Every row length the selection has a kernel for (scores in 8, 32 or 128 registers a lane, or left in memory),
+    on scores with ties, holes and boosted blocks: the lists and the scores left behind, bit for bit."""
+    g = ops.gpu
+    T, G = 2, 3
+    rng = np.random.default_rng(nblk * 31 + K)
+    sc = rng.integers(-50, 50, (T, G, nblk)).astype(np.float32) / 4            # many equal scores
+    sc[rng.random((T, G, nblk)) < 0.2] = -np.inf
+    sc[0, 0, : min(3, nblk)] += 1e30
+    sc[1, 2] = -np.inf                                                         # a row with nothing to choose
+    bs, sel = DevBuf.of(g, sc), DevBuf(g, T * G * K * 4)
+    ops.minimaxm3_idx_topk(bs, sel, T, G, nblk, K)
+    want_sel, want_left = orc.mm3_idx_topk(sc, K)
+    assert np.array_equal(sel.read(np.int32).reshape(T, G, K), want_sel)
+    assert np.array_equal(bs.read(np.float32).reshape(T, G, nblk).view(np.uint32), want_left.view(np.uint32))
+
+
 @pytest.mark.parametrize("q8", [False, True])
 @pytest.mark.parametrize("T,H,pos0,K", [(1, 128, 5000, 64), (3, 64, 2500, 512), (2, 160, 900, 16)])
 def test_glm_cell_pools(ops, q8, T, H, pos0, K):
