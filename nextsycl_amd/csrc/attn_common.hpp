@@ -102,6 +102,20 @@ __device__ __forceinline__ float wave_max(float v) {
         return __builtin_bit_cast(uint32_t, fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b)));
     }));
 }
+__device__ __forceinline__ float wave_sum(float v) {
+    return __builtin_bit_cast(float, wave_reduce_u32(__builtin_bit_cast(uint32_t, v), [](uint32_t a, uint32_t b) {
+        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b));
+    }));
+}
+// the sum over each row of 16 lanes, in every lane of the row
+__device__ __forceinline__ float row16_sum(float v) {
+    auto f = [](float x) { return __builtin_bit_cast(uint32_t, x); };
+    auto g = [](uint32_t x) { return __builtin_bit_cast(float, x); };
+    v += g(dpp_u32<0xB1>(f(v)));
+    v += g(dpp_u32<0x4E>(f(v)));
+    v += g(dpp_u32<0x141>(f(v)));
+    return v + g(dpp_u32<0x140>(f(v)));
+}
 __device__ __forceinline__ int wave_min(int v) {
     return (int) wave_reduce_u32((uint32_t) v, [](uint32_t a, uint32_t b) { return (uint32_t) min((int) a, (int) b); });
 }

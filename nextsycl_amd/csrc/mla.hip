@@ -473,32 +473,36 @@ __global__ __launch_bounds__(256) void mla_merge_kernel(const float* __restrict_
     }
 }
 
-// q~ = k_b q_nope: qa [T][H][L + R] = [k_b[h] q[t][h][:nope] | q[t][h][nope:]]; a work-group a (row, head), a thread two
-// latent rows of k_b (kernels/llm/deepseek2/ds2.cpp:176-184)
+// q~ = k_b q_nope: qa [T][H][L + R] = [k_b[h] q[t][h][:nope] | q[t][h][nope:]]; four work-groups a (row, head), a wave 32
+// latent rows of k_b four at a time (all 8 loads requested before the first is used): 16 lanes a row (16 bytes each: the wave's load is 1 KiB of consecutive memory), a
+// lane's 8 products summed in feature order, the 16 partial sums through DPP (kernels/llm/deepseek2/ds2.cpp:176-184)
 __global__ __launch_bounds__(256) void mla_absorb_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kb, float* __restrict__ qa,
                                                          int64_t H) {
     constexpr int NOPE = 128, R = 64;
-    __shared__ float qs[NOPE + R];
     const int64_t th = blockIdx.x, h = th % H;
-    const int tid = threadIdx.x;
-    if (tid < NOPE + R) qs[tid] = q[th * (NOPE + R) + tid];
-    __syncthreads();
-    for (int r = tid; r < ML; r += 256) {
-        const uint4* wr = reinterpret_cast<const uint4*>(kb + ((size_t) h * ML + r) * NOPE);
+    const int part = blockIdx.y;                                   // a quarter of the latent rows a work-group
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6, sub = lane & 15, rsel = lane >> 4;
+    float qv[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) qv[e] = q[th * (NOPE + R) + sub * 8 + e];
+    const int r0 = part * 128 + w * 32 + rsel;
+    const uint16_t* wbase = kb + ((size_t) h * ML + r0) * NOPE + sub * 8;
+    uint4 x[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) x[it] = *reinterpret_cast<const uint4*>(wbase + (size_t) it * 4 * NOPE);     // all in flight at once
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+        const uint32_t ww[4] = {x[it].x, x[it].y, x[it].z, x[it].w};
         float a = 0.0f;
 #pragma unroll
-        for (int c = 0; c < NOPE / 8; ++c) {
-            const uint4 x = wr[c];
-            const uint32_t ww[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-            for (int e = 0; e < 8; ++e) a += f16_to_f32((uint16_t) (ww[e >> 1] >> (16 * (e & 1)))) * qs[c * 8 + e];
-        }
-        qa[th * (ML + R) + r] = a;
+        for (int e = 0; e < 8; ++e) a += f16_to_f32((uint16_t) (ww[e >> 1] >> (16 * (e & 1)))) * qv[e];
+        a = row16_sum(a);
+        if (sub == 0) qa[th * (ML + R) + r0 + it * 4] = a;
     }
-    if (tid < R) qa[th * (ML + R) + ML + tid] = qs[NOPE + tid];
+    if (part == 0 && tid < R) qa[th * (ML + R) + ML + tid] = q[th * (NOPE + R) + NOPE + tid];
 }
 
-// out [T][H][V] = v_b u: a work-group a (row, head), a wave a value row at a time (kernels/llm/deepseek2/ds2.cpp:237-255)
+// out [T][H][V] = v_b u: four work-groups a (row, head), a wave a value row at a time (kernels/llm/deepseek2/ds2.cpp:237-255)
 __global__ __launch_bounds__(256) void mla_vb_kernel(const float* __restrict__ u, const uint16_t* __restrict__ vb, float* __restrict__ out,
                                                      int64_t H) {
     constexpr int V = 128;
@@ -507,15 +511,22 @@ __global__ __launch_bounds__(256) void mla_vb_kernel(const float* __restrict__ u
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     for (int i = tid; i < ML; i += 256) us[i] = u[th * ML + i];
     __syncthreads();
-    for (int r = w; r < V; r += 4) {
-        const uint4 x = reinterpret_cast<const uint4*>(vb + ((size_t) h * V + r) * ML)[lane];
-        const uint32_t ww[4] = {x.x, x.y, x.z, x.w};
+    // a quarter of the value rows a work-group, 8 a wave: their loads all requested before the first is used
+    const int r0 = blockIdx.y * 32 + w * 8;
+    uint4 x[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = reinterpret_cast<const uint4*>(vb + ((size_t) h * V + r0 + i) * ML)[lane];
+    float uv[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) uv[e] = us[lane * 8 + e];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t ww[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
         float a = 0.0f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) a += f16_to_f32((uint16_t) (ww[e >> 1] >> (16 * (e & 1)))) * us[lane * 8 + e];
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) a += __shfl_xor(a, o);
-        if (lane == 0) out[th * V + r] = a;
+        for (int e = 0; e < 8; ++e) a += f16_to_f32((uint16_t) (ww[e >> 1] >> (16 * (e & 1)))) * uv[e];
+        a = wave_sum(a);
+        if (lane == 0) out[th * V + r0 + i] = a;
     }
 }
 
@@ -714,10 +725,10 @@ int ns_ds2_mla_decode(ns_gpu* g, const float* q, const uint16_t* kb, const uint1
     float* u = qa + qa_f;
     float* part = u + u_f;
     NS_HIP(hipSetDevice(g->dev));
-    mla_absorb_kernel<<<(unsigned) rows, 256, 0, g->q>>>(q, kb, qa, H);
+    mla_absorb_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(q, kb, qa, H);
     NS_LAUNCHED("mla_absorb");
     if (mla_latent(g, "ns_ds2_mla_decode", 0, 0, 64, false, qa, cache, u, T, H, pos0, scale, part, g->own_scratch_floats - qa_f - u_f)) return -1;
-    mla_vb_kernel<<<(unsigned) rows, 256, 0, g->q>>>(u, vb, out, H);
+    mla_vb_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(u, vb, out, H);
     NS_LAUNCHED("mla_vb");
     return 0;
     NS_CATCH
