@@ -599,8 +599,7 @@ __global__ __launch_bounds__(MERGE_W * 64) void attn_merge_kernel(const float* _
         for (int c = 0; c < C; ++c) x[j][c] = *reinterpret_cast<const float2*>(pr + (int64_t) std::min(k + MERGE_W * j, ns - 1) * PS + 2 * (lane + 64 * c));
     float mx = -INFINITY;
     for (int s = lane; s < ns; s += 64) mx = fmaxf(mx, pr[(int64_t) s * PS + D]);
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    mx = wave_max(mx);
     // this wave's splits: nk of them, walked in batches of B after the first PF (slots past the last hold weight 0)
     const int nk = ns > k ? (ns - k + MERGE_W - 1) / MERGE_W : 0;
     const int njp = std::max(PF, (nk + B - 1) / B * B), nsz = MERGE_W * njp;
@@ -615,8 +614,7 @@ __global__ __launch_bounds__(MERGE_W * 64) void attn_merge_kernel(const float* _
         }
         wk[s] = wgt;
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) ls += __shfl_xor(ls, o);
+    ls = wave_sum(ls);
     // wk was written by this wave's own lanes: a wave's LDS operations complete in order
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
