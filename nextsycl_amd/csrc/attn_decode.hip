@@ -856,6 +856,12 @@ int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_
     NS_CATCH
 }
 
+// the merge of [rows][ns][D + 2] partials for the prompt kernel's key splits (the same kernel, the same layout)
+int ns_attn_merge_partials(ns_gpu* g, int64_t D, const float* part, int64_t ns, int qt, int64_t rows, void* out) {
+    if (ns > MERGE_MAX_NS) return ns_fail("ns_attn_prompt: more key splits than the merge holds");
+    return D == 128 ? launch_merge<128>(g, part, (int) ns, qt, rows, out) : launch_merge<256>(g, part, (int) ns, qt, rows, out);
+}
+
 // used by the exact-API routing in attn_api.cpp
 int ns_attn_decode_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T,
                        int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, int causal, float scale, void* out,

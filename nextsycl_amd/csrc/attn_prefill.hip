@@ -32,6 +32,9 @@
 #include <cstdlib>
 #include <type_traits>
 
+// attn_decode.hip: the merge of [rows][ns][D + 2] partials
+int ns_attn_merge_partials(ns_gpu* g, int64_t D, const float* part, int64_t ns, int qt, int64_t rows, void* out);
+
 namespace {
 
 constexpr int KT_TILE = 64;
@@ -52,6 +55,11 @@ struct PrefillParams {
     int64_t p0, win;
     float sl2;
     void* out;
+    // key splits (passes of few row blocks over many keys): work-group (x, y) takes the keys [k0 + y kbs, k0 + (y + 1) kbs)
+    // of its rows' own ranges and leaves a partial {O, m, l} a (row, head, split) for the decode path's merge kernel
+    int ns;
+    int64_t kbs, k0;
+    float* part;                // [T][Hq][ns][D + 2]
 };
 
 // a 16-byte chunk of a K or V row on its way from global memory to LDS (a plain vector type: arrays of it stay in registers)
@@ -87,8 +95,14 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     const int blk = nblk - 1 - unit / Hkv;
     const int r0 = blk * ROWS;
     const int rl = std::min(r0 + ROWS, p.T) - 1;                  // the block's last row
-    const int64_t kend = p.p0 + rl + 1;                           // keys [kbeg, kend) cover every row of the block
-    const int64_t kbeg = p.win > 0 ? std::max<int64_t>(0, p.p0 + r0 + 1 - p.win) : 0;
+    // keys [kbeg, kend) cover every row of the block; with key splits, the part of them in this work-group's split
+    const int split = blockIdx.y;
+    int64_t kend = p.p0 + rl + 1;
+    int64_t kbeg = p.win > 0 ? std::max<int64_t>(0, p.p0 + r0 + 1 - p.win) : 0;
+    if (p.ns > 1) {
+        kbeg = std::max(kbeg, p.k0 + split * p.kbs);
+        kend = std::max(kbeg, std::min(kend, p.k0 + (split + 1) * p.kbs));      // (none: an empty range at kbeg)
+    }
 
     // ---- this lane's two rows: positions, key ranges, Q^T operands. The queries carry the softmax scale (x log2 e) into
     // the 16-bit operand, so that the score product comes out in exponent units and needs no multiplication a score
@@ -100,8 +114,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         const bool live = row < p.T;
         const int rr = live ? row : p.T - 1;
         const int64_t pos = p.p0 + rr;
-        lo_r[rt] = live ? (p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0) : 1;
-        hi_r[rt] = live ? pos : 0;
+        lo_r[rt] = live ? std::max(kbeg, p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0) : 1;
+        hi_r[rt] = live ? std::min(pos, kend - 1) : 0;
         const int64_t qoff = (int64_t) rr * p.qs + (int64_t) hq * D + g4 * 8;
         if (p.qt == 0) {
             float4 raw[KB][2];
@@ -134,7 +148,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
     const uint8_t* vbase = p.vc + (int64_t) hk * p.head_stride;
     const int64_t t0 = kbeg / KT_TILE, t1 = (kend + KT_TILE - 1) / KT_TILE;
-    const int nt = (int) (t1 - t0);
+    const int nt = kend > kbeg ? (int) (t1 - t0) : 0;             // (a split past the block's last key: nothing to do)
     // From here on keys are counted from the first tile's first key (32-bit): tile k holds keys 64 k .. 64 k + 63, step
     // s = 2 k + h its 32-key half h
     const int64_t base = t0 * KT_TILE;
@@ -414,6 +428,33 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // ---- out = O / l. A lane holds dims 16 dt + 4 g4 .. + 3 of its rows: the wave's 32 x D block goes through LDS (the
     // tile buffers, free now) so that it leaves as whole rows, 16 bytes a lane and 4 (float32: 2) rows an instruction
     __syncthreads();                                              // every wave is done with the tiles
+    if (p.ns > 1) {
+        // ---- a key split's partial: the rows' unnormalized sums as float32, then (m, l) - D + 2 floats a (row, head, split),
+        // rows 8 bytes aligned: 8-byte pieces, 8 rows an instruction
+        const uint32_t rowp = D * 4 + 16;
+        const uint32_t ob = (uint32_t) w * 16 * rowp;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) {
+            const float lsum = rows_sum(l_r[rt]);
+            const uint32_t at = ob + (uint32_t) n * rowp + (uint32_t) (g4 * 16);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<__attribute__((address_space(3))) f4v*>(L + at + dt * 64) = o[rt][dt];
+            const int row = r0 + w * WROWS + rt * 16 + n;
+            if (g4 == 0 && row < p.T) {
+                float* pr = p.part + (((int64_t) row * p.Hq + hq) * p.ns + split) * (D + 2);
+                *reinterpret_cast<float2*>(pr + D) = float2{thr[rt] < 0.0f ? -INFINITY : -nbr[rt], lsum};
+            }
+            for (int c = lane; c < 16 * (D / 2); c += 64) {
+                const int rl_ = c / (D / 2), piece = c % (D / 2), prow = r0 + w * WROWS + rt * 16 + rl_;
+                if (prow < p.T) {
+                    typedef uint32_t u2v __attribute__((ext_vector_type(2)));
+                    const u2v x = *reinterpret_cast<const __attribute__((address_space(3))) u2v*>(L + ob + (uint32_t) rl_ * rowp + (uint32_t) piece * 8);
+                    *reinterpret_cast<u2v*>(p.part + (((int64_t) prow * p.Hq + hq) * p.ns + split) * (D + 2) + piece * 2) = x;
+                }
+            }
+        }
+        return;
+    }
     {
         const int esz = p.qt == 0 ? 4 : 2;
         const uint32_t rowb = (uint32_t) (D * esz), rowp = rowb + 16;    // bytes a row, padded in LDS
@@ -498,9 +539,28 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     if (((uintptr_t) kc | (uintptr_t) vc) % 16) return ns_fail(w + ": caches 16-byte aligned");
     if (rb % 16) return ns_fail(w + ": quantized cache rows with heads of 256 (shorter passes and other heads take the decode kernel)");
     // (512 work-groups of 256 rows: two for each of the chip's 256 CUs; NS_PREFILL_WAVES = 4 or 8 overrides: tuning, tests)
+    int64_t sns = 1, skbs = 0, sk0 = 0;
+    // Key splits. A pass of few rows over a long context - a chunk of a prompt behind 32K tokens, a long draft block - has
+    // too few (row block, head) pairs to fill the chip, each walking every key: its keys are cut into ns splits of whole
+    // tiles, a work-group a (row block, head, split), the partials merged by the decode path's merge kernel. ns is
+    // decided from the pass alone (128-row blocks x heads against ~512 work-groups; splits of at least 1024 keys), not
+    // from the work-group size, so both sizes sum a row in the same order. The partials live in the library's own
+    // scratch (the prompt entry points have no scratch argument): what fits bounds ns.
+    {
+        const int64_t kfirst = win > 0 ? std::max<int64_t>(0, p0 + 1 - win) : 0, keys = p0 + T - kfirst;
+        const int64_t pairs = ((T + 127) / 128) * Hq;
+        int64_t ns = std::min<int64_t>({(512 + pairs - 1) / pairs, keys / 1024, 64,
+                                        (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
+        if (const char* e = getenv("NS_PREFILL_SPLITS")) ns = std::min<int64_t>(atoll(e), (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2))));
+        if (ns >= 2) {
+            sk0 = kfirst / KT_TILE * KT_TILE;
+            skbs = ((p0 + T - sk0 + ns - 1) / ns + KT_TILE - 1) / KT_TILE * KT_TILE;
+            sns = (p0 + T - sk0 + skbs - 1) / skbs;
+        }
+    }
     // head size 256, 16-bit rows: a wave owns one 16-row tile, so 8 waves (two a SIMD, 128-row blocks) run the job 1.5 x
     // as fast as 4 (one a SIMD) whenever there are blocks enough for half the CUs
-    int PWs = D == 128 ? (((T + 255) / 256) * Hq >= 512 ? 8 : 4) : ((kt == 0 || kt == 3) && ((T + 127) / 128) * Hq >= 128 ? 8 : 4);
+    int PWs = D == 128 ? (((T + 255) / 256) * Hq * sns >= 512 ? 8 : 4) : ((kt == 0 || kt == 3) && T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
     if (const char* e = getenv("NS_PREFILL_WAVES"))
         if ((D == 128 || kt == 0 || kt == 3) && (atoi(e) == 4 || atoi(e) == 8)) PWs = atoi(e);
     const int64_t ROWS = rows_of((int) D, PWs);
@@ -524,14 +584,23 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     p.win = win;
     p.sl2 = (scale > 0.0f ? scale : 1.0f / sqrtf((float) D)) * 1.4426950408889634f;
     p.out = out;
+    p.ns = (int) sns;
+    p.kbs = skbs;
+    p.k0 = sk0;
+    p.part = g->own_scratch;
     const int64_t units = ((T + ROWS - 1) / ROWS) * Hkv;               // (row block, key head); padded to the 8 XCDs
-    dim3 grid((unsigned) ((units + 7) / 8 * 8 * (Hq / Hkv)));
+    dim3 grid((unsigned) ((units + 7) / 8 * 8 * (Hq / Hkv)), (unsigned) p.ns);
     if (ns_profile_mark(g, 0)) return -1;
     if ((D == 256 ? (PWs == 8 ? launch_prefill16<256, 8>(g, kt, p, grid) : launch_prefill<256, 4>(g, kt, p, grid))
                   : PWs == 8 ? launch_prefill<128, 8>(g, kt, p, grid) : launch_prefill<128, 4>(g, kt, p, grid)) != 0)
         return -1;
     NS_LAUNCHED("attn_prefill");
-    return ns_profile_mark(g, 1);
+    if (ns_profile_mark(g, 1)) return -1;
+    if (p.ns > 1) {
+        if (ns_attn_merge_partials(g, D, p.part, p.ns, qt, T * Hq, out)) return -1;
+        return ns_profile_mark(g, 2);
+    }
+    return 0;
     NS_CATCH
 }
 

@@ -80,6 +80,46 @@ def test_prefill_work_groups_of_8_waves(ops, monkeypatch, T, Hq, Hkv, D, p0, win
     assert np.array_equal(got8, got4)
 
 
+SPLIT = [
+    # T, Hq, Hkv, D, p0, win, kt, qt: few row blocks over many keys - the pass is cut into key splits and merged
+    (64, 8, 2, 128, 5000, 0, 0, F16),
+    (33, 4, 4, 128, 12000, 0, 3, BF16),
+    (300, 4, 1, 128, 9000, 3000, 0, F32),       # a window: the splits start at its first key
+    (40, 4, 2, 256, 4000, 0, 0, F32),
+    (130, 6, 2, 256, 2500, 0, 1, F16),          # quantized rows at head size 256
+    (17, 2, 1, 128, 40000, 0, 0, F32),
+]
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0,win,kt,qt", SPLIT)
+def test_prefill_key_splits(ops, T, Hq, Hkv, D, p0, win, kt, qt):
+    cap = p0 + T + 9
+    kc, vc = make_kv(kt, Hkv, D, cap, p0 + T, cfg=3)
+    qd, qf = make_q(qt, T, Hq, D, cfg=5)
+    got, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got, ref, qt, "prefill with key splits vs float64 closed form", kt=kt)
+
+
+@pytest.mark.parametrize("ns", [2, 5, 16])
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0,win", [(200, 4, 2, 128, 0, 0), (150, 2, 1, 128, 700, 90), (70, 4, 2, 256, 333, 0)])
+def test_prefill_forced_splits(ops, monkeypatch, ns, T, Hq, Hkv, D, p0, win):
+    """Splits forced onto short passes: splits wholly past a row block's last key, splits a window leaves empty, a last
+    split of a few keys - the same result as the unsplit pass within the path's bar, and the same whatever the
+    work-group size (bit for bit)."""
+    cap = p0 + T + 1
+    kc, vc = make_kv(0, Hkv, D, cap, p0 + T, cfg=1)
+    qd, qf = make_q(F32, T, Hq, D, cfg=2)
+    ref = orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, cap, p0, win=win)
+    monkeypatch.setenv("NS_PREFILL_SPLITS", str(ns))
+    monkeypatch.setenv("NS_PREFILL_WAVES", "8")
+    got8, _ = gpu_prompt(ops, F32, 0, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    monkeypatch.setenv("NS_PREFILL_WAVES", "4")
+    got4, _ = gpu_prompt(ops, F32, 0, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got8, ref, F32, "prefill with %d forced splits" % ns)
+    assert np.array_equal(got8, got4)
+
+
 def test_prefill_ring(ops):
     T, Hq, Hkv, D, cap, win, p0 = 150, 4, 2, 128, 512, 300, 900
     k = orc.randn(11, (p0 + T, Hkv * D))
