@@ -61,6 +61,7 @@ struct DecodeParams {
     int64_t p0, win;
     int64_t kbs, sp0;           // keys a split, the first split's index (absolute position / kbs)
     int ns;
+    int nz;                     // row chunks a (split, key head)
     float sl2;                  // scale x log2(e)
     float* part;                // [T][Hq][ns][D + 2]
     // block-sparse passes (one row a launch): the pass's keys are the listed blocks of 128 laid end to end - key j of
@@ -105,7 +106,13 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // the wave's index, known uniform to the compiler
-    const int split = blockIdx.x, hk = blockIdx.y, z = blockIdx.z;
+    // (split, key head, row chunk) of this work-group. Work-group ids go round the 8 XCDs, each with its own L2; the row
+    // chunks of one (split, head) read the same keys, so they take consecutive ids of ONE XCD and run there together:
+    // the keys come from HBM once and from that L2 for the other chunks. With one chunk this is the plain order, splits
+    // fastest. The grid is padded to a multiple of 8 (split, head) pairs; the padding leaves at once.
+    const int xj = blockIdx.x / 8, u = (xj / p.nz) * 8 + (int) (blockIdx.x % 8), z = xj % p.nz;
+    if (u >= p.ns * (p.Hq / p.G)) return;
+    const int split = u % p.ns, hk = u / p.ns;
     const int rows = p.T * p.G;
     const int64_t pass_end = p.p0 + p.T;
     const int64_t fmin = p.win > 0 ? std::max<int64_t>(0, p.p0 + 1 - p.win) : 0;
@@ -691,12 +698,16 @@ int launch_rt(ns_gpu* g, const DecodeParams& p, int rows, dim3 grid_xy) {
     // (quantized rows of 256: two row tiles and the staging registers do not fit the register file - one tile a chunk)
     constexpr bool ONE = D == 256 && (KT == 1 || KT == 2);
     const int RT = rows <= 16 || ONE ? 1 : 2;
-    dim3 grid(grid_xy.x, grid_xy.y, (unsigned) ((rows + RT * 16 - 1) / (RT * 16)));
+    DecodeParams c = p;
+    c.nz = (rows + RT * 16 - 1) / (RT * 16);
+    const int64_t pairs = (int64_t) grid_xy.x * grid_xy.y, wgs = (pairs + 7) / 8 * 8 * c.nz;
+    if (wgs >= (int64_t) 1 << 31) return ns_fail("ns_attn_decode: too many work-groups");
+    const dim3 grid((unsigned) wgs);
     if constexpr (ONE) {
-        attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(p);
+        attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(c);
     } else {
-        if (RT == 1) attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(p);
-        else attn_decode_kernel<D, 2, KT><<<grid, WAVES * 64, 0, g->q>>>(p);
+        if (RT == 1) attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(c);
+        else attn_decode_kernel<D, 2, KT><<<grid, WAVES * 64, 0, g->q>>>(c);
     }
     NS_LAUNCHED("attn_decode");
     return 0;
