@@ -508,14 +508,6 @@ int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
     return 0;
 }
 
-// 16-bit rows only (work-groups of 8 waves at D = 256)
-template <int D, int PW>
-int launch_prefill16(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
-    if (kt == 0) attn_prefill_kernel<D, false, 0, PW><<<grid, PW * 64, 0, g->q>>>(p);
-    else if (kt == 3) attn_prefill_kernel<D, true, 0, PW><<<grid, PW * 64, 0, g->q>>>(p);
-    else return ns_fail("ns_attn_prompt: internal: quantized rows in work-groups of 8 waves");
-    return 0;
-}
 
 }  // namespace
 
@@ -560,9 +552,9 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     }
     // head size 256, 16-bit rows: a wave owns one 16-row tile, so 8 waves (two a SIMD, 128-row blocks) run the job 1.5 x
     // as fast as 4 (one a SIMD) whenever there are blocks enough for half the CUs
-    int PWs = D == 128 ? (((T + 255) / 256) * Hq * sns >= 512 ? 8 : 4) : ((kt == 0 || kt == 3) && T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
+    int PWs = D == 128 ? (((T + 255) / 256) * Hq * sns >= 512 ? 8 : 4) : (T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
     if (const char* e = getenv("NS_PREFILL_WAVES"))
-        if ((D == 128 || kt == 0 || kt == 3) && (atoi(e) == 4 || atoi(e) == 8)) PWs = atoi(e);
+        if (atoi(e) == 4 || atoi(e) == 8) PWs = atoi(e);
     const int64_t ROWS = rows_of((int) D, PWs);
     if (T > (int64_t) 1 << 30 || ((T + ROWS - 1) / ROWS + 1) * Hq > (int64_t) 1 << 30) return ns_fail(w + ": too many rows or heads");
     if ((pm ? cap * Hkv : cap) * rb >= (int64_t) 1 << 32) return ns_fail(w + ": a key head's cache spans 4 GiB or more");
@@ -591,7 +583,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     const int64_t units = ((T + ROWS - 1) / ROWS) * Hkv;               // (row block, key head); padded to the 8 XCDs
     dim3 grid((unsigned) ((units + 7) / 8 * 8 * (Hq / Hkv)), (unsigned) p.ns);
     if (ns_profile_mark(g, 0)) return -1;
-    if ((D == 256 ? (PWs == 8 ? launch_prefill16<256, 8>(g, kt, p, grid) : launch_prefill<256, 4>(g, kt, p, grid))
+    if ((D == 256 ? (PWs == 8 ? launch_prefill<256, 8>(g, kt, p, grid) : launch_prefill<256, 4>(g, kt, p, grid))
                   : PWs == 8 ? launch_prefill<128, 8>(g, kt, p, grid) : launch_prefill<128, 4>(g, kt, p, grid)) != 0)
         return -1;
     NS_LAUNCHED("attn_prefill");

@@ -63,7 +63,8 @@ def test_prefill_seeded_shapes(ops, T, Hq, Hkv, D, p0, win, kt, qt):
 
 
 @pytest.mark.parametrize("T,Hq,Hkv,D,p0,win,kt,qt", [(700, 10, 2, 128, 300, 0, 3, BF16), (513, 4, 1, 128, 0, 400, 0, F32),
-                                                     (300, 8, 2, 256, 100, 0, 3, BF16), (260, 4, 1, 256, 0, 200, 0, F32)])
+                                                     (300, 8, 2, 256, 100, 0, 3, BF16), (260, 4, 1, 256, 0, 200, 0, F32),
+                                                     (200, 4, 2, 256, 60, 0, 1, F16), (140, 4, 1, 256, 0, 0, 2, F32)])
 def test_prefill_work_groups_of_8_waves(ops, monkeypatch, T, Hq, Hkv, D, p0, win, kt, qt):
     """Long passes run work-groups of 8 waves (blocks of 256 rows; 128 at head size 256), short ones of 4: the same rows,
     keys and order of a wave's arithmetic, so the two agree bit for bit; forced here on shapes the oracle finishes in
