@@ -45,6 +45,7 @@ constexpr int MTILE = 32, ML = 512;
 constexpr int mla_waves(int64_t group_rows, int64_t cells) { return group_rows <= 128 && cells <= 40960 ? 4 : 8; }
 // a split's partial of a row: u_s[512] = O_s / l_s as halfs (the split's own normalized result: bounded by the cache's
 // values, so half holds it; a quarter of the float32 form's bytes go to m and l), then m (log2 units), l, 2 of padding
+constexpr int SEL_DENSE_MAX = 2560;   // cells of a dense row in a selection pass (the reference's bound)
 constexpr int PSTRIDE = ML / 2 + 4;   // in floats: 1040 bytes, rows stay 16-byte aligned
 
 struct MlaParams {
@@ -414,7 +415,9 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
         }
         if (live && g4 == 0) {
             float* pr = prow + (int64_t) ri * p.ns * PSTRIDE;
-            pr[ML / 2] = m_r;
+            // (a row with more cells than the launch has splits for - a dense row of a selection pass past the length such
+            // passes are sized for - must not come out looking right: its partials' maxima are not numbers)
+            pr[ML / 2] = n_all > (int64_t) p.ns * p.kbs ? __builtin_nanf("") : m_r;
             pr[ML / 2 + 1] = l_row;
         }
     }
@@ -469,7 +472,7 @@ __global__ __launch_bounds__(256) void mla_merge_kernel(const float* __restrict_
     if (phase == 0) {
         const f4v t = ((ph[quad] + ph[64 + quad]) + ph[128 + quad]) + ph[192 + quad];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) store_o<QT>(u, row * ML + lat + i, L > 0.0f ? t[i] / L : 0.0f);
+        for (int i = 0; i < 4; ++i) store_o<QT>(u, row * ML + lat + i, L > 0.0f ? t[i] / L : L != L ? L : 0.0f);      // (a marked row stays NaN)
     }
 }
 
@@ -636,17 +639,18 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     if (!(scale > 0.0f)) return ns_fail(w + ": a positive scale");
     NS_HIP(hipSetDevice(g->dev));
     // With a selection (sel_cnt on the device) a row group holds one row's heads; a row's cell count is only known there:
-    // at most 4 K + 3 listed cells, or every earlier cell where its count is negative. Splits are sized for the listed
-    // form and enough of them cover a dense row.
+    // at most 4 K + 3 listed cells, or - where its count is negative - every earlier cell, which the reference allows up
+    // to 2,560 tokens only: its kernel keeps a row's scores in 2,560 floats of local memory, and the indexer lists pools
+    // past that (kernels/llm/glm5next/glm.cpp:1062-1067, 1085, 1258, 1274). The pass is sized for that many cells; a dense
+    // row beyond it comes out as NaNs (the kernel marks it), not as a plausible wrong answer.
     const bool per_t = sel_cnt != nullptr;
     if (per_t && (!sel || K < 0 || K > (int64_t) 1 << 24)) return ns_fail(w + ": a selection has cell pools and their count");
     if ((pos0 + T) * (int64_t) (q8 ? 544 : (512 + R) * 2) >= (int64_t) 1 << 32 && per_t) return ns_fail(w + ": a selection over a cache past 4 GiB");
     const int64_t rows = T * H;
     const int MW = mla_waves(per_t ? H : rows, pos0 + T), MROWS = MW * 16;
     const int64_t nz = per_t ? T * ((H + MROWS - 1) / MROWS) : (rows + MROWS - 1) / MROWS;
-    const int64_t listed = 4 * K + 3, cells = per_t ? std::max(pos0 + T, listed) : pos0 + T;
-    int64_t kbs = mla_kbs(per_t ? listed : cells, nz);
-    if (per_t) kbs = std::max(kbs, ((cells + 1023) / 1024 + MTILE - 1) / MTILE * MTILE);
+    const int64_t listed = 4 * K + 3, cells = per_t ? std::max(listed, std::min<int64_t>(pos0 + T, SEL_DENSE_MAX)) : pos0 + T;
+    int64_t kbs = mla_kbs(cells, nz);
     int64_t ns = (cells + kbs - 1) / kbs;
     // a caller's scratch may be smaller than the rule asks (the library's own, for the reference-named entry points):
     // fewer, longer splits then

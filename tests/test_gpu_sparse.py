@@ -111,3 +111,21 @@ def test_glm_cell_pools(ops, q8, T, H, pos0, K):
     # no counts: the dense pass, as before
     ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, scale, q8=q8)
     close(u.read(np.float32).reshape(T, H * L), orc.glm_mla_attend(qa, rows, q8, T, H, L, pos0, scale).reshape(T, H * L))
+
+
+def test_glm_dense_row_past_the_selection_bound_is_marked(ops):
+    """A selection pass is sized for its lists and for dense rows of up to 2,560 cells (the reference's bound: its kernel
+    keeps a row's scores in that many floats). A longer dense row must not come out as a plausible answer: NaNs."""
+    g = ops.gpu
+    T, H, L, pos0, K = 2, 16, 512, 2999, 16
+    n = pos0 + T
+    qa = orc.randn(1, (T, H * L), 0.3)
+    rows = orc.f2h(orc.randn(2, (n, L))).view(np.uint8).reshape(n, 2 * L)
+    sel = np.tile(np.arange(K, dtype=np.int32), (T, 1))
+    cnt = np.array([K, -1], np.int32)                     # row 0 listed, row 1 dense over 3001 cells
+    u = DevBuf(g, T * H * L * 4); u.fill(0)
+    ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, 0.05, sel=DevBuf.of(g, sel), sel_cnt=DevBuf.of(g, cnt), K=K)
+    got = u.read(np.float32).reshape(T, H * L)
+    want = orc.glm_mla_attend_sel(qa, rows, False, T, H, L, pos0, 0.05, sel, cnt, K)
+    close(got[:1], want.reshape(T, H * L)[:1])
+    assert np.isnan(got[1]).all()
