@@ -69,7 +69,8 @@ struct DecodeParams {
     // are not the row's
     const int32_t* sel;         // [Hkv][selK] block ids of this row, or null
     int selK;
-    int64_t sel_pos;
+    int selT;                   // rows of a block-list pass (each a row of its own in the kernel's numbering); else 1
+    int64_t sel_pos;            // the first row's position
 };
 
 template <int D, int KT>
@@ -111,8 +112,10 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // the keys come from HBM once and from that L2 for the other chunks. With one chunk this is the plain order, splits
     // fastest. The grid is padded to a multiple of 8 (split, head) pairs; the padding leaves at once.
     const int xj = blockIdx.x / 8, u = (xj / p.nz) * 8 + (int) (blockIdx.x % 8), z = xj % p.nz;
-    if (u >= p.ns * (p.Hq / p.G)) return;
-    const int split = u % p.ns, hk = u / p.ns;
+    // (a block-list pass holds selT rows with lists of their own: a row is one more factor of the pairs, tr its index)
+    const int Hkv = p.Hq / p.G;
+    if (u >= p.ns * Hkv * p.selT) return;
+    const int split = u % p.ns, hk = (u / p.ns) % Hkv, tr = u / (p.ns * Hkv);
     const int rows = p.T * p.G;
     const int64_t pass_end = p.p0 + p.T;
     const int64_t fmin = p.win > 0 ? std::max<int64_t>(0, p.p0 + 1 - p.win) : 0;
@@ -121,7 +124,8 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
     const uint8_t* vbase = p.vc + (int64_t) hk * p.head_stride;
     uint8_t* stage = lds + w * WREG;
-    const int32_t* selp = p.sel ? p.sel + (int64_t) hk * p.selK : nullptr;
+    const int32_t* selp = p.sel ? p.sel + ((int64_t) tr * Hkv + hk) * p.selK : nullptr;
+    const int64_t sel_pos = p.sel_pos + tr;
 
     // a key's row offset: keys outside [jb, je) are clamped into it (their scores are masked, their values meet P = 0).
     // A wrapped ring's slot is position % cap: the split's first key's slot once, then offsets from it with at most two
@@ -144,7 +148,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         if (!selp) return row_off(j0 + idx);
         const int blk = selp[(ti * TILE) >> 7];
         // (keys of a listed block past the row's position are masked: read the row's own key instead - the cache may end there)
-        return std::min<int64_t>((int64_t) (blk < 0 ? 0 : blk) * 128 + ((ti * TILE) & 127) + idx, p.sel_pos) * p.row_stride;
+        return std::min<int64_t>((int64_t) (blk < 0 ? 0 : blk) * 128 + ((ti * TILE) & 127) + idx, sel_pos) * p.row_stride;
     };
     // 16-bit rows: a tile's keys (which = 0) or values (1) on their way global -> LDS, 1 KiB a load: position cp of key kk
     // holds the row's 16-byte chunk cp ^ (kk % 16) (keys: the operand reads of 16 keys' same chunk meet no bank
@@ -287,7 +291,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         // checked on the host); a dead row reads row 0's and is zeroed
         // feature order of the k-blocks: plain (k-block kb, lane group g4: features 32 kb + 8 g4 ..), q8_0 keys: see load_tile
         auto foff = [&](int kb) { return KT == 1 ? 64 * (kb / 2) + 16 * g4 + 8 * (kb % 2) : 32 * kb + 8 * g4; };
-        const int64_t qoff = (int64_t) t * p.qs + ((int64_t) hk * p.G + gq) * D;
+        const int64_t qoff = (int64_t) (t + tr) * p.qs + ((int64_t) hk * p.G + gq) * D;
         if (p.qt == 0) {
             float4 raw[KB][2];
 #pragma unroll
@@ -424,7 +428,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         if (selp) {
             // (a listed block's keys count up to the row's own position; a hole in the list has none)
             const int blk = selp[j0 >> 7];
-            hi_tile = blk < 0 ? j0r - 1 : (int) ((j0 & ~(int64_t) 127) - jb + std::min<int64_t>(127, p.sel_pos - (int64_t) blk * 128));
+            hi_tile = blk < 0 ? j0r - 1 : (int) ((j0 & ~(int64_t) 127) - jb + std::min<int64_t>(127, sel_pos - (int64_t) blk * 128));
         }
         int lo_t[RT];
         unsigned span_t[RT];
@@ -577,7 +581,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             acc = k == 0 ? ok * f : acc + ok * f;
         }
         // partial rows are D + 2 floats: 8-byte aligned
-        float* pr = p.part + (((int64_t) t * p.Hq + hk * p.G + gq) * p.ns + split) * (D + 2);
+        float* pr = p.part + (((int64_t) (t + tr) * p.Hq + hk * p.G + gq) * p.ns + split) * (D + 2);
         *reinterpret_cast<float2*>(pr + c * 4) = float2{acc[0], acc[1]};
         *reinterpret_cast<float2*>(pr + c * 4 + 2) = float2{acc[2], acc[3]};
         if (c == 0) *reinterpret_cast<float2*>(pr + D) = float2{M, L};
@@ -737,6 +741,7 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
     const int64_t rb = kv_row_bytes(kt, D);
     const int esz = QT == 0 ? 4 : 2;
     DecodeParams p{};
+    p.selT = 1;
     p.qt = QT;
     p.kc = (const uint8_t*) kc;
     p.vc = (const uint8_t*) vc;
@@ -835,6 +840,8 @@ int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_
     if (K == 0) return ns_fill(g, out, 0, (size_t) (T * Hq * D) * sizeof(float));     // nothing listed: zeros (l = 0)
     const int64_t keys = K * 128, kbs = dec_kbs(keys, Hkv, D), ns = (keys + kbs - 1) / kbs;
     if ((size_t) (Hq * ns * (D + 2)) > scratch_floats) return ns_fail(w + ": the pass needs more scratch than the library keeps");
+    // every row in one launch and one merge where the partials of all rows fit the scratch; else a launch a row
+    const bool batched = (size_t) (T * Hq * ns * (D + 2)) <= scratch_floats && T * Hkv <= 65535;
     DecodeParams p{};
     p.qt = 0;
     p.qs = Hq * D;
@@ -856,6 +863,15 @@ int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_
     p.sl2 = scale * 1.4426950408889634f;
     p.part = scratch;
     p.selK = (int) K;
+    p.selT = 1;
+    if (batched) {
+        p.q = q;
+        p.sel = sel;
+        p.sel_pos = pos0;
+        p.selT = (int) T;
+        if (launch_kt<D>(g, 0, p, p.G, dim3((unsigned) ns, (unsigned) (Hkv * T)))) return -1;
+        return launch_merge<D>(g, scratch, (int) ns, 0, T * Hq, out);
+    }
     for (int64_t t = 0; t < T; ++t) {
         p.q = q + t * Hq * D;
         p.sel = sel + t * Hkv * K;
