@@ -16,6 +16,7 @@
 #include "kv_formats.hpp"
 #include "kv_pack.hpp"
 
+#include <algorithm>
 #include <cmath>
 
 namespace {
@@ -48,16 +49,22 @@ struct PreParams {
     int s0, s1, s2;
     int64_t cap;
     int ring;
+    int hpw;                          // heads of a row a wave walks (their rotation worked out once)
 };
 
-// output feature i of a head row: v(j) = x[j] * inv * w[j] (or x[j]), rotated as the mode says
-__device__ __forceinline__ float rope_feature(const PreParams& p, const float* x, const float* w, float inv, int i, int t, bool rot) {
-    auto v = [&](int j) { return w ? x[j] * inv * w[j] : x[j]; };
-    const float me = v(i);
-    if (!rot || p.mode == ROPE_NONE) return me;
+// the rotation of output feature i at row t: cosine and sine of its angle (on = false: the feature is not rotated). It
+// depends on the row and the feature only - not on the head - so a wave that walks several heads of a row works it out
+// once: powf, cosf and sinf are most of this kernel's arithmetic
+struct Rot {
+    float c, s;
+    bool on;
+};
+__device__ __forceinline__ Rot rope_cs(const PreParams& p, int i, int t) {
+    Rot r{1.0f, 0.0f, false};
+    if (p.mode == ROPE_NONE) return r;
     const int D = p.D;
     if (p.mode == ROPE_Q35) {
-        if (i >= p.n_rot) return me;
+        if (i >= p.n_rot) return r;
         const int hr = p.n_rot / 2, k = i < hr ? i : i - hr;
         float pos = (float) (p.p0 + t);
         if (p.pos3) {
@@ -66,7 +73,31 @@ __device__ __forceinline__ float rope_feature(const PreParams& p, const float* x
             pos = (float) p.pos3[t * 3 + c];
         }
         const float a = pos * powf(p.theta, -2.0f * (float) k / (float) p.n_rot);
-        const float c = cosf(a), sn = sinf(a);
+        return Rot{cosf(a), sinf(a), true};
+    }
+    if (p.mode == ROPE_MG_PAIRS || p.mode == ROPE_MG_HALVES) {
+        const bool halves = p.mode == ROPE_MG_HALVES;
+        const int pr = halves ? (i < D / 2 ? i : i - D / 2) : i / 2;
+        const float a = (float) (p.p0 + t) * powf(p.theta, -2.0f * (float) pr / (float) D);
+        return Rot{cosf(a), sinf(a), true};
+    }
+    // ROPE_MM3
+    if (i >= p.n_rot) return r;
+    const int hr = p.n_rot / 2, k = i % hr;
+    float th = (float) (p.p0 + t);
+    for (int j = 0; j < k; ++j) th *= p.ts;
+    return Rot{cosf(th), sinf(th), true};
+}
+
+// output feature i of a head row: v(j) = x[j] * inv * w[j] (or x[j]), rotated as the mode says by r = rope_cs(p, i, t)
+__device__ __forceinline__ float rope_feature(const PreParams& p, const float* x, const float* w, float inv, int i, bool rot, const Rot& r) {
+    auto v = [&](int j) { return w ? x[j] * inv * w[j] : x[j]; };
+    const float me = v(i);
+    if (!rot || !r.on) return me;
+    const int D = p.D;
+    const float c = r.c, sn = r.s;
+    if (p.mode == ROPE_Q35) {
+        const int hr = p.n_rot / 2;
         const float other = v(i < hr ? i + hr : i - hr);
         return i < hr ? me * c - other * sn : me * c + other * sn;
     }
@@ -74,57 +105,138 @@ __device__ __forceinline__ float rope_feature(const PreParams& p, const float* x
         const bool halves = p.mode == ROPE_MG_HALVES;
         const int pr = halves ? (i < D / 2 ? i : i - D / 2) : i / 2;
         const int i0 = halves ? pr : 2 * pr, i1 = halves ? pr + D / 2 : 2 * pr + 1;
-        const float a = (float) (p.p0 + t) * powf(p.theta, -2.0f * (float) pr / (float) D);
-        const float c = cosf(a), sn = sinf(a);
         const float a0 = i == i0 ? me : v(i0), a1 = i == i1 ? me : v(i1);
         return i == i0 ? a0 * c - a1 * sn : a0 * sn + a1 * c;
     }
     // ROPE_MM3
-    if (i >= p.n_rot) return me;
-    const int hr = p.n_rot / 2, k = i % hr;
-    float th = (float) (p.p0 + t);
-    for (int j = 0; j < k; ++j) th *= p.ts;
-    const float c = cosf(th), s = sinf(th);
+    const int hr = p.n_rot / 2;
     const float them = v(i < hr ? i + hr : i - hr);
-    return i < hr ? me * c - them * s : them * s + me * c;
+    return i < hr ? me * c - them * sn : them * sn + me * c;
 }
 
+// VEC: whole 4-feature groups pair up under the rotation (see below); MAXG: 4-feature groups a lane (1: D up to 256)
+template <bool VEC, int MAXG>
 __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
     const int lane = threadIdx.x & 63;
-    const int64_t rowid = (int64_t) blockIdx.x * 4 + (threadIdx.x >> 6);
+    // the wave's index as a scalar: the row, the head and its group's descriptor then live in scalar registers
+    const int64_t wid = (int64_t) blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
     int per_t = 0;
-    for (int gi = 0; gi < p.ngr; ++gi) per_t += p.gr[gi].heads;
-    if (rowid >= (int64_t) p.T * per_t) return;            // whole waves leave: no shuffle below misses a lane
-    const int t = (int) (rowid / per_t);
-    int h = (int) (rowid % per_t), gi = 0;
-    while (h >= p.gr[gi].heads) h -= p.gr[gi++].heads;
-    const PreGroup& G = p.gr[gi];
+#pragma unroll
+    for (int gi = 0; gi < 5; ++gi) per_t += gi < p.ngr ? p.gr[gi].heads : 0;
+    const int wpt = (per_t + p.hpw - 1) / p.hpw;           // waves a row: each walks hpw of the row's heads
+    if (wid >= (int64_t) p.T * wpt) return;                // whole waves leave: no shuffle below misses a lane
+    const int t = (int) (wid / wpt);
+    const int hfirst = (int) (wid % wpt) * p.hpw, hend = min(hfirst + p.hpw, per_t);
     const int D = p.D;
+    // the rotation of this lane's features at this row: the same for every head. One copy of the angle code, looped (eight
+    // unrolled copies cost the kernel half its waves in registers); the results go to registers by constant index
+    float rc[MAXG * 4], rs[MAXG * 4];
+    uint32_t onmask = 0;
+#pragma unroll
+    for (int q = 0; q < MAXG * 4; ++q) rc[q] = 1.0f, rs[q] = 0.0f;
+    const int nfeat = MAXG == 1 || D <= 256 ? 4 : 8;
+#pragma nounroll
+    for (int e = 0; e < nfeat; ++e) {
+        const int i = lane * 4 + (e >> 2) * 256 + (e & 3);
+        const Rot r = i < D ? rope_cs(p, i, t) : Rot{1.0f, 0.0f, false};
+#pragma unroll
+        for (int q = 0; q < MAXG * 4; ++q)
+            if (q == e) rc[q] = r.c, rs[q] = r.s;
+        onmask |= (r.on ? 1u : 0u) << e;
+    }
+    // the distance to a rotated feature's partner
+    const int pdist = p.mode == ROPE_MG_HALVES ? D / 2 : p.n_rot / 2;
+  for (int hh = hfirst; hh < hend; ++hh) {
+    // the head's group, picked by comparisons against constants' worth of indices: the descriptors stay in scalar
+    // registers (an index computed at run time would send the whole argument block through private memory)
+    int h = hh;
+    PreGroup G = p.gr[0];
+    {
+        int first = p.gr[0].heads;
+#pragma unroll
+        for (int k = 1; k < 5; ++k) {
+            if (k < p.ngr && hh >= first) {
+                G = p.gr[k];
+                h = hh - first;
+            }
+            first += k < p.ngr ? p.gr[k].heads : 0;
+        }
+    }
     const float* x = G.src + (int64_t) t * G.ss + (int64_t) h * G.hs;
-    // ---- the row's scale
+    // ---- the row's scale. A lane's own features come in one 16-byte load a group of four and stay in registers
+    float4 xo[MAXG];
+#pragma unroll
+    for (int c = 0; c < MAXG; ++c) {
+        const int i = lane * 4 + c * 256;
+        xo[c] = i < D ? *reinterpret_cast<const float4*>(x + i) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
     float inv = 1.0f;
     if (G.w) {
         float s = 0.0f;
-        for (int i = lane * 4; i < D; i += 256) {
-            const float4 a = *reinterpret_cast<const float4*>(x + i);
-            s += a.x * a.x;
-            s += a.y * a.y;
-            s += a.z * a.z;
-            s += a.w * a.w;
+#pragma unroll
+        for (int c = 0; c < MAXG; ++c) {
+            if (lane * 4 + c * 256 < D) {
+                s += xo[c].x * xo[c].x;
+                s += xo[c].y * xo[c].y;
+                s += xo[c].z * xo[c].z;
+                s += xo[c].w * xo[c].w;
+            }
         }
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) s += __shfl_xor(s, o);
         const float ms = s / (float) D + p.eps;
         inv = p.inv_sqrt ? 1.0f / sqrtf(ms) : rsqrtf(ms);
     }
-    // ---- this lane's features, all computed (every load done) before anything is stored
-    constexpr int MAXG = 2;                                  // D up to 512
+    // ---- this lane's features, all computed (every load done) before anything is stored. Where the partner of a rotated
+    // feature lies a whole number of 4-feature groups away (or inside the lane's own group: adjacent pairs) the partners
+    // come in one 16-byte load as well; other widths take the feature-by-feature form
     float y[MAXG][4];
+    if constexpr (VEC) {
 #pragma unroll
-    for (int c = 0; c < MAXG; ++c) {
-        const int i = lane * 4 + c * 256;
+        for (int c = 0; c < MAXG; ++c) {
+            const int i = lane * 4 + c * 256;
+            if (i >= D) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) y[c][j] = i < D ? rope_feature(p, x, G.w, inv, i + j, t, G.rope != 0) : 0.0f;
+                for (int j = 0; j < 4; ++j) y[c][j] = 0.0f;
+                continue;
+            }
+            const bool rotated = G.rope != 0 && (onmask >> (c * 4) & 1) != 0;
+            const int ip = !rotated || p.mode == ROPE_MG_PAIRS ? i : i < pdist ? i + pdist : i - pdist;
+            const float4 xp4 = rotated && ip != i ? *reinterpret_cast<const float4*>(x + ip) : xo[c];
+            float4 wo4 = make_float4(1.0f, 1.0f, 1.0f, 1.0f), wp4 = wo4;
+            if (G.w) {
+                wo4 = *reinterpret_cast<const float4*>(G.w + i);
+                wp4 = ip != i ? *reinterpret_cast<const float4*>(G.w + ip) : wo4;
+            }
+            const float xv[4] = {xo[c].x, xo[c].y, xo[c].z, xo[c].w}, xq[4] = {xp4.x, xp4.y, xp4.z, xp4.w};
+            const float wv[4] = {wo4.x, wo4.y, wo4.z, wo4.w}, wq[4] = {wp4.x, wp4.y, wp4.z, wp4.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float me = G.w ? xv[j] * inv * wv[j] : xv[j];
+                if (!rotated) {
+                    y[c][j] = me;
+                    continue;
+                }
+                const float cs = rc[c * 4 + j], sn = rs[c * 4 + j];
+                if (p.mode == ROPE_MG_PAIRS) {
+                    const float pt = G.w ? xv[j ^ 1] * inv * wv[j ^ 1] : xv[j ^ 1];
+                    y[c][j] = (j & 1) == 0 ? me * cs - pt * sn : pt * sn + me * cs;
+                } else {
+                    const float pt = G.w ? xq[j] * inv * wq[j] : xq[j];
+                    const bool first = i < pdist;
+                    if (p.mode == ROPE_Q35) y[c][j] = first ? me * cs - pt * sn : me * cs + pt * sn;
+                    else if (p.mode == ROPE_MG_HALVES) y[c][j] = first ? me * cs - pt * sn : pt * sn + me * cs;
+                    else y[c][j] = first ? me * cs - pt * sn : pt * sn + me * cs;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int c = 0; c < MAXG; ++c) {
+            const int i = lane * 4 + c * 256;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) y[c][j] = i < D ? rope_feature(p, x, G.w, inv, i + j, G.rope != 0, Rot{rc[c * 4 + j], rs[c * 4 + j], (onmask >> (c * 4 + j) & 1) != 0}) : 0.0f;
+        }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // loads above, stores below (source may be destination)
 #pragma unroll
@@ -178,15 +290,30 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
             }
         }
     }
+  }   // the wave's next head
 }
 
 int launch_pre(ns_gpu* g, const PreParams& p, const char* who) {
     NS_HIP(hipSetDevice(g->dev));
-    int64_t rows = 0;
-    for (int i = 0; i < p.ngr; ++i) rows += (int64_t) p.T * p.gr[i].heads;
-    if (rows <= 0) return 0;
-    if ((rows + 3) / 4 > (int64_t) 1 << 31) return ns_fail(std::string(who) + ": too many rows");
-    pre_attn_kernel<<<(unsigned) ((rows + 3) / 4), 256, 0, g->q>>>(p);
+    int64_t per_t = 0;
+    for (int i = 0; i < p.ngr; ++i) per_t += p.gr[i].heads;
+    if (per_t <= 0 || p.T <= 0) return 0;
+    // a wave a (row, head) while that leaves the chip short of waves (a decode step); a prompt's rows have waves to spare,
+    // and each then walks several heads of its row on one evaluation of the rotation
+    PreParams q = p;
+    q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, (int64_t) p.T * per_t / 8192));
+    const int64_t waves = (int64_t) p.T * ((per_t + q.hpw - 1) / q.hpw);
+    if ((waves + 3) / 4 > (int64_t) 1 << 31) return ns_fail(std::string(who) + ": too many rows");
+    // whole 4-feature groups pair up: no rotation, adjacent pairs, or partners a multiple of 4 features away
+    const bool vec = p.mode == ROPE_NONE || p.mode == ROPE_MG_PAIRS || (p.mode == ROPE_MG_HALVES ? p.D % 8 == 0 : p.n_rot % 8 == 0);
+    const dim3 grid((unsigned) ((waves + 3) / 4));
+    if (p.D <= 256) {
+        if (vec) pre_attn_kernel<true, 1><<<grid, 256, 0, g->q>>>(q);
+        else pre_attn_kernel<false, 1><<<grid, 256, 0, g->q>>>(q);
+    } else {
+        if (vec) pre_attn_kernel<true, 2><<<grid, 256, 0, g->q>>>(q);
+        else pre_attn_kernel<false, 2><<<grid, 256, 0, g->q>>>(q);
+    }
     NS_LAUNCHED(who);
     return 0;
 }
