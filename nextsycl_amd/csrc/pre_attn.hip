@@ -2,8 +2,9 @@
 // gfx950: the reference's separate entry points and one fused launch (norm + rotate + store, k never written as
 // float32). Bound: HBM, negligible volume (a few KB a token); the point of the fused form is two launches fewer a layer.
 //
-// One wave a (row, head); a lane four consecutive features (D up to 256; more: a lane several groups of four). Every
-// load of a wave precedes its stores, so source and destination may be the same rows. The arithmetic of an output
+// One wave a (row, head) - two or four rows of a head where a head row is 128 or 64 features, so no lane idles; a lane
+// four consecutive features (D up to 256; more: a lane several groups of four). In a prompt pass a wave walks several
+// heads of its rows on one evaluation of the rotation. Every load of a head precedes its stores, so source and destination may be the same rows. The arithmetic of an output
 // feature is one function (rope_feature) whatever entry point asks for it, and the quantized rows are kv_pack.hpp's:
 // the fused launch gives bit for bit what the separate calls give. Compiled with -ffp-contract=off (the packers).
 //
@@ -15,9 +16,12 @@
 #include "ns_pre.h"
 #include "kv_formats.hpp"
 #include "kv_pack.hpp"
+#include "attn_common.hpp"
 
 #include <algorithm>
 #include <cmath>
+#include <cstddef>
+#include <cstdlib>
 
 namespace {
 
@@ -118,16 +122,21 @@ __device__ __forceinline__ float rope_feature(const PreParams& p, const float* x
 template <bool VEC, int MAXG>
 __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
     const int lane = threadIdx.x & 63;
+    const int D = p.D;
+    // a head row of 64 or 128 features takes 16 or 32 lanes: the wave then carries 4 or 2 consecutive rows t of the same
+    // head at once (same group, same weights; the rotation is a lane's own anyway), and no lane idles
+    const int lph = MAXG == 1 && D == 64 ? 16 : MAXG == 1 && D == 128 ? 32 : 64;
+    const int rpw = 64 / lph, sub = lane / lph, li = lane - sub * lph;
     // the wave's index as a scalar: the row, the head and its group's descriptor then live in scalar registers
     const int64_t wid = (int64_t) blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
     int per_t = 0;
 #pragma unroll
     for (int gi = 0; gi < 5; ++gi) per_t += gi < p.ngr ? p.gr[gi].heads : 0;
-    const int wpt = (per_t + p.hpw - 1) / p.hpw;           // waves a row: each walks hpw of the row's heads
-    if (wid >= (int64_t) p.T * wpt) return;                // whole waves leave: no shuffle below misses a lane
-    const int t = (int) (wid / wpt);
+    const int wpt = (per_t + p.hpw - 1) / p.hpw;           // waves a group of rows: each walks hpw of the rows' heads
+    if (wid >= (int64_t) ((p.T + rpw - 1) / rpw) * wpt) return;   // whole waves leave: no shuffle below misses a lane
+    const int t = (int) (wid / wpt) * rpw + sub;
+    const bool row_live = t < p.T;                         // a lane past the last row loads zeros and stores nothing
     const int hfirst = (int) (wid % wpt) * p.hpw, hend = min(hfirst + p.hpw, per_t);
-    const int D = p.D;
     // the rotation of this lane's features at this row: the same for every head. One copy of the angle code, looped (eight
     // unrolled copies cost the kernel half its waves in registers); the results go to registers by constant index
     float rc[MAXG * 4], rs[MAXG * 4];
@@ -137,8 +146,8 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
     const int nfeat = MAXG == 1 || D <= 256 ? 4 : 8;
 #pragma nounroll
     for (int e = 0; e < nfeat; ++e) {
-        const int i = lane * 4 + (e >> 2) * 256 + (e & 3);
-        const Rot r = i < D ? rope_cs(p, i, t) : Rot{1.0f, 0.0f, false};
+        const int i = li * 4 + (e >> 2) * 256 + (e & 3);
+        const Rot r = i < D && row_live ? rope_cs(p, i, t) : Rot{1.0f, 0.0f, false};
 #pragma unroll
         for (int q = 0; q < MAXG * 4; ++q)
             if (q == e) rc[q] = r.c, rs[q] = r.s;
@@ -146,68 +155,97 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
     }
     // the distance to a rotated feature's partner
     const int pdist = p.mode == ROPE_MG_HALVES ? D / 2 : p.n_rot / 2;
-  for (int hh = hfirst; hh < hend; ++hh) {
-    // the head's group, picked by comparisons against constants' worth of indices: the descriptors stay in scalar
-    // registers (an index computed at run time would send the whole argument block through private memory)
-    int h = hh;
-    PreGroup G = p.gr[0];
-    {
-        int first = p.gr[0].heads;
+    // What a head needs from memory: its group, its row, the lane's own features and (VEC) their partners and weights.
+    // Every load is unconditional - a lane with nothing to do reads a valid address and drops the value - so the loads
+    // of the NEXT head can be in flight, counted, while this head is worked on: a head then costs about one memory
+    // latency a wave instead of two or three
+    struct HeadIn {
+        PreGroup G;
+        int h;
+        const float* x;
+        float4 xo[MAXG], xp[MAXG], wo[MAXG], wp[MAXG];
+    };
+    const int tl = row_live ? t : p.T - 1;
+    const PreGroup* groups = reinterpret_cast<const PreGroup*>((const char*) __builtin_amdgcn_kernarg_segment_ptr() + offsetof(PreParams, gr));
+    auto fetch = [&](int hh, HeadIn& in) __attribute__((always_inline)) {
+        // the head's group: its index from comparisons, its descriptor read from the kernel-argument block in memory at
+        // that index - scalar loads into scalar registers. (Indexing the by-value argument itself at run time would
+        // send the whole block through private memory; selecting among five descriptors held in registers overflows
+        // the scalar file)
+        int gi = 0, first = 0;
+        in.h = hh;
 #pragma unroll
-        for (int k = 1; k < 5; ++k) {
-            if (k < p.ngr && hh >= first) {
-                G = p.gr[k];
-                h = hh - first;
-            }
+        for (int k = 0; k < 4; ++k) {
             first += k < p.ngr ? p.gr[k].heads : 0;
+            if (k + 1 < p.ngr && hh >= first) gi = k + 1, in.h = hh - first;
         }
-    }
-    const float* x = G.src + (int64_t) t * G.ss + (int64_t) h * G.hs;
-    // ---- the row's scale. A lane's own features come in one 16-byte load a group of four and stay in registers
+        in.G = groups[gi];
+        in.x = in.G.src + (int64_t) tl * in.G.ss + (int64_t) in.h * in.G.hs;
+#pragma unroll
+        for (int c = 0; c < MAXG; ++c) {
+            const int i0 = li * 4 + c * 256, i = i0 < D ? i0 : 0;
+            in.xo[c] = *reinterpret_cast<const float4*>(in.x + i);
+            if constexpr (VEC) {
+                const bool rotated = in.G.rope != 0 && (onmask >> (c * 4) & 1) != 0;
+                const int ip = !rotated || p.mode == ROPE_MG_PAIRS ? i : i < pdist ? i + pdist : i - pdist;
+                const float* w = in.G.w ? in.G.w : in.x;
+                in.xp[c] = *reinterpret_cast<const float4*>(in.x + ip);
+                in.wo[c] = *reinterpret_cast<const float4*>(w + i);
+                in.wp[c] = *reinterpret_cast<const float4*>(w + ip);
+            }
+        }
+    };
+    HeadIn cur;
+    fetch(hfirst, cur);
+  for (int hh = hfirst; hh < hend; ++hh) {
+    HeadIn nxt;
+    fetch(hh + 1 < hend ? hh + 1 : hh, nxt);          // the last head reads itself again rather than branch
+    const PreGroup G = cur.G;
+    const int h = cur.h;
+    const float* x = cur.x;
+    // ---- the row's scale
     float4 xo[MAXG];
 #pragma unroll
-    for (int c = 0; c < MAXG; ++c) {
-        const int i = lane * 4 + c * 256;
-        xo[c] = i < D ? *reinterpret_cast<const float4*>(x + i) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    }
+    for (int c = 0; c < MAXG; ++c) xo[c] = li * 4 + c * 256 < D && row_live ? cur.xo[c] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     float inv = 1.0f;
     if (G.w) {
         float s = 0.0f;
 #pragma unroll
         for (int c = 0; c < MAXG; ++c) {
-            if (lane * 4 + c * 256 < D) {
-                s += xo[c].x * xo[c].x;
-                s += xo[c].y * xo[c].y;
-                s += xo[c].z * xo[c].z;
-                s += xo[c].w * xo[c].w;
-            }
+            s += xo[c].x * xo[c].x;
+            s += xo[c].y * xo[c].y;
+            s += xo[c].z * xo[c].z;
+            s += xo[c].w * xo[c].w;
         }
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) s += __shfl_xor(s, o);
+        // over the head row's lanes, pairwise as an exclusive-or butterfly would (lanes past the row carry zeros)
+        s = row16_sum(s);
+        float a, b;
+        if (lph > 16) {
+            pair16(s, a, b);
+            s = a + b;
+        }
+        if (lph > 32) {
+            pair32(s, a, b);
+            s = a + b;
+        }
         const float ms = s / (float) D + p.eps;
         inv = p.inv_sqrt ? 1.0f / sqrtf(ms) : rsqrtf(ms);
     }
-    // ---- this lane's features, all computed (every load done) before anything is stored. Where the partner of a rotated
-    // feature lies a whole number of 4-feature groups away (or inside the lane's own group: adjacent pairs) the partners
-    // come in one 16-byte load as well; other widths take the feature-by-feature form
+    // ---- this lane's features. Where the partner of a rotated feature lies a whole number of 4-feature groups away
+    // (or inside the lane's own group: adjacent pairs) the partners came in one 16-byte load as well; other widths
+    // take the feature-by-feature form
     float y[MAXG][4];
     if constexpr (VEC) {
 #pragma unroll
         for (int c = 0; c < MAXG; ++c) {
-            const int i = lane * 4 + c * 256;
-            if (i >= D) {
+            const int i = li * 4 + c * 256;
+            if (i >= D || !row_live) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) y[c][j] = 0.0f;
                 continue;
             }
             const bool rotated = G.rope != 0 && (onmask >> (c * 4) & 1) != 0;
-            const int ip = !rotated || p.mode == ROPE_MG_PAIRS ? i : i < pdist ? i + pdist : i - pdist;
-            const float4 xp4 = rotated && ip != i ? *reinterpret_cast<const float4*>(x + ip) : xo[c];
-            float4 wo4 = make_float4(1.0f, 1.0f, 1.0f, 1.0f), wp4 = wo4;
-            if (G.w) {
-                wo4 = *reinterpret_cast<const float4*>(G.w + i);
-                wp4 = ip != i ? *reinterpret_cast<const float4*>(G.w + ip) : wo4;
-            }
+            const float4 xp4 = cur.xp[c], wo4 = cur.wo[c], wp4 = cur.wp[c];
             const float xv[4] = {xo[c].x, xo[c].y, xo[c].z, xo[c].w}, xq[4] = {xp4.x, xp4.y, xp4.z, xp4.w};
             const float wv[4] = {wo4.x, wo4.y, wo4.z, wo4.w}, wq[4] = {wp4.x, wp4.y, wp4.z, wp4.w};
 #pragma unroll
@@ -225,7 +263,6 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
                     const float pt = G.w ? xq[j] * inv * wq[j] : xq[j];
                     const bool first = i < pdist;
                     if (p.mode == ROPE_Q35) y[c][j] = first ? me * cs - pt * sn : me * cs + pt * sn;
-                    else if (p.mode == ROPE_MG_HALVES) y[c][j] = first ? me * cs - pt * sn : pt * sn + me * cs;
                     else y[c][j] = first ? me * cs - pt * sn : pt * sn + me * cs;
                 }
             }
@@ -233,17 +270,17 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
     } else {
 #pragma unroll
         for (int c = 0; c < MAXG; ++c) {
-            const int i = lane * 4 + c * 256;
+            const int i = li * 4 + c * 256;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) y[c][j] = i < D ? rope_feature(p, x, G.w, inv, i + j, G.rope != 0, Rot{rc[c * 4 + j], rs[c * 4 + j], (onmask >> (c * 4 + j) & 1) != 0}) : 0.0f;
+            for (int j = 0; j < 4; ++j) y[c][j] = i < D && row_live ? rope_feature(p, x, G.w, inv, i + j, G.rope != 0, Rot{rc[c * 4 + j], rs[c * 4 + j], (onmask >> (c * 4 + j) & 1) != 0}) : 0.0f;
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // loads above, stores below (source may be destination)
 #pragma unroll
     for (int c = 0; c < MAXG; ++c) {
-        const int i = lane * 4 + c * 256;
+        const int i = li * 4 + c * 256;
         if (c * 256 >= D) break;
-        const bool live = i < D;
+        const bool live = i < D && row_live;
         if (G.dt < DST_CACHE) {
             if (!live) continue;
             const int64_t at = (int64_t) t * G.ds + (int64_t) h * D + i;
@@ -272,7 +309,7 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
                 *reinterpret_cast<ushort4*>(row + 2 * i) = o;
             } else {
                 // 8 lanes a block of 32: every lane takes part in the shuffles (dead lanes carry zeros, store nothing)
-                const int b = i / 32, ln = lane & 7;
+                const int b = i / 32, ln = li & 7;
                 float d;
                 if (kt == 1) {
                     const uint32_t wv = q8_0_pack4(y[c], d);
@@ -290,6 +327,7 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
             }
         }
     }
+    cur = nxt;
   }   // the wave's next head
 }
 
@@ -298,11 +336,15 @@ int launch_pre(ns_gpu* g, const PreParams& p, const char* who) {
     int64_t per_t = 0;
     for (int i = 0; i < p.ngr; ++i) per_t += p.gr[i].heads;
     if (per_t <= 0 || p.T <= 0) return 0;
-    // a wave a (row, head) while that leaves the chip short of waves (a decode step); a prompt's rows have waves to spare,
-    // and each then walks several heads of its row on one evaluation of the rotation
+    // a wave a (row group, head) while that leaves the chip short of waves (a decode step); a prompt's rows have waves to
+    // spare, and each then walks several heads of its rows on one evaluation of the rotation (most of a wave's
+    // arithmetic): about 4096 waves a launch measured best, the heads of a row group shared evenly among its waves
     PreParams q = p;
-    q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, (int64_t) p.T * per_t / 8192));
-    const int64_t waves = (int64_t) p.T * ((per_t + q.hpw - 1) / q.hpw);
+    const int64_t rpw = p.D == 64 ? 4 : p.D == 128 ? 2 : 1, tg = (p.T + rpw - 1) / rpw;
+    q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, tg * per_t / 4096));
+    q.hpw = (int) ((per_t + (per_t + q.hpw - 1) / q.hpw - 1) / ((per_t + q.hpw - 1) / q.hpw));
+    if (const char* e = getenv("NS_PRE_HPW")) q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, atoi(e)));   // sweeps
+    const int64_t waves = tg * ((per_t + q.hpw - 1) / q.hpw);
     if ((waves + 3) / 4 > (int64_t) 1 << 31) return ns_fail(std::string(who) + ": too many rows");
     // whole 4-feature groups pair up: no rotation, adjacent pairs, or partners a multiple of 4 features away
     const bool vec = p.mode == ROPE_NONE || p.mode == ROPE_MG_PAIRS || (p.mode == ROPE_MG_HALVES ? p.D % 8 == 0 : p.n_rot % 8 == 0);

@@ -140,6 +140,40 @@ def test_fused_equals_the_separate_calls_bit_for_bit(ops, kt, rope, D, n_rot):
         assert np.array_equal(qo3.read(np.uint16), conv(qo.read(np.float32)))
 
 
+@pytest.mark.parametrize("kt", [0, 1, 2, 3])
+@pytest.mark.parametrize("rope,D,n_rot", [(1, 64, 32), (1, 128, 64), (3, 128, 0), (1, 256, 64)])
+def test_a_prompt_pass_equals_its_rows_in_small_passes(ops, kt, rope, D, n_rot):
+    """A prompt-sized pass has each wave walk several heads of its rows (across the q / k / v groups) and, for heads of
+    64 and 128, several rows at once; a pass of 100 rows takes a wave a head. Both must give the same bytes. The row
+    count leaves the last wave's row group part empty."""
+    g = ops.gpu
+    T, Hq, Hkv, p0, theta, eps, step = 3001, 6, 3, 11, 1e6, 1e-6, 100
+    cap = p0 + T
+    q, k, v = orc.randn(41, (T, Hq * D)), orc.randn(42, (T, Hkv * D)), orc.randn(43, (T, Hkv * D))
+    qw, kw = ((1.0 + 0.1 * orc.randn(44 + i, (D,))).astype(np.float32) for i in range(2))
+    qb, kb, vb, qwb, kwb = (DevBuf.of(g, a) for a in (q, k, v, qw, kw))
+    nb = Hkv * cap * kv_row_bytes(kt, D)
+    kc1, vc1, kc2, vc2 = (DevBuf(g, nb) for _ in range(4))
+    for b in (kc1, vc1, kc2, vc2):
+        b.fill(0x5A)
+    qo1, qo2 = DevBuf(g, T * Hq * D * 2), DevBuf(g, T * Hq * D * 2)
+    ops.pre_store(rope, 1, kt, False, qb, Hq * D, D, qo1, Hq * D, kb, Hkv * D, D, vb, Hkv * D, qwb, kwb, eps, n_rot, theta, T, Hq, Hkv, D, cap, p0, kc1, vc1)
+    for t0 in range(0, T, step):
+        n = min(step, T - t0)
+        ops.pre_store(rope, 1, kt, False, qb.view(t0 * Hq * D * 4, n * Hq * D * 4), Hq * D, D, qo2.view(t0 * Hq * D * 2, n * Hq * D * 2), Hq * D,
+                      kb.view(t0 * Hkv * D * 4, n * Hkv * D * 4), Hkv * D, D, vb.view(t0 * Hkv * D * 4, n * Hkv * D * 4), Hkv * D, qwb, kwb, eps, n_rot,
+                      theta, n, Hq, Hkv, D, cap, p0 + t0, kc2, vc2)
+    assert np.array_equal(qo1.read(np.uint16), qo2.read(np.uint16))
+    assert np.array_equal(kc1.read(np.uint8), kc2.read(np.uint8))
+    assert np.array_equal(vc1.read(np.uint8), vc2.read(np.uint8))
+    # and the rows are the oracle's: the last ones, where the angle is largest
+    if rope == 1 and kt == 0:
+        lo = T - 4
+        want = orc.q35_norm_rope(q[lo:], 4, Hq, D, qw, eps, n_rot, theta, p0 + lo)
+        got = orc.h2f(qo1.read(np.uint16).reshape(T, Hq * D)[lo:])
+        assert np.abs(got - want).max() <= tol(want, p0 + T) + 2.0 ** -11 * np.abs(want).max()
+
+
 def test_pre_store_rejects_bad_arguments(ops):
     from nextsycl_amd import Error
     g = ops.gpu
