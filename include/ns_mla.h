@@ -21,8 +21,11 @@ typedef struct ns_gpu ns_gpu;
 
 /* The absorbed decode up to the latent sum (BASELINE's MLA configuration ends here): qa [T][H][512 + R] already absorbed
  * and rotated ([k_b q_nope | q_pe]), element type qt (0 float32, 1 half); cache rows [512 + R] half; u [T][H][512] of
- * type qt = softmax_i(scale qa . c_i) c_i[:512]. R 64 or 0; T 1..16. `scratch`: ns_mla_decode_latent_scratch floats.
- * This library's own entry point (the reference computes u inside ns_ds2_mla_decode / ns_mla_attend_sel) */
+ * type qt = softmax_i(scale qa . c_i) c_i[:512], row t over cells 0 .. pos0 + t. R 64 or 0. T 1..16 is a decode or
+ * verify pass; a prompt's rows (any T) run 16 a pass on the queue. `scratch`: ns_mla_decode_latent_scratch floats.
+ * This library's own entry point: the reference computes u inside ns_ds2_mla_decode / ns_mla_attend_sel at decode
+ * widths and, for prompts and contexts past 8192 cells, as a chain of half GEMMs and a masked softmax over the same
+ * rows (llm/deepseek2/src/engine.rs:1165-1253; kernels/llm/glm5next/glm.cpp:208-277, 1042-1060) */
 int64_t ns_mla_decode_latent_scratch(int64_t T, int64_t H, int64_t pos0);
 int ns_mla_decode_latent(ns_gpu* g, int qt, const void* qa, const uint16_t* cache, void* u, int64_t T, int64_t H, int64_t R, int64_t pos0,
                          float scale, float* scratch);

@@ -45,6 +45,7 @@ constexpr int MTILE = 32, ML = 512;
 constexpr int mla_waves(int64_t group_rows, int64_t cells) { return group_rows <= 128 && cells <= 40960 ? 4 : 8; }
 // a split's partial of a row: u_s[512] = O_s / l_s as halfs (the split's own normalized result: bounded by the cache's
 // values, so half holds it; a quarter of the float32 form's bytes go to m and l), then m (log2 units), l, 2 of padding
+constexpr int MLA_PASS_MAX = 256;    // rows of a prompt a pass of the latent kernel takes at most
 constexpr int SEL_DENSE_MAX = 2560;   // cells of a dense row in a selection pass (the reference's bound)
 constexpr int PSTRIDE = ML / 2 + 4;   // in floats: 1040 bytes, rows stay 16-byte aligned
 
@@ -56,6 +57,7 @@ struct MlaParams {
     int64_t pos0;
     int64_t kbs;         // cells a split
     int ns;
+    int flat;            // 1: work-group id = split * nz + row group (passes of fewer than 8 splits)
     float sl2;
     float* part;         // [T * H][ns][PSTRIDE]: {half u_s[512], float m, l, -, -}
     // a row's own cells (GLM's selection): sel_cnt[t] >= 0 -> the pools sel[t K ..][0, sel_cnt[t]) of 4 cells each, then
@@ -95,8 +97,10 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
     // Work-group ids go round the 8 XCDs (each with its own L2). The row groups of one cell split read the same tiles:
     // they get consecutive ids on one XCD, so that they run side by side and a tile comes from memory once. The grid is
     // padded to 8 splits a round; the padding's work-groups leave at once.
+    // (A pass of fewer than 8 splits - many row groups over few cells, a prompt's - would leave XCDs idle that way: its
+    // row groups are dealt over the XCDs instead, a split's groups in id order.)
     const int xcd = blockIdx.x % 8, xj = blockIdx.x / 8;
-    const int z = xj % p.nz, split = (xj / p.nz) * 8 + xcd;
+    const int z = p.flat ? blockIdx.x % p.nz : xj % p.nz, split = p.flat ? blockIdx.x / p.nz : (xj / p.nz) * 8 + xcd;
     if (split >= p.ns) return;
     const int rows = p.T * p.H;
     // a row group: 128 consecutive (row, head) pairs of the pass, or (per_t) 128 heads of one row t
@@ -633,7 +637,7 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     const std::string w(who);
     if (T <= 0) return 0;
     if (H <= 0 || pos0 < 0) return ns_fail(w + ": heads and a position");
-    if (T > 16) return ns_fail(w + ": 1..16 rows (decode widths)");
+    if (T > MLA_PASS_MAX) return ns_fail(w + ": more rows than a pass holds");
     if (!qa || !cache || !u || !scratch) return ns_fail(w + ": a null buffer");
     if (((uintptr_t) qa | (uintptr_t) cache | (uintptr_t) scratch) % 16) return ns_fail(w + ": buffers 16-byte aligned");
     if (!(scale > 0.0f)) return ns_fail(w + ": a positive scale");
@@ -676,7 +680,8 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     p.K = (int) K;
     p.per_t = per_t;
     p.nz = (int) nz;
-    dim3 grid((unsigned) ((ns + 7) / 8 * 8 * nz));
+    p.flat = ns < 8;
+    dim3 grid((unsigned) (p.flat ? ns * nz : (ns + 7) / 8 * 8 * nz));
     if (ns_profile_mark(g, 0)) return -1;
     if (MW == 4) {
         if (q8) mla_decode_kernel<0, true, 4><<<grid, 256, 0, g->q>>>(p);
@@ -699,10 +704,31 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
 
 extern "C" {
 
-int64_t ns_mla_decode_latent_scratch(int64_t T, int64_t H, int64_t pos0) {
-    if (T <= 0 || H <= 0) return 0;
+// A prompt's rows (T past 16) go through the same kernel a pass of rows after another on the queue: 16 rows x H heads
+// already fill the kernel's row groups, and a pass's arithmetic (2 x rows H x cells x 1088 flop) outweighs its read of
+// the cache, so nothing is gained by a second kernel. Every row of a pass walks the cells of the pass's last row (the
+// later ones masked), so a pass is 64 rows (behind a short context the masked work is small in absolute terms and a
+// pass costs its two launches), doubling up to MLA_PASS_MAX while the masked part stays under a quarter. The scratch is
+// the largest pass's.
+static int64_t mla_pass_rows(int64_t before, int64_t left) {
+    int64_t w = 64;
+    while (w < MLA_PASS_MAX && 8 * w <= before) w *= 2;
+    return std::min(w, left);
+}
+static int64_t mla_pass_scratch(int64_t T, int64_t H, int64_t pos0) {
     const int64_t rows = T * H, cells = pos0 + T, MROWS = mla_waves(rows, cells) * 16, nz = (rows + MROWS - 1) / MROWS, kbs = mla_kbs(cells, nz);
     return rows * ((cells + kbs - 1) / kbs) * PSTRIDE;
+}
+
+int64_t ns_mla_decode_latent_scratch(int64_t T, int64_t H, int64_t pos0) {
+    if (T <= 0 || H <= 0) return 0;
+    if (T <= 16) return mla_pass_scratch(T, H, pos0);
+    int64_t need = 0;
+    for (int64_t t0 = 0, n; t0 < T; t0 += n) {
+        n = mla_pass_rows(pos0 + t0, T - t0);
+        need = std::max(need, mla_pass_scratch(n, H, pos0 + t0));
+    }
+    return need;
 }
 
 int ns_mla_decode_latent(ns_gpu* g, int qt, const void* qa, const uint16_t* cache, void* u, int64_t T, int64_t H, int64_t R, int64_t pos0,
@@ -711,8 +737,16 @@ int ns_mla_decode_latent(ns_gpu* g, int qt, const void* qa, const uint16_t* cach
     if (T <= 0) return 0;
     if (qt != 0 && qt != 1) return ns_fail("ns_mla_decode_latent: rows of type 0 (float32) or 1 (half)");
     if (R != 0 && R != 64) return ns_fail("ns_mla_decode_latent: a rope part of 64 (DeepSeek's [512 | 64] rows) or none");
-    return mla_latent(g, "ns_mla_decode_latent", qt, qt, (int) R, false, qa, cache, u, T, H, pos0, scale, scratch,
-                      (size_t) ns_mla_decode_latent_scratch(T, H, pos0));
+    if (H <= 0 || pos0 < 0) return ns_fail("ns_mla_decode_latent: heads and a position");
+    if (!qa || !u) return ns_fail("ns_mla_decode_latent: a null buffer");
+    const int64_t e = qt == 0 ? 4 : 2;
+    for (int64_t t0 = 0, n; t0 < T; t0 += n) {
+        n = T <= 16 ? T : mla_pass_rows(pos0 + t0, T - t0);
+        if (mla_latent(g, "ns_mla_decode_latent", qt, qt, (int) R, false, (const char*) qa + t0 * H * (ML + R) * e, cache, (char*) u + t0 * H * ML * e, n, H,
+                       pos0 + t0, scale, scratch, (size_t) mla_pass_scratch(n, H, pos0 + t0)))
+            return -1;
+    }
+    return 0;
     NS_CATCH
 }
 
@@ -754,7 +788,7 @@ int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, i
                       const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
     NS_TRY
     if (T <= 0) return 0;
-    if (L != 512) return ns_fail("ns_mla_attend_sel: latent width 512");
+    if (L != 512 || T > 16) return ns_fail("ns_mla_attend_sel: latent width 512, at most 16 rows");
     return mla_latent(g, "ns_mla_attend_sel", 0, 0, 0, false, qa, c, u, T, H, pos0, scale, g->own_scratch, g->own_scratch_floats, sel, sel_cnt, K);
     NS_CATCH
 }

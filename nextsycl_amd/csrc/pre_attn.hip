@@ -1,12 +1,14 @@
 // pre_attn.hip: what runs in front of attention on every token - q / k RMS norm, rotary positions, the KV store - for
 // gfx950: the reference's separate entry points and one fused launch (norm + rotate + store, k never written as
-// float32). Bound: HBM, negligible volume (a few KB a token); the point of the fused form is two launches fewer a layer.
+// float32). Bound: HBM - a few KB a token at a decode step (the point of the fused form is two launches fewer a layer),
+// (Hq + 2 Hkv) D 4 bytes read and about half that written a row in a prompt pass.
 //
 // One wave a (row, head) - two or four rows of a head where a head row is 128 or 64 features, so no lane idles; a lane
-// four consecutive features (D up to 256; more: a lane several groups of four). In a prompt pass a wave walks several
-// heads of its rows on one evaluation of the rotation. Every load of a head precedes its stores, so source and destination may be the same rows. The arithmetic of an output
-// feature is one function (rope_feature) whatever entry point asks for it, and the quantized rows are kv_pack.hpp's:
-// the fused launch gives bit for bit what the separate calls give. Compiled with -ffp-contract=off (the packers).
+// four consecutive features (D up to 256; more: a lane two groups of four). In a prompt pass a wave walks several heads
+// of its rows on one evaluation of the rotation, the next head's loads in flight while it works on this one. Every load
+// of a head precedes its stores, so source and destination may be the same rows. The arithmetic of an output feature
+// is the same whatever entry point asks for it, and the quantized rows are kv_pack.hpp's: the fused launch gives bit
+// for bit what the separate calls give. Compiled with -ffp-contract=off (the packers).
 //
 // Reference behaviour kept: kernels/llm/qwen35/q35.cpp:220-279,350-386 (rotate-half over the first n_rot, angle
 // pos * theta^(-2 k / n_rot); interleaved position sections), kernels/llm/museglimmer/mg.cpp:157-190 (adjacent pairs or

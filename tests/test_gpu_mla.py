@@ -67,6 +67,25 @@ def test_latent_decode_seeded_shapes(ops, T, H, R, pos0, qt):
     _close(got, orc.mla_f64(qf, cache, T, H, pos0, scale, 512, R), "latent decode vs float64 closed form")
 
 
+@pytest.mark.parametrize("T,H,R,pos0,qt", [(40, 16, 64, 100, F16), (33, 128, 64, 0, F32), (17, 8, 0, 2000, F32), (64, 20, 64, 37, F16),
+                                            (300, 16, 64, 250, F16), (1100, 8, 64, 0, F32), (70, 16, 0, 5000, F32), (300, 4, 64, 1900, F16)])
+def test_latent_prompt_widths(ops, T, H, R, pos0, qt):
+    """A prompt's rows through the same entry point (the reference's GEMM chain + masked softmax over these rows:
+    llm/deepseek2/src/engine.rs:1165-1253): row t over cells 0 .. pos0 + t, against the float64 closed form. The passes
+    are 64 rows, wider (128, 256) behind long enough contexts: the cases cross each width."""
+    n = pos0 + T
+    cache = orc.f2h(orc.randn(9, (n, 512 + R), 0.5))
+    qa = orc.randn(10, (T, H, 512 + R))
+    scale = 1.0 / np.sqrt(192.0)
+    qd, qf = (qa, qa) if qt == F32 else (orc.f2h(qa), orc.h2f(orc.f2h(qa)))
+    got = _latent(ops, qt, qd, cache, T, H, R, pos0, scale)
+    _close(got, orc.mla_f64(qf, cache, T, H, pos0, scale, 512, R), "prompt rows vs float64 closed form")
+    # split anywhere, the rows are the same within the tolerance (another pass width sums in another order)
+    lo = T // 2
+    alone = _latent(ops, qt, qd[lo:], cache, T - lo, H, R, pos0 + lo, scale)
+    _close(alone, got[lo:], "the second half on its own")
+
+
 def test_config4_mla_decode_32k(ops):
     """BASELINE configs[3]: 128 heads, 512 latent + 64 rope, latent cache f16 ~N(0, 0.5), absorbed q of 576 a head,
     KV length 32768, scale 1/sqrt(192); output the 512-d latent a head, f16."""
