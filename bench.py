@@ -37,6 +37,10 @@ WORKLOADS = {
     "verify64k": ("decode", 4, 32, 4, 128, 65540, 0, 1, "MTP verify, 4 draft rows on a 65536-token f16 KV cache, 32 q heads / 4 kv heads, head_dim 128 (BASELINE configs[4])"),
     # MLA: Hq = heads, Hkv unused (one latent row a position), D = 512 latent + 64 rope
     "mla32k": ("mla", 1, 128, 1, 576, 32768, 0, 1, "DeepSeek-style absorbed MLA decode, 128 heads, 512 latent + 64 rope, f16 latent cache, KV 32768 (BASELINE configs[3])"),
+    # the callers either side of the path: a prompt chunk through the latent MLA entry point (the reference's GEMM chain),
+    # and the step in front of attention (q / k norm + rotary + KV store in one launch) at the prefill configuration
+    "mla_prompt8k": ("mla", 256, 128, 1, 576, 8192 + 256, 0, 1, "absorbed MLA, a 256-row prompt chunk behind 8192 cells, 128 heads, f16 latent cache"),
+    "pre_store8k": ("pre", 8192, 40, 8, 128, 8192, 3, 2, "q / k RMS norm + rotary + KV store, one launch, 8192 rows, 40 q / 8 kv heads of 128, bf16 rows and cache"),
 }
 
 
@@ -71,6 +75,15 @@ class Workload:
         self.p0 = kv - T
         self.flops, self.bytes = algorithmic(self.kind, T, Hq, Hkv, D, kv, kt, qt)
         self.i = 0
+        if self.kind == "pre":
+            rb = kv_bytes(kt, D)
+            self.bytes = T * (Hq + 2 * Hkv) * D * 4 + T * Hq * D * 2 + 2 * T * Hkv * rb       # float32 rows in; q rows, cache rows out
+            self.flops = 0
+            self.src = [DevBuf.of(g, orc.randn(0xB0B + i, (T, h * D))) for i, h in enumerate((Hq, Hkv, Hkv))]
+            self.w = [DevBuf.of(g, (1.0 + 0.1 * orc.randn(0xD00D + i, (D,))).astype(np.float32)) for i in range(2)]
+            self.out = DevBuf(g, T * Hq * D * 2)
+            self.caches = [(DevBuf(g, Hkv * kv * rb), DevBuf(g, Hkv * kv * rb)) for _ in range(nbuf)]
+            return
         if self.kind == "mla":
             self.caches = []
             host = orc.f2h(orc.randn(0xB0B, (kv, 576), 0.5))
@@ -107,7 +120,11 @@ class Workload:
         kc, vc = self.caches[self.i % len(self.caches)]
         self.i += 1
         o = self.ops
-        if self.kind == "mla":
+        if self.kind == "pre":
+            q, k, v = self.src
+            o.pre_store(1, self.qt, self.kt, False, q, self.Hq * self.D, self.D, self.out, self.Hq * self.D, k, self.Hkv * self.D, self.D, v,
+                        self.Hkv * self.D, self.w[0], self.w[1], 1e-6, self.D // 2, 1e6, self.T, self.Hq, self.Hkv, self.D, self.kv, 0, kc, vc)
+        elif self.kind == "mla":
             o.mla_decode_latent(1, self.q, kc, self.out, self.T, self.Hq, 64, self.p0, 192.0 ** -0.5, self.scratch)
         elif self.kind == "prefill":
             o.prompt(self.qt, self.kt, self.q, self.Hq * self.D, kc, vc, self.T, self.Hq, self.Hkv, self.D, self.kv, 0, self.out)
@@ -141,6 +158,9 @@ def timed(w, steps, warmup):
     # the events open gaps between the launches that the throughput pass must not see). Steps run back to back in short
     # runs and the last step of each run is read, so the kernel is timed on a busy stream like the one above - a
     # launch bracketed on an idle stream reads several microseconds long
+    if w.kind == "pre" or (w.kind == "mla" and w.T > 16):
+        # one launch a step (no marks inside) / several passes a step: the step itself, launched back to back, is the figure
+        return ms, ms * 1e6, 0.0
     w.ops.profile(True)
     main = merge = 0.0
     n = max(3, min(steps, 20))
@@ -167,6 +187,10 @@ def roofline(w, main_ns):
 
 
 def _roofline(w, main_ns):
+    if w.kind == "pre":
+        ach = w.bytes / main_ns
+        return {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
+                "kernel": "pre_attn_kernel", "kernel_us": round(main_ns / 1e3, 2)}
     if w.kind == "mla":
         ach = w.flops / main_ns / 1e3
         return {"bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_TFLOPS_BF16, "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS_BF16, 4),
@@ -185,6 +209,28 @@ def cpu_baseline(name):
     from oracle import orc
 
     kind, T, Hq, Hkv, D, kv, kt, qt, _ = WORKLOADS[name]
+    if kind == "pre":
+        # the q and k rows' norm + rotary through the numpy restatement (one core); the store is left out
+        w = np.ones(D, np.float32)
+        xq, xk = orc.randn(0xB0B, (T, Hq * D)), orc.randn(0xB0C, (T, Hkv * D))
+        t0 = time.perf_counter()
+        orc.q35_norm_rope(xq, T, Hq, D, w, 1e-6, D // 2, 1e6, 0)
+        orc.q35_norm_rope(xk, T, Hkv, D, w, 1e-6, D // 2, 1e6, 0)
+        dt = time.perf_counter() - t0
+        return {"value": round(T * (Hq + Hkv) * D * 8 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "norm + rotary of all %d q and k rows (float32 in and out), numpy restatement, no store" % T, "seconds": round(dt, 2)}
+    if kind == "mla":
+        # the restated kernel order on the last rows of the workload
+        rows = min(T, 2)
+        cache = orc.f2h(orc.randn(0xB0B, (kv, 576), 0.5))
+        qa = orc.h2f(orc.f2h(orc.randn(0xA11CE, (rows, Hq, 576))))
+        p0 = kv - rows
+        t0 = time.perf_counter()
+        orc.mla_decode_u(qa, cache, rows, Hq, p0, 192.0 ** -0.5)
+        dt = time.perf_counter() - t0
+        flops = sum(2 * Hq * (p0 + r + 1) * 1088 for r in range(rows))
+        return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+                "sample": "the last %d of %d rows, all %d heads, the whole %d-cell cache, restated kernel order (numpy)" % (rows, T, Hq, kv), "seconds": round(dt, 2)}
     k = orc.randn(0xB0B, (kv, Hkv * D))
     v = orc.randn(0xC0FFEE, (kv, Hkv * D))
     kc, vc = orc.kv_store(kt, k, v, Hkv, D, kv, 0)
@@ -247,14 +293,16 @@ def main():
     def run(name, steps, warmup):
         kind = WORKLOADS[name][0]
         # decode: rotate distinct caches totalling > 512 MB so the keys are read from HBM
-        nbuf = 1 if kind == "prefill" else 16 if kind == "mla" else max(4, int(np.ceil(600e6 / (2 * WORKLOADS[name][3] * WORKLOADS[name][5] * kv_bytes(WORKLOADS[name][6], WORKLOADS[name][4])))))
+        nbuf = 1 if kind == "prefill" else 16 if kind == "mla" else 4 if kind == "pre" else max(4, int(np.ceil(600e6 / (2 * WORKLOADS[name][3] * WORKLOADS[name][5] * kv_bytes(WORKLOADS[name][6], WORKLOADS[name][4])))))
         nbuf = min(nbuf, 40)
         w = Workload(ops, name, nbuf)
         ms, main_ns, merge_ns = timed(w, steps, warmup)
         return w, ms, main_ns, merge_ns
 
     w, ms, main_ns, merge_ns = run(a.workload, a.steps, a.warmup)
-    if w.kind == "mla":
+    if w.kind == "pre":
+        metric, unit, value = "pre-attention step HBM GB/s (algorithmic bytes), 1 MI355X", "GB/s", w.bytes / (ms * 1e-3) / 1e9
+    elif w.kind == "mla":
         metric, unit, value = "MLA decode attention TFLOP/s, 1 MI355X", "TFLOP/s", w.flops / (ms * 1e-3) / 1e12
     elif w.kind == "prefill":
         metric, unit, value = "prefill attention TFLOP/s (causal flops), 1 MI355X", "TFLOP/s", w.flops / (ms * 1e-3) / 1e12
@@ -276,13 +324,13 @@ def main():
     del w
     if not a.no_extra:
         others = {}
-        for name in ("decode32k", "decode4k", "decode128k_q8", "verify64k", "mla32k", "prefill8k"):
+        for name in ("decode32k", "decode4k", "decode128k_q8", "verify64k", "mla32k", "prefill8k", "mla_prompt8k", "pre_store8k"):
             if name == a.workload:
                 continue
             ww, m2, k2, g2 = run(name, max(10, a.steps), a.warmup)
             r = roofline(ww, k2)
-            others[name] = {"ms_per_step": round(m2, 5), "step_" + ("TFLOP/s" if ww.kind != "decode" else "GB/s"):
-                            round((ww.flops / (m2 * 1e-3) / 1e12) if ww.kind != "decode" else (ww.bytes / (m2 * 1e-3) / 1e9), 2), "roofline": r,
+            others[name] = {"ms_per_step": round(m2, 5), "step_" + ("TFLOP/s" if ww.kind not in ("decode", "pre") else "GB/s"):
+                            round((ww.flops / (m2 * 1e-3) / 1e12) if ww.kind not in ("decode", "pre") else (ww.bytes / (m2 * 1e-3) / 1e9), 2), "roofline": r,
                             "merge_kernel_us": round(g2 / 1e3, 2)}
             del ww
         line["others"] = others
