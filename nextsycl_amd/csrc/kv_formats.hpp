@@ -12,10 +12,7 @@ __device__ __forceinline__ uint16_t f32_to_f16(float f) {
 __device__ __forceinline__ float f16_to_f32(uint16_t b) { return (float) __builtin_bit_cast(_Float16, b); }
 // float -> bfloat16 bits, round to nearest even; NaN stays NaN
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-    uint32_t x = __builtin_bit_cast(uint32_t, f);
-    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t) ((x >> 16) | 0x40u);
-    x += 0x7fffu + ((x >> 16) & 1u);
-    return (uint16_t) (x >> 16);
+    return __builtin_bit_cast(uint16_t, (__bf16) f);        // gfx950 converts in hardware (v_cvt_pk_bf16_f32)
 }
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __builtin_bit_cast(float, (uint32_t) b << 16); }
 

@@ -157,6 +157,18 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
     }
     // the distance to a rotated feature's partner
     const int pdist = p.mode == ROPE_MG_HALVES ? D / 2 : p.n_rot / 2;
+    // Every rotary form is y = me cos -/+ partner sin, minus for the first feature of a pair (a - b is a + (-b) bit for
+    // bit, and the forms that write the sum the other way round add the same two products): the sign goes into the sine
+    // once, and a feature is one multiply-add pair with no branch. (VEC only; the other instance keeps rope_feature.)
+    float rss[MAXG * 4];
+#pragma unroll
+    for (int q = 0; q < MAXG * 4; ++q) {
+        const int i = li * 4 + (q >> 2) * 256 + (q & 3);
+        const bool first = p.mode == ROPE_MG_PAIRS ? (q & 1) == 0 : i < pdist;
+        rss[q] = first ? -rs[q] : rs[q];
+    }
+    const bool d_pow2 = (D & (D - 1)) == 0;
+    const float inv_d = 1.0f / (float) D;                  // exact for a power of two: s * inv_d is s / D bit for bit
     // What a head needs from memory: its group, its row, the lane's own features and (VEC) their partners and weights.
     // Every load is unconditional - a lane with nothing to do reads a valid address and drops the value - so the loads
     // of the NEXT head can be in flight, counted, while this head is worked on: a head then costs about one memory
@@ -230,7 +242,7 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
             pair32(s, a, b);
             s = a + b;
         }
-        const float ms = s / (float) D + p.eps;
+        const float ms = (d_pow2 ? s * inv_d : s / (float) D) + p.eps;
         inv = p.inv_sqrt ? 1.0f / sqrtf(ms) : rsqrtf(ms);
     }
     // ---- this lane's features. Where the partner of a rotated feature lies a whole number of 4-feature groups away
@@ -250,23 +262,17 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
             const float4 xp4 = cur.xp[c], wo4 = cur.wo[c], wp4 = cur.wp[c];
             const float xv[4] = {xo[c].x, xo[c].y, xo[c].z, xo[c].w}, xq[4] = {xp4.x, xp4.y, xp4.z, xp4.w};
             const float wv[4] = {wo4.x, wo4.y, wo4.z, wo4.w}, wq[4] = {wp4.x, wp4.y, wp4.z, wp4.w};
+            float me[4], pt[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const float me = G.w ? xv[j] * inv * wv[j] : xv[j];
-                if (!rotated) {
-                    y[c][j] = me;
-                    continue;
-                }
-                const float cs = rc[c * 4 + j], sn = rs[c * 4 + j];
-                if (p.mode == ROPE_MG_PAIRS) {
-                    const float pt = G.w ? xv[j ^ 1] * inv * wv[j ^ 1] : xv[j ^ 1];
-                    y[c][j] = (j & 1) == 0 ? me * cs - pt * sn : pt * sn + me * cs;
-                } else {
-                    const float pt = G.w ? xq[j] * inv * wq[j] : xq[j];
-                    const bool first = i < pdist;
-                    if (p.mode == ROPE_Q35) y[c][j] = first ? me * cs - pt * sn : me * cs + pt * sn;
-                    else y[c][j] = first ? me * cs - pt * sn : pt * sn + me * cs;
-                }
+                me[j] = G.w ? xv[j] * inv * wv[j] : xv[j];
+                pt[j] = G.w ? xq[j] * inv * wq[j] : xq[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float other = p.mode == ROPE_MG_PAIRS ? me[j ^ 1] : pt[j];
+                const float r = me[j] * rc[c * 4 + j] + other * rss[c * 4 + j];
+                y[c][j] = rotated ? r : me[j];
             }
         }
     } else {
