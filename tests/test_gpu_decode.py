@@ -198,3 +198,25 @@ def test_argument_errors(ops):
     assert k.attn_decode_t(raw, 0, 0, 0, None, 0, None, None, 0, 4, 1, 128, 64, 0, 0, 0.0, None, None) == 0
     with pytest.raises(Error):
         ops.decode(F32, 0, DevBuf(g, 16), 512, b, b, 1, 4, 1, 128, 64, 0, b, b)
+
+
+def test_alternating_shapes_repeat_their_bits(ops):
+    """Launches of several shapes alternate on one queue (other split counts, head counts, row tiles, sharing the scratch
+    sizes' rule): every launch gives the bits of its shape's first launch, and those are the oracle's rows."""
+    g = ops.gpu
+    shapes = [(1, 32, 8, 128, 3000), (2, 8, 2, 128, 700), (1, 16, 16, 128, 129), (1, 8, 2, 256, 2500), (4, 32, 4, 128, 2049)]
+    state = []
+    for i, (T, Hq, Hkv, D, p0) in enumerate(shapes):
+        cap = p0 + T
+        kc, vc = make_kv(0, Hkv, D, cap, cap, cfg=i)
+        qd, qf = make_q(F32, T, Hq, D, cfg=i)
+        state.append((T, Hq, Hkv, D, p0, cap, qd, kc, vc, (DevBuf.of(g, kc), DevBuf.of(g, vc)), orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, cap, p0)))
+    first = {}
+    for rep in range(10):
+        for i, (T, Hq, Hkv, D, p0, cap, qd, kc, vc, bufs, ref) in enumerate(state):
+            got, raw = gpu_decode(ops, F32, 0, qd, kc, vc, T, Hq, Hkv, D, cap, p0, bufs=bufs)
+            if rep == 0:
+                first[i] = raw.copy()
+                check_close(got, ref, F32, "shape %d" % i)
+            else:
+                assert np.array_equal(raw, first[i]), "launch %d of shape %d" % (rep, i)
