@@ -177,7 +177,7 @@ def timed(w, steps, warmup):
 # HBM bytes per launch of each workload's dominant kernel as rocprofv3 counted them (FETCH_SIZE + WRITE_SIZE per dispatch,
 # each scaled by what the same counter reads for a plain 1 GiB copy kernel); the runs are summarized under profiles/.
 # A counter run cannot be made from inside this script, so these are the recorded figures of those runs, not live ones.
-MEASURED_TRAFFIC = {"prefill8k": 183.5e6 + 83.9e6, "decode32k": 134.5e6 + 1.1e6, "mla32k": 39.5e6 + 17.4e6}
+MEASURED_TRAFFIC = {"prefill8k": 183.5e6 + 83.9e6, "decode32k": 134.5e6 + 1.1e6, "mla32k": 39.5e6 + 17.4e6, "pre_store8k": 235.1e6 + 117.4e6}
 
 
 def roofline(w, main_ns):
