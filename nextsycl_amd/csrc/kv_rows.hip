@@ -1,5 +1,6 @@
-// kv_rows.hip: the rows of a span of positions moved between caches of different geometry - a ring (slot = position %
-// cap) into position order for a checkpoint, a checkpoint back into a ring, one session's rings into another's. The
+// kv_rows.hip: byte work on device buffers - a queued fill (ns_fill), and the rows of a span of positions moved between
+// caches of different geometry: a ring (slot = position % cap) into position order for a checkpoint, a checkpoint back
+// into a ring, one session's rings into another's. The
 // reference's engines do this on the host as runs of copies, one or two a head and cache
 // (llm/museglimmer/src/engine.rs:1334-1346, 1475-1528; llm/qwen35/src/engine.rs:2977-3011); here it is one launch a
 // cache, every head at once, so a checkpoint is a handful of launches and ONE copy across PCIe.
@@ -7,6 +8,8 @@
 // Byte work, HBM-bound: a thread moves one unit (16, 8, 4 or 2 bytes - the widest that divides the row and the
 // addresses), consecutive threads consecutive units of a row and then the next position's row, so a wave reads and
 // writes whole lines except where the ring wraps. Bytes a launch: 2 x heads x positions x row bytes.
+#include <algorithm>
+
 #include "ns_internal.hpp"
 #include "ns_attn.h"
 
@@ -41,9 +44,35 @@ void launch_rows(ns_gpu* g, RowsCopy p, int64_t heads, int64_t row_bytes) {
     kv_rows_copy_kernel<U><<<dim3((unsigned) ((units + 255) / 256), (unsigned) heads), 256, 0, g->q>>>(p);
 }
 
+// bytes set to one value: 16-byte stores over the aligned body, byte stores over the ends
+__global__ void fill_kernel(uint8_t* dst, uint32_t word, uint32_t head, uint64_t units, uint32_t tail) {
+    const uint64_t i = (uint64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < units) reinterpret_cast<uint4*>(dst + head)[i] = make_uint4(word, word, word, word);
+    if (i < head) dst[i] = (uint8_t) word;
+    if (i < tail) dst[head + units * 16 + i] = (uint8_t) word;
+}
+
 }  // namespace
 
 extern "C" {
+
+// A queued fill (kernels/ns/ns.h's ns_fill). A kernel of this library's own rather than a memset node: a caller may
+// capture the queue into a graph, and memset nodes have replayed wrongly on this platform.
+int ns_fill(ns_gpu* g, void* dst, uint8_t value, size_t bytes) {
+    NS_TRY
+    if (!bytes) return 0;
+    if (!dst) return ns_fail("ns_fill: no buffer");
+    NS_HIP(hipSetDevice(g->dev));
+    uint8_t* d = (uint8_t*) dst;
+    const size_t head = std::min<size_t>(bytes, (16 - (uintptr_t) d % 16) % 16), units = (bytes - head) / 16, tail = bytes - head - units * 16;
+    const size_t threads = std::max<size_t>(units, 16), blocks = (threads + 255) / 256;
+    if (blocks >= (size_t) 1 << 31) return ns_fail("ns_fill: more than 2^39 bytes");
+    const uint32_t word = value * 0x01010101u;
+    fill_kernel<<<(unsigned) blocks, 256, 0, g->q>>>(d, word, (uint32_t) head, (uint64_t) units, (uint32_t) tail);
+    NS_LAUNCHED("ns_fill");
+    return 0;
+    NS_CATCH
+}
 
 int ns_attn_kv_rows_copy(ns_gpu* g, const void* src, int64_t scap, int64_t sbase, void* dst, int64_t dcap, int64_t dbase, int64_t heads,
                          int64_t row_bytes, int64_t from, int64_t to) {

@@ -290,15 +290,6 @@ int ns_elapsed(ns_gpu* g, int64_t t0, int64_t t1, double* ns) {
     NS_CATCH
 }
 
-int ns_fill(ns_gpu* g, void* dst, uint8_t value, size_t bytes) {
-    NS_TRY
-    if (!bytes) return 0;
-    NS_HIP(hipSetDevice(g->dev));
-    NS_HIP(hipMemsetAsync(dst, value, bytes, g->q));
-    return 0;
-    NS_CATCH
-}
-
 int ns_sync(ns_gpu* g) {
     NS_TRY
     NS_HIP(hipSetDevice(g->dev));

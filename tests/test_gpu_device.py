@@ -40,6 +40,19 @@ def test_copies_roundtrip(gpu):
     assert np.array_equal(v.read(np.uint32), x[256:256 + 1024])
 
 
+@pytest.mark.parametrize("at,n", [(0, 1), (3, 77), (5, 3), (16, 4096), (1, 15), (15, 17), (7, 100001), (0, 1 << 20)])
+def test_fill_any_alignment(gpu, at, n):
+    """ns_fill is a kernel of the library's own (16-byte stores over the aligned body, byte stores over the ends): the
+    span gets the value, the bytes either side keep theirs."""
+    total = at + n + 37
+    b = DevBuf(gpu, total)
+    b.fill(0x11)
+    a = gpu.api
+    assert a.fill(gpu.raw, b.ptr + at, 0xAB, n) == 0
+    got = b.read(np.uint8)
+    assert (got[:at] == 0x11).all() and (got[at:at + n] == 0xAB).all() and (got[at + n:] == 0x11).all()
+
+
 def test_copy_2d(gpu):
     a = gpu.api
     src = np.arange(32 * 64, dtype=np.uint8).reshape(32, 64)
