@@ -707,11 +707,11 @@ extern "C" {
 // A prompt's rows (T past 16) go through the same kernel a pass of rows after another on the queue: 16 rows x H heads
 // already fill the kernel's row groups, and a pass's arithmetic (2 x rows H x cells x 1088 flop) outweighs its read of
 // the cache, so nothing is gained by a second kernel. Every row of a pass walks the cells of the pass's last row (the
-// later ones masked), so a pass is 64 rows (behind a short context the masked work is small in absolute terms and a
-// pass costs its two launches), doubling up to MLA_PASS_MAX while the masked part stays under a quarter. The scratch is
+// later ones masked), so a pass is 128 rows (behind a short context the masked work is small in absolute terms and a
+// pass costs its two launches), 256 = MLA_PASS_MAX once the masked part stays under a quarter. The scratch is
 // the largest pass's.
 static int64_t mla_pass_rows(int64_t before, int64_t left) {
-    int64_t w = 64;
+    int64_t w = 128;
     while (w < MLA_PASS_MAX && 8 * w <= before) w *= 2;
     return std::min(w, left);
 }

@@ -72,7 +72,7 @@ def test_latent_decode_seeded_shapes(ops, T, H, R, pos0, qt):
 def test_latent_prompt_widths(ops, T, H, R, pos0, qt):
     """A prompt's rows through the same entry point (the reference's GEMM chain + masked softmax over these rows:
     llm/deepseek2/src/engine.rs:1165-1253): row t over cells 0 .. pos0 + t, against the float64 closed form. The passes
-    are 64 rows, wider (128, 256) behind long enough contexts: the cases cross each width."""
+    are 128 rows, 256 behind long enough contexts: the cases cross both widths."""
     n = pos0 + T
     cache = orc.f2h(orc.randn(9, (n, 512 + R), 0.5))
     qa = orc.randn(10, (T, H, 512 + R))
