@@ -18,7 +18,10 @@ def tol(ref, pos):
     return (4.0 * (1.0 + pos) * 2.0 ** -23 + 2e-6) * np.abs(ref).max()
 
 
-@pytest.mark.parametrize("D,n_rot,p0", [(128, 64, 3), (256, 64, 4095), (128, 128, 100000), (64, 32, 17), (128, 0, 5)])
+@pytest.mark.parametrize("D,n_rot,p0", [(128, 64, 3), (256, 64, 4095), (128, 128, 100000), (64, 32, 17), (128, 0, 5),
+                                        # rotated widths that are not whole 4-feature groups (the feature-by-feature
+                                        # instance), and heads past 256 features (two groups a lane), both ways
+                                        (128, 20, 9), (64, 6, 1000), (512, 64, 77), (384, 20, 5), (48, 12, 30)])
 def test_q35_norm_rope(ops, D, n_rot, p0):
     g = ops.gpu
     T, H, theta, eps = 6, 5, 1e6, 1e-6
@@ -58,9 +61,10 @@ def test_mg_norm_rope_in_place(ops, rope):
     assert np.abs(xb.read(np.float32).reshape(T, H * D) - want).max() <= tol(want, p0 + T)
 
 
-def test_minimaxm3_rope_and_attn_post(ops):
+@pytest.mark.parametrize("n_rot", [64, 20])        # whole 4-feature groups, and a width that is not
+def test_minimaxm3_rope_and_attn_post(ops, n_rot):
     g = ops.gpu
-    H, G, IH, HD, n_rot, base, eps, pos = 8, 2, 3, 128, 64, 5e6, 1e-6, 4321
+    H, G, IH, HD, base, eps, pos = 8, 2, 3, 128, 5e6, 1e-6, 4321
     T, row = 3, H * HD + 64
     x = orc.randn(17, (T, row))
     xb = DevBuf.of(g, x)
