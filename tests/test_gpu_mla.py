@@ -86,6 +86,26 @@ def test_latent_prompt_widths(ops, T, H, R, pos0, qt):
     _close(alone, got[lo:], "the second half on its own")
 
 
+def test_prompt_chunk_at_bench_size(ops):
+    """bench.py's `mla_prompt8k` at its full size (256 rows behind 8192 cells, 128 heads, half rows): the first and the
+    last row against the float64 closed form, and the last 16 rows against the same rows as a decode-width pass of their
+    own (another pass width, another summation order: within the tolerance)."""
+    g = ops.gpu
+    T, H, R, pos0 = 256, 128, 64, 8192
+    n = pos0 + T
+    scale = 1.0 / np.sqrt(192.0)
+    cache = orc.f2h(orc.randn(21, (n, 512 + R), 0.5))
+    qa = orc.f2h(orc.randn(22, (T, H, 512 + R)))
+    got = _latent(ops, F16, qa, cache, T, H, R, pos0, scale)
+    qf = orc.h2f(qa)
+    for t in (0, T - 1):
+        ref = orc.mla_f64(qf[t:t + 1], cache[:pos0 + t + 1], 1, H, pos0 + t, scale, 512, R)
+        _close(got[t:t + 1], ref, "row %d vs float64 closed form" % t)
+    lo = T - 16
+    alone = _latent(ops, F16, qa[lo:], cache, 16, H, R, pos0 + lo, scale)
+    _close(alone, got[lo:], "the last 16 rows as a pass of their own")
+
+
 def test_config4_mla_decode_32k(ops):
     """BASELINE configs[3]: 128 heads, 512 latent + 64 rope, latent cache f16 ~N(0, 0.5), absorbed q of 576 a head,
     KV length 32768, scale 1/sqrt(192); output the 512-d latent a head, f16."""
