@@ -178,6 +178,33 @@ def test_a_prompt_pass_equals_its_rows_in_small_passes(ops, kt, rope, D, n_rot):
         assert np.abs(got - want).max() <= tol(want, p0 + T) + 2.0 ** -11 * np.abs(want).max()
 
 
+def test_pre_store_at_bench_size(ops):
+    """bench.py's `pre_store8k` at its full size (8192 rows, 40 q / 8 kv heads of 128, bfloat16 rows and cache): the
+    caches bit for bit what the separate calls store, q rows bit for bit the separate call's float32 rows rounded, and
+    sampled rows against the oracle."""
+    g = ops.gpu
+    T, Hq, Hkv, D, n_rot, theta, eps, p0, kt = 8192, 40, 8, 128, 64, 1e6, 1e-6, 0, 3
+    cap = T
+    q, k, v = orc.randn(51, (T, Hq * D)), orc.randn(52, (T, Hkv * D)), orc.randn(53, (T, Hkv * D))
+    qw, kw = ((1.0 + 0.1 * orc.randn(54 + i, (D,))).astype(np.float32) for i in range(2))
+    qb, kb, vb, qwb, kwb = (DevBuf.of(g, a) for a in (q, k, v, qw, kw))
+    nb = Hkv * cap * kv_row_bytes(kt, D)
+    kc1, vc1, kc2, vc2 = (DevBuf(g, nb) for _ in range(4))
+    qo = DevBuf(g, T * Hq * D * 2)
+    ops.pre_store(1, 2, kt, False, qb, Hq * D, D, qo, Hq * D, kb, Hkv * D, D, vb, Hkv * D, qwb, kwb, eps, n_rot, theta, T, Hq, Hkv, D, cap, p0, kc1, vc1)
+    qf, kn = DevBuf(g, T * Hq * D * 4), DevBuf(g, T * Hkv * D * 4)
+    ops.q35_qk_norm_rope(qb, Hq * D, D, qf, Hq * D, T, Hq, D, qwb, eps, n_rot, theta, p0)
+    ops.q35_qk_norm_rope(kb, Hkv * D, D, kn, Hkv * D, T, Hkv, D, kwb, eps, n_rot, theta, p0)
+    ops.kv_store(kt, kn, Hkv * D, vb, Hkv * D, T, Hkv, D, cap, p0, kc2, vc2)
+    assert np.array_equal(kc1.read(np.uint8), kc2.read(np.uint8))
+    assert np.array_equal(vc1.read(np.uint8), vc2.read(np.uint8))
+    got = qo.read(np.uint16).reshape(T, Hq * D)
+    assert np.array_equal(got, orc.f2bf(qf.read(np.float32)).reshape(T, Hq * D))
+    for t in (0, 1, 4097, T - 1):
+        want = orc.q35_norm_rope(q[t:t + 1], 1, Hq, D, qw, eps, n_rot, theta, p0 + t)
+        assert np.abs(orc.bf2f(got[t:t + 1]) - want).max() <= tol(want, p0 + t) + 2.0 ** -8 * np.abs(want).max()
+
+
 def test_pre_store_rejects_bad_arguments(ops):
     from nextsycl_amd import Error
     g = ops.gpu
