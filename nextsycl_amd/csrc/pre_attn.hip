@@ -346,10 +346,11 @@ int launch_pre(ns_gpu* g, const PreParams& p, const char* who) {
     if (per_t <= 0 || p.T <= 0) return 0;
     // a wave a (row group, head) while that leaves the chip short of waves (a decode step); a prompt's rows have waves to
     // spare, and each then walks several heads of its rows on one evaluation of the rotation (most of a wave's
-    // arithmetic): about 4096 waves a launch measured best, the heads of a row group shared evenly among its waves
+    // arithmetic): about 4096 waves a launch measured best (8192 for the largest passes), the heads of a row group shared
+    // evenly among its waves
     PreParams q = p;
     const int64_t rpw = p.D == 64 ? 4 : p.D == 128 ? 2 : 1, tg = (p.T + rpw - 1) / rpw;
-    q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, tg * per_t / 4096));
+    q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, tg * per_t / (tg * per_t >= 131072 ? 8192 : 4096)));
     q.hpw = (int) ((per_t + (per_t + q.hpw - 1) / q.hpw - 1) / ((per_t + q.hpw - 1) / q.hpw));
     if (const char* e = getenv("NS_PRE_HPW")) q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, atoi(e)));   // sweeps
     const int64_t waves = tg * ((per_t + q.hpw - 1) / q.hpw);
