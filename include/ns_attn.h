@@ -126,17 +126,50 @@ int ns_q35_attn_prompt_kv(ns_gpu* g, int kt, const float* q, int64_t qs, const v
 int64_t ns_q35_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0);
 int ns_q35_attn(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
                 int64_t cap, int64_t p0, float* out, float* scratch);
-/* Replaces: kernels/llm/museglimmer/mg.h:27-33 (mg.cpp:208-253). causal 0 (the drafter's block: every row sees to the
- * pass's last key) is accepted for T <= 16 */
+/* Replaces: kernels/llm/museglimmer/mg.h:27-33 (mg.cpp:208-253). causal 0: the drafter's block - every row sees from
+ * its own window's first key to the pass's last key; up to 16 rows it is one launch of the split kernel cut by the
+ * first row's key count, longer blocks take the prompt kernel */
 int64_t ns_mg_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win, int causal);
 int ns_mg_attn(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
                int64_t win, int causal, float* out, float* scratch);
+/* The drafter's block under its silo name: ns_mg_attn with causal 0. Replaces: kernels/llm/museglimmer/silo/silo.h:53-58
+ * (silo/attn.cpp:280-315); the reference covers 1..16 rows of 4 query heads a key head */
+int64_t ns_mg_attn_block_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win);
+int ns_mg_attn_block(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
+                     int64_t win, float* out, float* scratch);
+/* The weights one decode row q [Hq][D] (float32, normed and rotated) gives the n keys of a head-major cache of form kt,
+ * reduced over the heads and ADDED to out [n]: their mean (mode 0) or their largest (mode 1); softmax in float32 with
+ * scale 1 / sqrt(D). scratch: 2 Hq floats (each head's largest score and sum). The scores are kept [Hq][n] in memory
+ * the library holds per ns_gpu (-1 when Hq x n exceeds it). D 128 or 256 (the reference: 256). Replaces:
+ * kernels/llm/qwen35/q35.h:37-38 (q35.cpp:464-506), bound at llm/qwen35/src/ffi.rs:111 */
+int ns_q35_attn_probs(ns_gpu* g, int kt, const float* q, const void* kc, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t n, int mode,
+                      float* scratch, float* out);
+
 /* GQA over a position-major half cache [position][G][128], q [T][H][128], explicit scale. sel NULL: dense; else
  * sel [T][G][K] names K blocks of 128 keys a (row, key head) (-1: none), cut at the row's own position (a row is a launch).
  * Replaces: kernels/llm/minimaxm3/mm3.h:33-37 (mm3.cpp:118-190). Needs scratch: this library keeps
  * ns_attn_decode_scratch(T, H, G, 128, pos0, 0) floats per ns_gpu for it (allocated at ns_gpu_open, 64 MiB) */
 int ns_llm_minimaxm3_attend(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
                             int64_t H, int64_t G, int64_t pos0, float scale);
+
+/* The MiniMax silo's names for the same passes. Replaces: kernels/llm/minimaxm3/silo/mm3s.h:14-33,61-62 (silo/attn.cpp,
+ * silo/attnx.cpp), bound at llm/minimaxm3/src/ffi.rs:164-171. One kernel family serves the vector-unit and the
+ * matrix-unit names. `_split`: S = ceil(keys / 128) and part (T G S 16 130 floats) are the caller's; this library's
+ * partials (splits of at least 128 keys) fit them and go there, else through the memory the library keeps per ns_gpu.
+ * `_x` forms: the reference ignores `scale` and uses 1 / sqrt(128); here a positive scale is honoured, anything else
+ * means 1 / sqrt(128). `_block`: a draft block, every row sees keys w0 .. pos0 + T - 1 (not causal), scale 1 / sqrt(128).
+ * `_supported`: heads of 128 and H a multiple of G (the reference: H = 16 G) */
+int ns_mm3s_attend_supported(int64_t H, int64_t G, int64_t head);
+int ns_mm3s_attend(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T, int64_t H,
+                   int64_t G, int64_t pos0, float scale);
+int ns_mm3s_attend_x(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T, int64_t H,
+                     int64_t G, int64_t pos0, float scale);
+int ns_mm3s_attend_split(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
+                         int64_t H, int64_t G, int64_t pos0, float scale, int64_t S, float* part);
+int ns_mm3s_attend_x_split(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
+                           int64_t H, int64_t G, int64_t pos0, float scale, int64_t S, float* part);
+int ns_mm3s_attend_block(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int64_t T, int64_t H, int64_t G, int64_t pos0,
+                         int64_t w0, int64_t S, float* part);
 
 /* kernels/llm/minimaxm3/mm3.h (indexer), mm3.cpp:59-116. The block indexer that fills `sel`: bs [T][G][nblk] = the largest
  * iq [T][G][128] . ik_j over block b's keys j <= pos0 + t (ik half [pos][128]); -inf for a block wholly past the row,
@@ -157,6 +190,11 @@ int ns_attn_profile(ns_gpu* g, int on);
  * rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled against. This library's own */
 int ns_attn_copy_probe(ns_gpu* g, void* dst, const void* src, size_t bytes);
 int ns_attn_profile_last(ns_gpu* g, double* main_ns, double* merge_ns);
+/* Tuning knobs for sweeps and tests (this library's own): knob 0 work-groups a decode pass aims for, 1 key splits and
+ * 2 waves a work-group (4 or 8) of a prompt pass, 3 work-groups an MLA pass aims for, 4 heads a wave of the
+ * pre-attention kernel; value 0 = the library's own choice. Each knob starts from its environment variable (NS_DEC_WGS,
+ * NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW), read once a process */
+int ns_attn_tune(int knob, int64_t value);
 
 #ifdef __cplusplus
 }

@@ -44,12 +44,21 @@ int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint1
 /* GLM-5.3's latent-only MLA over a half cache [n][512]: qa [T][H][512] float32 -> u [T][H][512] float32. sel_cnt NULL:
  * every row sees every earlier cell. Else row t's cells are the pools sel[t K ..][0, sel_cnt[t]) of 4 cells each (cells
  * 4 b .. 4 b + 3) followed by its incomplete pool 4 ((p + 1) / 4) .. p, p = pos0 + t; a negative sel_cnt[t] is a dense
- * row. Replaces: kernels/llm/glm5next/glm.h:65-66 (glm.cpp:1062-1067,1095-1102,1252-1264) */
+ * row. Any number of rows: rows with lists go 16 a pass on the queue, dense
+ * rows as a prompt's. Replaces: kernels/llm/glm5next/glm.h:65-66 (glm.cpp:1062-1067,1095-1102,1252-1264; latent width 512
+ * only - the reference also takes 256) */
 int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                       const int32_t* sel, const int32_t* sel_cnt, int64_t K);
-/* the same over q8 latent rows, at most 8 rows. Replaces: kernels/llm/glm5next/glm.h:79-80 (glm.cpp:1267-1276) */
+/* the same over q8 latent rows. Replaces: kernels/llm/glm5next/glm.h:79-80 (glm.cpp:1267-1276; the reference: at most 8 rows) */
 int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                          const int32_t* sel, const int32_t* sel_cnt, int64_t K);
+/* The dense form over a float32 latent cache c [n][512] (every row sees every earlier cell): the cells 0 .. pos0 + T - 1
+ * are rounded to half into memory the library keeps per ns_gpu and read from there (-1 when they do not fit beside the
+ * partials: ~48K cells). Replaces: kernels/llm/glm5next/glm.h:47 (glm.cpp:782-812) */
+int ns_mla_attend(ns_gpu* g, const float* qa, const float* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale);
+/* out [n][512] half = the q8 latent rows idx[i] of src, widened: half(scale x q), one rounding (a prompt pass's gather).
+ * Replaces: kernels/llm/glm5next/glm.h:78 (glm.cpp:1301-1325) */
+int ns_gather_q8_h(ns_gpu* g, const void* src, const int32_t* idx, uint16_t* out, int64_t n, int64_t L);
 /* rows x [n][512] float32 -> q8 latent rows y [n][544]: a block's scale amax / 127 rounded to half BEFORE the values are
  * divided by it, round half away from zero, clamp to +-127. Replaces: kernels/llm/glm5next/glm.h:77 (glm.cpp:1282-1299) */
 int ns_to_q8row(ns_gpu* g, const float* x, void* y, int64_t n, int64_t L);

@@ -12,6 +12,8 @@ from .core import Error, api
 from .sys import P, f32, i32, i64
 
 F32, F16, BF16 = 0, 1, 2                       # q / out element types (NS_F32, NS_F16, NS_BF16)
+# ns_attn_tune's knobs
+TUNE_DEC_WGS, TUNE_PREFILL_SPLITS, TUNE_PREFILL_WAVES, TUNE_MLA_WGS, TUNE_PRE_HPW = 0, 1, 2, 3, 4
 KV_F16, KV_Q8_0, KV_Q4_0, KV_BF16 = 0, 1, 2, 3   # cache forms
 ELT = {F32: 4, F16: 2, BF16: 2}
 
@@ -55,12 +57,22 @@ ATTN_H = {
     "ns_q35_attn": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P, P]),
     "ns_mg_attn_scratch": (i64, [i64, i64, i64, i64, i64, i64, i32]),
     "ns_mg_attn": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, i32, P, P]),
+    "ns_mg_attn_block_scratch": (i64, [i64, i64, i64, i64, i64, i64]),
+    "ns_mg_attn_block": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_q35_attn_probs": (i32, [P, i32, P, P, i64, i64, i64, i64, i64, i32, P, P]),
+    "ns_mm3s_attend_supported": (i32, [i64, i64, i64]),
+    "ns_mm3s_attend": (i32, [P, P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
+    "ns_mm3s_attend_x": (i32, [P, P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
+    "ns_mm3s_attend_split": (i32, [P, P, P, P, P, i64, P, i64, i64, i64, i64, f32, i64, P]),
+    "ns_mm3s_attend_x_split": (i32, [P, P, P, P, P, i64, P, i64, i64, i64, i64, f32, i64, P]),
+    "ns_mm3s_attend_block": (i32, [P, P, P, P, P, i64, i64, i64, i64, i64, i64, P]),
     "ns_llm_minimaxm3_attend": (i32, [P, P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
     "ns_llm_minimaxm3_idx_scores": (i32, [P, P, P, P, i64, i64, i64, i64, i64]),
     "ns_llm_minimaxm3_idx_topk": (i32, [P, P, P, i64, i64, i64, i64]),
     "ns_attn_profile": (i32, [P, i32]),
     "ns_attn_copy_probe": (i32, [P, P, P, C.c_size_t]),
     "ns_attn_profile_last": (i32, [P, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "ns_attn_tune": (i32, [i32, i64]),
 }
 
 
@@ -73,6 +85,8 @@ MLA_H = {
     "ns_mla_attend_sel": (i32, [P, P, P, P, i64, i64, i64, i64, f32, P, P, i64]),
     "ns_mla_attend_sel_q8": (i32, [P, P, P, P, i64, i64, i64, i64, f32, P, P, i64]),
     "ns_to_q8row": (i32, [P, P, P, i64, i64]),
+    "ns_mla_attend": (i32, [P, P, P, P, i64, i64, i64, i64, f32]),
+    "ns_gather_q8_h": (i32, [P, P, P, P, i64, i64]),
 }
 
 
@@ -138,6 +152,10 @@ class Ops:
         a, b = C.c_double(), C.c_double()
         self.ok(self.k.attn_profile_last(self.raw(), C.byref(a), C.byref(b)), "profile_last")
         return a.value, b.value
+
+    def tune(self, knob, value):
+        """A tuning knob (TUNE_*) to `value`; 0 restores the library's own choice."""
+        self.ok(self.k.attn_tune(knob, value), "tune")
 
     def copy_probe(self, dst, src, nbytes):
         _need(dst, nbytes, "copy_probe dst")
@@ -265,6 +283,25 @@ class Ops:
         self.ok(self.k.mg_attn(self.raw(), q.ptr, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, int(causal), out.ptr,
                                scratch.ptr if scratch is not None else None), "attention")
 
+    def mg_attn_block(self, q, kc, vc, T, Hq, Hkv, D, cap, p0, win, out, scratch):
+        """ns_mg_attn_block: the drafter's block (not causal)."""
+        _need(q, T * Hq * D * 4, "block q")
+        _need(out, T * Hq * D * 4, "block out")
+        _need(kc, self.cache_bytes(0, Hkv, cap, D), "block key cache")
+        _need(vc, self.cache_bytes(0, Hkv, cap, D), "block value cache")
+        if scratch is not None:
+            _need(scratch, self.k.mg_attn_block_scratch(T, Hq, Hkv, D, p0, win) * 4, "block scratch")
+        self.ok(self.k.mg_attn_block(self.raw(), q.ptr, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, out.ptr,
+                                     scratch.ptr if scratch is not None else None), "attention block")
+
+    def q35_attn_probs(self, kt, q, kc, Hq, Hkv, D, cap, n, mode, scratch, out):
+        """ns_q35_attn_probs: out [n] += the heads' weights of every key (mode 0 their mean, 1 their largest)."""
+        _need(q, Hq * D * 4, "attn_probs q")
+        _need(kc, self.cache_bytes(kt, Hkv, cap, D), "attn_probs key cache")
+        _need(scratch, 2 * Hq * 4, "attn_probs scratch")
+        _need(out, n * 4, "attn_probs out")
+        self.ok(self.k.q35_attn_probs(self.raw(), kt, q.ptr, kc.ptr, Hq, Hkv, D, cap, n, mode, scratch.ptr, out.ptr), "attn_probs")
+
     def q35_attn(self, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, out, scratch):
         if T > 0:
             _need(q, ((T - 1) * qs + Hq * D) * 4, "attention q")
@@ -317,6 +354,20 @@ class Ops:
         opt = lambda b: b.ptr if b is not None else None
         self.ok(f(self.raw(), qa.ptr, c.ptr, u.ptr, T, H, L, pos0, scale, opt(sel), opt(sel_cnt), K), "mla_attend")
 
+    def mla_attend_f32(self, qa, c, u, T, H, L, pos0, scale):
+        """ns_mla_attend: the dense form over a float32 latent cache [n][L]."""
+        _need(qa, T * H * L * 4, "mla_attend qa")
+        _need(c, (pos0 + T) * L * 4, "mla_attend cache")
+        _need(u, T * H * L * 4, "mla_attend u")
+        self.ok(self.k.mla_attend(self.raw(), qa.ptr, c.ptr, u.ptr, T, H, L, pos0, scale), "mla_attend")
+
+    def gather_q8_h(self, src, rows, idx, out, n, L):
+        """ns_gather_q8_h: out [n][L] half = the q8 latent rows idx[i] of src (`rows` of them), widened."""
+        _need(src, rows * (L // 32 * 2 + L), "gather_q8_h rows")
+        _need(idx, n * 4, "gather_q8_h indices")
+        _need(out, n * L * 2, "gather_q8_h out")
+        self.ok(self.k.gather_q8_h(self.raw(), src.ptr, idx.ptr, out.ptr, n, L), "gather_q8_h")
+
     def to_q8row(self, x, y, n, L):
         _need(x, n * L * 4, "to_q8row x")
         _need(y, n * (L // 32 * 2 + L), "to_q8row y")
@@ -331,6 +382,25 @@ class Ops:
             _need(sel, T * G * K * 4, "attend block lists")
         self.ok(self.k.llm_minimaxm3_attend(self.raw(), q.ptr, kc.ptr, vc.ptr, sel.ptr if sel is not None else None, K, out.ptr, T, H, G, pos0, scale),
                 "attend")
+
+    def mm3s_attend(self, form, q, kc, vc, out, T, H, G, pos0, scale, sel=None, K=0, S=0, part=None, w0=0):
+        """The MiniMax silo's names: form "", "x", "split", "x_split" or "block" (ns_mm3s_attend*)."""
+        _need(q, T * H * 128 * 4, "attend q")
+        _need(out, T * H * 128 * 4, "attend out")
+        _need(kc, (pos0 + T) * G * 128 * 2, "attend key cache")
+        _need(vc, (pos0 + T) * G * 128 * 2, "attend value cache")
+        if sel is not None:
+            _need(sel, T * G * K * 4, "attend block lists")
+        if form in ("split", "x_split", "block"):
+            _need(part, T * G * S * 16 * 130 * 4, "attend partials")
+        sp = sel.ptr if sel is not None else None
+        if form == "block":
+            rc = self.k.mm3s_attend_block(self.raw(), q.ptr, kc.ptr, vc.ptr, out.ptr, T, H, G, pos0, w0, S, part.ptr)
+        elif form in ("split", "x_split"):
+            rc = getattr(self.k, "mm3s_attend_" + form)(self.raw(), q.ptr, kc.ptr, vc.ptr, sp, K, out.ptr, T, H, G, pos0, scale, S, part.ptr)
+        else:
+            rc = getattr(self.k, "mm3s_attend" + ("_x" if form == "x" else ""))(self.raw(), q.ptr, kc.ptr, vc.ptr, sp, K, out.ptr, T, H, G, pos0, scale)
+        self.ok(rc, "mm3s_attend" + ("_" + form if form else ""))
 
     def minimaxm3_idx_scores(self, iq, ik, bs, T, G, nblk, pos0, local):
         _need(iq, T * G * 128 * 4, "idx_scores iq")

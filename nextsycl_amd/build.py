@@ -27,6 +27,7 @@ SOURCES = {
     "attn_decode.hip": [],
     "indexer.hip": [],
     "attn_prefill.hip": [],
+    "attn_probs.hip": [],
     "attn_api.cpp": [],
     "mla.hip": [],
 }

@@ -31,11 +31,13 @@
 #include "ns_internal.hpp"
 #include "ns_attn.h"
 #include "attn_common.hpp"
+#include "attn_host.hpp"
 #include "kv_formats.hpp"
 
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
+#include <string>
 #include <type_traits>
 
 namespace {
@@ -59,6 +61,7 @@ struct DecodeParams {
     int T, Hq, G;
     int causal;                 // 0: every row sees to the pass's last key (the drafter's block)
     int64_t p0, win;
+    int64_t kfirst;             // >= 0: every row's first key (a block whose rows all start at one key); else the window's
     int64_t kbs, sp0;           // keys a split, the first split's index (absolute position / kbs)
     int ns;
     int nz;                     // row chunks a (split, key head)
@@ -118,7 +121,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     const int split = u % p.ns, hk = (u / p.ns) % Hkv, tr = u / (p.ns * Hkv);
     const int rows = p.T * p.G;
     const int64_t pass_end = p.p0 + p.T;
-    const int64_t fmin = p.win > 0 ? std::max<int64_t>(0, p.p0 + 1 - p.win) : 0;
+    const int64_t fmin = p.kfirst >= 0 ? p.kfirst : p.win > 0 ? std::max<int64_t>(0, p.p0 + 1 - p.win) : 0;
     const int64_t jb = std::max((p.sp0 + split) * p.kbs, fmin), je = std::min((p.sp0 + split + 1) * p.kbs, pass_end);
 
     const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
@@ -281,7 +284,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         const int ri = (z * RT + rt) * 16 + n;
         const bool live = ri < rows;
         const int t = live ? ri / p.G : 0, gq = live ? ri % p.G : 0;
-        const int64_t pos = p.p0 + t, first = p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0;
+        const int64_t pos = p.p0 + t, first = p.kfirst >= 0 ? p.kfirst : p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0;
         live_r[rt] = live;
         // (a row whose last key lies before the split keeps an empty range; the differences fit 32 bits: a split's keys do)
         const int64_t hi64 = std::min(p.causal ? pos : pass_end - 1, je - 1);
@@ -681,11 +684,7 @@ __global__ __launch_bounds__(MERGE_W * 64) void attn_merge_kernel(const float* _
 // one a CU; 256 against 512 measured 17.6 against 23.2 us at 32K keys, and half the partials to merge); NS_DEC_WGS
 // overrides (tuning)
 int64_t target_wgs(int64_t D) {
-    static const int64_t v = [] {
-        const char* e = getenv("NS_DEC_WGS");
-        const int64_t x = e ? atoll(e) : 0;
-        return x > 0 ? x : 0;
-    }();
+    const int64_t v = ns_tune_get(NS_TUNE_DEC_WGS);
     return v > 0 ? v : D == 256 ? 256 : 512;
 }
 // keys a split for a row that sees `keys` keys: a multiple of 128 (4 waves x 32-key tiles)
@@ -737,9 +736,10 @@ int launch_merge(ns_gpu* g, const float* part, int ns, int qt, int64_t rh, void*
 
 template <int D, int QT>
 int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv,
-                 int64_t cap, int64_t p0, int64_t win, int causal, float scale, void* out, float* scratch) {
+                 int64_t cap, int64_t p0, int64_t win, const DecodeExtra& x, float scale, void* out, float* scratch) {
     const int64_t rb = kv_row_bytes(kt, D);
     const int esz = QT == 0 ? 4 : 2;
+    const int causal = x.causal;
     DecodeParams p{};
     p.selT = 1;
     p.qt = QT;
@@ -753,18 +753,21 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
     p.G = (int) (Hq / Hkv);
     p.causal = causal;
     p.win = win;
+    p.kfirst = x.kfirst;
     p.sl2 = (scale > 0.0f ? scale : 1.0f / sqrtf((float) D)) * 1.4426950408889634f;
     const int64_t last = p0 + T - 1;
-    auto kb_of = [&](int64_t r) {
-        const int64_t pos = causal ? p0 + r : last;
-        return dec_kbs(pos + 1 - row_first(p0 + r, win), Hkv, D);
-    };
+    auto first_of = [&](int64_t r) { return x.kfirst >= 0 ? x.kfirst : row_first(p0 + r, win); };
+    auto kb_of = [&](int64_t r) { return dec_kbs(p0 + r + 1 - first_of(r), Hkv, D); };
+    // A causal pass is one launch when its rows' own split sizes agree, else a launch a row (a row's bits must not depend
+    // on the rows that share its pass). A pass that is not causal is always one launch, cut by its first row's key count
+    // (the longest: every row ends at the pass's last key) - kernels/llm/museglimmer/silo/attn.cpp:282-291
     bool same = true;
-    for (int64_t r = 1; r < T; ++r) same = same && kb_of(r) == kb_of(0);
-    const int64_t nsa = ns_attn_decode_scratch(T, Hq, Hkv, D, p0, win) / (T * Hq * (D + 2));
+    if (causal)
+        for (int64_t r = 1; r < T; ++r) same = same && kb_of(r) == kb_of(0);
+    const int64_t nsa = (x.scratch_floats > 0 ? x.scratch_floats : ns_attn_decode_scratch(T, Hq, Hkv, D, p0, win)) / (T * Hq * (D + 2));
     auto launch = [&](int64_t r0, int64_t nr, int64_t kb) -> int {
-        const int64_t pp = p0 + r0, sp0 = row_first(pp, win) / kb, ns = (pp + nr - 1) / kb - sp0 + 1;
-        if (ns > nsa) return ns_fail("ns_attn_decode: internal: more splits than the scratch holds");
+        const int64_t pp = p0 + r0, sp0 = first_of(r0) / kb, ns = (pp + nr - 1) / kb - sp0 + 1;
+        if (ns > nsa) return ns_fail("ns_attn_decode: more key splits than the scratch holds");
         DecodeParams c = p;
         c.q = (const uint8_t*) q + r0 * qs * esz;
         c.qs = qs;
@@ -774,12 +777,13 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
         c.sp0 = sp0;
         c.ns = (int) ns;
         c.part = scratch + r0 * Hq * nsa * (D + 2);
-        if (ns_profile_mark(g, 0)) return -1;
+        if (x.marks && ns_profile_mark(g, 0)) return -1;
         if (launch_kt<D>(g, kt, c, (int) (nr * c.G), dim3((unsigned) ns, (unsigned) Hkv))) return -1;
-        if (ns_profile_mark(g, 1)) return -1;
+        if (x.marks && ns_profile_mark(g, 1)) return -1;
         if (launch_merge<D>(g, c.part, (int) ns, QT, nr * Hq, (uint8_t*) out + r0 * Hq * D * esz)) return -1;
-        return ns_profile_mark(g, 2);
+        return x.marks ? ns_profile_mark(g, 2) : 0;
     };
+    if (!causal) return launch(0, T, dec_kbs(last + 1 - first_of(0), Hkv, D));
     if (same) return launch(0, T, kb_of(0));
     for (int64_t r = 0; r < T; ++r)
         if (launch(r, 1, kb_of(r))) return -1;
@@ -787,7 +791,8 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
 }
 
 int decode_checked(ns_gpu* g, const char* who, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T,
-                   int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, int causal, float scale, void* out, float* scratch) {
+                   int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, const DecodeExtra& x, float scale, void* out,
+                   float* scratch) {
     NS_TRY
     const std::string w(who);
     if (T <= 0) return 0;
@@ -797,6 +802,7 @@ int decode_checked(ns_gpu* g, const char* who, int qt, int kt, int pm, const voi
     if (kt < 0 || kt > 3) return ns_fail(w + ": a cache form 0 (half), 1 (q8_0), 2 (q4_0) or 3 (bfloat16)");
     if (qt < 0 || qt > 2) return ns_fail(w + ": rows of type 0 (float32), 1 (half) or 2 (bfloat16)");
     if (p0 < 0 || cap <= 0 || win < 0) return ns_fail(w + ": a position, a capacity and a window of 0 or more");
+    if (x.kfirst > p0) return ns_fail(w + ": a block's first key lies at or before its first row");
     if (Hkv > 65535) return ns_fail(w + ": at most 65535 key heads");
     const int64_t need = pm ? p0 + T : (win > 0 ? std::min(p0 + T, win + T - 1) : p0 + T);
     if (need > cap) return ns_fail(w + (win > 0 ? ": the cache's ring is shorter than the window and the pass" : ": past the cache's capacity"));
@@ -807,7 +813,7 @@ int decode_checked(ns_gpu* g, const char* who, int qt, int kt, int pm, const voi
     if (((uintptr_t) kc | (uintptr_t) vc) % 16 && (kt == 0 || kt == 3)) return ns_fail(w + ": caches 16-byte aligned");
     if (((uintptr_t) kc | (uintptr_t) vc) % 8) return ns_fail(w + ": caches 8-byte aligned");
     NS_HIP(hipSetDevice(g->dev));
-#define NS_DISPATCH(DD, QQ) return decode_typed<DD, QQ>(g, kt, pm, q, qs, kc, vc, T, Hq, Hkv, cap, p0, win, causal, scale, out, scratch)
+#define NS_DISPATCH(DD, QQ) return decode_typed<DD, QQ>(g, kt, pm, q, qs, kc, vc, T, Hq, Hkv, cap, p0, win, x, scale, out, scratch)
     if (D == 128) {
         if (qt == 0) NS_DISPATCH(128, 0);
         if (qt == 1) NS_DISPATCH(128, 1);
@@ -855,6 +861,7 @@ int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_
     p.Hq = (int) Hq;
     p.G = (int) (Hq / Hkv);
     p.causal = 1;
+    p.kfirst = -1;
     p.p0 = keys - 1;            // in the kernel's numbering the row sees every listed key; sel_pos cuts the real ones
     p.win = 0;
     p.kbs = kbs;
@@ -891,9 +898,9 @@ int ns_attn_merge_partials(ns_gpu* g, int64_t D, const float* part, int64_t ns, 
 
 // used by the exact-API routing in attn_api.cpp
 int ns_attn_decode_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T,
-                       int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, int causal, float scale, void* out,
+                       int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, const DecodeExtra& x, float scale, void* out,
                        float* scratch) {
-    return decode_checked(g, who, qt, kt, pm, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, win, causal, scale, out, scratch);
+    return decode_checked(g, who, qt, kt, pm, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, win, x, scale, out, scratch);
 }
 
 extern "C" {
@@ -919,7 +926,7 @@ int64_t ns_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, in
 
 int ns_attn_decode_t(ns_gpu* g, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq,
                      int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out, float* scratch) {
-    return decode_checked(g, "ns_attn_decode_t", qt, kt, pm, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, win, 1, scale, out, scratch);
+    return decode_checked(g, "ns_attn_decode_t", qt, kt, pm, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, win, DecodeExtra{}, scale, out, scratch);
 }
 
 int ns_q35_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) {
@@ -928,12 +935,12 @@ int ns_q35_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) 
 int64_t ns_q35_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0) { return ns_attn_decode_scratch(T, Hq, Hkv, D, p0, 0); }
 int ns_q35_attn_decode(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
                        int64_t cap, int64_t p0, float* out, float* scratch) {
-    return decode_checked(g, "ns_q35_attn_decode", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, 1, 0.0f, out, scratch);
+    return decode_checked(g, "ns_q35_attn_decode", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, DecodeExtra{}, 0.0f, out, scratch);
 }
 int ns_q35_attn_decode_kv(ns_gpu* g, int kt, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv,
                           int64_t D, int64_t cap, int64_t p0, float* out, float* scratch) {
     if (kt < 0 || kt > 2) return ns_fail("ns_q35_attn_decode_kv: a cache form 0 (half), 1 (q8_0) or 2 (q4_0)");
-    return decode_checked(g, "ns_q35_attn_decode_kv", 0, kt, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, 1, 0.0f, out, scratch);
+    return decode_checked(g, "ns_q35_attn_decode_kv", 0, kt, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, DecodeExtra{}, 0.0f, out, scratch);
 }
 
 int ns_mg_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) { return ns_q35_attn_decode_supported(T, Hq, Hkv, D); }
@@ -942,7 +949,7 @@ int64_t ns_mg_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
 }
 int ns_mg_attn_decode(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap,
                       int64_t p0, int64_t win, float* out, float* scratch) {
-    return decode_checked(g, "ns_mg_attn_decode", 0, 0, 0, q, Hq * D, kc, vc, T, Hq, Hkv, D, cap, p0, win, 1, 0.0f, out, scratch);
+    return decode_checked(g, "ns_mg_attn_decode", 0, 0, 0, q, Hq * D, kc, vc, T, Hq, Hkv, D, cap, p0, win, DecodeExtra{}, 0.0f, out, scratch);
 }
 
 }  // extern "C"

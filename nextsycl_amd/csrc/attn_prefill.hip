@@ -25,6 +25,7 @@
 #include "ns_internal.hpp"
 #include "ns_attn.h"
 #include "attn_common.hpp"
+#include "attn_host.hpp"
 #include "kv_formats.hpp"
 
 #include <algorithm>
@@ -32,8 +33,6 @@
 #include <cstdlib>
 #include <type_traits>
 
-// attn_decode.hip: the merge of [rows][ns][D + 2] partials
-int ns_attn_merge_partials(ns_gpu* g, int64_t D, const float* part, int64_t ns, int qt, int64_t rows, void* out);
 
 namespace {
 
@@ -53,6 +52,8 @@ struct PrefillParams {
     int wrap;
     int T, Hq, G;
     int64_t p0, win;
+    int causal;                 // 0: every row sees to the pass's last key (a draft block)
+    int64_t kfirst;             // >= 0: every row's first key, instead of its own window's
     float sl2;
     void* out;
     // key splits (passes of few row blocks over many keys): work-group (x, y) takes the keys [k0 + y kbs, k0 + (y + 1) kbs)
@@ -65,6 +66,10 @@ struct PrefillParams {
 // a 16-byte chunk of a K or V row on its way from global memory to LDS (a plain vector type: arrays of it stay in registers)
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
 
+// The queries enter the first product as they are given (16-bit rows bit for bit, float32 rows rounded once) and the
+// softmax scale (x log2 e) rides in one fused multiply-add a score. Folding the scale into the 16-bit query operand
+// instead saves that instruction but rounds 16-bit queries a second time (bfloat16 at 8192 rows: relative L2 against
+// the closed form 2.3e-3 instead of 1.5e-3)
 template <int D, bool BF, int KT, int PW>
 __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_prefill_kernel(const PrefillParams p) {
     static_assert(D == 128 || D == 256, "head size 128 or 256");
@@ -97,15 +102,14 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     const int rl = std::min(r0 + ROWS, p.T) - 1;                  // the block's last row
     // keys [kbeg, kend) cover every row of the block; with key splits, the part of them in this work-group's split
     const int split = blockIdx.y;
-    int64_t kend = p.p0 + rl + 1;
-    int64_t kbeg = p.win > 0 ? std::max<int64_t>(0, p.p0 + r0 + 1 - p.win) : 0;
+    int64_t kend = p.causal ? p.p0 + rl + 1 : p.p0 + p.T;
+    int64_t kbeg = p.kfirst >= 0 ? p.kfirst : p.win > 0 ? std::max<int64_t>(0, p.p0 + r0 + 1 - p.win) : 0;
     if (p.ns > 1) {
         kbeg = std::max(kbeg, p.k0 + split * p.kbs);
         kend = std::max(kbeg, std::min(kend, p.k0 + (split + 1) * p.kbs));      // (none: an empty range at kbeg)
     }
 
-    // ---- this lane's two rows: positions, key ranges, Q^T operands. The queries carry the softmax scale (x log2 e) into
-    // the 16-bit operand, so that the score product comes out in exponent units and needs no multiplication a score
+    // ---- this lane's two rows: positions, key ranges, Q^T operands
     int64_t lo_r[RT], hi_r[RT];
     s8v qreg[RT][KB];
 #pragma unroll
@@ -114,8 +118,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         const bool live = row < p.T;
         const int rr = live ? row : p.T - 1;
         const int64_t pos = p.p0 + rr;
-        lo_r[rt] = live ? std::max(kbeg, p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0) : 1;
-        hi_r[rt] = live ? std::min(pos, kend - 1) : 0;
+        lo_r[rt] = live ? std::max(kbeg, p.kfirst >= 0 ? p.kfirst : p.win > 0 ? std::max<int64_t>(0, pos + 1 - p.win) : 0) : 1;
+        hi_r[rt] = live ? std::min(p.causal ? pos : p.p0 + p.T - 1, kend - 1) : 0;
         const int64_t qoff = (int64_t) rr * p.qs + (int64_t) hq * D + g4 * 8;
         if (p.qt == 0) {
             float4 raw[KB][2];
@@ -128,7 +132,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             for (int kb = 0; kb < KB; ++kb) {
                 const float f[8] = {raw[kb][0].x, raw[kb][0].y, raw[kb][0].z, raw[kb][0].w, raw[kb][1].x, raw[kb][1].y, raw[kb][1].z, raw[kb][1].w};
 #pragma unroll
-                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = to16<BF>(f[i] * p.sl2);
+                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = to16<BF>(f[i]);
             }
         } else {
             uint4 raw[KB];
@@ -140,7 +144,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const uint16_t b16 = (uint16_t) (ww[i >> 1] >> (16 * (i & 1)));
-                    qreg[rt][kb][i] = to16<BF>((p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16)) * p.sl2);
+                    // rows of the operand type pass through bit for bit; the other 16-bit type is rounded once
+                    qreg[rt][kb][i] = (p.qt == 2) == BF ? (short) b16 : to16<BF>(p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16));
                 }
             }
         }
@@ -162,19 +167,16 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // the wave's own steps: from its first row's first key to its last row's last; steps in between that no row's edge
     // crosses need no mask
     const int wrow0 = r0 + w * WROWS, wrow1 = std::min(wrow0 + WROWS - 1, p.T - 1);
-    const int w_full_end = (int) (p.p0 + wrow0 + 1 - base);
-    const int w_full_beg = p.win > 0 ? (int) (std::max<int64_t>(0, p.p0 + wrow1 + 1 - p.win) - base) : 0;
+    const int w_full_end = (int) ((p.causal ? p.p0 + wrow0 + 1 : p.p0 + p.T) - base);
+    const int w_full_beg = p.kfirst >= 0 ? (int) (p.kfirst - base) : p.win > 0 ? (int) (std::max<int64_t>(0, p.p0 + wrow1 + 1 - p.win) - base) : 0;
 
     // Online softmax state, in base-2 exponent units (scores x scale x log2 e): nbr = minus the reference the weights
     // are taken against, thr = how far a score may exceed it before the reference moves (-inf while the row has seen no
     // key: the first one sets it), l_r = this lane's own share of the row's sum
-    // (nb4: nbr in all four slots of an accumulator, the value the score products start from)
     float nbr[RT], thr[RT], l_r[RT];
-    f4v nb4[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         nbr[rt] = 0.0f;
-        nb4[rt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
         thr[rt] = -INFINITY;
         l_r[rt] = 0.0f;
     }
@@ -271,8 +273,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     s8v pb[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) pb[rt] = s8v{0, 0, 0, 0, 0, 0, 0, 0};
-    // S^T of one 32-key half (LDS byte offset kl) against the wave's 32 rows, in exponent units and counted from the
-    // row's reference: the accumulators start at nbr
+    // S^T of one 32-key half (LDS byte offset kl) against the wave's 32 rows: the raw dot products
     auto scores = [&](f4v (&s)[RT][2], uint32_t kl) {
 #pragma unroll
         for (int kt2 = 0; kt2 < 2; ++kt2) {
@@ -282,7 +283,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                 ka[kb] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + kl + k_rd + kt2 * 16 * KS + kb * 64);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
-                f4v acc = mfma16<BF>(ka[0], qreg[rt][0], nb4[rt]);
+                f4v acc = mfma16<BF>(ka[0], qreg[rt][0], f4v{0.0f, 0.0f, 0.0f, 0.0f});
 #pragma unroll
                 for (int kb = 1; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
                 s[rt][kt2] = acc;
@@ -314,7 +315,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) a[rt][e] = sc[rt][e >> 2][e & 3];
+            for (int e = 0; e < 8; ++e) a[rt][e] = __builtin_fmaf(sc[rt][e >> 2][e & 3], p.sl2, nbr[rt]);
         if (masked) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -351,7 +352,6 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
                 nbr[rt] -= delta;
-                nb4[rt] = f4v{nbr[rt], nbr[rt], nbr[rt], nbr[rt]};
 #pragma unroll
                 for (int e = 0; e < 8; ++e) a[rt][e] -= delta;
                 thr[rt] = (fresh && nokey) ? -INFINITY : 8.0f;
@@ -512,7 +512,8 @@ int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
 }  // namespace
 
 int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T,
-                       int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out) {
+                       int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, int causal, int64_t kfirst, float scale,
+                       void* out) {
     NS_TRY
     const std::string w(who);
     if (T <= 0) return 0;
@@ -521,6 +522,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     if (kt < 0 || kt > 3) return ns_fail(w + ": a cache form 0 (half), 1 (q8_0), 2 (q4_0) or 3 (bfloat16)");
     if (qt < 0 || qt > 2) return ns_fail(w + ": rows of type 0 (float32), 1 (half) or 2 (bfloat16)");
     if (p0 < 0 || cap <= 0 || win < 0) return ns_fail(w + ": a position, a capacity and a window of 0 or more");
+    if (kfirst > p0) return ns_fail(w + ": a block's first key lies at or before its first row");
     const int64_t need = pm ? p0 + T : (win > 0 ? std::min(p0 + T, win + T - 1) : p0 + T);
     if (need > cap) return ns_fail(w + (win > 0 ? ": the cache's ring is shorter than the window and the pass" : ": past the cache's capacity"));
     if (!q || !kc || !vc || !out) return ns_fail(w + ": a null buffer");
@@ -539,13 +541,14 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // from the work-group size, so both sizes sum a row in the same order. The partials live in the library's own
     // scratch (the prompt entry points have no scratch argument): what fits bounds ns.
     {
-        const int64_t kfirst = win > 0 ? std::max<int64_t>(0, p0 + 1 - win) : 0, keys = p0 + T - kfirst;
+        const int64_t kf = kfirst >= 0 ? kfirst : win > 0 ? std::max<int64_t>(0, p0 + 1 - win) : 0, keys = p0 + T - kf;
         const int64_t pairs = ((T + 127) / 128) * Hq;
         int64_t ns = std::min<int64_t>({(512 + pairs - 1) / pairs, keys / 1024, 64,
                                         (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
-        if (const char* e = getenv("NS_PREFILL_SPLITS")) ns = std::min<int64_t>(atoll(e), (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2))));
+        // (a forced count - tests - stays within what the scratch and the merge kernel hold)
+        if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_SPLITS)) ns = std::min<int64_t>({forced, 2048, (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
         if (ns >= 2) {
-            sk0 = kfirst / KT_TILE * KT_TILE;
+            sk0 = kf / KT_TILE * KT_TILE;
             skbs = ((p0 + T - sk0 + ns - 1) / ns + KT_TILE - 1) / KT_TILE * KT_TILE;
             sns = (p0 + T - sk0 + skbs - 1) / skbs;
         }
@@ -553,8 +556,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // head size 256, 16-bit rows: a wave owns one 16-row tile, so 8 waves (two a SIMD, 128-row blocks) run the job 1.5 x
     // as fast as 4 (one a SIMD) whenever there are blocks enough for half the CUs
     int PWs = D == 128 ? (((T + 255) / 256) * Hq * sns >= 512 ? 8 : 4) : (T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
-    if (const char* e = getenv("NS_PREFILL_WAVES"))
-        if (atoi(e) == 4 || atoi(e) == 8) PWs = atoi(e);
+    if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_WAVES); forced == 4 || forced == 8) PWs = (int) forced;
     const int64_t ROWS = rows_of((int) D, PWs);
     if (T > (int64_t) 1 << 30 || ((T + ROWS - 1) / ROWS + 1) * Hq > (int64_t) 1 << 30) return ns_fail(w + ": too many rows or heads");
     if ((pm ? cap * Hkv : cap) * rb >= (int64_t) 1 << 32) return ns_fail(w + ": a key head's cache spans 4 GiB or more");
@@ -574,6 +576,8 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     p.G = (int) (Hq / Hkv);
     p.p0 = p0;
     p.win = win;
+    p.causal = causal;
+    p.kfirst = kfirst;
     p.sl2 = (scale > 0.0f ? scale : 1.0f / sqrtf((float) D)) * 1.4426950408889634f;
     p.out = out;
     p.ns = (int) sns;
@@ -600,7 +604,7 @@ extern "C" {
 
 int ns_attn_prompt_t(ns_gpu* g, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq,
                      int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out) {
-    return ns_attn_prompt_any(g, "ns_attn_prompt_t", qt, kt, pm, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, win, scale, out);
+    return ns_attn_prompt_any(g, "ns_attn_prompt_t", qt, kt, pm, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, win, 1, -1, scale, out);
 }
 
 }  // extern "C"

@@ -118,6 +118,7 @@ int ns_attn_kv_store(ns_gpu* g, int kt, int ring, const float* k, int64_t ks, co
     if (kt < 0 || kt > 3) return ns_fail("ns_attn_kv_store: a cache form 0 (half), 1 (q8_0), 2 (q4_0) or 3 (bfloat16)");
     if (Hkv <= 0 || D <= 0 || D % 32 || ks % 4 || vs % 4) return ns_fail("ns_attn_kv_store: heads of a multiple of 32, row strides a multiple of 4");
     if (p0 < 0 || cap <= 0) return ns_fail("ns_attn_kv_store: a position and a capacity");
+    if (!g || !k || !v || !kc || !vc) return ns_fail("ns_attn_kv_store: a null buffer");
     if (ring && (kt == 1 || kt == 2)) return ns_fail("ns_attn_kv_store: ring caches are half or bfloat16");
     if (ring ? T > cap : p0 + T > cap) return ns_fail("ns_attn_kv_store: past the cache's capacity");
     if (((uintptr_t) k | (uintptr_t) v) % 16 || ((uintptr_t) kc | (uintptr_t) vc) % 8) return ns_fail("ns_attn_kv_store: rows 16-byte aligned, caches 8-byte aligned");
@@ -163,6 +164,8 @@ int ns_attn_kv_dequant(ns_gpu* g, int kt, const void* rows, int64_t n, int64_t D
     NS_TRY
     if (n <= 0) return 0;
     if (kt < 0 || kt > 3 || D <= 0 || D % 32) return ns_fail("ns_attn_kv_dequant: a cache form 0..3, rows of a multiple of 32");
+    if (stride < kv_row_bytes(kt, D) || ((uintptr_t) rows | (uintptr_t) stride) % 2) return ns_fail("ns_attn_kv_dequant: rows at least a row apart, 2-byte aligned");
+    if (!g || !rows || !out) return ns_fail("ns_attn_kv_dequant: a null buffer");
     NS_HIP(hipSetDevice(g->dev));
     kv_dequant_kernel<<<blocks_for(n * D, 256), 256, 0, g->q>>>(kt, (const uint8_t*) rows, n, D, stride, out);
     NS_LAUNCHED("kv_dequant");
@@ -184,7 +187,9 @@ int ns_attn_copy_probe(ns_gpu* g, void* dst, const void* src, size_t bytes) {
 int ns_q35_fwht32(ns_gpu* g, float* x, int64_t rows, int64_t n, int64_t stride) {
     NS_TRY
     if (rows <= 0) return 0;
-    if (n % 32) return ns_fail("ns_q35_fwht32: rows of a multiple of 32");
+    if (n <= 0 || n % 32) return ns_fail("ns_q35_fwht32: rows of a multiple of 32");
+    if (stride < n) return ns_fail("ns_q35_fwht32: rows at least a row apart");
+    if (!g || !x) return ns_fail("ns_q35_fwht32: a null buffer");
     NS_HIP(hipSetDevice(g->dev));
     const int64_t nb = n / 32;
     fwht32_kernel<<<blocks_for(rows * nb, 256), 256, 0, g->q>>>(x, rows, nb, stride);

@@ -29,6 +29,7 @@
 #include "ns_internal.hpp"
 #include "ns_mla.h"
 #include "attn_common.hpp"
+#include "attn_host.hpp"
 #include "kv_formats.hpp"
 
 #include <algorithm>
@@ -615,15 +616,39 @@ __global__ __launch_bounds__(256) void to_q8row_kernel(const float* __restrict__
     }
 }
 
+// float32 -> half, 8 values a thread (a float32 latent cache's rows on their way to the latent kernel)
+__global__ __launch_bounds__(256) void to_half_kernel(const float* __restrict__ x, uint16_t* __restrict__ y, int64_t n8) {
+    const int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (i >= n8) return;
+    const float4 a = reinterpret_cast<const float4*>(x)[2 * i], b = reinterpret_cast<const float4*>(x)[2 * i + 1];
+    typedef uint16_t us8v __attribute__((ext_vector_type(8)));
+    const us8v h = {f32_to_f16(a.x), f32_to_f16(a.y), f32_to_f16(a.z), f32_to_f16(a.w), f32_to_f16(b.x), f32_to_f16(b.y), f32_to_f16(b.z), f32_to_f16(b.w)};
+    reinterpret_cast<us8v*>(y)[i] = h;
+}
+
+// out [n][512] half = the q8 latent rows idx[i] of src widened: half(scale x q), one rounding (the product is exact in
+// float32); a thread 8 values (kernels/llm/glm5next/glm.cpp:1301-1325)
+__global__ __launch_bounds__(256) void gather_q8_h_kernel(const uint8_t* __restrict__ src, const int32_t* __restrict__ idx, uint16_t* __restrict__ out,
+                                                          int64_t n) {
+    const int64_t gi = (int64_t) blockIdx.x * 256 + threadIdx.x, r = gi / 64;
+    const int c = (int) (gi % 64);
+    if (r >= n) return;
+    const uint8_t* row = src + (int64_t) idx[r] * (ML / 32 * 2 + ML);
+    const float d = f16_to_f32(reinterpret_cast<const uint16_t*>(row)[c / 4]);
+    const uint2 qv = *reinterpret_cast<const uint2*>(row + 32 + c * 8);
+    const uint32_t ww[2] = {qv.x, qv.y};
+    typedef uint16_t us8v __attribute__((ext_vector_type(8)));
+    us8v h;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) h[e] = f32_to_f16(d * (float) (int8_t) (ww[e >> 2] >> (8 * (e & 3))));
+    reinterpret_cast<us8v*>(out)[r * 64 + c] = h;
+}
+
 // ---- host side --------------------------------------------------------------------------------------------------------
 
 int64_t mla_target_wgs() {
-    static const int64_t v = [] {
-        const char* e = getenv("NS_MLA_WGS");
-        const int64_t x = e ? atoll(e) : 0;
-        return x > 0 ? x : 256;
-    }();
-    return v;
+    const int64_t v = ns_tune_get(NS_TUNE_MLA_WGS);
+    return v > 0 ? v : 256;
 }
 // cells a split: ~mla_target_wgs() work-groups over the pass, whole 32-cell tiles, at least 2 tiles
 int64_t mla_kbs(int64_t cells, int64_t groups) {
@@ -776,7 +801,8 @@ int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint1
                     float freq_base, float freq_scale, float ext_factor, float mscale, float corr0, float corr1) {
     NS_TRY
     if (T <= 0) return 0;
-    if (R % 2 != 0) return ns_fail("ns_ds2_kv_store: an even rotated width");
+    if (L <= 0 || R < 0 || R % 2 != 0 || pos0 < 0) return ns_fail("ns_ds2_kv_store: a latent width, an even rotated width and a position");
+    if (!g || !kv || !w || !cache) return ns_fail("ns_ds2_kv_store: a null buffer");
     NS_HIP(hipSetDevice(g->dev));
     ds2_kv_store_kernel<<<(unsigned) T, 256, 0, g->q>>>(kv, w, eps, cache, L, R, pos0, freq_base, freq_scale, ext_factor, mscale, corr0, corr1);
     NS_LAUNCHED("ds2_kv_store");
@@ -784,12 +810,27 @@ int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint1
     NS_CATCH
 }
 
+// GLM's latent-only MLA through the library's own scratch, any number of rows: rows with cell lists of their own go 16 a
+// pass (a row group holds one row's heads, so wider passes gain nothing), dense rows as a prompt's do
+static int mla_sel_rows(ns_gpu* g, const char* who, bool q8, const float* qa, const void* c, float* u, int64_t T, int64_t H, int64_t pos0,
+                        float scale, const int32_t* sel, const int32_t* sel_cnt, int64_t K, float* scratch, size_t scratch_floats) {
+    if (H <= 0 || pos0 < 0) return ns_fail(std::string(who) + ": heads and a position");
+    if (!qa || !u) return ns_fail(std::string(who) + ": a null buffer");
+    for (int64_t t0 = 0, n; t0 < T; t0 += n) {
+        n = T <= 16 ? T : sel_cnt ? std::min<int64_t>(16, T - t0) : mla_pass_rows(pos0 + t0, T - t0);
+        if (mla_latent(g, who, 0, 0, 0, q8, qa + t0 * H * ML, c, u + t0 * H * ML, n, H, pos0 + t0, scale, scratch, scratch_floats,
+                       sel_cnt ? sel + t0 * K : nullptr, sel_cnt ? sel_cnt + t0 : nullptr, K))
+            return -1;
+    }
+    return 0;
+}
+
 int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                       const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
     NS_TRY
     if (T <= 0) return 0;
-    if (L != 512 || T > 16) return ns_fail("ns_mla_attend_sel: latent width 512, at most 16 rows");
-    return mla_latent(g, "ns_mla_attend_sel", 0, 0, 0, false, qa, c, u, T, H, pos0, scale, g->own_scratch, g->own_scratch_floats, sel, sel_cnt, K);
+    if (L != 512) return ns_fail("ns_mla_attend_sel: latent width 512");
+    return mla_sel_rows(g, "ns_mla_attend_sel", false, qa, c, u, T, H, pos0, scale, sel, sel_cnt, K, g->own_scratch, g->own_scratch_floats);
     NS_CATCH
 }
 
@@ -797,8 +838,41 @@ int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, in
                          const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
     NS_TRY
     if (T <= 0) return 0;
-    if (L != 512 || T > 8) return ns_fail("ns_mla_attend_sel_q8: latent width 512, at most 8 rows");
-    return mla_latent(g, "ns_mla_attend_sel_q8", 0, 0, 0, true, qa, c, u, T, H, pos0, scale, g->own_scratch, g->own_scratch_floats, sel, sel_cnt, K);
+    if (L != 512) return ns_fail("ns_mla_attend_sel_q8: latent width 512");
+    return mla_sel_rows(g, "ns_mla_attend_sel_q8", true, qa, c, u, T, H, pos0, scale, sel, sel_cnt, K, g->own_scratch, g->own_scratch_floats);
+    NS_CATCH
+}
+
+// the dense form over a float32 latent cache c [n][512]: its rows 0 .. pos0 + T - 1 are rounded to half into the
+// library's scratch (the half cache's own rounding) and the latent kernel reads those
+int ns_mla_attend(ns_gpu* g, const float* qa, const float* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale) {
+    NS_TRY
+    if (T <= 0) return 0;
+    if (L != 512) return ns_fail("ns_mla_attend: latent width 512");
+    if (pos0 < 0 || !c) return ns_fail("ns_mla_attend: a position and a cache");
+    if ((uintptr_t) c % 16) return ns_fail("ns_mla_attend: the cache 16-byte aligned");
+    const int64_t cells = pos0 + T, ch_floats = (cells * ML / 2 + 3) / 4 * 4;     // the half rows, counted in floats
+    if ((size_t) ch_floats + (size_t) (H > 0 ? 16 * H * PSTRIDE : 0) > g->own_scratch_floats)
+        return ns_fail("ns_mla_attend: more cells than the library's scratch holds as half rows (use a half cache and ns_mla_attend_sel)");
+    NS_HIP(hipSetDevice(g->dev));
+    uint16_t* ch = (uint16_t*) g->own_scratch;
+    to_half_kernel<<<(unsigned) ((cells * ML / 8 + 255) / 256), 256, 0, g->q>>>(c, ch, cells * ML / 8);
+    NS_LAUNCHED("to_half");
+    return mla_sel_rows(g, "ns_mla_attend", false, qa, ch, u, T, H, pos0, scale, nullptr, nullptr, 0, g->own_scratch + ch_floats,
+                        g->own_scratch_floats - (size_t) ch_floats);
+    NS_CATCH
+}
+
+int ns_gather_q8_h(ns_gpu* g, const void* src, const int32_t* idx, uint16_t* out, int64_t n, int64_t L) {
+    NS_TRY
+    if (n <= 0) return 0;
+    if (L != 512) return ns_fail("ns_gather_q8_h: latent width 512");
+    if (!src || !idx || !out) return ns_fail("ns_gather_q8_h: a null buffer");
+    if ((uintptr_t) src % 8 || (uintptr_t) out % 16) return ns_fail("ns_gather_q8_h: rows 8-byte, the output 16-byte aligned");
+    NS_HIP(hipSetDevice(g->dev));
+    gather_q8_h_kernel<<<(unsigned) ((n * 64 + 255) / 256), 256, 0, g->q>>>((const uint8_t*) src, idx, out, n);
+    NS_LAUNCHED("gather_q8_h");
+    return 0;
     NS_CATCH
 }
 
@@ -806,6 +880,8 @@ int ns_to_q8row(ns_gpu* g, const float* x, void* y, int64_t n, int64_t L) {
     NS_TRY
     if (n <= 0) return 0;
     if (L != 512) return ns_fail("ns_to_q8row: latent width 512");
+    if (!g || !x || !y) return ns_fail("ns_to_q8row: a null buffer");
+    if ((uintptr_t) x % 16 || (uintptr_t) y % 4) return ns_fail("ns_to_q8row: float rows 16-byte, q8 rows 4-byte aligned");
     NS_HIP(hipSetDevice(g->dev));
     to_q8row_kernel<<<(unsigned) ((n * 16 + 255) / 256), 256, 0, g->q>>>(x, (uint8_t*) y, n);
     NS_LAUNCHED("to_q8row");

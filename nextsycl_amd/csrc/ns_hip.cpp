@@ -9,6 +9,12 @@ thread_local std::string g_err;
 constexpr size_t EV_RING = 1 << 16;
 constexpr size_t OWN_SCRATCH_FLOATS = (size_t) 16 << 20;   // 64 MiB
 
+// the event of a ticket the ring still holds, or null: tickets are 0 .. next_ev - 1, the ring keeps the last EV_RING
+hipEvent_t ticket_event(ns_gpu* g, int64_t t) {
+    if (t < 0 || t >= g->next_ev || g->next_ev - t > (int64_t) EV_RING) return nullptr;
+    return g->ev[(size_t) t % EV_RING];
+}
+
 int bad_index(int index, int n) { return ns_fail("no GPU " + std::to_string(index) + " (" + std::to_string(n) + " found)"); }
 
 // the event of ticket slot t, created on first use
@@ -250,7 +256,8 @@ int ns_stream_copy(ns_gpu* g, void* dst, const void* src, size_t bytes, const in
     NS_HIP(hipSetDevice(g->dev));
     hipStream_t s = lane ? g->cq2 : g->cq;
     for (int i = 0; i < ndeps; ++i) {
-        hipEvent_t e = g->ev[(size_t) after[i] % EV_RING];
+        if (!after) return ns_fail("ns_stream_copy: tickets to wait for, but no list");
+        hipEvent_t e = ticket_event(g, after[i]);
         if (!e) return ns_fail("ns_stream_copy: ticket " + std::to_string(after[i]) + " was never issued");
         NS_HIP(hipStreamWaitEvent(s, e, 0));
     }
@@ -267,7 +274,7 @@ int ns_stream_copy(ns_gpu* g, void* dst, const void* src, size_t bytes, const in
 int ns_await(ns_gpu* g, int64_t t) {
     NS_TRY
     NS_HIP(hipSetDevice(g->dev));
-    hipEvent_t e = t >= 0 ? g->ev[(size_t) t % EV_RING] : nullptr;
+    hipEvent_t e = ticket_event(g, t);
     if (!e) return ns_fail("ns_await: ticket " + std::to_string(t) + " was never issued");
     NS_HIP(hipStreamWaitEvent(g->q, e, 0));
     return 0;
@@ -279,7 +286,7 @@ int ns_stamp(ns_gpu* g, int64_t* ticket) { return ns_mark(g, ticket); }
 int ns_elapsed(ns_gpu* g, int64_t t0, int64_t t1, double* ns) {
     NS_TRY
     NS_HIP(hipSetDevice(g->dev));
-    hipEvent_t a = t0 >= 0 ? g->ev[(size_t) t0 % EV_RING] : nullptr, b = t1 >= 0 ? g->ev[(size_t) t1 % EV_RING] : nullptr;
+    hipEvent_t a = ticket_event(g, t0), b = ticket_event(g, t1);
     if (!a || !b) return ns_fail("ns_elapsed: a ticket that was never issued");
     NS_HIP(hipEventSynchronize(a));
     NS_HIP(hipEventSynchronize(b));

@@ -19,6 +19,7 @@
 #include "kv_formats.hpp"
 #include "kv_pack.hpp"
 #include "attn_common.hpp"
+#include "attn_host.hpp"
 
 #include <algorithm>
 #include <cmath>
@@ -352,7 +353,7 @@ int launch_pre(ns_gpu* g, const PreParams& p, const char* who) {
     const int64_t rpw = p.D == 64 ? 4 : p.D == 128 ? 2 : 1, tg = (p.T + rpw - 1) / rpw;
     q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, tg * per_t / (tg * per_t >= 131072 ? 8192 : 4096)));
     q.hpw = (int) ((per_t + (per_t + q.hpw - 1) / q.hpw - 1) / ((per_t + q.hpw - 1) / q.hpw));
-    if (const char* e = getenv("NS_PRE_HPW")) q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, atoi(e)));   // sweeps
+    if (const int64_t forced = ns_tune_get(NS_TUNE_PRE_HPW)) q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, forced));   // sweeps
     const int64_t waves = tg * ((per_t + q.hpw - 1) / q.hpw);
     if ((waves + 3) / 4 > (int64_t) 1 << 31) return ns_fail(std::string(who) + ": too many rows");
     // whole 4-feature groups pair up: no rotation, adjacent pairs, or partners a multiple of 4 features away

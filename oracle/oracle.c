@@ -435,8 +435,8 @@ ORC_API int orc_attn_exact(const float* q, int64_t qs, const uint8_t* kc, const 
 /* The closed form in float64 on the stored values: out[r][hq][:] = sum_j softmax_j(scale q.k_j) v_j over the keys
  * the row sees; no key visible -> 0. q is float32 (the caller rounds it to f16 / bf16 first when the config says so).
  * scale <= 0: 1 / sqrt(D). */
-ORC_API int orc_attn_f64(const float* q, int64_t qs, const uint8_t* kc, const uint8_t* vc, int kt, int pm, int64_t T, int64_t Hq, int64_t Hkv,
-                         int64_t D, int64_t cap, int64_t p0, int64_t win, int causal, double scale, double* out) {
+static int attn_f64_impl(const float* q, int64_t qs, const uint8_t* kc, const uint8_t* vc, int kt, int pm, int64_t T, int64_t Hq, int64_t Hkv,
+                         int64_t D, int64_t cap, int64_t p0, int64_t win, int causal, int64_t kfirst, double scale, double* out) {
     if (T <= 0) return 0;
     if (Hkv <= 0 || Hq % Hkv || orc_kv_row_bytes(kt, D) < 0) return -1;
     const int64_t per = Hq / Hkv, rb = orc_kv_row_bytes(kt, D);
@@ -444,7 +444,7 @@ ORC_API int orc_attn_f64(const float* q, int64_t qs, const uint8_t* kc, const ui
 #pragma omp parallel for collapse(2) schedule(dynamic)
     for (int64_t r = 0; r < T; ++r)
         for (int64_t hq = 0; hq < Hq; ++hq) {
-            const int64_t pos = p0 + r, end = causal ? pos + 1 : p0 + T, first = win > 0 ? imax(0, pos + 1 - win) : 0, hk = hq / per;
+            const int64_t pos = p0 + r, end = causal ? pos + 1 : p0 + T, first = kfirst >= 0 ? kfirst : win > 0 ? imax(0, pos + 1 - win) : 0, hk = hq / per;
             const int64_t n = end - first;
             double* o = out + (r * Hq + hq) * D;
             for (int64_t d = 0; d < D; ++d) o[d] = 0.0;
@@ -469,6 +469,57 @@ ORC_API int orc_attn_f64(const float* q, int64_t qs, const uint8_t* kc, const ui
             for (int64_t d = 0; d < D; ++d) o[d] /= l;
             free(s);
         }
+    return 0;
+}
+ORC_API int orc_attn_f64(const float* q, int64_t qs, const uint8_t* kc, const uint8_t* vc, int kt, int pm, int64_t T, int64_t Hq, int64_t Hkv,
+                         int64_t D, int64_t cap, int64_t p0, int64_t win, int causal, double scale, double* out) {
+    return attn_f64_impl(q, qs, kc, vc, kt, pm, T, Hq, Hkv, D, cap, p0, win, causal, -1, scale, out);
+}
+/* the same closed form for a draft block whose rows all start at one key: every row sees kfirst .. p0 + T - 1 (not
+ * causal) - kernels/llm/minimaxm3/silo/attnx.cpp:36,60,86 (`pos = pos0 + T - 1`, `total = pos + 1 - w0`, `j0 = c0 + w0`) */
+ORC_API int orc_attn_f64_block(const float* q, int64_t qs, const uint8_t* kc, const uint8_t* vc, int kt, int pm, int64_t T, int64_t Hq, int64_t Hkv,
+                               int64_t D, int64_t cap, int64_t p0, int64_t kfirst, double scale, double* out) {
+    if (kfirst < 0 || kfirst > p0) return -1;
+    return attn_f64_impl(q, qs, kc, vc, kt, pm, T, Hq, Hkv, D, cap, p0, 0, 0, kfirst, scale, out);
+}
+
+/* The weights one row's heads give every key, reduced over the heads and ADDED to out [n] - kernels/llm/qwen35/q35.cpp:464-506:
+ * score(h, j) = (sum_i q[h][i] k_j[i], i ascending, float32) / sqrt(D); per head m = max_j, z = sum_j exp(score - m); per key
+ * acc = sum_h p / Hq (mode 0, heads ascending) or max_h p (mode 1), p = exp(score - m) / z. The reference's per-head
+ * reductions run over a work-group in an order SYCL leaves open; here the sum over j is ascending. */
+ORC_API int orc_attn_probs(int kt, const float* q, const uint8_t* kc, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t n, int mode,
+                           float* out) {
+    if (n <= 0) return 0;
+    if (n > cap || Hkv <= 0 || Hq % Hkv || orc_kv_row_bytes(kt, D) < 0) return -1;
+    const int64_t G = Hq / Hkv, rb = orc_kv_row_bytes(kt, D);
+    const float scale = 1.0f / sqrtf((float) D);
+    float* sc = (float*) malloc(sizeof(float) * (size_t) (Hq * n));
+    float* mz = (float*) malloc(sizeof(float) * (size_t) (2 * Hq));
+#pragma omp parallel for schedule(static)
+    for (int64_t h = 0; h < Hq; ++h) {
+        float m = -INFINITY;
+        for (int64_t j = 0; j < n; ++j) {
+            const uint8_t* row = kc + ((h / G) * cap + j) * rb;
+            float a = 0.0f;
+            for (int64_t i = 0; i < D; ++i) a += q[h * D + i] * orc_kv_value(row, kt, D, i);
+            sc[h * n + j] = a * scale;
+            m = fmaxf(m, sc[h * n + j]);
+        }
+        float z = 0.0f;
+        for (int64_t j = 0; j < n; ++j) z += expf(sc[h * n + j] - m);
+        mz[2 * h] = m;
+        mz[2 * h + 1] = z;
+    }
+    for (int64_t j = 0; j < n; ++j) {
+        float acc = 0.0f;
+        for (int64_t h = 0; h < Hq; ++h) {
+            const float p = expf(sc[h * n + j] - mz[2 * h]) / mz[2 * h + 1];
+            acc = mode == 1 ? fmaxf(acc, p) : acc + p / (float) Hq;
+        }
+        out[j] += acc;
+    }
+    free(sc);
+    free(mz);
     return 0;
 }
 
@@ -895,6 +946,44 @@ ORC_API void orc_glm_mla_attend_sel(const float* qa, const uint8_t* cache, int q
 ORC_API void orc_glm_mla_attend(const float* qa, const uint8_t* cache, int q8, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0,
                                 float scale) {
     orc_glm_mla_attend_sel(qa, cache, q8, u, T, H, L, pos0, scale, NULL, NULL, 0);
+}
+
+/* GLM-5.3's dense MLA over a float32 latent cache c [n][L], two passes (the largest score, then the weights and the sum)
+ * - kernels/llm/glm5next/glm.cpp:782-812. The reference sums a score's L products across 256 work-items (an order SYCL
+ * leaves open); here feature-ascending in float32. */
+ORC_API void orc_glm_mla_attend_f32(const float* qa, const float* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale) {
+#pragma omp parallel for collapse(2) schedule(dynamic)
+    for (int64_t t = 0; t < T; ++t)
+        for (int64_t h = 0; h < H; ++h) {
+            const float* qr = qa + (t * H + h) * L;
+            const int64_t n = pos0 + t + 1;
+            float mx = -INFINITY;
+            for (int64_t s = 0; s < n; ++s) {
+                float dot = 0.0f;
+                for (int64_t r = 0; r < L; ++r) dot += qr[r] * c[s * L + r];
+                mx = fmaxf(mx, dot * scale);
+            }
+            float* o = u + (t * H + h) * L;
+            for (int64_t r = 0; r < L; ++r) o[r] = 0.0f;
+            float sum = 0.0f;
+            for (int64_t s = 0; s < n; ++s) {
+                float dot = 0.0f;
+                for (int64_t r = 0; r < L; ++r) dot += qr[r] * c[s * L + r];
+                const float p = expf(dot * scale - mx);
+                sum += p;
+                for (int64_t r = 0; r < L; ++r) o[r] += p * c[s * L + r];
+            }
+            for (int64_t r = 0; r < L; ++r) o[r] /= sum;
+        }
+}
+
+/* out [n][L] half = the q8 latent rows idx[i] of src widened: half(h2f(scale) x (float) q) - kernels/llm/glm5next/glm.cpp:1301-1325 */
+ORC_API void orc_glm_gather_q8_h(const uint8_t* src, const int32_t* idx, uint16_t* out, int64_t n, int64_t L) {
+    const int64_t nb = L / 32, rb = nb * 2 + L;
+    for (int64_t i = 0; i < n; ++i) {
+        const uint8_t* row = src + (int64_t) idx[i] * rb;
+        for (int64_t f = 0; f < L; ++f) out[i * L + f] = orc_f2h(orc_h2f(ld16(row + 2 * (f / 32))) * (float) (int8_t) row[nb * 2 + f]);
+    }
 }
 
 /* ------------------------------------------------------------------------------------ norm + rotary positions */

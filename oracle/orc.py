@@ -44,6 +44,10 @@ def lib():
             "orc_q35_attn_decode_scratch": (i64, [i64, i64, i64, i64, i64]),
             "orc_attn_exact": (C.c_int, [P, i64, P, P, C.c_int, C.c_int, i64, i64, i64, i64, i64, i64, i64, C.c_int, i64, C.c_int, P]),
             "orc_attn_f64": (C.c_int, [P, i64, P, P, C.c_int, C.c_int, i64, i64, i64, i64, i64, i64, i64, C.c_int, f64, P]),
+            "orc_attn_f64_block": (C.c_int, [P, i64, P, P, C.c_int, C.c_int, i64, i64, i64, i64, i64, i64, i64, f64, P]),
+            "orc_attn_probs": (C.c_int, [C.c_int, P, P, i64, i64, i64, i64, i64, C.c_int, P]),
+            "orc_glm_mla_attend_f32": (None, [P, P, P, i64, i64, i64, i64, f32]),
+            "orc_glm_gather_q8_h": (None, [P, P, P, i64, i64]),
             "orc_attn_flash_model": (C.c_int, [P, i64, P, P, C.c_int, C.c_int, i64, i64, i64, i64, i64, i64, i64, i64, P]),
             "orc_mm3_attend": (C.c_int, [P, P, P, P, i64, i64, i64, i64, f32]),
             "orc_mm3_attend_sel": (C.c_int, [P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
@@ -198,6 +202,26 @@ def attn_f64(q, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=0, causal=True, pm=False
     return out
 
 
+def attn_f64_block(q, kc, vc, kt, T, Hq, Hkv, D, cap, p0, kfirst, pm=False, scale=0.0):
+    """A draft block: every row sees keys kfirst .. p0 + T - 1 (not causal)."""
+    q = _c(q, np.float32).reshape(T, Hq * D)
+    out = np.empty((T, Hq * D), np.float64)
+    rc = lib().orc_attn_f64_block(_p(q), Hq * D, _p(kc), _p(vc), kt, int(pm), T, Hq, Hkv, D, cap, p0, kfirst, float(scale), _p(out))
+    if rc:
+        raise ValueError("orc_attn_f64_block: bad arguments")
+    return out
+
+
+def attn_probs(kt, q, kc, Hq, Hkv, D, cap, n, mode, out=None):
+    """out [n] += the heads' weights of each key: their mean (mode 0) or largest (1) - ns_q35_attn_probs."""
+    q = _c(q, np.float32)
+    out = np.zeros(n, np.float32) if out is None else _c(out, np.float32).copy()
+    rc = lib().orc_attn_probs(kt, _p(q), _p(kc), Hq, Hkv, D, cap, n, mode, _p(out))
+    if rc:
+        raise ValueError("orc_attn_probs: bad arguments")
+    return out
+
+
 def attn_flash_model(q, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=0, kbs=0, pm=False):
     q = _c(q, np.float32).reshape(T, Hq * D)
     out = np.empty((T, Hq * D), np.float32)
@@ -283,6 +307,22 @@ def glm_mla_attend(qa, cache, q8, T, H, L, pos0, scale):
     u = np.empty((T, H, L), np.float32)
     lib().orc_glm_mla_attend(_p(qa), _p(cache), int(q8), _p(u), T, H, L, pos0, float(scale))
     return u
+
+
+def glm_mla_attend_f32(qa, c, T, H, L, pos0, scale):
+    """ns_mla_attend: the dense form over a float32 latent cache c [n][L]."""
+    qa, c = _c(qa, np.float32), _c(c, np.float32)
+    u = np.empty((T, H, L), np.float32)
+    lib().orc_glm_mla_attend_f32(_p(qa), _p(c), _p(u), T, H, L, pos0, float(scale))
+    return u
+
+
+def glm_gather_q8_h(src, idx, L):
+    """ns_gather_q8_h: the q8 latent rows idx of src widened to half bits [n][L]."""
+    src, idx = np.ascontiguousarray(src, np.uint8), _c(idx, np.int32)
+    out = np.empty((idx.size, L), np.uint16)
+    lib().orc_glm_gather_q8_h(_p(src), _p(idx), _p(out), idx.size, L)
+    return out
 
 
 # ---- comparisons -------------------------------------------------------------------------------------------------

@@ -25,6 +25,20 @@ def gpu():
     g.close()
 
 
+@pytest.fixture
+def tune(ops):
+    """Sets the library's tuning knobs (ns_attn_tune) for one test; every knob touched goes back to 0 = the default."""
+    touched = set()
+
+    def set_knob(knob, value):
+        touched.add(knob)
+        ops.tune(knob, value)
+
+    yield set_knob
+    for k in touched:
+        ops.tune(k, 0)
+
+
 @pytest.fixture(scope="session")
 def ops(gpu):
     from nextsycl_amd.attn import Ops

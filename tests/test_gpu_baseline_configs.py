@@ -1,6 +1,6 @@
 """BASELINE.json's configurations at their full sizes, through the C ABI, against the oracle: the decode-side ones
-(configs 1, 3, 5 and the 32K target) in full against the float64 closed form; the 8192-row prefill (config 2) on sampled
-rows against the closed form plus size-independent properties over the whole output."""
+(configs 1, 3, 5 and the 32K target) in full against the float64 closed form; the 8192-row prefill (config 2) on three
+whole 256-row blocks against the closed form plus size-independent properties over the whole output."""
 import numpy as np
 import pytest
 
@@ -69,8 +69,16 @@ def test_config5_mtp_verify_64k(ops):
         assert np.array_equal(one, raw[t]), t
 
 
-def test_config2_prefill_8k(ops):
-    """configs[1]: seq 8192, 40 / 8 heads (G = 5), head 128, bf16 Q / K / V and output, causal."""
+# The float32-output variant of the bf16 prefill kernel is held to a fixed bound: relative L2 2.0e-3 against the float64
+# closed form on whole 256-row blocks. What is left in it is the rounding of the softmax weights to bfloat16 for the second
+# product (~1.5e-3 on its own); the queries enter the first product exactly as given.
+CONFIG2_F32_REL_L2 = 2.0e-3
+
+
+def test_config2_prefill_8k(ops, record_property):
+    """configs[1]: seq 8192, 40 / 8 heads (G = 5), head 128, bf16 Q / K / V and output, causal. Three whole 256-row blocks
+    (the first, a middle one, the last: every wave and row tile of a work-group, every head) against the float64 closed
+    form, plus size-independent properties over the whole output."""
     T, Hq, Hkv, D = 8192, 40, 8, 128
     g = ops.gpu
     kc, vc = make_kv(3, Hkv, D, T, T, cfg=2)
@@ -78,18 +86,20 @@ def test_config2_prefill_8k(ops):
     bufs = (DevBuf.of(g, kc), DevBuf.of(g, vc))
     got, raw = gpu_prompt(ops, BF16, 3, qd, kc, vc, T, Hq, Hkv, D, T, 0, bufs=bufs)
     assert np.isfinite(got).all() and raw.shape == (T * Hq * D,)
-    # sampled rows (block edges, wave edges, first and last) of every head against the float64 closed form
-    rows = [0, 1, 15, 16, 31, 32, 127, 128, 129, 1000, 4095, 4096, 5555, 8063, 8064, 8190, 8191]
-    for r in rows:
-        ref = orc.attn_f64(qf[r:r + 1], kc, vc, 3, 1, Hq, Hkv, D, T, r)
-        check_close(got[r:r + 1], ref, BF16, "config 2, row %d" % r, kt=3)
-    # the float32-output variant of the same kernel: the kernel's own error without the output's bfloat16 rounding,
-    # and the bfloat16 output is exactly its rounding
+    # the float32-output variant of the same kernel: the kernel's own error without the output's bfloat16 rounding; the
+    # bfloat16 output is exactly its rounding
     got32, _ = gpu_prompt(ops, F32, 3, qf, kc, vc, T, Hq, Hkv, D, T, 0, bufs=bufs)
     assert np.array_equal(orc.f2bf(got32).ravel(), raw)
-    ref = np.concatenate([orc.attn_f64(qf[r:r + 1], kc, vc, 3, 1, Hq, Hkv, D, T, r) for r in rows[-8:]])
-    mx, rel, _ = orc.compare(np.concatenate([got32[r:r + 1] for r in rows[-8:]]), ref)
-    assert mx <= 2e-3 and rel <= 1e-3 + 2.0 ** -9, (mx, rel)
+    worst = [0.0, 0.0]
+    for r0 in (0, 4096, 7936):
+        ref = orc.attn_f64(qf[r0:r0 + 256], kc, vc, 3, 256, Hq, Hkv, D, T, r0)
+        check_close(got[r0:r0 + 256], ref, BF16, "config 2, rows %d.." % r0, kt=3)
+        mx, rel, _ = orc.compare(got32[r0:r0 + 256], ref)
+        print("config 2, float32 output, rows %d..%d: max-abs %.3e, relative L2 %.3e" % (r0, r0 + 255, mx, rel))
+        worst = [max(worst[0], mx), max(worst[1], rel)]
+        assert rel <= CONFIG2_F32_REL_L2 and mx <= 2e-3 + 2.0 ** -9 * np.abs(ref).max(), (r0, mx, rel)
+    record_property("config2_f32_max_abs", worst[0])
+    record_property("config2_f32_rel_l2", worst[1])
     # row 0 sees one key: its output is that key's value row, exactly
     V0 = orc.kv_dequant(vc[:, 0], 3, D)            # [Hkv][D]
     assert np.array_equal(got[0].reshape(Hq, D), np.repeat(V0, Hq // Hkv, axis=0))

@@ -1,0 +1,190 @@
+"""The entry points an engine binds beyond the typed kernels - the drafter's block (not causal), the MiniMax silo's
+names, ns_q35_attn_probs, ns_mla_attend, ns_gather_q8_h, longer ns_mla_attend_sel passes - through the C ABI against the
+oracle (pinned in tests/test_oracle_boundary.py, tests/test_oracle_attention.py). Attention within max-abs 2e-3 /
+relative L2 1e-3 of the float64 closed form; byte formats bit for bit."""
+import numpy as np
+import pytest
+
+from helpers import check_close, make_kv, make_q
+from nextsycl_amd import DevBuf
+from nextsycl_amd.attn import F32
+from oracle import orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _ring_caches(Hkv, D, cap, n, seed):
+    """Half ring caches [Hkv][cap][D] holding the last `cap` of positions 0 .. n - 1 (slot = position % cap)."""
+    k, v = orc.randn(seed, (n, Hkv * D)), orc.randn(seed + 1, (n, Hkv * D))
+    kc = np.zeros((Hkv, cap, 2 * D), np.uint8)
+    vc = np.zeros((Hkv, cap, 2 * D), np.uint8)
+    for s in range(0, n, 64):
+        e = min(n, s + 64)
+        orc.kv_store(0, k[s:e], v[s:e], Hkv, D, cap, s, kc=kc, vc=vc, ring=True)
+    return kc, vc
+
+
+# the drafter's block as the engine calls it: ns_mg_attn(win = the draft window, causal = 0). The last four shapes are ones
+# whose rows' own split sizes differ (a 128-multiple is crossed inside the block): the pass must still be one launch
+# cut by its first row's key count
+BLOCKS = [(2, 8, 2, 128, 5000, 0), (8, 16, 4, 128, 3000, 2048), (16, 8, 2, 128, 9000, 4096), (16, 32, 8, 128, 20000, 8192),
+          (8, 32, 8, 128, 8190, 8192), (5, 16, 8, 256, 4094, 4096), (16, 32, 16, 128, 4090, 4096), (3, 32, 16, 256, 2046, 2048),
+          (4, 8, 2, 128, 100, 0), (16, 4, 1, 128, 0, 0)]
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0,win", BLOCKS)
+def test_block_that_is_not_causal(ops, T, Hq, Hkv, D, p0, win):
+    g = ops.gpu
+    cap = p0 + T if win == 0 else win + T - 1 + 3
+    if win == 0:
+        kc, vc = make_kv(0, Hkv, D, cap, p0 + T, cfg=T)
+    else:
+        kc, vc = _ring_caches(Hkv, D, cap, p0 + T, 100 + T)
+    qd, qf = make_q(F32, T, Hq, D, cfg=p0 % 7)
+    ref = orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, cap, p0, win=win, causal=False)
+    qb, kb, vb = DevBuf.of(g, qd), DevBuf.of(g, kc), DevBuf.of(g, vc)
+    ob = DevBuf(g, T * Hq * D * 4); ob.fill(0xFF)
+    sc = DevBuf(g, 4 * ops.k.mg_attn_scratch(T, Hq, Hkv, D, p0, win, 0))
+    ops.mg_attn(qb, kb, vb, T, Hq, Hkv, D, cap, p0, win, False, ob, sc)
+    got = ob.read(np.float32).reshape(T, -1)
+    check_close(got, ref, F32, "ns_mg_attn, not causal")
+    # the silo's name for it: the same launch, the same bits
+    ob2 = DevBuf(g, T * Hq * D * 4); ob2.fill(0xFF)
+    sc2 = DevBuf(g, 4 * ops.k.mg_attn_block_scratch(T, Hq, Hkv, D, p0, win))
+    ops.mg_attn_block(qb, kb, vb, T, Hq, Hkv, D, cap, p0, win, ob2, sc2)
+    assert np.array_equal(ob2.read(np.float32).reshape(T, -1), got)
+    # and it differs from the causal pass wherever a row has later rows behind it
+    if T > 1:
+        assert np.abs(orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, cap, p0, win=win)[0] - ref[0]).max() > 1e-4
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0,win", [(40, 8, 2, 128, 700, 0), (70, 4, 1, 128, 3000, 512), (33, 4, 2, 256, 300, 0), (300, 4, 2, 128, 0, 0)])
+def test_long_block_that_is_not_causal(ops, T, Hq, Hkv, D, p0, win):
+    """More than 16 rows: the prompt kernel with every row ending at the pass's last key (kernels/llm/museglimmer/mg.cpp:58,
+    227-229 runs any row count that way)."""
+    g = ops.gpu
+    cap = p0 + T if win == 0 else win + T - 1 + 5
+    kc, vc = make_kv(0, Hkv, D, cap, p0 + T, cfg=1) if win == 0 else _ring_caches(Hkv, D, cap, p0 + T, 300)
+    qd, qf = make_q(F32, T, Hq, D, cfg=2)
+    ob = DevBuf(g, T * Hq * D * 4); ob.fill(0xFF)
+    ops.mg_attn(DevBuf.of(g, qd), DevBuf.of(g, kc), DevBuf.of(g, vc), T, Hq, Hkv, D, cap, p0, win, False, ob, None)
+    check_close(ob.read(np.float32).reshape(T, -1), orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, cap, p0, win=win, causal=False), F32,
+                "ns_mg_attn, not causal, prompt kernel")
+
+
+def _mm3_inputs(T, H, G, pos0, seed=0):
+    n = pos0 + T
+    q = orc.randn(60 + seed, (T, H * 128))
+    kc, _ = orc.randn_f16(61 + seed, (n, G, 128)); vc, _ = orc.randn_f16(62 + seed, (n, G, 128))
+    return n, q, kc, vc
+
+
+@pytest.mark.parametrize("T,H,G,pos0", [(1, 32, 2, 4000), (4, 16, 1, 700), (40, 32, 2, 900)])
+def test_mm3s_names_are_the_shared_kernels(ops, T, H, G, pos0):
+    """ns_mm3s_attend / _x / _split / _x_split give ns_llm_minimaxm3_attend's bits (one kernel family behind every name),
+    dense and with block lists; the split forms go through the caller's `part`."""
+    g = ops.gpu
+    n, q, kc, vc = _mm3_inputs(T, H, G, pos0)
+    scale = 1.0 / np.sqrt(128.0)
+    assert ops.k.mm3s_attend_supported(H, G, 128) == 1 and ops.k.mm3s_attend_supported(H, G, 64) == 0
+    qb, kb, vb = DevBuf.of(g, q), DevBuf.of(g, kc), DevBuf.of(g, vc)
+    nblk = (n + 127) // 128
+    K = min(6, nblk)
+    rng = np.random.default_rng(3)
+    sel = np.stack([np.stack([rng.permutation(nblk)[:K] for _ in range(G)]) for _ in range(T)]).astype(np.int32)
+    sel[-1, -1, 0] = nblk - 1
+    for lists in (None, sel):
+        sb = DevBuf.of(g, lists) if lists is not None else None
+        kk = K if lists is not None else 0
+        base = DevBuf(g, T * H * 128 * 4); base.fill(0xFF)
+        ops.minimaxm3_attend(qb, kb, vb, base, T, H, G, pos0, scale, sel=sb, K=kk)
+        want = base.read(np.float32)
+        close_to = orc.mm3_attend(q, kc, vc, T, H, G, pos0, scale, sel=lists, K=kk)
+        check_close(want.reshape(T, -1), close_to.astype(np.float64), F32, "minimaxm3_attend")
+        S = kk if lists is not None else nblk
+        for form in ("", "x", "split", "x_split"):
+            ob = DevBuf(g, T * H * 128 * 4); ob.fill(0xFF)
+            part = DevBuf(g, T * G * S * 16 * 130 * 4) if "split" in form else None
+            if part is not None:
+                part.fill(0xFF)
+            # the matrix-unit names take any scale that is not positive as 1 / sqrt(128)
+            ops.mm3s_attend(form, qb, kb, vb, ob, T, H, G, pos0, 0.0 if form.startswith("x") else scale, sel=sb, K=kk, S=S, part=part)
+            assert np.array_equal(ob.read(np.float32), want), (form, lists is not None)
+            if part is not None and T <= 16 and H == 16 * G:
+                assert not np.all(part.read(np.uint8) == 0xFF), "the caller's part was not used"
+
+
+@pytest.mark.parametrize("T,H,G,pos0,w0", [(8, 32, 2, 3000, 1234), (16, 16, 1, 5000, 0), (4, 16, 1, 227 - 3, 100), (24, 32, 2, 2000, 777)])
+def test_mm3s_attend_block(ops, T, H, G, pos0, w0):
+    """A draft block: every row sees keys w0 .. pos0 + T - 1. (The third shape: 128 keys that straddle a 128-key boundary -
+    one split more than the caller's S = 1 holds, so the partials go through the library's own memory.)"""
+    g = ops.gpu
+    n, q, kc, vc = _mm3_inputs(T, H, G, pos0, seed=5)
+    S = (n - w0 + 127) // 128
+    part = DevBuf(g, T * G * S * 16 * 130 * 4)
+    ob = DevBuf(g, T * H * 128 * 4); ob.fill(0xFF)
+    ops.mm3s_attend("block", DevBuf.of(g, q), DevBuf.of(g, kc), DevBuf.of(g, vc), ob, T, H, G, pos0, 0.0, S=S, part=part, w0=w0)
+    ref = orc.attn_f64_block(q, kc.view(np.uint8), vc.view(np.uint8), 0, T, H, G, 128, n, pos0, w0, pm=True)
+    check_close(ob.read(np.float32).reshape(T, -1), ref, F32, "ns_mm3s_attend_block")
+
+
+@pytest.mark.parametrize("kt,Hq,Hkv,D,cap,n", [(0, 12, 2, 256, 3000, 2777), (1, 12, 2, 256, 900, 900), (2, 6, 1, 256, 500, 333),
+                                               (0, 32, 8, 128, 1500, 1499), (1, 8, 8, 128, 70, 1)])
+def test_q35_attn_probs(ops, kt, Hq, Hkv, D, cap, n):
+    g = ops.gpu
+    k = orc.randn(70 + kt, (cap, Hkv * D))
+    kc, _ = orc.kv_store(kt, k, k, Hkv, D, cap, 0)
+    q = orc.randn(71, (Hq, D), 0.6)
+    base = np.linspace(0.0, 0.5, n).astype(np.float32)
+    qb, kb = DevBuf.of(g, q), DevBuf.of(g, kc)
+    for mode in (0, 1):
+        ob = DevBuf.of(g, base)
+        sc = DevBuf(g, 2 * Hq * 4)
+        ops.q35_attn_probs(kt, qb, kb, Hq, Hkv, D, cap, n, mode, sc, ob)
+        got = ob.read(np.float32)
+        want = orc.attn_probs(kt, q, kc, Hq, Hkv, D, cap, n, mode, out=base)
+        # float32 softmax weights summed in another order: a few ulps of the largest weight
+        assert np.abs(got - want).max() <= 2e-6 + 1e-5 * np.abs(want - base).max(), (mode, np.abs(got - want).max())
+        if mode == 0:
+            assert abs(float((got.astype(np.float64) - base).sum()) - 1.0) < 1e-4
+
+
+def test_glm_dense_over_a_float32_cache(ops):
+    g = ops.gpu
+    L, scale = 512, 0.044
+    for T, H, pos0 in ((1, 64, 2047), (5, 16, 300), (40, 8, 100)):
+        n = pos0 + T
+        qa, c = orc.randn(80, (T, H * L), 0.3), orc.randn(81, (n, L))
+        u = DevBuf(g, T * H * L * 4); u.fill(0xFF)
+        ops.mla_attend_f32(DevBuf.of(g, qa), DevBuf.of(g, c), u, T, H, L, pos0, scale)
+        want = orc.glm_mla_attend_f32(qa, c, T, H, L, pos0, scale).reshape(T, H * L)
+        check_close(u.read(np.float32).reshape(T, H * L), want.astype(np.float64), F32, "ns_mla_attend")
+
+
+def test_gather_q8_rows_as_half(ops):
+    g = ops.gpu
+    L, rows, n = 512, 300, 1000
+    y = orc.glm_to_q8row(orc.randn(90, (rows, L), 2.0), L)
+    idx = np.random.default_rng(1).integers(0, rows, n).astype(np.int32)
+    out = DevBuf(g, n * L * 2); out.fill(0xFF)
+    ops.gather_q8_h(DevBuf.of(g, y), rows, DevBuf.of(g, idx), out, n, L)
+    assert np.array_equal(out.read(np.uint16).reshape(n, L), orc.glm_gather_q8_h(y, idx, L))
+
+
+@pytest.mark.parametrize("q8", [False, True])
+def test_glm_cell_pools_of_a_long_pass(ops, q8):
+    """More rows than one pass of the selection kernel takes (16): queued pass after pass, each row with its own list."""
+    g = ops.gpu
+    T, H, L, pos0, K, scale = 40, 16, 512, 3000, 32, 0.044
+    n = pos0 + T
+    qa = orc.randn(91, (T, H * L), 0.3)
+    x = orc.randn(92, (n, L))
+    rows = orc.glm_to_q8row(x, L) if q8 else orc.f2h(x).view(np.uint8).reshape(n, 2 * L)
+    rng = np.random.default_rng(9)
+    npool = (pos0 + 1) // 4
+    sel = np.stack([rng.permutation(npool)[:K] for _ in range(T)]).astype(np.int32)
+    cnt = rng.integers(0, K + 1, T).astype(np.int32)
+    u = DevBuf(g, T * H * L * 4); u.fill(0xFF)
+    ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, scale, q8=q8, sel=DevBuf.of(g, sel), sel_cnt=DevBuf.of(g, cnt), K=K)
+    want = orc.glm_mla_attend_sel(qa, rows, q8, T, H, L, pos0, scale, sel, cnt, K)
+    check_close(u.read(np.float32).reshape(T, H * L), want.reshape(T, H * L).astype(np.float64), F32, "ns_mla_attend_sel, 40 rows")

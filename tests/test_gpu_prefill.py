@@ -5,7 +5,7 @@ import pytest
 
 from helpers import check_close, gpu_decode, gpu_prompt, make_kv, make_q
 from nextsycl_amd import DevBuf
-from nextsycl_amd.attn import BF16, F16, F32
+from nextsycl_amd.attn import BF16, F16, F32, TUNE_PREFILL_SPLITS, TUNE_PREFILL_WAVES
 from oracle import orc
 
 pytestmark = pytest.mark.gpu
@@ -65,16 +65,16 @@ def test_prefill_seeded_shapes(ops, T, Hq, Hkv, D, p0, win, kt, qt):
 @pytest.mark.parametrize("T,Hq,Hkv,D,p0,win,kt,qt", [(700, 10, 2, 128, 300, 0, 3, BF16), (513, 4, 1, 128, 0, 400, 0, F32),
                                                      (300, 8, 2, 256, 100, 0, 3, BF16), (260, 4, 1, 256, 0, 200, 0, F32),
                                                      (200, 4, 2, 256, 60, 0, 1, F16), (140, 4, 1, 256, 0, 0, 2, F32)])
-def test_prefill_work_groups_of_8_waves(ops, monkeypatch, T, Hq, Hkv, D, p0, win, kt, qt):
+def test_prefill_work_groups_of_8_waves(ops, tune, T, Hq, Hkv, D, p0, win, kt, qt):
     """Long passes run work-groups of 8 waves (blocks of 256 rows; 128 at head size 256), short ones of 4: the same rows,
     keys and order of a wave's arithmetic, so the two agree bit for bit; forced here on shapes the oracle finishes in
     seconds."""
     cap = p0 + T + 5
     kc, vc = make_kv(kt, Hkv, D, cap, p0 + T)
     qd, qf = make_q(qt, T, Hq, D)
-    monkeypatch.setenv("NS_PREFILL_WAVES", "8")
+    tune(TUNE_PREFILL_WAVES, 8)
     got8, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
-    monkeypatch.setenv("NS_PREFILL_WAVES", "4")
+    tune(TUNE_PREFILL_WAVES, 4)
     got4, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
     ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
     check_close(got8, ref, qt, "prefill (8 waves) vs float64 closed form", kt=kt)
@@ -104,7 +104,7 @@ def test_prefill_key_splits(ops, T, Hq, Hkv, D, p0, win, kt, qt):
 
 @pytest.mark.parametrize("ns", [2, 5, 16])
 @pytest.mark.parametrize("T,Hq,Hkv,D,p0,win", [(200, 4, 2, 128, 0, 0), (150, 2, 1, 128, 700, 90), (70, 4, 2, 256, 333, 0)])
-def test_prefill_forced_splits(ops, monkeypatch, ns, T, Hq, Hkv, D, p0, win):
+def test_prefill_forced_splits(ops, tune, ns, T, Hq, Hkv, D, p0, win):
     """Splits forced onto short passes: splits wholly past a row block's last key, splits a window leaves empty, a last
     split of a few keys - the same result as the unsplit pass within the path's bar, and the same whatever the
     work-group size (bit for bit)."""
@@ -112,10 +112,10 @@ def test_prefill_forced_splits(ops, monkeypatch, ns, T, Hq, Hkv, D, p0, win):
     kc, vc = make_kv(0, Hkv, D, cap, p0 + T, cfg=1)
     qd, qf = make_q(F32, T, Hq, D, cfg=2)
     ref = orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, cap, p0, win=win)
-    monkeypatch.setenv("NS_PREFILL_SPLITS", str(ns))
-    monkeypatch.setenv("NS_PREFILL_WAVES", "8")
+    tune(TUNE_PREFILL_SPLITS, ns)
+    tune(TUNE_PREFILL_WAVES, 8)
     got8, _ = gpu_prompt(ops, F32, 0, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
-    monkeypatch.setenv("NS_PREFILL_WAVES", "4")
+    tune(TUNE_PREFILL_WAVES, 4)
     got4, _ = gpu_prompt(ops, F32, 0, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
     check_close(got8, ref, F32, "prefill with %d forced splits" % ns)
     assert np.array_equal(got8, got4)

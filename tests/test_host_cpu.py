@@ -68,6 +68,47 @@ def test_pure_functions_without_a_gpu(handle):
     assert handle.ns_last_error() is not None
 
 
+def test_null_buffers_are_refused_before_any_launch(handle):
+    """Entry points that launch kernels check their pointers and strides on the host: a forgotten buffer is -1 with the
+    reason, not a GPU fault. (No ns_gpu here either: nothing may touch the device before the checks pass.)"""
+    i64, P, f32 = C.c_int64, C.c_void_p, C.c_float
+    handle.ns_last_error.restype = C.c_char_p
+    buf = C.create_string_buffer(4096)
+    b = C.addressof(buf) // 16 * 16 + 16
+
+    def refused(name, argtypes, args, word):
+        f = getattr(handle, name)
+        f.restype, f.argtypes = C.c_int, argtypes
+        assert f(*args) == -1, name
+        assert word in handle.ns_last_error().decode(), (name, handle.ns_last_error())
+
+    st = [P, C.c_int, C.c_int, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]
+    refused("ns_attn_kv_store", st, (None, 0, 0, b, 128, b, 128, 1, 1, 128, 4, 0, b, None), "null")
+    refused("ns_attn_kv_store", st, (None, 0, 0, None, 128, b, 128, 1, 1, 128, 4, 0, b, b), "null")
+    refused("ns_attn_kv_dequant", [P, C.c_int, P, i64, i64, i64, P], (None, 1, b, 2, 128, 136, None), "null")
+    refused("ns_attn_kv_dequant", [P, C.c_int, P, i64, i64, i64, P], (None, 1, b, 2, 128, 100, b), "a row apart")
+    refused("ns_q35_fwht32", [P, P, i64, i64, i64], (None, None, 2, 64, 64), "null")
+    refused("ns_q35_fwht32", [P, P, i64, i64, i64], (None, b, 2, 64, 32), "a row apart")
+    ds = [P, P, P, f32, P, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32]
+    refused("ns_ds2_kv_store", ds, (None, b, None, 1e-6, b, 1, 512, 64, 0, 1e4, 1.0, 0.0, 1.0, 0.0, 0.0), "null")
+    refused("ns_to_q8row", [P, P, P, i64, i64], (None, b, None, 1, 512), "null")
+    refused("ns_gather_q8_h", [P, P, P, P, i64, i64], (None, b, None, b, 1, 512), "null")
+    refused("ns_gather_q8_h", [P, P, P, P, i64, i64], (None, b, b, b, 1, 256), "512")
+    refused("ns_attn_tune", [C.c_int, i64], (9, 1), "knob")
+    refused("ns_attn_tune", [C.c_int, i64], (0, -1), "knob")
+    handle.ns_attn_tune.restype = C.c_int
+    assert handle.ns_attn_tune(0, 0) == 0
+    # the new pure functions
+    bs = handle.ns_mg_attn_block_scratch
+    bs.restype, bs.argtypes = i64, [i64] * 6
+    ds_ = handle.ns_attn_decode_scratch
+    ds_.restype, ds_.argtypes = i64, [i64] * 6
+    assert bs(8, 32, 8, 128, 5000, 4096) == ds_(8, 32, 8, 128, 5000, 4096) and bs(17, 32, 8, 128, 5000, 0) == 0
+    sup = handle.ns_mm3s_attend_supported
+    sup.restype, sup.argtypes = C.c_int, [i64] * 3
+    assert sup(64, 4, 128) == 1 and sup(64, 4, 64) == 0 and sup(63, 4, 128) == 0
+
+
 def test_row_bytes_and_errors():
     assert [kv_row_bytes(k, 128) for k in (0, 1, 2, 3)] == [256, 136, 72, 256]
     assert [kv_row_bytes(k, 256) for k in (0, 1, 2)] == [512, 272, 144]      # llm/qwen35/src/engine.rs:54-60
