@@ -86,6 +86,17 @@ int64_t ns_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, in
 int ns_attn_decode_t(ns_gpu* g, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq,
                      int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out, float* scratch);
 
+/* ns_attn_decode_t without a scratch argument and without any allocation: the partials go through an array that is part
+ * of the library's code object (NS_ATTN_STATIC_SCRATCH_FLOATS floats = 16 MiB, held by every GPU the library runs on
+ * until the process ends; its address is looked up at ns_gpu_open). No counterpart in the reference: it is for callers
+ * that cannot allocate - code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. Same
+ * arguments, same result bit for bit. -1 when ns_attn_decode_scratch(T, Hq, Hkv, D, p0, win) exceeds the array (take
+ * ns_attn_decode_t with a buffer of the caller's then). Every call on a GPU shares that GPU's array: calls that overlap
+ * on one GPU race */
+#define NS_ATTN_STATIC_SCRATCH_FLOATS (4 << 20)
+int ns_attn_decode_static(ns_gpu* g, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq,
+                          int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out);
+
 /* Replaces: kernels/llm/qwen35/silo/silo.h:46-59 (silo/attn.cpp:375-435). The reference covers D 256 with 6 query
  * heads a key head and 1..8 rows; here D 128 or 256, any Hq a multiple of Hkv, 1..16 rows */
 int ns_q35_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);

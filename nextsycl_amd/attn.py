@@ -40,6 +40,7 @@ ATTN_H = {
     "ns_q35_fwht32": (i32, [P, P, i64, i64, i64]),
     "ns_attn_decode_scratch": (i64, [i64, i64, i64, i64, i64, i64]),
     "ns_attn_decode_t": (i32, [P, i32, i32, i32, P, i64, P, P, i64, i64, i64, i64, i64, i64, i64, f32, P, P]),
+    "ns_attn_decode_static": (i32, [P, i32, i32, i32, P, i64, P, P, i64, i64, i64, i64, i64, i64, i64, f32, P]),
     "ns_q35_attn_decode_supported": (i32, [i64, i64, i64, i64]),
     "ns_q35_attn_decode_scratch": (i64, [i64, i64, i64, i64, i64]),
     "ns_q35_attn_decode": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P, P]),
@@ -230,6 +231,17 @@ class Ops:
         _need(vc, self.cache_bytes(kt, Hkv, cap, D), "decode value cache")
         self.ok(self.k.attn_decode_t(self.raw(), qt, kt, int(pm), q.ptr, qs, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, scale, out.ptr,
                                      scratch.ptr if scratch is not None else None), "attention decode")
+
+    def decode_static(self, qt, kt, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, out, win=0, pm=False, scale=0.0):
+        """ns_attn_decode_static: the typed decode with the partials in the library's device-resident array - no scratch
+        buffer, no allocation."""
+        if T > 0:
+            _need(q, ((T - 1) * qs + Hq * D) * ELT[qt], "decode q")
+            _need(out, T * Hq * D * ELT[qt], "decode out")
+        _need(kc, self.cache_bytes(kt, Hkv, cap, D), "decode key cache")
+        _need(vc, self.cache_bytes(kt, Hkv, cap, D), "decode value cache")
+        self.ok(self.k.attn_decode_static(self.raw(), qt, kt, int(pm), q.ptr, qs, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, scale, out.ptr),
+                "attention decode (static scratch)")
 
     def q35_attn_decode_kv(self, kt, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, out, scratch):
         if T > 0:

@@ -37,6 +37,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
+#include <mutex>
 #include <string>
 #include <type_traits>
 
@@ -903,7 +904,49 @@ int ns_attn_decode_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     return decode_checked(g, who, qt, kt, pm, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, win, x, scale, out, scratch);
 }
 
+// ---- a decode entry point that allocates nothing ---------------------------------------------------------------------
+// Callers under HIP graph capture, tight serving loops and harnesses that forbid allocation cannot hand over a scratch
+// buffer they would have to hipMalloc first. ns_attn_decode_static is ns_attn_decode_t with the partials in an array that
+// is part of the library's code object: each GPU the library runs on holds its own copy, at its own address, until the
+// process ends. In host code the array's name is only a handle for hipGetSymbolAddress - never a device address - so
+// the address is looked up once a device (ns_gpu_open calls ns_attn_static_scratch_init with the device current) and
+// every launch is given that pointer. Nothing in it has to start at zero: a pass writes every partial it later merges.
+// Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two ns_gpu of one device, or two streams)
+// race.
+static __device__ __align__(256) float ns_static_scratch[NS_ATTN_STATIC_SCRATCH_FLOATS];
+
+namespace {
+constexpr int STATIC_MAX_DEVS = 64;
+float* static_scratch_ptr[STATIC_MAX_DEVS] = {};
+std::mutex static_scratch_mu;
+}  // namespace
+
+int ns_attn_static_scratch_init(int dev) {
+    if (dev < 0 || dev >= STATIC_MAX_DEVS) return ns_fail("ns_attn_decode_static: device index past the table");
+    std::lock_guard<std::mutex> lock(static_scratch_mu);
+    if (static_scratch_ptr[dev]) return 0;
+    void* ptr = nullptr;
+    NS_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(ns_static_scratch)));
+    if (!ptr) return ns_fail("ns_attn_decode_static: the scratch array has no address on this device");
+    static_scratch_ptr[dev] = (float*) ptr;
+    return 0;
+}
+
 extern "C" {
+
+int ns_attn_decode_static(ns_gpu* g, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq,
+                          int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out) {
+    if (T <= 0) return 0;
+    if (!g || g->dev < 0 || g->dev >= STATIC_MAX_DEVS || !static_scratch_ptr[g->dev]) return ns_fail("ns_attn_decode_static: the device's scratch array was not set up");
+    if (T > 16 || Hq <= 0 || Hkv <= 0 || (D != 128 && D != 256)) return ns_fail("ns_attn_decode_static: 1..16 rows, heads of 128 or 256");
+    const int64_t need = ns_attn_decode_scratch(T, Hq, Hkv, D, p0, win);
+    if (need > (int64_t) NS_ATTN_STATIC_SCRATCH_FLOATS)
+        return ns_fail("ns_attn_decode_static: the pass needs " + std::to_string(need) + " floats of scratch, the array holds " +
+                       std::to_string((int64_t) NS_ATTN_STATIC_SCRATCH_FLOATS) + " (use ns_attn_decode_t with a buffer of the caller's)");
+    DecodeExtra x;
+    x.marks = false;                                   // (the profiling events are created on first use: an allocation)
+    return decode_checked(g, "ns_attn_decode_static", qt, kt, pm, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, win, x, scale, out, static_scratch_ptr[g->dev]);
+}
 
 int64_t ns_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win) {
     if (T <= 0 || Hq <= 0 || Hkv <= 0) return 0;

@@ -123,7 +123,8 @@ int ns_gpu_open(int index, ns_gpu** out) {
     if (ns_hip_check(hipStreamCreateWithFlags(&g->q, hipStreamNonBlocking), "compute stream") ||
         ns_hip_check(hipStreamCreateWithFlags(&g->cq, hipStreamNonBlocking), "copy stream 0") ||
         ns_hip_check(hipStreamCreateWithFlags(&g->cq2, hipStreamNonBlocking), "copy stream 1") ||
-        ns_hip_check(hipMalloc((void**) &g->own_scratch, OWN_SCRATCH_FLOATS * sizeof(float)), "library scratch")) {
+        ns_hip_check(hipMalloc((void**) &g->own_scratch, OWN_SCRATCH_FLOATS * sizeof(float)), "library scratch") ||
+        ns_attn_static_scratch_init(index)) {
         ns_gpu_close(g);
         return -1;
     }

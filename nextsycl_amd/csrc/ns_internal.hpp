@@ -29,6 +29,10 @@ struct ns_gpu {
 // records profile event i on the compute stream when profiling is on (creates it on first use); 0 or -1
 int ns_profile_mark(ns_gpu* g, int i);
 
+// attn_decode.hip: looks up, once a device and with that device current, the address of the device-resident scratch
+// array that ns_attn_decode_static uses (called by ns_gpu_open); 0 or -1
+int ns_attn_static_scratch_init(int dev);
+
 // sets the calling thread's error text (ns_last_error) and returns -1
 int ns_fail(const std::string& what);
 // -1 with "hip: <what>: <error string>" when e is an error, else 0
