@@ -50,6 +50,12 @@ __device__ __forceinline__ s4v lds_read_tr16(void* lds_addr) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// the largest of three numbers as one instruction (for values that are never NaN: fmaxf would first quieten each input)
+__device__ __forceinline__ float max3f(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 
 // Reductions over the 4 lanes {n, n + 16, n + 32, n + 48} that hold one query row's scores. The partner's value comes
 // by v_permlane16_swap / v_permlane32_swap (vector instructions: given two copies of v they return, in every lane, the

@@ -172,13 +172,16 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 
     // Online softmax state, in base-2 exponent units (scores x scale x log2 e): nbr = minus the reference the weights
     // are taken against, thr = how far a score may exceed it before the reference moves (-inf while the row has seen no
-    // key: the first one sets it), l_r = this lane's own share of the row's sum
-    float nbr[RT], thr[RT], l_r[RT];
+    // key: the first one sets it). The row's sum of weights l4 comes out of the matrix unit: a product of the rounded weights
+    // with an operand of ones beside each step's V^T P^T (every slot of l4 then holds the whole row's sum - no vector
+    // additions, no cross-lane step, and numerator and denominator carry the very same rounded weights)
+    float nbr[RT], thr[RT];
+    f4v l4[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         nbr[rt] = 0.0f;
         thr[rt] = -INFINITY;
-        l_r[rt] = 0.0f;
+        l4[rt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
     }
     f4v o[RT][DT];
 #pragma unroll
@@ -274,29 +277,62 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) pb[rt] = s8v{0, 0, 0, 0, 0, 0, 0, 0};
     // S^T of one 32-key half (LDS byte offset kl) against the wave's 32 rows: the raw dot products
-    auto scores = [&](f4v (&s)[RT][2], uint32_t kl) {
+    // (the operands of a block's first matrix instructions are read a block earlier - kread / vread - so that their LDS
+    // latency passes under the other block's work instead of at the head of this one)
+    constexpr int VPRE = D == 128 ? DT : 4;                       // value operands read ahead
+    constexpr int KPRE = D == 128 ? 2 : 1;                        // 16-key halves whose key operands are read ahead
+    auto kread = [&](s8v (&ka)[KPRE][KB], uint32_t kl) {
 #pragma unroll
-        for (int kt2 = 0; kt2 < 2; ++kt2) {
-            s8v ka[KB];
+        for (int kt2 = 0; kt2 < KPRE; ++kt2)
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb)
-                ka[kb] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + kl + k_rd + kt2 * 16 * KS + kb * 64);
+                ka[kt2][kb] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + kl + k_rd + kt2 * 16 * KS + kb * 64);
+    };
+    auto vread1 = [&](uint32_t vl, int dt) {
+        const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + vl + v_rd + dt * 32));
+        const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + vl + v_rd + dt * 32 + 16 * VS));
+        return s8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    auto vread = [&](s8v (&va)[VPRE], uint32_t vl) {
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) {
-                f4v acc = mfma16<BF>(ka[0], qreg[rt][0], f4v{0.0f, 0.0f, 0.0f, 0.0f});
+        for (int dt = 0; dt < VPRE; ++dt) va[dt] = vread1(vl, dt);
+    };
+    auto scores = [&](f4v (&s)[RT][2], uint32_t kl, const s8v (&kpre)[KPRE][KB]) {
+        if constexpr (KPRE == 2) {
+            // every operand is in registers: the 2 RT chains of dependent products advance side by side
 #pragma unroll
-                for (int kb = 1; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
-                s[rt][kt2] = acc;
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int kt2 = 0; kt2 < 2; ++kt2)
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+                        s[rt][kt2] = mfma16<BF>(kpre[kt2][kb], qreg[rt][kb], kb == 0 ? f4v{0.0f, 0.0f, 0.0f, 0.0f} : s[rt][kt2]);
+        } else {
+#pragma unroll
+            for (int kt2 = 0; kt2 < 2; ++kt2) {
+                s8v ka[KB];
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+                    ka[kb] = kt2 == 0 ? kpre[0][kb] : *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + kl + k_rd + kt2 * 16 * KS + kb * 64);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+                    f4v acc = mfma16<BF>(ka[0], qreg[rt][0], f4v{0.0f, 0.0f, 0.0f, 0.0f});
+#pragma unroll
+                    for (int kb = 1; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
+                    s[rt][kt2] = acc;
+                }
             }
         }
     };
     // O^T += V^T P^T of one 32-key half (LDS byte offset vl) with the weights in pb
-    auto weigh = [&](uint32_t vl) {
+    constexpr short ONE16 = BF ? (short) 0x3F80 : (short) 0x3C00;
+    const s8v ones = {ONE16, ONE16, ONE16, ONE16, ONE16, ONE16, ONE16, ONE16};
+    auto weigh = [&](uint32_t vl, const s8v (&vpre)[VPRE]) {
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) l4[rt] = mfma16<BF>(ones, pb[rt], l4[rt]);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
-            const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + vl + v_rd + dt * 32));
-            const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + vl + v_rd + dt * 32 + 16 * VS));
-            const s8v va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            const s8v va = dt < VPRE ? vpre[dt] : vread1(vl, dt);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
         }
@@ -308,14 +344,15 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     //   (only if some row's score outgrew its reference by more than 2^8: move the references, rescale; the weights may
     //    otherwise exceed 1, by at most 2^8: harmless in float32 sums and 16-bit operands, and the final division by
     //    the row's sum makes the result the same function of the inputs)
-    //   B: S^T of step s + 1              ||   weights of step s = exp2(arguments), their sum, rounding to 16 bit
+    //   B: S^T of step s + 1              ||   weights of step s = exp2(arguments), rounded to 16 bit
+    // Every LDS operand of a block is requested a block ahead (vread at the step's start, kread at the head of A), and
+    // sched_group_barrier deals the vector instructions out between the matrix instructions.
     // The mask is applied under a wave-uniform branch: steps no row's causal or window edge crosses pay no comparison.
     auto step = [&](f4v (&sc)[RT][2], f4v (&sn)[RT][2], uint32_t kl_next, uint32_t vl_prev, int j0, bool masked) {
         float a[RT][8], amax[RT];
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) a[rt][e] = __builtin_fmaf(sc[rt][e >> 2][e & 3], p.sl2, nbr[rt]);
+        s8v vpre[VPRE], kpre[KPRE][KB];
+        vread(vpre, vl_prev);
+        // (the mask goes onto the raw scores: minus infinity stays minus infinity under the positive scale)
         if (masked) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -328,17 +365,30 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const int j = (e >> 2) * 16 + g4 * 4 + (e & 3);
-                    a[rt][e] = (unsigned) (j - lo) <= span ? a[rt][e] : -INFINITY;
+                    sc[rt][e >> 2][e & 3] = (unsigned) (j - lo) <= span ? sc[rt][e >> 2][e & 3] : -INFINITY;
                 }
             }
         }
         __builtin_amdgcn_s_setprio(1);
-        weigh(vl_prev);
+        kread(kpre, kl_next);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[rt][e] = __builtin_fmaf(sc[rt][e >> 2][e & 3], p.sl2, nbr[rt]);
+        weigh(vl_prev, vpre);
         bool grow = false;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-            amax[rt] = fmaxf(fmaxf(fmaxf(fmaxf(fmaxf(fmaxf(fmaxf(a[rt][0], a[rt][1]), a[rt][2]), a[rt][3]), a[rt][4]), a[rt][5]), a[rt][6]), a[rt][7]);
+            amax[rt] = max3f(max3f(max3f(a[rt][0], a[rt][1], a[rt][2]), a[rt][3], a[rt][4]), max3f(a[rt][5], a[rt][6], a[rt][7]), a[rt][7]);
             grow |= amax[rt] > thr[rt];
+        }
+        if constexpr (D == 128) {
+            // the matrix instructions of this block with two vector instructions between each
+#pragma unroll
+            for (int i = 0; i < RT * DT + RT; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+            }
         }
         if (__any(grow)) {
 #pragma unroll
@@ -348,7 +398,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                 const bool nokey = mx == -INFINITY;
                 const float delta = fresh ? (nokey ? 0.0f : mx) : fmaxf(mx, 0.0f);
                 const float c = fresh ? 1.0f : fast_exp2(-delta);
-                l_r[rt] *= c;
+                l4[rt] *= c;
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
                 nbr[rt] -= delta;
@@ -357,21 +407,24 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                 thr[rt] = (fresh && nokey) ? -INFINITY : 8.0f;
             }
         }
-        scores(sn, kl_next);
+        scores(sn, kl_next, kpre);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-            float sum = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float pv = fast_exp2(a[rt][e]);                // -inf -> 0
-                sum += pv;
-                pb[rt][e] = to16<BF>(pv);
+            for (int e = 0; e < 8; ++e) pb[rt][e] = to16<BF>(fast_exp2(a[rt][e]));      // -inf -> 0
+        }
+        if constexpr (D == 128) {
+            // a matrix instruction, an exponential, and a conversion after every other
+#pragma unroll
+            for (int i = 0; i < RT * 2 * KB; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
+                if (i & 1) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
             }
-            l_r[rt] += sum;
         }
         // the step's results are complete here, in program order: nothing of it drifts past the next barrier or branch
-        if constexpr (RT == 2) asm volatile("" : "+v"(pb[0]), "+v"(pb[1]), "+v"(l_r[0]), "+v"(l_r[1]));
-        else asm volatile("" : "+v"(pb[0]), "+v"(l_r[0]));
+        if constexpr (RT == 2) asm volatile("" : "+v"(pb[0]), "+v"(pb[1]));
+        else asm volatile("" : "+v"(pb[0]));
         __builtin_amdgcn_s_setprio(0);
     };
 
@@ -401,7 +454,11 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         fetch(stk, kbase, 1);
         fetch(stv, vbase, 1);
         __syncthreads();
-        scores(sA, 0);
+        {
+            s8v kpre[KPRE][KB];
+            kread(kpre, 0);
+            scores(sA, 0, kpre);
+        }
         for (int k = 0; k < nt; k += 2) {
             // tile k: buffers 0
             stash_k(stk, 1);
@@ -422,7 +479,11 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             step(sB, sA, 0, V0 + VBUF, 64 * k + 96, !(64 * k + 96 >= w_full_beg && 64 * k + 128 <= w_full_end));
         }
         // the last step's product
-        weigh(V0 + (uint32_t) ((nt - 1) & 1) * VBUF + 32 * VS);
+        {
+            s8v vpre[VPRE];
+            vread(vpre, V0 + (uint32_t) ((nt - 1) & 1) * VBUF + 32 * VS);
+            weigh(V0 + (uint32_t) ((nt - 1) & 1) * VBUF + 32 * VS, vpre);
+        }
     }
 
     // ---- out = O / l. A lane holds dims 16 dt + 4 g4 .. + 3 of its rows: the wave's 32 x D block goes through LDS (the
@@ -435,7 +496,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         const uint32_t ob = (uint32_t) w * 16 * rowp;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-            const float lsum = rows_sum(l_r[rt]);
+            const float lsum = l4[rt][0];
             const uint32_t at = ob + (uint32_t) n * rowp + (uint32_t) (g4 * 16);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<__attribute__((address_space(3))) f4v*>(L + at + dt * 64) = o[rt][dt];
@@ -463,7 +524,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         uint8_t* const orow = reinterpret_cast<uint8_t*>(p.out) + (int64_t) hq * rowb;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
-            const float lsum = rows_sum(l_r[rt]);
+            const float lsum = l4[rt][0];
             const float inv = lsum > 0.0f ? 1.0f / lsum : 0.0f;
             const uint32_t at = ob + (uint32_t) n * rowp + (uint32_t) (g4 * 4 * esz);
 #pragma unroll
