@@ -127,7 +127,7 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
     const int rr = live ? ri : rows - 1;
     const int64_t hi_r = !live ? -1 : p.per_t ? je - 1 : std::min(p.pos0 + rr / p.H, je - 1);
     s8v qreg[KB];
-    {
+    auto load_queries = [&]() {
         const int64_t qoff = (int64_t) rr * DK + g4 * 8;
         if (p.qt == 0) {
 #pragma unroll
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
                 for (int i = 0; i < 8; ++i) qreg[kb][i] = live ? raw[i] : (short) 0;
             }
         }
-    }
+    };
     float nbr = 0.0f, thr = -INFINITY, l_r = 0.0f;
     const int hi_rel = (int) std::max<int64_t>(std::min<int64_t>(hi_r - jb, (int64_t) 1 << 30), -1);
     f4v o[DT];
@@ -226,8 +226,32 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
     // last 64 units again, so that every wave has the same count in flight).
     constexpr int NU = MTILE * RCH, NDMA = (NU + MW * 64 - 1) / (MW * 64);
     static_assert(NU % 64 == 0, "whole instructions a tile");
+    // (a whole tile of a dense split: lane offsets that do not depend on the tile, worked out once)
+    // (the 8-wave form has no registers to spare for them)
+    constexpr bool DMA_PRE = MW == 4 && !Q8;
+    uint32_t dma_off[DMA_PRE ? NDMA : 1];
+    if constexpr (DMA_PRE) {
+#pragma unroll
+        for (int i = 0; i < NDMA; ++i) {
+            const int u0 = std::min(i * MW * 64 + w * 64, NU - 64);
+            const int u = u0 + lane, r = u / RCH, c = std::min(u % RCH, CPR - 1);
+            dma_off[i] = (uint32_t) (r * CROW + c * 16);
+        }
+    }
     auto dma = [&](lds_u8* dst, int it_) {
         const bool plain = !selt && (it_ + 1) * MTILE - 1 <= last_rel;
+        if constexpr (DMA_PRE) {
+            if (plain) {
+                const uint8_t* sp = split_base + (int64_t) it_ * MTILE * CROW;
+#pragma unroll
+                for (int i = 0; i < NDMA; ++i) {
+                    const int u0 = std::min(i * MW * 64 + w * 64, NU - 64);
+                    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (sp + dma_off[i]),
+                                                     (__attribute__((address_space(3))) void*) (dst + u0 * 16), 16, 0, 0);
+                }
+                return;
+            }
+        }
         const uint8_t* sp = selt ? p.cache : split_base + (plain ? (int64_t) it_ * MTILE * CROW : 0);
 #pragma unroll
         for (int i = 0; i < NDMA; ++i) {
@@ -360,31 +384,167 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
             asm volatile("" ::: "memory");
         }
     };
-    if (nt > 0) {
-        if constexpr (Q8) {
+    // Half rows: the same three parts software-pipelined over the tiles, so that the one wave a SIMD holds keeps its matrix
+    // pipe fed while the vector unit works - a tile's step is two straight-line blocks,
+    //   1: S^T of tile it + 1 (its buffer landed a step ago)   ||   weights of tile it = exp2(arguments), sum, rounding
+    //   2: O^T += C^T P^T of tile it                           ||   exponent arguments of tile it + 1 and their largest
+    // then (rarely) the move of the reference, the wait for tile it + 2's transfers and the barrier. Past the split's last
+    // tile block 1 scores whatever the next buffer holds: every such cell is masked.
+    float a_cur[8];
+    auto args_of = [&](const f4v (&s)[2], int it, float (&a)[8]) -> float {
+        const int hi = hi_rel - it * MTILE;                    // cells 0 .. hi of this tile are the row's
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int j = (e >> 2) * 16 + g4 * 4 + (e & 3);
+            a[e] = j <= hi ? __builtin_fmaf(s[e >> 2][e & 3], p.sl2, nbr) : -INFINITY;
+        }
+        return fmaxf(fmaxf(fmaxf(a[0], a[1]), fmaxf(a[2], a[3])), fmaxf(fmaxf(a[4], a[5]), fmaxf(a[6], a[7])));
+    };
+    auto regrow = [&](float amax, float (&a)[8]) {
+        if (__any(amax > thr)) {
+            const float mx = rows_max(amax);
+            const bool fresh = thr < 0.0f, nokey = mx == -INFINITY;
+            const float delta = fresh ? (nokey ? 0.0f : mx) : fmaxf(mx, 0.0f);
+            const float c = fresh ? 1.0f : fast_exp2(-delta);
+            l_r *= c;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) o[dt] *= c;
+            nbr -= delta;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) a[e] -= delta;
+            thr = (fresh && nokey) ? -INFINITY : 8.0f;
+        }
+    };
+    auto scores_of = [&](lds_u8* rd, f4v (&s)[2]) {
+        s[0] = s[1] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+        auto ld = [&](int kb, int ct) {
+            return *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(rd + s_rd[kb & 1] + ct * 16 * RSTRIDE + (kb >> 1) * 128);
+        };
+        constexpr int AHEAD = MW == 4 ? 3 : 1;                 // kb steps (two reads each) in flight
+        s8v fa[AHEAD + 1][2];
+#pragma unroll
+        for (int kb = 0; kb < AHEAD; ++kb) {
+            fa[kb][0] = ld(kb, 0);
+            fa[kb][1] = ld(kb, 1);
+        }
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            if (kb + AHEAD < KB) {
+                fa[(kb + AHEAD) % (AHEAD + 1)][0] = ld(kb + AHEAD, 0);
+                fa[(kb + AHEAD) % (AHEAD + 1)][1] = ld(kb + AHEAD, 1);
+            }
+            s[0] = mfma16<false>(fa[kb % (AHEAD + 1)][0], qreg[kb], s[0]);
+            s[1] = mfma16<false>(fa[kb % (AHEAD + 1)][1], qreg[kb], s[1]);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * AHEAD, 0);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            if (kb + AHEAD < KB) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+            if (kb % 2 == 0 && kb < 16) __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);      // an exponential of the tile before
+        }
+    };
+    auto weigh_of = [&](lds_u8* rd, const s8v pb) {
+        auto ldt = [&](int dt) {
+            const lds_u8* src = rd + v_rd[dt & 3] + (dt >> 2) * 128;
+            const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) src);
+            const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (src + 16 * RSTRIDE));
+            return s8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        };
+        constexpr int AHEAD = MW == 4 ? 6 : 2;
+        s8v va[AHEAD + 1];
+#pragma unroll
+        for (int dt = 0; dt < AHEAD; ++dt) va[dt] = ldt(dt);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            if (dt + AHEAD < DT) va[(dt + AHEAD) % (AHEAD + 1)] = ldt(dt + AHEAD);
+            o[dt] = mfma16<false>(va[dt % (AHEAD + 1)], pb, o[dt]);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 2 * AHEAD, 0);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            if (dt + AHEAD < DT) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+    };
+    auto pstep = [&](lds_u8* rd, lds_u8* nx1, lds_u8* nx2, int it) {
+        if (it + 2 < nt) dma(nx2, it + 2);
+        // ---- block 1
+        f4v s[2];
+        scores_of(nx1, s);
+        s8v pb;
+        {
+            float sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float pv = fast_exp2(a_cur[e]);               // -inf -> 0
+                sum += pv;
+                pb[e] = to16<false>(pv);
+            }
+            l_r += sum;
+        }
+        // ---- block 2
+        weigh_of(rd, pb);
+        const float amax = args_of(s, it + 1, a_cur);
+        regrow(amax, a_cur);
+        if (it + 2 < nt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    if constexpr (Q8) {
+        load_queries();
+        if (nt > 0) {
             fetch(0, 0, H1);
             stash(B0, 0, H1);
             fetch(0, H1, NLD);
             stash(B0, H1, NLD);
-        } else {
-            dma(B0, 0);
-            if (nt > 1) dma(B1, 1);
-            if (nt > 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
-            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
-    }
-    if constexpr (Q8) {
         __syncthreads();
-    } else {
+        for (int it = 0; it < nt; it += 3) {
+            step(B0, B1, B2, it);
+            if (it + 1 >= nt) break;
+            step(B1, B2, B0, it + 1);
+            if (it + 2 >= nt) break;
+            step(B2, B0, B1, it + 2);
+        }
+    } else if constexpr (MW == 8) {
+        // (two waves a SIMD overlap each other; the pipelined form's extra live registers would spill at 256 a wave)
+        if (nt > 0) dma(B0, 0);
+        if (nt > 1) dma(B1, 1);
+        load_queries();
+        if (nt > 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-    }
-    for (int it = 0; it < nt; it += 3) {
-        step(B0, B1, B2, it);
-        if (it + 1 >= nt) break;
-        step(B1, B2, B0, it + 1);
-        if (it + 2 >= nt) break;
-        step(B2, B0, B1, it + 2);
+        for (int it = 0; it < nt; it += 3) {
+            step(B0, B1, B2, it);
+            if (it + 1 >= nt) break;
+            step(B1, B2, B0, it + 1);
+            if (it + 2 >= nt) break;
+            step(B2, B0, B1, it + 2);
+        }
+    } else {
+        // the first two tiles are on their way before the queries are loaded
+        if (nt > 0) dma(B0, 0);
+        if (nt > 1) dma(B1, 1);
+        load_queries();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (nt > 0) {
+            f4v s[2];
+            scores_of(B0, s);
+            const float amax = args_of(s, 0, a_cur);
+            regrow(amax, a_cur);
+        }
+        for (int it = 0; it < nt; it += 3) {
+            pstep(B0, B1, B2, it);
+            if (it + 1 >= nt) break;
+            pstep(B1, B2, B0, it + 1);
+            if (it + 2 >= nt) break;
+            pstep(B2, B0, B1, it + 2);
+        }
     }
 
     // ---- the split's partial {u_s = O / l as halfs, m, l}. A lane holds latents 16 dt + 4 g4 .. + 3 of its row: the
@@ -430,47 +590,63 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
 
 // the splits of a row merged: u = sum_s u_s w_s / sum_s w_s, w_s = l_s 2^(m_s - M). Two work-groups of 256 threads a row,
 // 256 latents each: a thread sums 4 latents (one 8-byte load a split) over every fourth split, then the four phases are
-// added in a fixed order.
+// added in a fixed order. A thread's first 32 loads are requested before anything else, so that they travel while the
+// splits' (m, l) are fetched and turned into weights: one memory latency a row instead of three.
 template <int QT>
 __global__ __launch_bounds__(256) void mla_merge_kernel(const float* __restrict__ part, int ns, void* __restrict__ u) {
     __shared__ float wsh[1024];
-    __shared__ float red[256];
+    __shared__ float red[8];
     __shared__ f4v ph[256];
     const int64_t row = blockIdx.x;
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const float* pr = part + row * ns * PSTRIDE;
-    float mx = -INFINITY;
-    for (int s = tid; s < ns; s += 256) mx = fmaxf(mx, pr[s * PSTRIDE + ML / 2]);
-    red[tid] = mx;
-    __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if (tid < o) red[tid] = fmaxf(red[tid], red[tid + o]);
-        __syncthreads();
-    }
-    mx = red[0];
-    __syncthreads();
-    float ls = 0.0f;
-    for (int s = tid; s < ns; s += 256) {
-        const float m = pr[s * PSTRIDE + ML / 2];
-        const float wgt = m == -INFINITY ? 0.0f : pr[s * PSTRIDE + ML / 2 + 1] * fast_exp2(m - mx);
-        wsh[s] = wgt;
-        ls += wgt;
-    }
-    red[tid] = ls;
-    __syncthreads();
-    for (int o = 128; o > 0; o >>= 1) {
-        if (tid < o) red[tid] += red[tid + o];
-        __syncthreads();
-    }
-    const float L = red[0];
     const int quad = tid & 63, phase = tid >> 6;
     const int lat = blockIdx.y * 256 + quad * 4;
     typedef _Float16 h4v __attribute__((ext_vector_type(4)));
+    constexpr int CH = 32;                                         // loads a thread keeps in flight
+    h4v hv[CH];
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int sp = phase + 4 * i;
+        hv[i] = sp < ns ? *reinterpret_cast<const h4v*>(reinterpret_cast<const _Float16*>(pr + sp * PSTRIDE) + lat) : h4v{0, 0, 0, 0};
+    }
+    // (m, l) of up to 1024 splits: 4 a thread
+    float mv[4], lv[4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int sp = tid + 256 * k;
+        const float2 ml = sp < ns ? *reinterpret_cast<const float2*>(pr + sp * PSTRIDE + ML / 2) : float2{-INFINITY, 0.0f};
+        mv[k] = ml.x;
+        lv[k] = ml.y;
+        mx = fmaxf(mx, ml.x);                                      // (a marked split's NaN does not take part in the maximum)
+    }
+    mx = wave_max(mx);
+    if (lane == 0) red[wv] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float ls = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int sp = tid + 256 * k;
+        const float wgt = mv[k] == -INFINITY ? 0.0f : lv[k] * fast_exp2(mv[k] - mx);
+        if (sp < ns) wsh[sp] = wgt;
+        ls += wgt;
+    }
+    ls = wave_sum(ls);
+    if (lane == 0) red[4 + wv] = ls;
+    __syncthreads();
+    const float L = (red[4] + red[5]) + (red[6] + red[7]);
     f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int sp = phase + 4 * i;
+        if (sp < ns) acc += f4v{(float) hv[i][0], (float) hv[i][1], (float) hv[i][2], (float) hv[i][3]} * wsh[sp];
+    }
 #pragma unroll 8
-    for (int s = phase; s < ns; s += 4) {
-        const h4v h = *reinterpret_cast<const h4v*>(reinterpret_cast<const _Float16*>(pr + s * PSTRIDE) + lat);
-        acc += f4v{(float) h[0], (float) h[1], (float) h[2], (float) h[3]} * wsh[s];
+    for (int sp = phase + 4 * CH; sp < ns; sp += 4) {
+        const h4v h = *reinterpret_cast<const h4v*>(reinterpret_cast<const _Float16*>(pr + sp * PSTRIDE) + lat);
+        acc += f4v{(float) h[0], (float) h[1], (float) h[2], (float) h[3]} * wsh[sp];
     }
     ph[tid] = acc;
     __syncthreads();
