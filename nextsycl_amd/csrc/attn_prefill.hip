@@ -65,6 +65,8 @@ struct PrefillParams {
 
 // a 16-byte chunk of a K or V row on its way from global memory to LDS (a plain vector type: arrays of it stay in registers)
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));
+// the same at an address that is only 8-byte aligned (q8_0 / q4_0 rows of 128 values are 136 / 72 bytes long)
+typedef uint32_t u4a8 __attribute__((ext_vector_type(4), aligned(8)));
 
 // The queries enter the first product as they are given (16-bit rows bit for bit, float32 rows rounded once) and the
 // softmax scale (x log2 e) rides in one fused multiply-add a score. Folding the scale into the 16-bit query operand
@@ -236,7 +238,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         }
 #pragma unroll
         for (int i = 0; i < NST; ++i) {
-            st.raw[i] = *reinterpret_cast<const u4v*>(sp + off[i]);
+            if constexpr (KT != 0 && D == 128) st.raw[i] = *reinterpret_cast<const u4a8*>(sp + off[i]);
+            else st.raw[i] = *reinterpret_cast<const u4v*>(sp + off[i]);
             if constexpr (KT != 0) st.sc[i] = *reinterpret_cast<const uint16_t*>(sp + off[i] + sc_rel);
         }
     };
@@ -559,12 +562,13 @@ int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
         attn_prefill_kernel<D, false, 0, PW><<<grid, TH, 0, g->q>>>(p);
     } else if (kt == 3) {
         attn_prefill_kernel<D, true, 0, PW><<<grid, TH, 0, g->q>>>(p);
-    } else if constexpr (D == 256) {
-        // (quantized rows are a multiple of 16 bytes at D = 256 only: the caller has checked)
-        if (kt == 1) attn_prefill_kernel<D, false, 1, PW><<<grid, TH, 0, g->q>>>(p);
-        else attn_prefill_kernel<D, false, 2, PW><<<grid, TH, 0, g->q>>>(p);
+    } else if (kt == 1) {
+        attn_prefill_kernel<D, false, 1, PW><<<grid, TH, 0, g->q>>>(p);
+    } else if constexpr (D == 256 || PW == 4) {
+        attn_prefill_kernel<D, false, 2, PW><<<grid, TH, 0, g->q>>>(p);
     } else {
-        return ns_fail("ns_attn_prompt: internal: quantized rows at this head size");
+        // (a q4_0 tile of 128-value rows is 256 chunks: fewer than 8 waves have threads - the caller takes 4 waves)
+        return ns_fail("ns_attn_prompt: internal: q4_0 rows of 128 values take 4 waves");
     }
     return 0;
 }
@@ -589,10 +593,9 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     if (!q || !kc || !vc || !out) return ns_fail(w + ": a null buffer");
     if ((uintptr_t) q % 16 || qs % (qt == 0 ? 4 : 8) || (uintptr_t) out % 16) return ns_fail(w + ": query and output rows 16-byte aligned");
     const int64_t rb = kv_row_bytes(kt, D);
-    // rows are fetched in 16-byte chunks, so a row's size must keep that alignment: every 16-bit row does, q8_0 / q4_0
-    // rows do at D = 256 (272 / 144 bytes; the reference's quantized prompt form is D = 256 only), not at D = 128 (136 / 72)
-    if (((uintptr_t) kc | (uintptr_t) vc) % 16) return ns_fail(w + ": caches 16-byte aligned");
-    if (rb % 16) return ns_fail(w + ": quantized cache rows with heads of 256 (shorter passes and other heads take the decode kernel)");
+    // rows are fetched in 16-byte chunks: every 16-bit row keeps that alignment, q8_0 / q4_0 rows do at D = 256 (272 / 144
+    // bytes; the reference's quantized prompt form is D = 256 only); at D = 128 (136 / 72 bytes) the chunks are 8-byte aligned
+    if (((uintptr_t) kc | (uintptr_t) vc) % (rb % 16 ? 8 : 16)) return ns_fail(w + (rb % 16 ? ": caches 8-byte aligned" : ": caches 16-byte aligned"));
     // (512 work-groups of 256 rows: two for each of the chip's 256 CUs; NS_PREFILL_WAVES = 4 or 8 overrides: tuning, tests)
     int64_t sns = 1, skbs = 0, sk0 = 0;
     // Key splits. A pass of few rows over a long context - a chunk of a prompt behind 32K tokens, a long draft block - has
@@ -618,6 +621,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // as fast as 4 (one a SIMD) whenever there are blocks enough for half the CUs
     int PWs = D == 128 ? (((T + 255) / 256) * Hq * sns >= 512 ? 8 : 4) : (T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
     if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_WAVES); forced == 4 || forced == 8) PWs = (int) forced;
+    if (kt == 2 && D == 128) PWs = 4;                                 // (a q4_0 tile of 128-value rows has chunks for 256 threads)
     const int64_t ROWS = rows_of((int) D, PWs);
     if (T > (int64_t) 1 << 30 || ((T + ROWS - 1) / ROWS + 1) * Hq > (int64_t) 1 << 30) return ns_fail(w + ": too many rows or heads");
     if ((pm ? cap * Hkv : cap) * rb >= (int64_t) 1 << 32) return ns_fail(w + ": a key head's cache spans 4 GiB or more");

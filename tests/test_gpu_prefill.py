@@ -35,13 +35,14 @@ def test_prefill_small(ops, T, Hq, Hkv, p0, win, kt, qt):
 
 
 def _random_cases(n, seed):
-    """Seeded shapes over what the kernel branches on: rows around the block sizes, groups, head size (256 also over
-    quantized caches), a context before the pass, windows shorter and longer than a tile and than the pass."""
+    """Seeded shapes over what the kernel branches on: rows around the block sizes, groups, head size, every cache form
+    (q8_0 / q4_0 rows of 128 values are 136 / 72 bytes: 8-byte aligned chunks), a context before the pass, windows shorter
+    and longer than a tile and than the pass."""
     rng = np.random.default_rng(seed)
     out = []
     for _ in range(n):
         D = int(rng.choice([128, 128, 256]))
-        kt = int(rng.choice([0, 3, 1, 2])) if D == 256 else int(rng.choice([0, 3]))
+        kt = int(rng.choice([0, 3, 1, 2]))
         Hkv = int(rng.integers(1, 3))
         G = int(rng.choice([1, 2, 4, 5, 8]))
         T = int(rng.choice([rng.integers(17, 70), rng.integers(70, 300), rng.integers(300, 600)]))
@@ -79,6 +80,29 @@ def test_prefill_work_groups_of_8_waves(ops, tune, T, Hq, Hkv, D, p0, win, kt, q
     ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
     check_close(got8, ref, qt, "prefill (8 waves) vs float64 closed form", kt=kt)
     assert np.array_equal(got8, got4)
+
+
+QROWS128 = [
+    # T, Hq, Hkv, p0, win, kt, qt        q8_0 / q4_0 rows of 128 values: both work-group sizes, a window, key splits
+    (17, 4, 1, 0, 0, 1, F32),
+    (700, 16, 2, 300, 0, 1, F16),        # blocks of 256 rows (8 waves)
+    (700, 16, 2, 300, 0, 2, F16),        # q4_0: 4 waves always
+    (260, 8, 2, 1000, 200, 1, F32),
+    (150, 4, 1, 64, 0, 2, F32),
+    (64, 8, 1, 9000, 0, 1, F16),         # key splits
+    (64, 8, 1, 9000, 0, 2, F32),
+]
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,p0,win,kt,qt", QROWS128)
+def test_prefill_quantized_rows_of_128(ops, T, Hq, Hkv, p0, win, kt, qt):
+    D = 128
+    cap = p0 + T + 1                     # (an odd row count: the second cache starts 8 bytes off a 16-byte boundary)
+    kc, vc = make_kv(kt, Hkv, D, cap, p0 + T)
+    qd, qf = make_q(qt, T, Hq, D)
+    got, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got, ref, qt, "prefill, q8_0 / q4_0 rows of 128", kt=kt)
 
 
 SPLIT = [
@@ -181,9 +205,6 @@ def test_reference_named_prompt_entry_points(ops):
     ob.fill(0)
     ops.q35_attn(qb, Hq * D, bufs[0], bufs[1], T, Hq, Hkv, D, cap, p0, ob, None)
     assert np.array_equal(ob.read(np.float32).reshape(T, -1), want)
-    # quantized rows at heads of 128 are not 16-byte rows: rejected with the reason (the reference's form is D = 256)
-    assert k.q35_attn_prompt_kv(g.raw, 1, qb.ptr, Hq * D, bufs[0].ptr, bufs[1].ptr, T, Hq, Hkv, D, cap, p0, ob.ptr) == -1
-    assert "heads of 256" in k.api.error()
     assert k.attn_prompt_t(g.raw, 0, 0, 0, qb.ptr, Hq * D, bufs[0].ptr, bufs[1].ptr, T, Hq, Hkv, 64, cap, p0, 0, 0.0, ob.ptr) == -1
     assert "heads of 128 or 256" in k.api.error()
 
@@ -210,9 +231,10 @@ def test_prefill_heads_of_256_and_quantized_rows(ops, T, Hq, Hkv, p0, win, kt, q
     check_close(got, ref, qt, "prefill, heads of 256", kt=kt)
 
 
-def test_q35_prompt_kv_entry_point(ops):
-    """ns_q35_attn_prompt_kv as the engine calls it (llm/qwen35/src/engine.rs:1598-1617): float32 rows, D = 256, Hq = 6 Hkv."""
-    T, Hq, Hkv, D, p0 = 90, 12, 2, 256, 40
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0", [(90, 12, 2, 256, 40), (300, 16, 2, 128, 500), (1100, 16, 1, 128, 0)])
+def test_q35_prompt_kv_entry_point(ops, T, Hq, Hkv, D, p0):
+    """ns_q35_attn_prompt_kv as the engine calls it (llm/qwen35/src/engine.rs:1598-1617): float32 rows, D = 256, Hq = 6 Hkv;
+    and over heads of 128 (136- / 72-byte rows: the cache form of the 128K q8_0 decode configuration taking a prompt)."""
     cap = p0 + T
     g = ops.gpu
     qd, qf = make_q(F32, T, Hq, D)
