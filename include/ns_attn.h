@@ -116,15 +116,15 @@ int ns_mg_attn_decode(ns_gpu* g, const float* q, const void* kc, const void* vc,
 /* Typed causal flash attention of T rows at positions p0.. against caches that already hold positions 0 .. p0 + T - 1
  * (the engine stores a pass's keys first: llm/museglimmer/src/engine.rs:856-860). No scratch argument: a pass of few rows
  * over a long context is cut into key splits whose partials live in memory the library keeps per ns_gpu (calls on one
- * ns_gpu are ordered by its stream). D 128 or 256; kt 0 (half) or 3 (bfloat16), and at D 256 also 1 (q8_0) and 2 (q4_0):
- * the cache's rows are read in 16-byte chunks */
+ * ns_gpu are ordered by its stream). D 128 or 256; kt 0 (half), 1 (q8_0), 2 (q4_0) or 3 (bfloat16). 16-bit caches
+ * 16-byte aligned; quantized ones 16-byte aligned at D 256 (272- / 144-byte rows) and 8-byte aligned at D 128 (136 / 72) */
 int ns_attn_prompt_t(ns_gpu* g, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq,
                      int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, float scale, void* out);
 /* Replaces: kernels/llm/museglimmer/silo/silo.h:44-48 (silo/attn.cpp:378-392) */
 int ns_mg_attn_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);
 int ns_mg_attn_prompt(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap,
                       int64_t p0, int64_t win, float* out);
-/* Replaces: kernels/llm/qwen35/silo/silo.h:43-45,57-58 (silo/attn.cpp:375-400); _kv: kt 0, 1, 2 at D 256 as there, 0 at D 128 */
+/* Replaces: kernels/llm/qwen35/silo/silo.h:43-45,57-58 (silo/attn.cpp:375-400); _kv: kt 0, 1, 2 (the reference: at D 256) */
 int ns_q35_attn_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);
 int ns_q35_attn_prompt(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
                        int64_t cap, int64_t p0, float* out);
