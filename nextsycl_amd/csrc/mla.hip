@@ -738,21 +738,33 @@ __device__ void yarn_cs(float pos, int i0, int n_dims, float freq_base, float fr
 __global__ __launch_bounds__(256) void ds2_kv_store_kernel(const float* __restrict__ kv, const float* __restrict__ wgt, float eps,
                                                            uint16_t* __restrict__ cache, int64_t L, int64_t R, int64_t pos0, float freq_base,
                                                            float freq_scale, float ext_factor, float mscale, float corr0, float corr1) {
-    __shared__ float red[256];
+    // the sum of squares in float64 (every product exact, the sum good to 1e-16: whatever the order of the additions, its
+    // rounding to float32 is the same number) - the normalized half of a row is then the same bits on any machine
+    __shared__ double red[256];
     const int64_t t = blockIdx.x;
     const int tid = threadIdx.x;
     const float* xr = kv + t * (L + R);
-    float ss = 0.0f;
-    for (int64_t i = tid; i < L; i += 256) ss += xr[i] * xr[i];
+    double ss = 0.0;
+    for (int64_t i = tid; i < L; i += 256) ss += (double) xr[i] * (double) xr[i];
     red[tid] = ss;
     __syncthreads();
     for (int o = 128; o > 0; o >>= 1) {
         if (tid < o) red[tid] += red[tid + o];
         __syncthreads();
     }
-    const float inv = 1.0f / sqrtf(red[0] / (float) L + eps);
+    // (the quotient, the root and the reciprocal through float64 and back: each is then the correctly rounded float32
+    // result whatever the compiler makes of a float32 division or square root)
+    const float arg = (float) ((double) (float) red[0] / (double) (float) L) + eps;
+    const float root = (float) sqrt((double) arg);
+    const float inv = (float) (1.0 / (double) root);
     uint16_t* o = cache + (pos0 + t) * (L + R);
-    for (int64_t i = tid; i < L; i += 256) o[i] = f32_to_f16(xr[i] * inv * wgt[i]);
+    // (the float32 product passes through a register of its own: left to itself the compiler folds the last multiply
+    // into the conversion - one rounding to half where the cache's rule has two)
+    for (int64_t i = tid; i < L; i += 256) {
+        float y = xr[i] * inv * wgt[i];
+        asm volatile("" : "+v"(y));
+        o[i] = f32_to_f16(y);
+    }
     for (int64_t i = tid; i < R / 2; i += 256) {
         const int i0 = (int) (2 * i);
         float c, s;

@@ -188,3 +188,23 @@ def test_glm_cell_pools_of_a_long_pass(ops, q8):
     ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, scale, q8=q8, sel=DevBuf.of(g, sel), sel_cnt=DevBuf.of(g, cnt), K=K)
     want = orc.glm_mla_attend_sel(qa, rows, q8, T, H, L, pos0, scale, sel, cnt, K)
     check_close(u.read(np.float32).reshape(T, H * L), want.reshape(T, H * L).astype(np.float64), F32, "ns_mla_attend_sel, 40 rows")
+
+
+@pytest.mark.parametrize("q8", [False, True])
+def test_glm_cell_pools_at_100k_tokens(ops, q8):
+    """Selection lists over a 100K-token latent cache: 4 rows x 64 heads, 512 pools (2048 cells) a row picked from the whole
+    context, against the reference-order restatement."""
+    g = ops.gpu
+    T, H, L, pos0, K, scale = 4, 64, 512, 100000, 512, 0.044
+    n = pos0 + T
+    qa = orc.randn(93, (T, H * L), 0.3)
+    x = orc.randn(94, (n, L))
+    rows = orc.glm_to_q8row(x, L) if q8 else orc.f2h(x).view(np.uint8).reshape(n, 2 * L)
+    rng = np.random.default_rng(10)
+    npool = (pos0 + 1) // 4
+    sel = np.stack([rng.choice(npool, K, replace=False) for _ in range(T)]).astype(np.int32)
+    cnt = np.array([K, K - 1, 7, K], np.int32)
+    u = DevBuf(g, T * H * L * 4); u.fill(0xFF)
+    ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, scale, q8=q8, sel=DevBuf.of(g, sel), sel_cnt=DevBuf.of(g, cnt), K=K)
+    want = orc.glm_mla_attend_sel(qa, rows, q8, T, H, L, pos0, scale, sel, cnt, K)
+    check_close(u.read(np.float32).reshape(T, H * L), want.reshape(T, H * L).astype(np.float64), F32, "ns_mla_attend_sel at 100K tokens")
