@@ -44,6 +44,21 @@ WORKLOADS = {
 }
 
 
+def randn(seed, shape, sigma=1.0):
+    """Seeded N(0, sigma) float32 (numpy's PCG64): the bench's own input generator."""
+    return (np.random.default_rng(seed).standard_normal(shape, dtype=np.float32) * np.float32(sigma)).astype(np.float32)
+
+
+def f2h(x):
+    return np.ascontiguousarray(x, np.float32).astype(np.float16).view(np.uint16)
+
+
+def f2bf(x):
+    """float32 -> bfloat16 bits, round to nearest even."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
 def kv_bytes(kt, D):
     return {0: 2 * D, 1: D + D // 16, 2: D // 2 + D // 16, 3: 2 * D}[kt]
 
@@ -66,7 +81,6 @@ class Workload:
 
     def __init__(self, ops, name, nbuf):
         from nextsycl_amd import DevBuf
-        from oracle import orc
 
         self.ops, self.name = ops, name
         self.kind, self.T, self.Hq, self.Hkv, self.D, self.kv, self.kt, self.qt, self.desc = WORKLOADS[name]
@@ -79,17 +93,17 @@ class Workload:
             rb = kv_bytes(kt, D)
             self.bytes = T * (Hq + 2 * Hkv) * D * 4 + T * Hq * D * 2 + 2 * T * Hkv * rb       # float32 rows in; q rows, cache rows out
             self.flops = 0
-            self.src = [DevBuf.of(g, orc.randn(0xB0B + i, (T, h * D))) for i, h in enumerate((Hq, Hkv, Hkv))]
-            self.w = [DevBuf.of(g, (1.0 + 0.1 * orc.randn(0xD00D + i, (D,))).astype(np.float32)) for i in range(2)]
+            self.src = [DevBuf.of(g, randn(0xB0B + i, (T, h * D))) for i, h in enumerate((Hq, Hkv, Hkv))]
+            self.w = [DevBuf.of(g, (1.0 + 0.1 * randn(0xD00D + i, (D,))).astype(np.float32)) for i in range(2)]
             self.out = DevBuf(g, T * Hq * D * 2)
             self.caches = [(DevBuf(g, Hkv * kv * rb), DevBuf(g, Hkv * kv * rb)) for _ in range(nbuf)]
             return
         if self.kind == "mla":
             self.caches = []
-            host = orc.f2h(orc.randn(0xB0B, (kv, 576), 0.5))
+            host = f2h(randn(0xB0B, (kv, 576), 0.5))
             for b in range(nbuf):
                 self.caches.append((DevBuf.of(g, host), None))
-            self.q = DevBuf.of(g, orc.f2h(orc.randn(0xA11CE, (T, Hq, 576))))
+            self.q = DevBuf.of(g, f2h(randn(0xA11CE, (T, Hq, 576))))
             self.out = DevBuf(g, T * Hq * 512 * 2)
             self.scratch = DevBuf(g, 4 * ops.mla_latent_scratch(T, Hq, self.p0))
             return
@@ -101,8 +115,8 @@ class Workload:
             if b == 0:
                 for s in range(0, kv, chunk):
                     n = min(chunk, kv - s)
-                    k = DevBuf.of(g, orc.randn(0xB0B + s, (n, Hkv * D)))
-                    v = DevBuf.of(g, orc.randn(0xC0FFEE + s, (n, Hkv * D)))
+                    k = DevBuf.of(g, randn(0xB0B + s, (n, Hkv * D)))
+                    v = DevBuf.of(g, randn(0xC0FFEE + s, (n, Hkv * D)))
                     ops.kv_store(kt, k, Hkv * D, v, Hkv * D, n, Hkv, D, kv, s, kc, vc)
             else:
                 # further caches: the same rows at other addresses (what the rotation needs is distinct memory)
@@ -110,8 +124,8 @@ class Workload:
                 g.api.copy_dev(g.raw, vc.ptr, self.caches[0][1].ptr, vc.len)
             g.sync()
             self.caches.append((kc, vc))
-        q = orc.randn(0xA11CE, (T, Hq * D))
-        qd = q if qt == 0 else (orc.f2h(q) if qt == 1 else orc.f2bf(q))
+        q = randn(0xA11CE, (T, Hq * D))
+        qd = q if qt == 0 else (f2h(q) if qt == 1 else f2bf(q))
         self.q = DevBuf.of(g, qd)
         self.out = DevBuf(g, T * Hq * D * (4 if qt == 0 else 2))
         self.scratch = DevBuf(g, max(4, 4 * ops.decode_scratch(T, Hq, Hkv, D, self.p0))) if self.kind == "decode" else None
@@ -175,14 +189,22 @@ def timed(w, steps, warmup):
 
 
 # HBM bytes per launch of each workload's dominant kernel as rocprofv3 counted them (FETCH_SIZE + WRITE_SIZE per dispatch,
-# each scaled by what the same counter reads for a plain 1 GiB copy kernel); the runs are summarized under profiles/.
-# A counter run cannot be made from inside this script, so these are the recorded figures of those runs, not live ones.
-MEASURED_TRAFFIC = {"prefill8k": 183.5e6 + 83.9e6, "decode32k": 134.5e6 + 1.1e6, "mla32k": 39.5e6 + 17.4e6, "pre_store8k": 235.1e6 + 117.4e6}
+# each scaled by what the same counter reads for a plain copy kernel of known size). A counter run cannot be made from
+# inside this script: the figure is read from the committed summary of that run, profiles/<kernel>_<workload>.md (its line
+# "traffic_bytes_per_launch: N"), and is null where no such summary exists.
+def measured_traffic(kernel, workload):
+    import re
+    path = os.path.join(ROOT, "profiles", "%s_%s.md" % (kernel, workload))
+    try:
+        m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), re.M)
+    except OSError:
+        return None
+    return float(m.group(1)) if m else None
 
 
 def roofline(w, main_ns):
     r = _roofline(w, main_ns)
-    r["traffic"] = MEASURED_TRAFFIC.get(w.name)
+    r["traffic"] = measured_traffic(r["kernel"], w.name)
     return r
 
 
@@ -205,54 +227,58 @@ def _roofline(w, main_ns):
 
 
 def cpu_baseline(name):
-    """The CPU oracle on a bounded sample of the workload, timed on this host's cores."""
+    """The CPU oracle (the C restatement of the reference's exact kernels, OpenMP over rows x heads) on a bounded sample of
+    the workload, timed on this host's cores: a few seconds a workload, so that the default run stays within minutes."""
     from oracle import orc
 
     kind, T, Hq, Hkv, D, kv, kt, qt, _ = WORKLOADS[name]
     if kind == "pre":
-        # the q and k rows' norm + rotary through the numpy restatement (one core); the store is left out
+        # the q and k rows' norm + rotary (the C restatement, one thread) on the first rows; the store is left out
+        rows = min(T, 1024)
         w = np.ones(D, np.float32)
-        xq, xk = orc.randn(0xB0B, (T, Hq * D)), orc.randn(0xB0C, (T, Hkv * D))
+        xq, xk = randn(0xB0B, (rows, Hq * D)), randn(0xB0C, (rows, Hkv * D))
         t0 = time.perf_counter()
-        orc.q35_norm_rope(xq, T, Hq, D, w, 1e-6, D // 2, 1e6, 0)
-        orc.q35_norm_rope(xk, T, Hkv, D, w, 1e-6, D // 2, 1e6, 0)
+        orc.q35_norm_rope(xq, rows, Hq, D, w, 1e-6, D // 2, 1e6, 0)
+        orc.q35_norm_rope(xk, rows, Hkv, D, w, 1e-6, D // 2, 1e6, 0)
         dt = time.perf_counter() - t0
-        return {"value": round(T * (Hq + Hkv) * D * 8 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-                "sample": "norm + rotary of all %d q and k rows (float32 in and out), numpy restatement, no store" % T, "seconds": round(dt, 2)}
+        return {"value": round(rows * (Hq + Hkv) * D * 8 / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+                "sample": "norm + rotary of the first %d of %d q and k rows (float32 in and out), no store" % (rows, T), "seconds": round(dt, 2)}
     if kind == "mla":
-        # the restated kernel order on the last rows of the workload
-        rows = min(T, 2)
-        cache = orc.f2h(orc.randn(0xB0B, (kv, 576), 0.5))
-        qa = orc.h2f(orc.f2h(orc.randn(0xA11CE, (rows, Hq, 576))))
+        # the restated kernel order (16 streams a (row, head), exp) on the last rows and a quarter of the heads
+        rows, heads = min(T, 2), max(1, Hq // 4)
+        cache = f2h(randn(0xB0B, (kv, 576), 0.5))
+        qa = orc.h2f(f2h(randn(0xA11CE, (rows, heads, 576))))
         p0 = kv - rows
         t0 = time.perf_counter()
-        orc.mla_decode_u(qa, cache, rows, Hq, p0, 192.0 ** -0.5)
+        orc.mla_decode_u(qa, cache, rows, heads, p0, 192.0 ** -0.5)
         dt = time.perf_counter() - t0
-        flops = sum(2 * Hq * (p0 + r + 1) * 1088 for r in range(rows))
-        return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": 1, "kind": "port",
-                "sample": "the last %d of %d rows, all %d heads, the whole %d-cell cache, restated kernel order (numpy)" % (rows, T, Hq, kv), "seconds": round(dt, 2)}
-    k = orc.randn(0xB0B, (kv, Hkv * D))
-    v = orc.randn(0xC0FFEE, (kv, Hkv * D))
+        flops = sum(2 * heads * (p0 + r + 1) * 1088 for r in range(rows))
+        return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": orc.threads(), "kind": "port",
+                "sample": "the last %d of %d rows, %d of %d heads, the whole %d-cell cache, reference-order float32 kernel" % (rows, T, heads, Hq, kv),
+                "seconds": round(dt, 2)}
+    k = randn(0xB0B, (kv, Hkv * D))
+    v = randn(0xC0FFEE, (kv, Hkv * D))
     kc, vc = orc.kv_store(kt, k, v, Hkv, D, kv, 0)
     if kind == "prefill":
         rows = 1024          # the last 1024 query rows against the whole cache (~10-20 s on 16 cores)
         p0 = kv - rows
-        q = orc.bf2f(orc.f2bf(orc.randn(0xA11CE, (rows, Hq * D))))
+        q = orc.bf2f(f2bf(randn(0xA11CE, (rows, Hq * D))))
         sample = "last %d of %d query rows (positions %d..%d), all %d heads, full %d-key cache, reference-order float32 kernel" % (rows, T, p0, kv - 1, Hq, kv)
         flops = 4 * D * Hq * (rows * p0 + rows * (rows + 1) // 2)
         t0 = time.perf_counter()
         orc.attn_exact(q, kc, vc, kt, rows, Hq, Hkv, D, kv, p0, groups=max(1, Hq // 4))
         dt = time.perf_counter() - t0
         return {"value": round(flops / dt / 1e12, 5), "unit": "TFLOP/s", "cores": orc.threads(), "kind": "port", "sample": sample, "seconds": round(dt, 2)}
-    reps = 3
-    q = orc.randn(0xA11CE, (T, Hq * D))
+    q = randn(0xA11CE, (T, Hq * D))
     flops, nbytes = algorithmic(kind, T, Hq, Hkv, D, kv, kt, qt)
+    reps, dt = 0, 0.0
     t0 = time.perf_counter()
-    for _ in range(reps):
+    while reps < 3 and dt < 5.0:
         orc.attn_exact(q, kc, vc, kt, T, Hq, Hkv, D, kv, kv - T, groups=max(1, Hq // 4))
-    dt = (time.perf_counter() - t0) / reps
-    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": orc.threads(), "kind": "port",
-            "sample": "the whole workload, %d passes, reference-order float32 kernel" % reps, "seconds": round(dt * reps, 2)}
+        reps += 1
+        dt = time.perf_counter() - t0
+    return {"value": round(nbytes * reps / dt / 1e9, 3), "unit": "GB/s", "cores": orc.threads(), "kind": "port",
+            "sample": "the whole workload, %d passes, reference-order float32 kernel" % reps, "seconds": round(dt, 2)}
 
 
 def main():
@@ -312,7 +338,7 @@ def main():
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {0: "f32", 1: "f16", 2: "bf16"}[w.qt] if w.kt in (0, 3) else "q8_0/f16",
-        "data": "synthetic (seeded xorshift64* + Box-Muller N(0,1))",
+        "data": "synthetic (seeded numpy PCG64 N(0,1))",
         "config": {"workload": w.desc, "name": a.workload, "rows": w.T, "q_heads": w.Hq, "kv_heads": w.Hkv, "head_dim": w.D, "kv_len": w.kv,
                    "kv_form": {0: "f16", 1: "q8_0", 2: "q4_0", 3: "bf16"}[w.kt], "flops_per_step": w.flops, "bytes_per_step": w.bytes,
                    "untimed_settle_ms": SETTLE_MS},
@@ -333,6 +359,8 @@ def main():
                             round((ww.flops / (m2 * 1e-3) / 1e12) if ww.kind not in ("decode", "pre") else (ww.bytes / (m2 * 1e-3) / 1e9), 2), "roofline": r,
                             "merge_kernel_us": round(g2 / 1e3, 2)}
             del ww
+            if not a.no_cpu:
+                others[name]["cpu_baseline"] = cpu_baseline(name)
         line["others"] = others
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(a.workload)
