@@ -36,6 +36,11 @@ int ns_mla_decode_latent(ns_gpu* g, int qt, const void* qa, const uint16_t* cach
  * kernels/llm/deepseek2/ds2.h:32-37 (ds2.cpp:139-258, 262-270) */
 int ns_ds2_mla_decode(ns_gpu* g, const float* q, const uint16_t* kb, const uint16_t* vb, const uint16_t* cache, float* out, int64_t T, int64_t H,
                       int64_t pos0, float scale);
+/* The same with kv_b as the model file stores it - Q6_K, [H x (nope + V)] rows of L = 512 (two 210-byte blocks a row): per
+ * head its 128 k rows (k_i[c]: q~[c] = sum_i q_nope[i] k_i[c]), then its 128 v rows - decoded where it is read. Replaces:
+ * kernels/llm/deepseek2/ds2.h:38-41 (ds2.cpp:117-134,157-173,237-246,272-281) */
+int ns_ds2_mla_decode_q6k(ns_gpu* g, const float* q, const void* kvb, const uint16_t* cache, float* out, int64_t T, int64_t H, int64_t pos0,
+                          float scale);
 /* The latent cache's rows pos0 .. pos0 + T - 1 from kv [T][L + R] float32: the first L RMS-normed with w (eps), the last
  * R rotated by ggml's YaRN rope on adjacent pairs. Replaces: kernels/llm/deepseek2/ds2.h:28-31 (ds2.cpp:85-112) */
 int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint16_t* cache, int64_t T, int64_t L, int64_t R, int64_t pos0,

@@ -82,6 +82,7 @@ MLA_H = {
     "ns_mla_decode_latent_scratch": (i64, [i64, i64, i64]),
     "ns_mla_decode_latent": (i32, [P, i32, P, P, P, i64, i64, i64, i64, f32, P]),
     "ns_ds2_mla_decode": (i32, [P, P, P, P, P, P, i64, i64, i64, f32]),
+    "ns_ds2_mla_decode_q6k": (i32, [P, P, P, P, P, i64, i64, i64, f32]),
     "ns_ds2_kv_store": (i32, [P, P, P, f32, P, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32]),
     "ns_mla_attend_sel": (i32, [P, P, P, P, i64, i64, i64, i64, f32, P, P, i64]),
     "ns_mla_attend_sel_q8": (i32, [P, P, P, P, i64, i64, i64, i64, f32, P, P, i64]),
@@ -346,6 +347,14 @@ class Ops:
         _need(cache, (pos0 + T) * 576 * 2, "mla_decode cache")
         _need(out, T * H * 128 * 4, "mla_decode out")
         self.ok(self.k.ds2_mla_decode(self.raw(), q.ptr, kb.ptr, vb.ptr, cache.ptr, out.ptr, T, H, pos0, scale), "mla_decode")
+
+    def mla_decode_q6k(self, q, kvb, cache, out, T, H, pos0, scale):
+        """ns_ds2_mla_decode_q6k: q [T][H][192], kv_b as Q6_K rows ([H][256] rows of 420 bytes), cache half [.., 576] -> out [T][H][128]."""
+        _need(q, T * H * 192 * 4, "mla_decode_q6k q")
+        _need(kvb, H * 256 * 420, "mla_decode_q6k kv_b")
+        _need(cache, (pos0 + T) * 576 * 2, "mla_decode_q6k cache")
+        _need(out, T * H * 128 * 4, "mla_decode_q6k out")
+        self.ok(self.k.ds2_mla_decode_q6k(self.raw(), q.ptr, kvb.ptr, cache.ptr, out.ptr, T, H, pos0, scale), "mla_decode_q6k")
 
     def ds2_kv_store(self, kv, w, eps, cache, T, L, R, pos0, freq_base, freq_scale, ext_factor, mscale, corr0, corr1):
         _need(kv, T * (L + R) * 4, "kv_store kv")

@@ -714,6 +714,69 @@ __global__ __launch_bounds__(256) void mla_vb_kernel(const float* __restrict__ u
     }
 }
 
+// ---- k_b / v_b as the model file stores them: Q6_K rows of 512 (two blocks of 210 bytes: ql [128], qh [64], int8 scales
+// [16], a half d), per head its 128 k rows and then its 128 v rows (kernels/llm/deepseek2/ds2.cpp:117-134). A lane owns the
+// columns 8 lane .. 8 lane + 7 of a row: eight consecutive values of one 32-value group, so one scale, eight ql bytes (low
+// or high nibbles) and eight qh bytes (two bits each). value = d x scale x (q - 32), the products in that order, in float32.
+__device__ __forceinline__ void q6k_cols8(const uint8_t* row, int lane, float (&v)[8]) {
+    const uint8_t* b = row + (lane >> 5) * 210;                   // the row's block: columns 0..255 / 256..511
+    const int j = (lane & 31) * 8, n = j >> 7, gq = (j & 127) >> 5, l0 = j & 31;
+    const uint16_t* ql = reinterpret_cast<const uint16_t*>(b + 64 * n + (gq & 1) * 32 + l0);       // (blocks are 2-byte aligned)
+    const uint16_t* qh = reinterpret_cast<const uint16_t*>(b + 128 + 32 * n + l0);
+    const float ds = f16_to_f32(*reinterpret_cast<const uint16_t*>(b + 208)) * (float) (int8_t) b[192 + 8 * n + 2 * gq + (l0 >> 4)];
+    const int shift = 2 * gq;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int lb = (ql[e >> 1] >> (8 * (e & 1))) & 0xFF, hb = (qh[e >> 1] >> (8 * (e & 1))) & 0xFF;
+        const int lo = gq < 2 ? (lb & 0xF) : (lb >> 4);
+        v[e] = ds * (float) ((lo | (((hb >> shift) & 3) << 4)) - 32);
+    }
+}
+
+// q~ = sum_i q_nope[i] k_i over a head's 128 Q6_K k rows: a work-group a (row, head), a wave every fourth k row, a lane 8
+// columns; the four waves' sums added in wave order (kernels/llm/deepseek2/ds2.cpp:157-173)
+__global__ __launch_bounds__(256) void mla_absorb_q6k_kernel(const float* __restrict__ q, const uint8_t* __restrict__ kvb, float* __restrict__ qa,
+                                                             int64_t H) {
+    constexpr int NOPE = 128, R = 64, V = 128, ROWB = 420;
+    __shared__ float part[4][ML];
+    const int64_t th = blockIdx.x, h = th % H;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const float* qr = q + th * (NOPE + R);
+    float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    for (int i = w; i < NOPE; i += 4) {
+        float v[8];
+        q6k_cols8(kvb + ((size_t) h * (NOPE + V) + i) * ROWB, lane, v);
+        const float qi = qr[i];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += qi * v[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[w][lane * 8 + e] = acc[e];
+    __syncthreads();
+    for (int c = tid; c < ML; c += 256) qa[th * (ML + R) + c] = ((part[0][c] + part[1][c]) + part[2][c]) + part[3][c];
+    if (tid < R) qa[th * (ML + R) + ML + tid] = qr[NOPE + tid];
+}
+
+// out [T][H][V] = v_b u over a head's 128 Q6_K v rows: a wave a value row at a time (kernels/llm/deepseek2/ds2.cpp:237-246)
+__global__ __launch_bounds__(256) void mla_vb_q6k_kernel(const float* __restrict__ u, const uint8_t* __restrict__ kvb, float* __restrict__ out,
+                                                         int64_t H) {
+    constexpr int NOPE = 128, V = 128, ROWB = 420;
+    const int64_t th = blockIdx.x, h = th % H;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    float uv[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) uv[e] = u[th * ML + lane * 8 + e];
+    for (int r = blockIdx.y * 32 + w; r < blockIdx.y * 32 + 32; r += 4) {
+        float v[8];
+        q6k_cols8(kvb + ((size_t) h * (NOPE + V) + NOPE + r) * ROWB, lane, v);
+        float a = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a += v[e] * uv[e];
+        a = wave_sum(a);
+        if (lane == 0) out[th * V + r] = a;
+    }
+}
+
 // ggml's rope_yarn angle of pair i0 (kernels/llm/deepseek2/ds2.cpp:15-34): the angle by repeated products, as it does
 __device__ float yarn_ramp(float low, float high, int i0) {
     const float y = ((float) (i0 / 2) - low) / fmaxf(0.001f, high - low);
@@ -981,6 +1044,28 @@ int ns_ds2_mla_decode(ns_gpu* g, const float* q, const uint16_t* kb, const uint1
     if (mla_latent(g, "ns_ds2_mla_decode", 0, 0, 64, false, qa, cache, u, T, H, pos0, scale, part, g->own_scratch_floats - qa_f - u_f)) return -1;
     mla_vb_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(u, vb, out, H);
     NS_LAUNCHED("mla_vb");
+    return 0;
+    NS_CATCH
+}
+
+int ns_ds2_mla_decode_q6k(ns_gpu* g, const float* q, const void* kvb, const uint16_t* cache, float* out, int64_t T, int64_t H, int64_t pos0,
+                          float scale) {
+    NS_TRY
+    if (T <= 0) return 0;
+    if (H <= 0 || pos0 < 0 || T > 16) return ns_fail("ns_ds2_mla_decode_q6k: 1..16 rows, heads and a position");
+    if (!q || !kvb || !cache || !out) return ns_fail("ns_ds2_mla_decode_q6k: a null buffer");
+    if ((uintptr_t) kvb % 2) return ns_fail("ns_ds2_mla_decode_q6k: kv_b 2-byte aligned");
+    const size_t rows = (size_t) (T * H), qa_f = (rows * (ML + 64) + 3) / 4 * 4, u_f = rows * ML;
+    if (qa_f + u_f + rows * PSTRIDE > g->own_scratch_floats) return ns_fail("ns_ds2_mla_decode_q6k: the pass needs more scratch than the library keeps");
+    float* qa = g->own_scratch;
+    float* u = qa + qa_f;
+    float* part = u + u_f;
+    NS_HIP(hipSetDevice(g->dev));
+    mla_absorb_q6k_kernel<<<(unsigned) rows, 256, 0, g->q>>>(q, (const uint8_t*) kvb, qa, H);
+    NS_LAUNCHED("mla_absorb_q6k");
+    if (mla_latent(g, "ns_ds2_mla_decode_q6k", 0, 0, 64, false, qa, cache, u, T, H, pos0, scale, part, g->own_scratch_floats - qa_f - u_f)) return -1;
+    mla_vb_q6k_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(u, (const uint8_t*) kvb, out, H);
+    NS_LAUNCHED("mla_vb_q6k");
     return 0;
     NS_CATCH
 }

@@ -842,6 +842,78 @@ ORC_API void orc_mla_decode_u(const float* qa, const uint16_t* cache, float* u, 
         }
 }
 
+/* Q6_K (210 bytes a 256 values): ql [128], qh [64], int8 scales [16], half d. The 32 values of block half n, quarter gq at
+ * l = 0..31: (low or high nibble of ql[64 n + (gq & 1) 32 + l]) | two bits of qh[32 n + l] << 4, less 32, times d x
+ * scale[8 n + 2 gq + l / 16], the products in that order - kernels/llm/deepseek2/ds2.cpp:117-134. Columns [32 k, 32 k + 32)
+ * of a 512-wide row (two blocks). */
+static void q6k_cols32(const uint8_t* row, int k, float* v) {
+    const uint8_t* b = row + (k / 8) * 210;
+    const int j = (k % 8) * 32, n = j / 128, gq = (j % 128) / 32;
+    uint16_t dh;
+    memcpy(&dh, b + 208, 2);
+    const float d = orc_h2f(dh);
+    const uint8_t* ql = b + 64 * n + (gq & 1) * 32;
+    const uint8_t* qh = b + 128 + 32 * n;
+    const int shift = 2 * gq;
+    for (int l = 0; l < 32; ++l) {
+        const int lo = gq < 2 ? (ql[l] & 0xF) : (ql[l] >> 4);
+        const int q = (lo | (((qh[l] >> shift) & 3) << 4)) - 32;
+        v[l] = d * (float) (int8_t) b[192 + 8 * n + 2 * gq + l / 16] * (float) q;
+    }
+}
+
+/* a Q6_K row of 512 widened to float32 (the rule above) */
+ORC_API void orc_q6k_row512(const uint8_t* row, float* out) {
+    for (int k = 0; k < 16; ++k) q6k_cols32(row, k, out + 32 * k);
+}
+
+/* q~ over kv_b as the file stores it (Q6_K, per head 128 k rows then 128 v rows, each [512]): q~[c] = sum_i q_nope[i]
+ * k_i[c], 16 streams (stream s: rows s, s + 16, ..) added in stream order - kernels/llm/deepseek2/ds2.cpp:157-173 */
+ORC_API void orc_mla_absorb_q6k(const float* q, const uint8_t* kvb, float* qa, int64_t T, int64_t H) {
+    enum { L = 512, R = 64, NOPE = 128, V = 128, NSG = 16 };
+#pragma omp parallel for collapse(2)
+    for (int64_t t = 0; t < T; ++t)
+        for (int64_t h = 0; h < H; ++h) {
+            const float* qr = q + (t * H + h) * (NOPE + R);
+            float* o = qa + (t * H + h) * (L + R);
+            float part[NSG][L];
+            memset(part, 0, sizeof(part));
+            for (int s = 0; s < NSG; ++s)
+                for (int i = s; i < NOPE; i += NSG) {
+                    float row[L];
+                    orc_q6k_row512(kvb + ((size_t) h * (NOPE + V) + i) * 420, row);
+                    for (int c = 0; c < L; ++c) part[s][c] += qr[i] * row[c];
+                }
+            for (int c = 0; c < L; ++c) {
+                float a = 0.0f;
+                for (int s = 0; s < NSG; ++s) a += part[s][c];
+                o[c] = a;
+            }
+            for (int f = 0; f < R; ++f) o[L + f] = qr[NOPE + f];
+        }
+}
+
+/* out = v_b u over the Q6_K v rows: a lane 32 columns in order, 16 lanes reduced - kernels/llm/deepseek2/ds2.cpp:237-246 */
+ORC_API void orc_mla_vb_q6k(const float* u, const uint8_t* kvb, float* out, int64_t T, int64_t H) {
+    enum { L = 512, NOPE = 128, V = 128 };
+#pragma omp parallel for collapse(2)
+    for (int64_t t = 0; t < T; ++t)
+        for (int64_t h = 0; h < H; ++h)
+            for (int64_t r = 0; r < V; ++r) {
+                float row[L], lane[16];
+                orc_q6k_row512(kvb + ((size_t) h * (NOPE + V) + NOPE + r) * 420, row);
+                const float* uu = u + (t * H + h) * L;
+                for (int ln = 0; ln < 16; ++ln) {
+                    float a = 0.0f;
+                    for (int f = 0; f < 32; ++f) a += row[ln * 32 + f] * uu[ln * 32 + f];
+                    lane[ln] = a;
+                }
+                for (int o = 8; o > 0; o >>= 1)
+                    for (int ln = 0; ln < o; ++ln) lane[ln] += lane[ln + o];
+                out[(t * H + h) * V + r] = lane[0];
+            }
+}
+
 /* out [T][H][V] = v_b u: vb half [H][V][L] - kernels/llm/deepseek2/ds2.cpp:237-255 (lane ln sums columns
  * (k*16 + ln)*8 .. +8 for k = 0..3, then the 16 lanes are reduced) */
 ORC_API void orc_mla_vb(const float* u, const uint16_t* vb, float* out, int64_t T, int64_t H, int64_t L, int64_t V) {

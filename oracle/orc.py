@@ -58,6 +58,9 @@ def lib():
             "orc_mla_absorb": (None, [P, P, P, i64, i64, i64, i64, i64]),
             "orc_mla_decode_u": (None, [P, P, P, i64, i64, i64, i64, i64, f32]),
             "orc_mla_vb": (None, [P, P, P, i64, i64, i64, i64]),
+            "orc_q6k_row512": (None, [P, P]),
+            "orc_mla_absorb_q6k": (None, [P, P, P, i64, i64]),
+            "orc_mla_vb_q6k": (None, [P, P, P, i64, i64]),
             "orc_mla_f64": (None, [P, P, P, i64, i64, i64, i64, i64, f64]),
             "orc_glm_mla_attend": (None, [P, P, C.c_int, P, i64, i64, i64, i64, f32]),
             "orc_q35_norm_rope": (C.c_int, [P, i64, i64, P, i64, i64, i64, i64, P, f32, i64, f32, i64, P, i64, i64, i64]),
@@ -284,6 +287,29 @@ def mla_vb(u, vb, T, H, L=512, V=128):
     u, vb = _c(u, np.float32), _c(vb, np.uint16)
     out = np.empty((T, H, V), np.float32)
     lib().orc_mla_vb(_p(u), _p(vb), _p(out), T, H, L, V)
+    return out
+
+
+def q6k_rows512(rows):
+    """Q6_K rows of 512 values (420 bytes each) widened to float32 [n][512]."""
+    rows = _c(rows, np.uint8).reshape(-1, 420)
+    out = np.empty((rows.shape[0], 512), np.float32)
+    for i in range(rows.shape[0]):
+        lib().orc_q6k_row512(_p(rows[i]), _p(out[i]))
+    return out
+
+
+def mla_absorb_q6k(q, kvb, T, H):
+    q, kvb = _c(q, np.float32), _c(kvb, np.uint8)
+    qa = np.empty((T, H, 576), np.float32)
+    lib().orc_mla_absorb_q6k(_p(q), _p(kvb), _p(qa), T, H)
+    return qa
+
+
+def mla_vb_q6k(u, kvb, T, H):
+    u, kvb = _c(u, np.float32), _c(kvb, np.uint8)
+    out = np.empty((T, H, 128), np.float32)
+    lib().orc_mla_vb_q6k(_p(u), _p(kvb), _p(out), T, H)
     return out
 
 

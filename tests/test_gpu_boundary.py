@@ -208,3 +208,29 @@ def test_glm_cell_pools_at_100k_tokens(ops, q8):
     ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, scale, q8=q8, sel=DevBuf.of(g, sel), sel_cnt=DevBuf.of(g, cnt), K=K)
     want = orc.glm_mla_attend_sel(qa, rows, q8, T, H, L, pos0, scale, sel, cnt, K)
     check_close(u.read(np.float32).reshape(T, H * L), want.reshape(T, H * L).astype(np.float64), F32, "ns_mla_attend_sel at 100K tokens")
+
+
+@pytest.mark.parametrize("T,H,pos0", [(1, 16, 700), (3, 128, 2000), (16, 8, 5)])
+def test_ds2_mla_decode_with_q6k_weights(ops, T, H, pos0):
+    """ns_ds2_mla_decode_q6k: kv_b read as the file stores it (Q6_K rows), against the float64 chain over the widened rows."""
+    from test_oracle_boundary import random_q6k_rows
+    g = ops.gpu
+    n = pos0 + T
+    kvb = random_q6k_rows(31, H * 256).reshape(H, 256, 420)
+    cache = orc.f2h(orc.randn(32, (n, 576), 0.5))
+    q = orc.randn(33, (T, H, 192))
+    scale = 1.0 / np.sqrt(192.0)
+    out = DevBuf(g, T * H * 128 * 4); out.fill(0xFF)
+    ops.mla_decode_q6k(DevBuf.of(g, q), DevBuf.of(g, kvb), DevBuf.of(g, cache), out, T, H, pos0, scale)
+    w = orc.q6k_rows512(kvb).reshape(H, 256, 512).astype(np.float64)
+    qa64 = np.concatenate([np.einsum("hic,thi->thc", w[:, :128], q[:, :, :128].astype(np.float64)), q[:, :, 128:]], axis=2)
+    u64 = orc.mla_f64(qa64.astype(np.float32), cache, T, H, pos0, scale)
+    want = np.einsum("hvc,thc->thv", w[:, 128:], u64)
+    got = out.read(np.float32).reshape(T, H * 128)
+    # the result is small (weights of 1e-3 x 6-bit values): the bar relative to its own size
+    mx, rel, _ = orc.compare(got, want.reshape(T, H * 128))
+    assert rel <= 1e-3 and mx <= 2e-3 * max(1.0, np.abs(want).max()), (mx, rel)
+    # the restated chain agrees with the float64 one as well
+    qa = orc.mla_absorb_q6k(q, kvb, T, H)
+    ref = orc.mla_vb_q6k(orc.mla_decode_u(qa, cache, T, H, pos0, scale), kvb, T, H)
+    assert orc.compare(ref.reshape(T, H * 128), want.reshape(T, H * 128))[1] <= 1e-4

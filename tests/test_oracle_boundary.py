@@ -82,3 +82,59 @@ def test_gather_q8_known_answers():
     y = orc.glm_to_q8row(orc.randn(7, (5, L)), L)
     want = (orc.h2f(y[:, :32].view(np.uint16).copy()).repeat(32, axis=1) * y[:, 32:].view(np.int8).astype(np.float32)).astype(np.float16).view(np.uint16)
     assert np.array_equal(orc.glm_gather_q8_h(y, np.arange(5, dtype=np.int32), L), want)
+
+
+def _q6k_numpy(blocks):
+    """ggml dequantize_row_q6_K restated in numpy. blocks uint8 [nb][210] -> float32 [nb][256]:
+    for each half n (128 values) and l = 0..31: q1 = (ql[l] & 15) | ((qh[l] >> 0) & 3) << 4, q2 = (ql[l + 32] & 15) | ((qh[l] >> 2) & 3) << 4,
+    q3 = (ql[l] >> 4) | ((qh[l] >> 4) & 3) << 4, q4 = (ql[l + 32] >> 4) | ((qh[l] >> 6) & 3) << 4, each less 32;
+    y[l + 32 g] = d * sc[l / 16 + 2 g] * q_g."""
+    nb = blocks.shape[0]
+    ql = blocks[:, :128].astype(np.int32).reshape(nb, 2, 64)
+    qh = blocks[:, 128:192].astype(np.int32).reshape(nb, 2, 32)
+    sc = blocks[:, 192:208].view(np.int8).astype(np.float32).reshape(nb, 2, 8)
+    d = blocks[:, 208:210].copy().view(np.float16).astype(np.float32).reshape(nb, 1, 1)
+    out = np.zeros((nb, 2, 4, 32), np.float32)
+    is_ = np.arange(32) // 16
+    for g, (src, hi, sh) in enumerate(((ql[:, :, :32], False, 0), (ql[:, :, 32:], False, 2), (ql[:, :, :32], True, 4), (ql[:, :, 32:], True, 6))):
+        lo = (src >> 4) if hi else (src & 15)
+        q = (lo | (((qh >> sh) & 3) << 4)) - 32
+        out[:, :, g, :] = (d * sc[:, :, is_ + 2 * g]).astype(np.float32) * q.astype(np.float32)
+    return out.reshape(nb, 256)
+
+
+def random_q6k_rows(seed, n):
+    """n Q6_K rows of 512 values: random 6-bit values and scales, d near 1e-3 (the size of real kv_b weights)."""
+    rng = np.random.default_rng(seed)
+    b = np.zeros((n * 2, 210), np.uint8)
+    b[:, :192] = rng.integers(0, 256, (n * 2, 192), dtype=np.uint8)
+    b[:, 192:208] = rng.integers(-60, 61, (n * 2, 16)).astype(np.int8).view(np.uint8)
+    b[:, 208:210] = (rng.uniform(5e-4, 2e-3, n * 2).astype(np.float16)).view(np.uint8).reshape(n * 2, 2)
+    return b.reshape(n, 420)
+
+
+def test_q6k_rows_against_the_published_rule():
+    rows = random_q6k_rows(5, 40)
+    rows[0].reshape(2, 210)[:, :192] = 0
+    rows[1].reshape(2, 210)[:, :192] = 0xFF
+    want = _q6k_numpy(rows.reshape(-1, 210)).reshape(40, 512)
+    assert np.array_equal(orc.q6k_rows512(rows), want)
+    # all-zero ql / qh: every value is -32 times its block's d x scale
+    ds = np.repeat(rows[0].reshape(2, 210)[:, 192:208].view(np.int8).astype(np.float32), 16, axis=1) * rows[0].reshape(2, 210)[:, 208:210].copy().view(np.float16).astype(np.float32)
+    assert np.array_equal(want[0].reshape(2, 256), ds * np.float32(-32.0))
+    assert np.array_equal(want[1].reshape(2, 256), np.repeat(rows[1].reshape(2, 210)[:, 192:208].view(np.int8).astype(np.float32), 16, axis=1) *
+                          rows[1].reshape(2, 210)[:, 208:210].copy().view(np.float16).astype(np.float32) * np.float32(31.0))
+
+
+def test_q6k_absorb_and_value_projection_against_the_definition():
+    T, H = 2, 3
+    kvb = random_q6k_rows(6, H * 256).reshape(H, 256, 420)
+    q = orc.randn(7, (T, H, 192))
+    w = orc.q6k_rows512(kvb).reshape(H, 256, 512).astype(np.float64)
+    qa = orc.mla_absorb_q6k(q, kvb, T, H)
+    want = np.einsum("hic,thi->thc", w[:, :128], q[:, :, :128].astype(np.float64))
+    assert np.abs(qa[:, :, :512] - want).max() < 1e-4 * np.abs(want).max() and np.array_equal(qa[:, :, 512:], q[:, :, 128:])
+    u = orc.randn(8, (T, H, 512))
+    out = orc.mla_vb_q6k(u, kvb, T, H)
+    want = np.einsum("hvc,thc->thv", w[:, 128:], u.astype(np.float64))
+    assert np.abs(out - want).max() < 1e-4 * np.abs(want).max()
