@@ -68,6 +68,10 @@ struct MlaParams {
     const int32_t* sel_cnt;
     int K, per_t;
     int nz;              // row groups
+    // a pass of one split needs no merge: the kernel writes its rows' results themselves, u [T * H][512] of type ot
+    // (0 float32, 1 half), and the partials are not used
+    void* u;
+    int ot;
 };
 
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));   // a 16-byte chunk in flight (a plain vector: stays in registers)
@@ -553,6 +557,45 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
     const float l_row = rows_sum(l_r);
     const float m_r = thr < 0.0f ? -INFINITY : -nbr;
     const float inv_l = l_row > 0.0f ? 1.0f / l_row : 0.0f;
+    if (p.ns == 1 && p.u) {
+        // ---- one split: the rows' results, through the same staging (512 bytes a row and pass: 256 halfs, or 128 floats).
+        // (a dense row of a selection pass past the length such passes are sized for comes out as NaNs, not as a
+        // plausible wrong answer)
+        constexpr int OROW = 512 + 16;
+        lds_u8* const ob = (w < 4 ? B0 : B1) + (w & 3) * 16 * OROW;
+        typedef _Float16 h4v __attribute__((ext_vector_type(4)));
+        const float sc = n_all > p.kbs ? __builtin_nanf("") : inv_l;
+        const int passes = p.ot == 0 ? 4 : 2, dpp = DT / passes;      // passes over the latents, 16-latent tiles a pass
+        const int64_t rowb = p.ot == 0 ? ML * 4 : ML * 2;
+        for (int hp = 0; hp < passes; ++hp) {
+#pragma unroll
+            for (int d2 = 0; d2 < DT / 2; ++d2) {
+                if (d2 < dpp) {
+                    // (o indexed through a constant-trip loop: the accumulators stay in registers)
+                    f4v v = o[0];
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) v = dt == hp * dpp + d2 ? o[dt] : v;
+                    v = v * sc;
+                    if (p.ot == 0) {
+                        *reinterpret_cast<__attribute__((address_space(3))) f4v*>(ob + n * OROW + (d2 * 16 + g4 * 4) * 4) = v;
+                    } else {
+                        const h4v h = {(_Float16) v[0], (_Float16) v[1], (_Float16) v[2], (_Float16) v[3]};
+                        *reinterpret_cast<__attribute__((address_space(3))) h4v*>(ob + n * OROW + (d2 * 16 + g4 * 4) * 2) = h;
+                    }
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const int id = c * 64 + lane, r = id >> 5, piece = id & 31;
+                const int rg = (p.per_t ? z % zpt : z) * MROWS + w * 16 + r;
+                const bool ok = p.per_t ? rg < p.H : rg < rows;
+                const int64_t rrow = p.per_t ? (int64_t) tz * p.H + rg : rg;
+                const u4v x = *reinterpret_cast<const __attribute__((address_space(3))) u4v*>(ob + r * OROW + piece * 16);
+                if (ok) *reinterpret_cast<u4v*>(reinterpret_cast<uint8_t*>(p.u) + rrow * rowb + hp * 512 + piece * 16) = x;
+            }
+        }
+        return;
+    }
     {
         constexpr int OROW = 256 * 2 + 16;                        // bytes a staged row of 256 halfs, padded
         lds_u8* const ob = (w < 4 ? B0 : B1) + (w & 3) * 16 * OROW;   // 4 waves x 8,448 bytes in each of the first two buffers
@@ -957,6 +1000,8 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     p.per_t = per_t;
     p.nz = (int) nz;
     p.flat = ns < 8;
+    p.u = ns == 1 ? u : nullptr;
+    p.ot = ot;
     dim3 grid((unsigned) (p.flat ? ns * nz : (ns + 7) / 8 * 8 * nz));
     if (ns_profile_mark(g, 0)) return -1;
     if (MW == 4) {
@@ -970,9 +1015,11 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     }
     NS_LAUNCHED("mla_decode");
     if (ns_profile_mark(g, 1)) return -1;
-    if (ot == 0) mla_merge_kernel<0><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
-    else mla_merge_kernel<1><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
-    NS_LAUNCHED("mla_merge");
+    if (ns > 1) {
+        if (ot == 0) mla_merge_kernel<0><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
+        else mla_merge_kernel<1><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
+        NS_LAUNCHED("mla_merge");
+    }
     return ns_profile_mark(g, 2);
 }
 
