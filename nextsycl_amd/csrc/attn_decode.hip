@@ -25,7 +25,7 @@
 // {O[D], m (log2 units), l}; a second kernel merges the splits: out = sum O_s 2^(m_s - M) / sum l_s 2^(m_s - M).
 //
 // Reference behaviour kept: kernels/llm/qwen35/silo/attn.cpp:100-104,261-290,321-370 (split form, partial layout,
-// merge, one launch when the rows' split sizes agree else a row at a time), kernels/llm/museglimmer/silo/attn.cpp:51-55,
+// merge, one launch when the rows' split sizes agree - here: a launch a run of rows whose sizes agree), kernels/llm/museglimmer/silo/attn.cpp:51-55,
 // 86-92,120-127 (absolute split positions, ring slots, window), and the rounding model of both (16-bit operands,
 // float32 scores, softmax and accumulation; quantized values rounded to half as staged).
 #include "ns_internal.hpp"
@@ -682,15 +682,19 @@ __global__ __launch_bounds__(MERGE_W * 64) void attn_merge_kernel(const float* _
 // ---- host side ----------------------------------------------------------------------------------------------------
 
 // work-groups the key splits aim for (key heads x splits): two a CU at head size 128, one at 256 (its LDS footprint admits
-// one a CU; 256 against 512 measured 17.6 against 23.2 us at 32K keys, and half the partials to merge); NS_DEC_WGS
-// overrides (tuning)
-int64_t target_wgs(int64_t D) {
+// one a CU; 256 against 512 measured 17.6 against 23.2 us at 32K keys, and half the partials to merge). A split's partial
+// is written and read again for every query row on it - T x G rows of D + 2 floats against the split's 2 kbs rows of
+// keys and values - so 16-bit caches whose key heads serve 8 or more query heads take half as many, twice as long
+// splits (G = 8, 64K keys, 4 rows: 30.9 -> 29.7 us; G = 16, 4 rows: 44.7 -> 40.5; one row: within 0.5 us either way);
+// quantized rows keep the two work-groups a CU their arithmetic needs (128K keys of q8_0: 35.0 against 37.8 us).
+// The rule may depend on the heads and the cache form, never on the rows of a pass. NS_DEC_WGS overrides (tuning)
+int64_t target_wgs(int64_t D, int64_t G, int kt) {
     const int64_t v = ns_tune_get(NS_TUNE_DEC_WGS);
-    return v > 0 ? v : D == 256 ? 256 : 512;
+    return v > 0 ? v : D == 256 || (G >= 8 && (kt == 0 || kt == 3)) ? 256 : 512;
 }
 // keys a split for a row that sees `keys` keys: a multiple of 128 (4 waves x 32-key tiles)
-int64_t dec_kbs(int64_t keys, int64_t Hkv, int64_t D) {
-    const int64_t t = target_wgs(D), want = (keys * Hkv + t - 1) / t;
+int64_t dec_kbs(int64_t keys, int64_t Hkv, int64_t D, int64_t G, int kt) {
+    const int64_t t = target_wgs(D, G, kt), want = (keys * Hkv + t - 1) / t;
     return std::max<int64_t>(128, (want + 127) / 128 * 128);
 }
 inline int64_t row_first(int64_t pos, int64_t win) { return win > 0 ? std::max<int64_t>(0, pos - win + 1) : 0; }
@@ -758,13 +762,13 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
     p.sl2 = (scale > 0.0f ? scale : 1.0f / sqrtf((float) D)) * 1.4426950408889634f;
     const int64_t last = p0 + T - 1;
     auto first_of = [&](int64_t r) { return x.kfirst >= 0 ? x.kfirst : row_first(p0 + r, win); };
-    auto kb_of = [&](int64_t r) { return dec_kbs(p0 + r + 1 - first_of(r), Hkv, D); };
-    // A causal pass is one launch when its rows' own split sizes agree, else a launch a row (a row's bits must not depend
-    // on the rows that share its pass). A pass that is not causal is always one launch, cut by its first row's key count
-    // (the longest: every row ends at the pass's last key) - kernels/llm/museglimmer/silo/attn.cpp:282-291
-    bool same = true;
-    if (causal)
-        for (int64_t r = 1; r < T; ++r) same = same && kb_of(r) == kb_of(0);
+    auto kb_of = [&](int64_t r) { return dec_kbs(p0 + r + 1 - first_of(r), Hkv, D, Hq / Hkv, kt); };
+    // A causal pass is one launch when its rows' own split sizes agree (a row's bits must not depend on the rows that
+    // share its pass). Where they do not - the pass straddles a key count at which the split size steps - the reference
+    // launches a row at a time (kernels/llm/qwen35/silo/attn.cpp:344-350); here each run of consecutive rows with one
+    // split size is a launch: every row is still cut by its own split size, and a pass has two runs, not T launches
+    // (8 rows across the step at 65536 keys: 212 -> 58 us). A pass that is not causal is always one launch, cut by its
+    // first row's key count (the longest: every row ends at the pass's last key) - kernels/llm/museglimmer/silo/attn.cpp:282-291
     const int64_t nsa = (x.scratch_floats > 0 ? x.scratch_floats : ns_attn_decode_scratch(T, Hq, Hkv, D, p0, win)) / (T * Hq * (D + 2));
     auto launch = [&](int64_t r0, int64_t nr, int64_t kb) -> int {
         const int64_t pp = p0 + r0, sp0 = first_of(r0) / kb, ns = (pp + nr - 1) / kb - sp0 + 1;
@@ -784,10 +788,14 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
         if (launch_merge<D>(g, c.part, (int) ns, QT, nr * Hq, (uint8_t*) out + r0 * Hq * D * esz)) return -1;
         return x.marks ? ns_profile_mark(g, 2) : 0;
     };
-    if (!causal) return launch(0, T, dec_kbs(last + 1 - first_of(0), Hkv, D));
-    if (same) return launch(0, T, kb_of(0));
-    for (int64_t r = 0; r < T; ++r)
-        if (launch(r, 1, kb_of(r))) return -1;
+    if (!causal) return launch(0, T, dec_kbs(last + 1 - first_of(0), Hkv, D, Hq / Hkv, kt));
+    for (int64_t r = 0; r < T;) {
+        const int64_t kb = kb_of(r);
+        int64_t r1 = r + 1;
+        while (r1 < T && kb_of(r1) == kb) ++r1;
+        if (launch(r, r1 - r, kb)) return -1;
+        r = r1;
+    }
     return 0;
 }
 
@@ -845,7 +853,7 @@ int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_
     if ((uintptr_t) q % 16 || ((uintptr_t) kc | (uintptr_t) vc) % 16) return ns_fail(w + ": rows 16-byte aligned");
     NS_HIP(hipSetDevice(g->dev));
     if (K == 0) return ns_fill(g, out, 0, (size_t) (T * Hq * D) * sizeof(float));     // nothing listed: zeros (l = 0)
-    const int64_t keys = K * 128, kbs = dec_kbs(keys, Hkv, D), ns = (keys + kbs - 1) / kbs;
+    const int64_t keys = K * 128, kbs = dec_kbs(keys, Hkv, D, Hq / Hkv, 0), ns = (keys + kbs - 1) / kbs;
     if ((size_t) (Hq * ns * (D + 2)) > scratch_floats) return ns_fail(w + ": the pass needs more scratch than the library keeps");
     // every row in one launch and one merge where the partials of all rows fit the scratch; else a launch a row
     const bool batched = (size_t) (T * Hq * ns * (D + 2)) <= scratch_floats && T * Hkv <= 65535;
@@ -951,18 +959,19 @@ int ns_attn_decode_static(ns_gpu* g, int qt, int kt, int pm, const void* q, int6
 int64_t ns_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win) {
     if (T <= 0 || Hq <= 0 || Hkv <= 0) return 0;
     int64_t ns = 1;
-    // a row launched alone: its own split size over its own keys
-    for (int64_t r = 0; r < T; ++r) {
-        const int64_t pos = p0 + r, first = row_first(pos, win), kb = dec_kbs(pos + 1 - first, Hkv, D);
-        ns = std::max(ns, pos / kb - first / kb + 1);
-    }
-    // the pass in one launch: from its first row's first key to its last row's last; causal or not, the last row's
-    // key count bounds every row's
-    const int64_t f0 = row_first(p0, win), last = p0 + T - 1;
-    for (int64_t r = 0; r < T; ++r) {
-        const int64_t kb = dec_kbs(last + 1 - row_first(p0 + r, win), Hkv, D), kb2 = dec_kbs(p0 + r + 1 - row_first(p0 + r, win), Hkv, D);
-        ns = std::max(ns, last / kb - f0 / kb + 1);
-        ns = std::max(ns, last / kb2 - f0 / kb2 + 1);
+    // (the cache form is not an argument: the count holds for the 16-bit rule and the quantized one)
+    for (int kt = 0; kt < 2; ++kt) {
+        auto kbs = [&](int64_t keys) { return dec_kbs(keys, Hkv, D, Hq / Hkv, kt); };
+        // a run of rows launched on its own: the row's own split size over its own first key to the pass's last
+        // the pass in one launch: from its first row's first key to its last row's last; causal or not, the last row's
+        // key count bounds every row's
+        const int64_t f0 = row_first(p0, win), last = p0 + T - 1;
+        for (int64_t r = 0; r < T; ++r) {
+            const int64_t pos = p0 + r, first = row_first(pos, win), kb = kbs(last + 1 - first), kb2 = kbs(pos + 1 - first);
+            ns = std::max(ns, pos / kb2 - first / kb2 + 1);
+            ns = std::max(ns, last / kb - f0 / kb + 1);
+            ns = std::max(ns, last / kb2 - f0 / kb2 + 1);
+        }
     }
     return T * Hq * ns * (D + 2);
 }
