@@ -168,24 +168,25 @@ def timed(w, steps, warmup):
         w.step()
     g.sync()
     ms = (time.perf_counter() - t0) * 1e3 / steps
-    # the dominant kernel alone: HIP events on the library's compute stream around each launch (a pass of its own:
-    # the events open gaps between the launches that the throughput pass must not see). Steps run back to back in short
-    # runs and the last step of each run is read, so the kernel is timed on a busy stream like the one above - a
-    # launch bracketed on an idle stream reads several microseconds long
-    if w.kind == "pre" or (w.kind == "mla" and w.T > 16):
-        # one launch a step (no marks inside) / several passes a step: the step itself, launched back to back, is the figure
+    # the dominant kernel alone: the same steps with the library told to queue its main kernel only (no merge launch),
+    # back to back between two HIP event stamps on the library's compute stream - the kernel's own launch duration on a
+    # busy queue, what rocprofv3's kernel trace reports. (Events around every single launch open gaps and read ~3 us long
+    # for kernels of 20 us.) The merge kernel's share is the rest of the step.
+    if w.kind == "pre" or w.kind == "prefill" or (w.kind == "mla" and w.T > 16):
+        # one launch a step / several passes a step: the step itself, launched back to back, is the figure
         return ms, ms * 1e6, 0.0
-    w.ops.profile(True)
-    main = merge = 0.0
-    n = max(3, min(steps, 20))
+    w.ops.profile(2)
+    for _ in range(8):
+        w.step()
+    g.sync()
+    n = max(steps, 50)
+    t0 = g.stamp()
     for _ in range(n):
-        for _ in range(6):
-            w.step()
-        a, b = w.ops.profile_last()
-        main += a
-        merge += b
-    w.ops.profile(False)
-    return ms, main / n, merge / n
+        w.step()
+    t1 = g.stamp()
+    main = g.elapsed_ns(t0, t1) / n
+    w.ops.profile(0)
+    return ms, main, max(0.0, ms * 1e6 - main)
 
 
 # HBM bytes per launch of each workload's dominant kernel as rocprofv3 counted them (FETCH_SIZE + WRITE_SIZE per dispatch,

@@ -192,10 +192,13 @@ int ns_llm_minimaxm3_idx_topk(ns_gpu* g, float* bs, int32_t* sel, int64_t T, int
 
 /* ---- measurement ---------------------------------------------------------------------------------------------------- */
 
-/* This library's own (the reference times kernels from the host side: llm/qwen35/src/probe.rs:105-113). on != 0: every
+/* This library's own (the reference times kernels from the host side: llm/qwen35/src/probe.rs:105-113). on = 1: every
  * attention call records HIP events on the compute stream before its main kernel, between it and the merge kernel, and
  * after; ns_attn_profile_last waits for the last call's and returns the two kernels' device times in nanoseconds
- * (merge_ns 0 for a call without a merge). Off by default: the events add gaps between the launches */
+ * (merge_ns 0 for a call without a merge). The events open gaps between the launches and read a few microseconds long
+ * for kernels this short, so: on = 2: attention calls queue their main kernel ONLY - no merge launch, the output is NOT
+ * written - and a run of such calls between two ns_stamp's divided by its length is that kernel's own launch duration
+ * on a busy queue. on = 0 (the default): neither */
 int ns_attn_profile(ns_gpu* g, int on);
 /* a plain device-to-device copy kernel (16 bytes a thread, reads `bytes`, writes `bytes`): the kernel of known size that
  * rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled against. This library's own */

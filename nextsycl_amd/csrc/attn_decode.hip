@@ -785,6 +785,7 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
         if (x.marks && ns_profile_mark(g, 0)) return -1;
         if (launch_kt<D>(g, kt, c, (int) (nr * c.G), dim3((unsigned) ns, (unsigned) Hkv))) return -1;
         if (x.marks && ns_profile_mark(g, 1)) return -1;
+        if (g->main_only) return 0;
         if (launch_merge<D>(g, c.part, (int) ns, QT, nr * Hq, (uint8_t*) out + r0 * Hq * D * esz)) return -1;
         return x.marks ? ns_profile_mark(g, 2) : 0;
     };

@@ -657,7 +657,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
         return -1;
     NS_LAUNCHED("attn_prefill");
     if (ns_profile_mark(g, 1)) return -1;
-    if (p.ns > 1) {
+    if (p.ns > 1 && !g->main_only) {
         if (ns_attn_merge_partials(g, D, p.part, p.ns, qt, T * Hq, out)) return -1;
         return ns_profile_mark(g, 2);
     }

@@ -46,7 +46,8 @@ int ns_profile_mark(ns_gpu* g, int i) {
 extern "C" {
 
 int ns_attn_profile(ns_gpu* g, int on) {
-    g->profile = on != 0;
+    g->profile = on == 1;
+    g->main_only = on == 2;
     g->pev_used = 0;
     return 0;
 }
