@@ -50,16 +50,17 @@ int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint1
  * every row sees every earlier cell. Else row t's cells are the pools sel[t K ..][0, sel_cnt[t]) of 4 cells each (cells
  * 4 b .. 4 b + 3) followed by its incomplete pool 4 ((p + 1) / 4) .. p, p = pos0 + t; a negative sel_cnt[t] is a dense
  * row. Any number of rows: rows with lists go 16 a pass on the queue, dense
- * rows as a prompt's. Replaces: kernels/llm/glm5next/glm.h:65-66 (glm.cpp:1062-1067,1095-1102,1252-1264; latent width 512
- * only - the reference also takes 256) */
+ * rows as a prompt's. L = 512, or 256 (cache [n][256], qa and u [T][H][256]): the narrow cache's cells 0 .. pos0 + T - 1, the
+ * rows and the results are widened with zeros into memory the library keeps per ns_gpu for the call (-1 when they do not
+ * fit: ~60,000 cells). Replaces: kernels/llm/glm5next/glm.h:65-66 (glm.cpp:1062-1067,1095-1102,1252-1264) */
 int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                       const int32_t* sel, const int32_t* sel_cnt, int64_t K);
 /* the same over q8 latent rows. Replaces: kernels/llm/glm5next/glm.h:79-80 (glm.cpp:1267-1276; the reference: at most 8 rows) */
 int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                          const int32_t* sel, const int32_t* sel_cnt, int64_t K);
-/* The dense form over a float32 latent cache c [n][512] (every row sees every earlier cell): the cells 0 .. pos0 + T - 1
- * are rounded to half into memory the library keeps per ns_gpu and read from there (-1 when they do not fit beside the
- * partials: ~48K cells). Replaces: kernels/llm/glm5next/glm.h:47 (glm.cpp:782-812) */
+/* The dense form over a float32 latent cache c [n][L], L = 512 or 256 (every row sees every earlier cell): the cells
+ * 0 .. pos0 + T - 1 are rounded to half into memory the library keeps per ns_gpu and read from there (-1 when they do not
+ * fit beside the partials: ~48K cells). Replaces: kernels/llm/glm5next/glm.h:47 (glm.cpp:782-812) */
 int ns_mla_attend(ns_gpu* g, const float* qa, const float* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale);
 /* out [n][512] half = the q8 latent rows idx[i] of src, widened: half(scale x q), one rounding (a prompt pass's gather).
  * Replaces: kernels/llm/glm5next/glm.h:78 (glm.cpp:1301-1325) */

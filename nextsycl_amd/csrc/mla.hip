@@ -920,6 +920,25 @@ __global__ __launch_bounds__(256) void to_half_kernel(const float* __restrict__ 
     reinterpret_cast<us8v*>(y)[i] = h;
 }
 
+// rows of Ls values into rows of Ld: the first min(Ls, Ld) copied (float32 -> half rounds), the rest zeros. A latent cache
+// of width 256 and its absorbed rows are widened to the kernel's 512 this way (a zero latent adds nothing to a score or
+// to a sum) and the results' first 256 values taken back out
+__device__ __forceinline__ void put_as(float* d, float v) { *d = v; }
+__device__ __forceinline__ void put_as(uint16_t* d, float v) { *d = f32_to_f16(v); }
+__device__ __forceinline__ void put_as(uint16_t* d, uint16_t v) { *d = v; }
+template <class S, class Dt>
+__global__ __launch_bounds__(256) void widen_rows_kernel(const S* __restrict__ src, Dt* __restrict__ dst, int64_t rows, int Ls, int Ld) {
+    const int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x, per = Ld / 4, r = i / per;
+    if (r >= rows) return;
+    const int c0 = (int) (i % per) * 4;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const int f = c0 + k;
+        if (f < Ls) put_as(dst + r * Ld + f, src[r * Ls + f]);
+        else put_as(dst + r * Ld + f, S(0));
+    }
+}
+
 // out [n][512] half = the q8 latent rows idx[i] of src widened: half(scale x q), one rounding (the product is exact in
 // float32); a thread 8 values (kernels/llm/glm5next/glm.cpp:1301-1325)
 __global__ __launch_bounds__(256) void gather_q8_h_kernel(const uint8_t* __restrict__ src, const int32_t* __restrict__ idx, uint16_t* __restrict__ out,
@@ -1145,11 +1164,41 @@ static int mla_sel_rows(ns_gpu* g, const char* who, bool q8, const float* qa, co
     return 0;
 }
 
+// A latent width of 256 (the reference's other width, kernels/llm/glm5next/glm.cpp:1257) rides on the 512-wide kernel: the
+// cache's rows 0 .. pos0 + T - 1 (half, or float32 rounded to half: CT), the absorbed rows and the results pass through
+// the library's scratch, widened with zeros / narrowed again. What the scratch does not hold is refused.
+extern "C++" {
+template <class CT>
+static int mla_narrow(ns_gpu* g, const char* who, const float* qa, const CT* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
+                      const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
+    const std::string w(who);
+    if (H <= 0 || pos0 < 0) return ns_fail(w + ": heads and a position");
+    if (!qa || !c || !u) return ns_fail(w + ": a null buffer");
+    const int64_t cells = pos0 + T, rows = T * H;
+    const size_t c_f = (size_t) cells * ML / 2, q_f = (size_t) rows * ML, u_f = q_f;        // floats of scratch each takes
+    if (c_f + q_f + u_f + (size_t) (16 * H) * PSTRIDE > g->own_scratch_floats)
+        return ns_fail(w + ": a latent width of 256 is widened in the library's scratch, which does not hold " + std::to_string(cells) + " cells and " +
+                       std::to_string(rows) + " rows");
+    NS_HIP(hipSetDevice(g->dev));
+    uint16_t* cw = (uint16_t*) g->own_scratch;
+    float* qw = g->own_scratch + c_f;
+    float* uw = qw + q_f;
+    widen_rows_kernel<CT, uint16_t><<<(unsigned) ((cells * (ML / 4) + 255) / 256), 256, 0, g->q>>>(c, cw, cells, (int) L, ML);
+    widen_rows_kernel<float, float><<<(unsigned) ((rows * (ML / 4) + 255) / 256), 256, 0, g->q>>>(qa, qw, rows, (int) L, ML);
+    NS_LAUNCHED("widen_rows");
+    if (mla_sel_rows(g, who, false, qw, cw, uw, T, H, pos0, scale, sel, sel_cnt, K, uw + u_f, g->own_scratch_floats - (c_f + q_f + u_f))) return -1;
+    widen_rows_kernel<float, float><<<(unsigned) ((rows * (L / 4) + 255) / 256), 256, 0, g->q>>>(uw, u, rows, ML, (int) L);
+    NS_LAUNCHED("narrow_rows");
+    return 0;
+}
+}  // extern "C++"
+
 int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                       const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
     NS_TRY
     if (T <= 0) return 0;
-    if (L != 512) return ns_fail("ns_mla_attend_sel: latent width 512");
+    if (L == 256) return mla_narrow<uint16_t>(g, "ns_mla_attend_sel", qa, c, u, T, H, L, pos0, scale, sel, sel_cnt, K);
+    if (L != 512) return ns_fail("ns_mla_attend_sel: latent width 256 or 512");
     return mla_sel_rows(g, "ns_mla_attend_sel", false, qa, c, u, T, H, pos0, scale, sel, sel_cnt, K, g->own_scratch, g->own_scratch_floats);
     NS_CATCH
 }
@@ -1168,7 +1217,8 @@ int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, in
 int ns_mla_attend(ns_gpu* g, const float* qa, const float* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale) {
     NS_TRY
     if (T <= 0) return 0;
-    if (L != 512) return ns_fail("ns_mla_attend: latent width 512");
+    if (L == 256) return mla_narrow<float>(g, "ns_mla_attend", qa, c, u, T, H, L, pos0, scale, nullptr, nullptr, 0);
+    if (L != 512) return ns_fail("ns_mla_attend: latent width 256 or 512");
     if (pos0 < 0 || !c) return ns_fail("ns_mla_attend: a position and a cache");
     if ((uintptr_t) c % 16) return ns_fail("ns_mla_attend: the cache 16-byte aligned");
     const int64_t cells = pos0 + T, ch_floats = (cells * ML / 2 + 3) / 4 * 4;     // the half rows, counted in floats

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 from helpers import check_close, make_kv, make_q
-from nextsycl_amd import DevBuf
+from nextsycl_amd import DevBuf, Error
 from nextsycl_amd.attn import F32
 from oracle import orc
 
@@ -234,3 +234,35 @@ def test_ds2_mla_decode_with_q6k_weights(ops, T, H, pos0):
     qa = orc.mla_absorb_q6k(q, kvb, T, H)
     ref = orc.mla_vb_q6k(orc.mla_decode_u(qa, cache, T, H, pos0, scale), kvb, T, H)
     assert orc.compare(ref.reshape(T, H * 128), want.reshape(T, H * 128))[1] <= 1e-4
+
+
+def test_glm_latent_width_256(ops):
+    """The reference's other latent width (kernels/llm/glm5next/glm.cpp:1257): a half cache dense and with cell pools, a
+    float32 cache dense - against the reference-order restatement at L = 256; and the refusal, with its reason, of a
+    cache the widening does not hold."""
+    g = ops.gpu
+    L, scale = 256, 0.0625
+    for T, H, pos0, K in ((1, 64, 2000, 0), (5, 16, 300, 0), (20, 8, 3000, 24), (3, 32, 20000, 128)):
+        n = pos0 + T
+        qa, x = orc.randn(95, (T, H * L), 0.3), orc.randn(96, (n, L))
+        rows = orc.f2h(x).view(np.uint8).reshape(n, 2 * L)
+        rng = np.random.default_rng(11)
+        sel = cnt = None
+        if K:
+            npool = (pos0 + 1) // 4
+            sel = np.stack([rng.permutation(npool)[:K] for _ in range(T)]).astype(np.int32)
+            cnt = rng.integers(0, K + 1, T).astype(np.int32)
+        u = DevBuf(g, T * H * L * 4); u.fill(0xFF)
+        ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, scale, sel=DevBuf.of(g, sel) if K else None,
+                       sel_cnt=DevBuf.of(g, cnt) if K else None, K=K)
+        want = orc.glm_mla_attend_sel(qa, rows, False, T, H, L, pos0, scale, sel, cnt, K) if K else orc.glm_mla_attend(qa, rows, False, T, H, L, pos0, scale)
+        check_close(u.read(np.float32).reshape(T, H * L), want.reshape(T, H * L).astype(np.float64), F32, "ns_mla_attend_sel at L = 256, %d rows" % T)
+        if not K and pos0 < 3000:
+            u.fill(0xFF)
+            ops.mla_attend_f32(DevBuf.of(g, qa), DevBuf.of(g, x), u, T, H, L, pos0, scale)
+            want = orc.glm_mla_attend_f32(qa, x, T, H, L, pos0, scale).reshape(T, H * L)
+            check_close(u.read(np.float32).reshape(T, H * L), want.astype(np.float64), F32, "ns_mla_attend at L = 256")
+    # 100K cells widened to 512 halfs each are 100 MB: more than the library's scratch
+    big = DevBuf(g, 100001 * 2 * L)
+    with pytest.raises(Error, match="widened in the library's scratch"):
+        ops.mla_attend(DevBuf(g, 8 * L * 4), big, DevBuf(g, 8 * L * 4), 1, 8, L, 100000, scale)
