@@ -1092,47 +1092,49 @@ int ns_mla_decode_latent(ns_gpu* g, int qt, const void* qa, const uint16_t* cach
     NS_CATCH
 }
 
+// one body for both weight forms (kvb != NULL: Q6_K rows). More rows than a decode pass holds are queued 16 at a time - the
+// reference's kernel takes any row count (kernels/llm/deepseek2/ds2.cpp:262-281), its engine sends prompts elsewhere
+static int ds2_decode(ns_gpu* g, const char* who, const float* q, const uint16_t* kb, const uint16_t* vb, const uint8_t* kvb, const uint16_t* cache,
+                      float* out, int64_t T, int64_t H, int64_t pos0, float scale) {
+    const std::string w(who);
+    if (T <= 0) return 0;
+    if (H <= 0 || pos0 < 0) return ns_fail(w + ": heads and a position");
+    if (!q || !cache || !out || (kvb ? false : !kb || !vb)) return ns_fail(w + ": a null buffer");
+    if (kvb && (uintptr_t) kvb % 2) return ns_fail(w + ": kv_b 2-byte aligned");
+    NS_HIP(hipSetDevice(g->dev));
+    for (int64_t t0 = 0; t0 < T; t0 += 16) {
+        const int64_t n = std::min<int64_t>(16, T - t0);
+        // the library's own scratch (the reference's signature has none): the absorbed queries, u, then the partials
+        const size_t rows = (size_t) (n * H), qa_f = (rows * (ML + 64) + 3) / 4 * 4, u_f = rows * ML;
+        if (qa_f + u_f + rows * PSTRIDE > g->own_scratch_floats) return ns_fail(w + ": the pass needs more scratch than the library keeps");
+        float* qa = g->own_scratch;
+        float* u = qa + qa_f;
+        float* part = u + u_f;
+        const float* qp = q + t0 * H * 192;
+        float* op = out + t0 * H * 128;
+        if (kvb) mla_absorb_q6k_kernel<<<(unsigned) rows, 256, 0, g->q>>>(qp, kvb, qa, H);
+        else mla_absorb_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(qp, kb, qa, H);
+        NS_LAUNCHED("mla_absorb");
+        if (mla_latent(g, who, 0, 0, 64, false, qa, cache, u, n, H, pos0 + t0, scale, part, g->own_scratch_floats - qa_f - u_f)) return -1;
+        if (kvb) mla_vb_q6k_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(u, kvb, op, H);
+        else mla_vb_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(u, vb, op, H);
+        NS_LAUNCHED("mla_vb");
+    }
+    return 0;
+}
+
 int ns_ds2_mla_decode(ns_gpu* g, const float* q, const uint16_t* kb, const uint16_t* vb, const uint16_t* cache, float* out, int64_t T, int64_t H,
                       int64_t pos0, float scale) {
     NS_TRY
-    if (T <= 0) return 0;
-    if (H <= 0 || pos0 < 0 || T > 16) return ns_fail("ns_ds2_mla_decode: 1..16 rows, heads and a position");
-    if (!q || !kb || !vb || !cache || !out) return ns_fail("ns_ds2_mla_decode: a null buffer");
-    // the library's own scratch (the reference's signature has none): the absorbed queries, u, then the partials
-    const size_t rows = (size_t) (T * H), qa_f = (rows * (ML + 64) + 3) / 4 * 4, u_f = rows * ML;
-    if (qa_f + u_f + rows * PSTRIDE > g->own_scratch_floats) return ns_fail("ns_ds2_mla_decode: the pass needs more scratch than the library keeps");
-    float* qa = g->own_scratch;
-    float* u = qa + qa_f;
-    float* part = u + u_f;
-    NS_HIP(hipSetDevice(g->dev));
-    mla_absorb_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(q, kb, qa, H);
-    NS_LAUNCHED("mla_absorb");
-    if (mla_latent(g, "ns_ds2_mla_decode", 0, 0, 64, false, qa, cache, u, T, H, pos0, scale, part, g->own_scratch_floats - qa_f - u_f)) return -1;
-    mla_vb_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(u, vb, out, H);
-    NS_LAUNCHED("mla_vb");
-    return 0;
+    return ds2_decode(g, "ns_ds2_mla_decode", q, kb, vb, nullptr, cache, out, T, H, pos0, scale);
     NS_CATCH
 }
 
 int ns_ds2_mla_decode_q6k(ns_gpu* g, const float* q, const void* kvb, const uint16_t* cache, float* out, int64_t T, int64_t H, int64_t pos0,
                           float scale) {
     NS_TRY
-    if (T <= 0) return 0;
-    if (H <= 0 || pos0 < 0 || T > 16) return ns_fail("ns_ds2_mla_decode_q6k: 1..16 rows, heads and a position");
-    if (!q || !kvb || !cache || !out) return ns_fail("ns_ds2_mla_decode_q6k: a null buffer");
-    if ((uintptr_t) kvb % 2) return ns_fail("ns_ds2_mla_decode_q6k: kv_b 2-byte aligned");
-    const size_t rows = (size_t) (T * H), qa_f = (rows * (ML + 64) + 3) / 4 * 4, u_f = rows * ML;
-    if (qa_f + u_f + rows * PSTRIDE > g->own_scratch_floats) return ns_fail("ns_ds2_mla_decode_q6k: the pass needs more scratch than the library keeps");
-    float* qa = g->own_scratch;
-    float* u = qa + qa_f;
-    float* part = u + u_f;
-    NS_HIP(hipSetDevice(g->dev));
-    mla_absorb_q6k_kernel<<<(unsigned) rows, 256, 0, g->q>>>(q, (const uint8_t*) kvb, qa, H);
-    NS_LAUNCHED("mla_absorb_q6k");
-    if (mla_latent(g, "ns_ds2_mla_decode_q6k", 0, 0, 64, false, qa, cache, u, T, H, pos0, scale, part, g->own_scratch_floats - qa_f - u_f)) return -1;
-    mla_vb_q6k_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(u, (const uint8_t*) kvb, out, H);
-    NS_LAUNCHED("mla_vb_q6k");
-    return 0;
+    if (T > 0 && !kvb) return ns_fail("ns_ds2_mla_decode_q6k: a null buffer");
+    return ds2_decode(g, "ns_ds2_mla_decode_q6k", q, nullptr, nullptr, (const uint8_t*) kvb, cache, out, T, H, pos0, scale);
     NS_CATCH
 }
 

@@ -210,7 +210,7 @@ def test_glm_cell_pools_at_100k_tokens(ops, q8):
     check_close(u.read(np.float32).reshape(T, H * L), want.reshape(T, H * L).astype(np.float64), F32, "ns_mla_attend_sel at 100K tokens")
 
 
-@pytest.mark.parametrize("T,H,pos0", [(1, 16, 700), (3, 128, 2000), (16, 8, 5)])
+@pytest.mark.parametrize("T,H,pos0", [(1, 16, 700), (3, 128, 2000), (16, 8, 5), (37, 8, 300)])
 def test_ds2_mla_decode_with_q6k_weights(ops, T, H, pos0):
     """ns_ds2_mla_decode_q6k: kv_b read as the file stores it (Q6_K rows), against the float64 chain over the widened rows."""
     from test_oracle_boundary import random_q6k_rows

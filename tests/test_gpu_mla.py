@@ -144,6 +144,26 @@ def test_full_ds2_mla_decode(ops):
     _close(want, want64, "the restated chain itself")
 
 
+def test_full_ds2_mla_decode_of_more_rows_than_a_pass(ops):
+    """ns_ds2_mla_decode takes any row count, as the reference's kernel does (kernels/llm/deepseek2/ds2.cpp:262-270): 41
+    rows are three queued passes, every row at its own position."""
+    T, H, pos0 = 41, 8, 250
+    n = pos0 + T
+    g = ops.gpu
+    cache = orc.f2h(orc.randn(5, (n, 576), 0.5))
+    q = orc.randn(6, (T, H, 192))
+    kb = orc.f2h(orc.randn(7, (H, 512, 128), 0.09))
+    vb = orc.f2h(orc.randn(8, (H, 128, 512), 0.05))
+    scale = 0.0722
+    out = DevBuf(g, T * H * 128 * 4)
+    out.fill(0xFF)
+    ops.mla_decode(DevBuf.of(g, q), DevBuf.of(g, kb), DevBuf.of(g, vb), DevBuf.of(g, cache), out, T, H, pos0, scale)
+    got = out.read(np.float32).reshape(T, H, 128)
+    qa64 = np.concatenate([np.einsum("hrc,thc->thr", orc.h2f(kb).astype(np.float64), q[:, :, :128].astype(np.float64)), q[:, :, 128:]], axis=2)
+    u64 = orc.mla_f64(qa64.astype(np.float32), cache, T, H, pos0, scale)
+    _close(got, np.einsum("hvl,thl->thv", orc.h2f(vb).astype(np.float64), u64), "ns_ds2_mla_decode, 41 rows")
+
+
 def test_ds2_kv_store(ops):
     g = ops.gpu
     T, L, R, pos0 = 37, 512, 64, 40
