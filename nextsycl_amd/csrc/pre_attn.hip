@@ -170,53 +170,62 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
     }
     const bool d_pow2 = (D & (D - 1)) == 0;
     const float inv_d = 1.0f / (float) D;                  // exact for a power of two: s * inv_d is s / D bit for bit
-    // What a head needs from memory: its group, its row, the lane's own features and (VEC) their partners and weights.
+    // The wave walks its heads group by group: a group's descriptor (scalar registers, read from the kernel-argument block
+    // at a scalar index - indexing the by-value argument at run time would send it through private memory), the lane's row
+    // bases in the group's source and destination, its weights and which of its features the group rotates are worked out
+    // once a group; a head then costs two 64-bit additions an address, its loads, its arithmetic and its stores.
     // Every load is unconditional - a lane with nothing to do reads a valid address and drops the value - so the loads
-    // of the NEXT head can be in flight, counted, while this head is worked on: a head then costs about one memory
-    // latency a wave instead of two or three
+    // of the next two heads are in flight while this head is worked on
     struct HeadIn {
-        PreGroup G;
-        int h;
         const float* x;
-        float4 xo[MAXG], xp[MAXG], wo[MAXG], wp[MAXG];
+        float4 xo[MAXG], xp[MAXG];
     };
     const int tl = row_live ? t : p.T - 1;
     const PreGroup* groups = reinterpret_cast<const PreGroup*>((const char*) __builtin_amdgcn_kernarg_segment_ptr() + offsetof(PreParams, gr));
-    auto fetch = [&](int hh, HeadIn& in) __attribute__((always_inline)) {
-        // the head's group: its index from comparisons, its descriptor read from the kernel-argument block in memory at
-        // that index - scalar loads into scalar registers. (Indexing the by-value argument itself at run time would
-        // send the whole block through private memory; selecting among five descriptors held in registers overflows
-        // the scalar file)
-        int gi = 0, first = 0;
-        in.h = hh;
+    int gfirst = 0;
+    for (int gi = 0; gi < p.ngr; ++gi) {
+    const PreGroup G = groups[gi];
+    const int g0 = gfirst;
+    gfirst += G.heads;
+    const int ha = max(hfirst, g0) - g0, hb = min(hend, gfirst) - g0;     // this wave's heads of the group
+    if (ha >= hb) continue;
+    // ---- once a group: the lane's own features and their partners in the row, the weights of both
+    const float* xrow = G.src + (int64_t) tl * G.ss;
+    int io[MAXG], ipn[MAXG];
+    bool rot_c[MAXG];
+    float4 wo[MAXG], wp[MAXG];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            first += k < p.ngr ? p.gr[k].heads : 0;
-            if (k + 1 < p.ngr && hh >= first) gi = k + 1, in.h = hh - first;
+    for (int c = 0; c < MAXG; ++c) {
+        const int i0 = li * 4 + c * 256, i = i0 < D ? i0 : 0;
+        rot_c[c] = G.rope != 0 && (onmask >> (c * 4) & 1) != 0;
+        io[c] = i;
+        ipn[c] = !rot_c[c] || p.mode == ROPE_MG_PAIRS ? i : i < pdist ? i + pdist : i - pdist;
+        if constexpr (VEC) {
+            const float* w = G.w ? G.w : xrow;
+            wo[c] = *reinterpret_cast<const float4*>(w + io[c]);
+            wp[c] = *reinterpret_cast<const float4*>(w + ipn[c]);
         }
-        in.G = groups[gi];
-        in.x = in.G.src + (int64_t) tl * in.G.ss + (int64_t) in.h * in.G.hs;
+    }
+    auto fetch = [&](int h, HeadIn& in) __attribute__((always_inline)) {
+        in.x = xrow + (int64_t) h * G.hs;
 #pragma unroll
         for (int c = 0; c < MAXG; ++c) {
-            const int i0 = li * 4 + c * 256, i = i0 < D ? i0 : 0;
-            in.xo[c] = *reinterpret_cast<const float4*>(in.x + i);
-            if constexpr (VEC) {
-                const bool rotated = in.G.rope != 0 && (onmask >> (c * 4) & 1) != 0;
-                const int ip = !rotated || p.mode == ROPE_MG_PAIRS ? i : i < pdist ? i + pdist : i - pdist;
-                const float* w = in.G.w ? in.G.w : in.x;
-                in.xp[c] = *reinterpret_cast<const float4*>(in.x + ip);
-                in.wo[c] = *reinterpret_cast<const float4*>(w + i);
-                in.wp[c] = *reinterpret_cast<const float4*>(w + ip);
-            }
+            in.xo[c] = *reinterpret_cast<const float4*>(in.x + io[c]);
+            if constexpr (VEC) in.xp[c] = *reinterpret_cast<const float4*>(in.x + ipn[c]);
         }
     };
-    HeadIn cur;
-    fetch(hfirst, cur);
-  for (int hh = hfirst; hh < hend; ++hh) {
-    HeadIn nxt;
-    fetch(hh + 1 < hend ? hh + 1 : hh, nxt);          // the last head reads itself again rather than branch
-    const PreGroup G = cur.G;
-    const int h = cur.h;
+    // where the lane's results go: a plain row's element (t, h = 0, feature i), or the cache row of head 0 at the row's slot
+    const int kt = G.dt - DST_CACHE;
+    const int64_t slot = p.ring ? (p.p0 + t) % p.cap : p.p0 + t;
+    const int64_t rb = G.dt >= DST_CACHE ? kv_row_bytes(kt, D) : 0;
+    uint8_t* const crow0 = reinterpret_cast<uint8_t*>(G.dst) + slot * rb;
+    const int64_t at0 = (int64_t) t * G.ds, at20 = (int64_t) t * G.ds2;
+    HeadIn cur, nxt;
+    fetch(ha, cur);
+    fetch(ha + 1 < hb ? ha + 1 : ha, nxt);
+  for (int h = ha; h < hb; ++h) {
+    HeadIn nx2;
+    fetch(h + 2 < hb ? h + 2 : hb - 1, nx2);          // two heads ahead; the last heads read the last again rather than branch
     const float* x = cur.x;
     // ---- the row's scale
     float4 xo[MAXG];
@@ -259,8 +268,8 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
                 for (int j = 0; j < 4; ++j) y[c][j] = 0.0f;
                 continue;
             }
-            const bool rotated = G.rope != 0 && (onmask >> (c * 4) & 1) != 0;
-            const float4 xp4 = cur.xp[c], wo4 = cur.wo[c], wp4 = cur.wp[c];
+            const bool rotated = rot_c[c];
+            const float4 xp4 = cur.xp[c], wo4 = wo[c], wp4 = wp[c];
             const float xv[4] = {xo[c].x, xo[c].y, xo[c].z, xo[c].w}, xq[4] = {xp4.x, xp4.y, xp4.z, xp4.w};
             const float wv[4] = {wo4.x, wo4.y, wo4.z, wo4.w}, wq[4] = {wp4.x, wp4.y, wp4.z, wp4.w};
             float me[4], pt[4];
@@ -292,7 +301,7 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
         const bool live = i < D && row_live;
         if (G.dt < DST_CACHE) {
             if (!live) continue;
-            const int64_t at = (int64_t) t * G.ds + (int64_t) h * D + i;
+            const int64_t at = at0 + (int64_t) h * D + i;
             if (G.dt == DST_F32) {
                 *reinterpret_cast<float4*>(reinterpret_cast<float*>(G.dst) + at) = make_float4(y[c][0], y[c][1], y[c][2], y[c][3]);
             } else {
@@ -302,14 +311,12 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
                 *reinterpret_cast<ushort4*>(reinterpret_cast<uint16_t*>(G.dst) + at) = o;
             }
             if (G.dst2) {
-                const int64_t at2 = (int64_t) t * G.ds2 + (int64_t) h * D + i;
+                const int64_t at2 = at20 + (int64_t) h * D + i;
                 *reinterpret_cast<ushort4*>(reinterpret_cast<uint16_t*>(G.dst2) + at2) =
                     make_ushort4(f32_to_f16(y[c][0]), f32_to_f16(y[c][1]), f32_to_f16(y[c][2]), f32_to_f16(y[c][3]));
             }
         } else {
-            const int kt = G.dt - DST_CACHE;
-            const int64_t slot = p.ring ? (p.p0 + t) % p.cap : p.p0 + t;
-            uint8_t* row = reinterpret_cast<uint8_t*>(G.dst) + ((int64_t) h * p.cap + slot) * kv_row_bytes(kt, D);
+            uint8_t* row = crow0 + (int64_t) h * p.cap * rb;
             if (kt == 0 || kt == 3) {
                 if (!live) continue;
                 ushort4 o;
@@ -337,7 +344,9 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
         }
     }
     cur = nxt;
-  }   // the wave's next head
+    nxt = nx2;
+  }   // the group's next head
+    }   // the wave's next group
 }
 
 int launch_pre(ns_gpu* g, const PreParams& p, const char* who) {
@@ -347,11 +356,10 @@ int launch_pre(ns_gpu* g, const PreParams& p, const char* who) {
     if (per_t <= 0 || p.T <= 0) return 0;
     // a wave a (row group, head) while that leaves the chip short of waves (a decode step); a prompt's rows have waves to
     // spare, and each then walks several heads of its rows on one evaluation of the rotation (most of a wave's
-    // arithmetic): about 4096 waves a launch measured best (8192 for the largest passes), the heads of a row group shared
-    // evenly among its waves
+    // arithmetic): about 4096 waves a launch measured best, the heads of a row group shared evenly among its waves
     PreParams q = p;
     const int64_t rpw = p.D == 64 ? 4 : p.D == 128 ? 2 : 1, tg = (p.T + rpw - 1) / rpw;
-    q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, tg * per_t / (tg * per_t >= 131072 ? 8192 : 4096)));
+    q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, tg * per_t / 4096));
     q.hpw = (int) ((per_t + (per_t + q.hpw - 1) / q.hpw - 1) / ((per_t + q.hpw - 1) / q.hpw));
     if (const int64_t forced = ns_tune_get(NS_TUNE_PRE_HPW)) q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, forced));   // sweeps
     const int64_t waves = tg * ((per_t + q.hpw - 1) / q.hpw);
