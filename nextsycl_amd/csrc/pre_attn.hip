@@ -25,6 +25,7 @@
 #include <cmath>
 #include <cstddef>
 #include <cstdlib>
+#include <type_traits>
 
 namespace {
 
@@ -215,11 +216,16 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
         }
     };
     // where the lane's results go: a plain row's element (t, h = 0, feature i), or the cache row of head 0 at the row's slot
-    const int kt = G.dt - DST_CACHE;
     const int64_t slot = p.ring ? (p.p0 + t) % p.cap : p.p0 + t;
-    const int64_t rb = G.dt >= DST_CACHE ? kv_row_bytes(kt, D) : 0;
+    const int64_t rb = G.dt >= DST_CACHE ? kv_row_bytes(G.dt - DST_CACHE, D) : 0;
     uint8_t* const crow0 = reinterpret_cast<uint8_t*>(G.dst) + slot * rb;
     const int64_t at0 = (int64_t) t * G.ds, at20 = (int64_t) t * G.ds2;
+    // the group's heads, one copy of the loop a destination form and "has weights" (both are the group's, not a head's:
+    // decided here, the loop holds no select or branch on them)
+    auto walk = [&](auto dt_c, auto w_c) __attribute__((always_inline)) {
+    constexpr int DTK = decltype(dt_c)::value;
+    constexpr bool HASW = decltype(w_c)::value;
+    constexpr int kt = DTK - DST_CACHE;
     HeadIn cur, nxt;
     fetch(ha, cur);
     fetch(ha + 1 < hb ? ha + 1 : ha, nxt);
@@ -232,7 +238,7 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
 #pragma unroll
     for (int c = 0; c < MAXG; ++c) xo[c] = li * 4 + c * 256 < D && row_live ? cur.xo[c] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     float inv = 1.0f;
-    if (G.w) {
+    if constexpr (HASW) {
         float s = 0.0f;
 #pragma unroll
         for (int c = 0; c < MAXG; ++c) {
@@ -275,8 +281,8 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
             float me[4], pt[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                me[j] = G.w ? xv[j] * inv * wv[j] : xv[j];
-                pt[j] = G.w ? xq[j] * inv * wq[j] : xq[j];
+                me[j] = HASW ? xv[j] * inv * wv[j] : xv[j];
+                pt[j] = HASW ? xq[j] * inv * wq[j] : xq[j];
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -290,7 +296,7 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
         for (int c = 0; c < MAXG; ++c) {
             const int i = li * 4 + c * 256;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) y[c][j] = i < D && row_live ? rope_feature(p, x, G.w, inv, i + j, G.rope != 0, Rot{rc[c * 4 + j], rs[c * 4 + j], (onmask >> (c * 4 + j) & 1) != 0}) : 0.0f;
+            for (int j = 0; j < 4; ++j) y[c][j] = i < D && row_live ? rope_feature(p, x, HASW ? G.w : nullptr, inv, i + j, G.rope != 0, Rot{rc[c * 4 + j], rs[c * 4 + j], (onmask >> (c * 4 + j) & 1) != 0}) : 0.0f;
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // loads above, stores below (source may be destination)
@@ -299,14 +305,14 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
         const int i = li * 4 + c * 256;
         if (c * 256 >= D) break;
         const bool live = i < D && row_live;
-        if (G.dt < DST_CACHE) {
+        if constexpr (DTK < DST_CACHE) {
             if (!live) continue;
             const int64_t at = at0 + (int64_t) h * D + i;
-            if (G.dt == DST_F32) {
+            if constexpr (DTK == DST_F32) {
                 *reinterpret_cast<float4*>(reinterpret_cast<float*>(G.dst) + at) = make_float4(y[c][0], y[c][1], y[c][2], y[c][3]);
             } else {
                 ushort4 o;
-                if (G.dt == DST_F16) o = make_ushort4(f32_to_f16(y[c][0]), f32_to_f16(y[c][1]), f32_to_f16(y[c][2]), f32_to_f16(y[c][3]));
+                if constexpr (DTK == DST_F16) o = make_ushort4(f32_to_f16(y[c][0]), f32_to_f16(y[c][1]), f32_to_f16(y[c][2]), f32_to_f16(y[c][3]));
                 else o = make_ushort4(f32_to_bf16(y[c][0]), f32_to_bf16(y[c][1]), f32_to_bf16(y[c][2]), f32_to_bf16(y[c][3]));
                 *reinterpret_cast<ushort4*>(reinterpret_cast<uint16_t*>(G.dst) + at) = o;
             }
@@ -317,17 +323,17 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
             }
         } else {
             uint8_t* row = crow0 + (int64_t) h * p.cap * rb;
-            if (kt == 0 || kt == 3) {
+            if constexpr (kt == 0 || kt == 3) {
                 if (!live) continue;
                 ushort4 o;
-                if (kt == 0) o = make_ushort4(f32_to_f16(y[c][0]), f32_to_f16(y[c][1]), f32_to_f16(y[c][2]), f32_to_f16(y[c][3]));
+                if constexpr (kt == 0) o = make_ushort4(f32_to_f16(y[c][0]), f32_to_f16(y[c][1]), f32_to_f16(y[c][2]), f32_to_f16(y[c][3]));
                 else o = make_ushort4(f32_to_bf16(y[c][0]), f32_to_bf16(y[c][1]), f32_to_bf16(y[c][2]), f32_to_bf16(y[c][3]));
                 *reinterpret_cast<ushort4*>(row + 2 * i) = o;
             } else {
                 // 8 lanes a block of 32: every lane takes part in the shuffles (dead lanes carry zeros, store nothing)
                 const int b = i / 32, ln = li & 7;
                 float d;
-                if (kt == 1) {
+                if constexpr (kt == 1) {
                     const uint32_t wv = q8_0_pack4(y[c], d);
                     if (live) {
                         *reinterpret_cast<uint32_t*>(row + i) = wv;
@@ -346,6 +352,20 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
     cur = nxt;
     nxt = nx2;
   }   // the group's next head
+    };
+    auto walk_w = [&](auto w_c) __attribute__((always_inline)) {
+        switch (G.dt) {
+            case DST_F32: walk(std::integral_constant<int, DST_F32>{}, w_c); break;
+            case DST_F16: walk(std::integral_constant<int, DST_F16>{}, w_c); break;
+            case DST_BF16: walk(std::integral_constant<int, DST_BF16>{}, w_c); break;
+            case DST_CACHE + 0: walk(std::integral_constant<int, DST_CACHE + 0>{}, w_c); break;
+            case DST_CACHE + 1: walk(std::integral_constant<int, DST_CACHE + 1>{}, w_c); break;
+            case DST_CACHE + 2: walk(std::integral_constant<int, DST_CACHE + 2>{}, w_c); break;
+            default: walk(std::integral_constant<int, DST_CACHE + 3>{}, w_c); break;
+        }
+    };
+    if (G.w) walk_w(std::true_type{});
+    else walk_w(std::false_type{});
     }   // the wave's next group
 }
 
