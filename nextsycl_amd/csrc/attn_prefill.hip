@@ -351,7 +351,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // Every LDS operand of a block is requested a block ahead (vread at the step's start, kread at the head of A), and
     // sched_group_barrier deals the vector instructions out between the matrix instructions.
     // The mask is applied under a wave-uniform branch: steps no row's causal or window edge crosses pay no comparison.
-    auto step = [&](f4v (&sc)[RT][2], f4v (&sn)[RT][2], uint32_t kl_next, uint32_t vl_prev, int j0, bool masked) {
+    auto step = [&](f4v (&sc)[RT][2], f4v (&sn)[RT][2], uint32_t kl_next, uint32_t vl_prev, int j0, bool masked, bool bar_mid = false) {
         float a[RT][8], amax[RT];
         s8v vpre[VPRE], kpre[KPRE][KB];
         vread(vpre, vl_prev);
@@ -393,6 +393,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                 __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
             }
         }
+        if (bar_mid) __syncthreads();
         if (__any(grow)) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -438,6 +439,12 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     //   step 2k+1 : V(k+1) registers -> LDS, fetch V(k+2); A reads V(k) half 0,   B reads K(k+1) half 0
     // A wave runs steps sb - 1 .. se of its own (the one before its first computes nothing it keeps except the scores of
     // the first; the one after its last adds the last step's product); all waves take part in the staging of every tile.
+    // 8 waves of 128-wide heads: the upper four meet a tile's barrier a block earlier in their own stream - inside the
+    // tile's first step, between its product with the values and its scores, whose key operands (and the values') are all
+    // in registers by then, so nothing they read later can be overwritten by a wave that is already past the barrier. The
+    // two waves of a SIMD then run half a step apart: one asks LDS for its value operands while the other is between
+    // reads (config 2: -1 % of the kernel's time)
+    const bool upper = D == 128 && PW == 8 && KPRE == 2 && VPRE == DT && w >= PW / 2;
     if (nt > 0) {
         Stage stk, stv;
         f4v sA[RT][2], sB[RT][2];
@@ -466,8 +473,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             // tile k: buffers 0
             stash_k(stk, 1);
             fetch(stk, kbase, k + 2);
-            step(sA, sB, 32 * KS, V0 + VBUF + 32 * VS, 64 * k, !(64 * k >= w_full_beg && 64 * k + 32 <= w_full_end));
-            __syncthreads();
+            step(sA, sB, 32 * KS, V0 + VBUF + 32 * VS, 64 * k, !(64 * k >= w_full_beg && 64 * k + 32 <= w_full_end), upper);
+            if (!upper) __syncthreads();
             stash_v(stv, 1);
             fetch(stv, vbase, k + 2);
             step(sB, sA, KBUF, V0, 64 * k + 32, !(64 * k + 32 >= w_full_beg && 64 * k + 64 <= w_full_end));
@@ -475,8 +482,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             // tile k + 1: buffers 1
             stash_k(stk, 0);
             fetch(stk, kbase, k + 3);
-            step(sA, sB, KBUF + 32 * KS, V0 + 32 * VS, 64 * k + 64, !(64 * k + 64 >= w_full_beg && 64 * k + 96 <= w_full_end));
-            __syncthreads();
+            step(sA, sB, KBUF + 32 * KS, V0 + 32 * VS, 64 * k + 64, !(64 * k + 64 >= w_full_beg && 64 * k + 96 <= w_full_end), upper);
+            if (!upper) __syncthreads();
             stash_v(stv, 0);
             fetch(stv, vbase, k + 3);
             step(sB, sA, 0, V0 + VBUF, 64 * k + 96, !(64 * k + 96 >= w_full_beg && 64 * k + 128 <= w_full_end));
