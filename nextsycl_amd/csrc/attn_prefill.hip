@@ -83,7 +83,22 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // the transposing reads of the values) meet no bank conflict - 16 bytes apart the key reads would, two ways
     constexpr int KS = D * 2 + 32, VS = D * 2 + 32;
     constexpr int KBUF = KT_TILE * KS, VBUF = KT_TILE * VS;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * (KBUF + VBUF)];
+    // DMA: 8 waves over 16-bit rows of 128 stage their tiles global -> LDS directly (global_load_lds_dwordx4: no register in
+    // between, no LDS write instruction, a tile requested two tiles ahead). The tiles are unpadded 256-byte rows, a row's
+    // 16-byte chunks exclusive-ored into place by its key (keys: chunk c of key r at position c ^ (r % 16); values:
+    // c ^ 2 (r % 8)) so that neither the operand reads of 16 keys' same chunk nor the transposing reads meet a bank
+    // conflict; three buffers a stream, each an array of its own so that the compiler can tell a transfer's target from
+    // the arrays being read (it waits for every transfer in flight before a read it cannot tell apart)
+    constexpr bool DMA = D == 128 && KT == 0 && PW == 8;
+    constexpr int TB = KT_TILE * 256;
+    constexpr int TBP = TB + 512;                                 // (two waves' output staging, 8448 B each, go through one array)
+    __shared__ __attribute__((aligned(16))) uint8_t lds[DMA ? 16 : 2 * (KBUF + VBUF)];
+    __shared__ __attribute__((aligned(1024))) uint8_t dk0[DMA ? TBP : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t dk1[DMA ? TBP : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t dk2[DMA ? TBP : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t dv0[DMA ? TBP : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t dv1[DMA ? TBP : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t dv2[DMA ? TBP : 16];
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -274,8 +289,75 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     auto stash_k = [&](const Stage& st, int buf) { put(st, (uint32_t) (buf * KBUF) + k_wr, KS); };
     auto stash_v = [&](const Stage& st, int buf) { put(st, V0 + (uint32_t) (buf * VBUF) + v_wr, VS); };
 
+    // DMA: a wave's two 1 KiB instructions a tile and stream: instruction j fills rows 4 (2 w + j) .. + 3 of the tile (16
+    // lanes a row: lane l position l % 16 of row 4 (2 w + j) + l / 16), so it fetches the chunk that belongs there. Whole
+    // tiles of an unwrapped cache: a wave-uniform tile address plus lane offsets worked out once; else the row is clamped
+    // into the pass's keys (masked anyway) and a ring's slot worked out, as the register path does
+    uint32_t koff[DMA ? 2 : 1], voff[DMA ? 2 : 1];
+    if constexpr (DMA) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int r = (w * 2 + j) * 4 + (lane >> 4), cp = lane & 15;
+            koff[j] = (uint32_t) (r * p.row_stride) + (uint32_t) ((cp ^ (r & 15)) << 4);
+            voff[j] = (uint32_t) (r * p.row_stride) + (uint32_t) ((cp ^ (2 * (r & 7))) << 4);
+        }
+    }
+    // (one transfer instruction: 64 lanes x 16 bytes from base + the lane's offset to 1 KiB of LDS at dst, wave-uniform.
+    // Written out so that the compiler's wait-count pass does not see a memory instruction that writes LDS - it would
+    // make every later LDS read wait for all earlier ones; the waits these transfers need are the tile barrier's)
+    auto dma16 = [&](const uint8_t* base_, uint32_t off, lds_u8* dst) __attribute__((always_inline)) {
+        const uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t) (uintptr_t) dst);
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"                   // (m0 is reserved: nothing of the compiler's lives in it across this)
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m), "v"(off), "s"(base_) : "memory", "m0");
+#pragma clang diagnostic pop
+    };
+    auto dma = [&](lds_u8* dst, const uint8_t* cache, int krel, auto which_c) __attribute__((always_inline)) {
+        constexpr bool VAL = decltype(which_c)::value;
+        if (krel >= plain0 && krel <= plain1) {
+            const uint8_t* sp = cache + (base + (int64_t) krel * KT_TILE) * p.row_stride;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                dma16(sp, VAL ? voff[j] : koff[j], dst + (w * 2 + j) * 1024);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int r = (w * 2 + j) * 4 + (lane >> 4), cp = lane & 15;
+                const int rel = std::min(std::max(krel * KT_TILE - kbeg32 + r, 0), kspan);
+                int64_t slot = kbeg_slot + rel;
+                if (p.wrap) {
+                    slot = slot >= p.cap ? slot - p.cap : slot;
+                    slot = slot >= p.cap ? slot - p.cap : slot;
+                }
+                const uint32_t off = (uint32_t) (slot * p.row_stride) + (uint32_t) ((VAL ? cp ^ (2 * (r & 7)) : cp ^ (r & 15)) << 4);
+                dma16(cache, off, dst + (w * 2 + j) * 1024);
+            }
+        }
+    };
+    // a tile's barrier. DMA: this wave's transfers of the tile about to be read are done when at most the two younger
+    // requests (2 instructions each) are still in flight, and every LDS read it has issued has returned (a wave past the
+    // barrier may request a transfer into a buffer this wave read from); a bare barrier then - no fence over the
+    // transfers still in flight
+    auto tile_barrier = [&]() __attribute__((always_inline)) {
+        if constexpr (DMA) {
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else {
+            __syncthreads();
+        }
+    };
     const uint32_t k_rd = (uint32_t) (n * KS + g4 * 16);                          // + kt2 * 16 * KS + kb * 64
     const uint32_t v_rd = (uint32_t) ((g4 * 4 + (n >> 2)) * VS + (n & 3) * 8);    // + dt * 32 (+ 16 * VS)
+    // (DMA tiles: where the lane's key-operand chunk kb and value-operand column tile dt sit in their swizzled rows)
+    uint32_t k_rd4[DMA ? KB : 1], v_rd8[DMA ? DT : 1];
+    if constexpr (DMA) {
+        const int kkv = g4 * 4 + (n >> 2);
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) k_rd4[kb] = (uint32_t) (n * 256 + (((kb * 4 + g4) ^ n) << 4));
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) v_rd8[dt] = (uint32_t) (kkv * 256 + ((dt ^ (kkv & 7)) << 5) + (((n & 3) >> 1) << 4) + (n & 1) * 8);
+    }
     s8v pb[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) pb[rt] = s8v{0, 0, 0, 0, 0, 0, 0, 0};
@@ -284,23 +366,32 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // latency passes under the other block's work instead of at the head of this one)
     constexpr int VPRE = D == 128 ? DT : 4;                       // value operands read ahead
     constexpr int KPRE = D == 128 ? 2 : 1;                        // 16-key halves whose key operands are read ahead
-    auto kread = [&](s8v (&ka)[KPRE][KB], uint32_t kl) {
+    // (kl / vl: where the 32-key half starts - a pointer into the tile buffers)
+    auto kread = [&](s8v (&ka)[KPRE][KB], const lds_u8* kl) __attribute__((always_inline)) {
 #pragma unroll
         for (int kt2 = 0; kt2 < KPRE; ++kt2)
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-                ka[kt2][kb] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + kl + k_rd + kt2 * 16 * KS + kb * 64);
+            for (int kb = 0; kb < KB; ++kb) {
+                if constexpr (DMA) ka[kt2][kb] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(kl + k_rd4[kb] + kt2 * 16 * 256);
+                else ka[kt2][kb] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(kl + k_rd + kt2 * 16 * KS + kb * 64);
+            }
     };
-    auto vread1 = [&](uint32_t vl, int dt) {
-        const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + vl + v_rd + dt * 32));
-        const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (L + vl + v_rd + dt * 32 + 16 * VS));
-        return s8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    auto vread1 = [&](const lds_u8* vl, int dt) __attribute__((always_inline)) {
+        if constexpr (DMA) {
+            const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (vl + v_rd8[dt]));
+            const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (vl + v_rd8[dt] + 16 * 256));
+            return s8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        } else {
+            const s4v lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (vl + v_rd + dt * 32));
+            const s4v hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s4v*) (vl + v_rd + dt * 32 + 16 * VS));
+            return s8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        }
     };
-    auto vread = [&](s8v (&va)[VPRE], uint32_t vl) {
+    auto vread = [&](s8v (&va)[VPRE], const lds_u8* vl) __attribute__((always_inline)) {
 #pragma unroll
         for (int dt = 0; dt < VPRE; ++dt) va[dt] = vread1(vl, dt);
     };
-    auto scores = [&](f4v (&s)[RT][2], uint32_t kl, const s8v (&kpre)[KPRE][KB]) {
+    auto scores = [&](f4v (&s)[RT][2], const lds_u8* kl, const s8v (&kpre)[KPRE][KB]) __attribute__((always_inline)) {
         if constexpr (KPRE == 2) {
             // every operand is in registers: the 2 RT chains of dependent products advance side by side
 #pragma unroll
@@ -316,7 +407,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                 s8v ka[KB];
 #pragma unroll
                 for (int kb = 0; kb < KB; ++kb)
-                    ka[kb] = kt2 == 0 ? kpre[0][kb] : *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(L + kl + k_rd + kt2 * 16 * KS + kb * 64);
+                    ka[kb] = kt2 == 0 ? kpre[0][kb] : *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(kl + k_rd + kt2 * 16 * KS + kb * 64);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
                     f4v acc = mfma16<BF>(ka[0], qreg[rt][0], f4v{0.0f, 0.0f, 0.0f, 0.0f});
@@ -330,7 +421,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // O^T += V^T P^T of one 32-key half (LDS byte offset vl) with the weights in pb
     constexpr short ONE16 = BF ? (short) 0x3F80 : (short) 0x3C00;
     const s8v ones = {ONE16, ONE16, ONE16, ONE16, ONE16, ONE16, ONE16, ONE16};
-    auto weigh = [&](uint32_t vl, const s8v (&vpre)[VPRE]) {
+    auto weigh = [&](const lds_u8* vl, const s8v (&vpre)[VPRE]) __attribute__((always_inline)) {
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) l4[rt] = mfma16<BF>(ones, pb[rt], l4[rt]);
 #pragma unroll
@@ -351,7 +442,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // Every LDS operand of a block is requested a block ahead (vread at the step's start, kread at the head of A), and
     // sched_group_barrier deals the vector instructions out between the matrix instructions.
     // The mask is applied under a wave-uniform branch: steps no row's causal or window edge crosses pay no comparison.
-    auto step = [&](f4v (&sc)[RT][2], f4v (&sn)[RT][2], uint32_t kl_next, uint32_t vl_prev, int j0, bool masked, bool bar_mid = false) {
+    auto step = [&](f4v (&sc)[RT][2], f4v (&sn)[RT][2], const lds_u8* kl_next, const lds_u8* vl_prev, int j0, bool masked, bool bar_mid = false) __attribute__((always_inline)) {
         float a[RT][8], amax[RT];
         s8v vpre[VPRE], kpre[KPRE][KB];
         vread(vpre, vl_prev);
@@ -393,7 +484,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                 __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
             }
         }
-        if (bar_mid) __syncthreads();
+        if (bar_mid) tile_barrier();
         if (__any(grow)) {
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt) {
@@ -446,12 +537,61 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // reads (config 2: -1 % of the kernel's time)
     const bool upper = D == 128 && PW == 8 && KPRE == 2 && VPRE == DT && w >= PW / 2;
     if (nt > 0) {
-        Stage stk, stv;
         f4v sA[RT][2], sB[RT][2];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int kt2 = 0; kt2 < 2; ++kt2) sA[rt][kt2] = sB[rt][kt2] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+      if constexpr (DMA) {
+        // ---- three buffers a stream, tile k in buffer k % 3:
+        //   step 2k   : request K(k+2);  A reads V(k-1) half 1, B's operands K(k) half 1
+        //   barrier (the upper waves: inside step 2k, see above)
+        //   step 2k+1 : request V(k+2);  A reads V(k) half 0,   B's operands K(k+1) half 0
+        const std::false_type KEYS;
+        const std::true_type VALUES;
+        lds_u8* const K0 = (lds_u8*) dk0; lds_u8* const K1 = (lds_u8*) dk1; lds_u8* const K2 = (lds_u8*) dk2;
+        lds_u8* const W0 = (lds_u8*) dv0; lds_u8* const W1 = (lds_u8*) dv1; lds_u8* const W2 = (lds_u8*) dv2;
+        dma(K0, kbase, 0, KEYS);
+        dma(W0, vbase, 0, VALUES);
+        dma(K1, kbase, 1, KEYS);
+        dma(W1, vbase, 1, VALUES);
+        {   // the V buffer step 0 "adds" with zero weights must hold numbers
+            const u4v z = {0u, 0u, 0u, 0u};
+            for (uint32_t at = (uint32_t) tid * 16; at < (uint32_t) TB; at += PW * 64 * 16)
+                *reinterpret_cast<__attribute__((address_space(3))) u4v*>(W2 + at) = z;
+        }
+        tile_barrier();
+        {
+            s8v kpre[KPRE][KB];
+            kread(kpre, K0);
+            scores(sA, K0, kpre);
+        }
+        // one tile: its two steps; kb / vb: the tile's own buffers, kn: the next tile's keys, vp: the tile before's values,
+        // k2 / v2: where the tile after the next goes
+        auto tile = [&](int k, lds_u8* kb, lds_u8* vb, lds_u8* kn, lds_u8* vp, lds_u8* k2, lds_u8* v2) __attribute__((always_inline)) {
+            dma(k2, kbase, k + 2, KEYS);
+            step(sA, sB, kb + 32 * 256, vp + 32 * 256, 64 * k, !(64 * k >= w_full_beg && 64 * k + 32 <= w_full_end), upper);
+            if (!upper) tile_barrier();
+            dma(v2, vbase, k + 2, VALUES);
+            step(sB, sA, kn, vb, 64 * k + 32, !(64 * k + 32 >= w_full_beg && 64 * k + 64 <= w_full_end));
+        };
+        for (int k = 0; k < nt; k += 3) {
+            tile(k, K0, W0, K1, W2, K2, W2);
+            if (k + 1 >= nt) break;
+            tile(k + 1, K1, W1, K2, W0, K0, W0);
+            if (k + 2 >= nt) break;
+            tile(k + 2, K2, W2, K0, W1, K1, W1);
+        }
+        // the last step's product
+        {
+            s8v vpre[VPRE];
+            lds_u8* const vl = ((nt - 1) % 3 == 0 ? W0 : (nt - 1) % 3 == 1 ? W1 : W2) + 32 * 256;
+            vread(vpre, vl);
+            weigh(vl, vpre);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // (transfers past the last tile land in buffers the output goes through)
+      } else {
+        Stage stk, stv;
         fetch(stk, kbase, 0);
         fetch(stv, vbase, 0);
         {   // the V buffer step 0 "adds" with zero weights must hold numbers
@@ -466,50 +606,54 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         __syncthreads();
         {
             s8v kpre[KPRE][KB];
-            kread(kpre, 0);
-            scores(sA, 0, kpre);
+            kread(kpre, L);
+            scores(sA, L, kpre);
         }
         for (int k = 0; k < nt; k += 2) {
             // tile k: buffers 0
             stash_k(stk, 1);
             fetch(stk, kbase, k + 2);
-            step(sA, sB, 32 * KS, V0 + VBUF + 32 * VS, 64 * k, !(64 * k >= w_full_beg && 64 * k + 32 <= w_full_end), upper);
+            step(sA, sB, L + 32 * KS, L + V0 + VBUF + 32 * VS, 64 * k, !(64 * k >= w_full_beg && 64 * k + 32 <= w_full_end), upper);
             if (!upper) __syncthreads();
             stash_v(stv, 1);
             fetch(stv, vbase, k + 2);
-            step(sB, sA, KBUF, V0, 64 * k + 32, !(64 * k + 32 >= w_full_beg && 64 * k + 64 <= w_full_end));
+            step(sB, sA, L + KBUF, L + V0, 64 * k + 32, !(64 * k + 32 >= w_full_beg && 64 * k + 64 <= w_full_end));
             if (k + 1 >= nt) break;
             // tile k + 1: buffers 1
             stash_k(stk, 0);
             fetch(stk, kbase, k + 3);
-            step(sA, sB, KBUF + 32 * KS, V0 + 32 * VS, 64 * k + 64, !(64 * k + 64 >= w_full_beg && 64 * k + 96 <= w_full_end), upper);
+            step(sA, sB, L + KBUF + 32 * KS, L + V0 + 32 * VS, 64 * k + 64, !(64 * k + 64 >= w_full_beg && 64 * k + 96 <= w_full_end), upper);
             if (!upper) __syncthreads();
             stash_v(stv, 0);
             fetch(stv, vbase, k + 3);
-            step(sB, sA, 0, V0 + VBUF, 64 * k + 96, !(64 * k + 96 >= w_full_beg && 64 * k + 128 <= w_full_end));
+            step(sB, sA, L, L + V0 + VBUF, 64 * k + 96, !(64 * k + 96 >= w_full_beg && 64 * k + 128 <= w_full_end));
         }
         // the last step's product
         {
             s8v vpre[VPRE];
-            vread(vpre, V0 + (uint32_t) ((nt - 1) & 1) * VBUF + 32 * VS);
-            weigh(V0 + (uint32_t) ((nt - 1) & 1) * VBUF + 32 * VS, vpre);
+            lds_u8* const vl = L + V0 + (uint32_t) ((nt - 1) & 1) * VBUF + 32 * VS;
+            vread(vpre, vl);
+            weigh(vl, vpre);
         }
+      }
     }
 
     // ---- out = O / l. A lane holds dims 16 dt + 4 g4 .. + 3 of its rows: the wave's 32 x D block goes through LDS (the
     // tile buffers, free now) so that it leaves as whole rows, 16 bytes a lane and 4 (float32: 2) rows an instruction
     __syncthreads();                                              // every wave is done with the tiles
+    // (DMA: the tile buffers are arrays of their own; two waves' staging regions go through each of the first four)
+    lds_u8* const OB = DMA ? ((w & 3) == 0 ? (lds_u8*) dk0 : (w & 3) == 1 ? (lds_u8*) dk1 : (w & 3) == 2 ? (lds_u8*) dk2 : (lds_u8*) dv0) + (w >> 2) * 16 * (D * 4 + 16)
+                           : L + w * 16 * (D * 4 + 16);
     if (p.ns > 1) {
         // ---- a key split's partial: the rows' unnormalized sums as float32, then (m, l) - D + 2 floats a (row, head, split),
         // rows 8 bytes aligned: 8-byte pieces, 8 rows an instruction
         const uint32_t rowp = D * 4 + 16;
-        const uint32_t ob = (uint32_t) w * 16 * rowp;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             const float lsum = l4[rt][0];
-            const uint32_t at = ob + (uint32_t) n * rowp + (uint32_t) (g4 * 16);
+            const uint32_t at = (uint32_t) n * rowp + (uint32_t) (g4 * 16);
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<__attribute__((address_space(3))) f4v*>(L + at + dt * 64) = o[rt][dt];
+            for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<__attribute__((address_space(3))) f4v*>(OB + at + dt * 64) = o[rt][dt];
             const int row = r0 + w * WROWS + rt * 16 + n;
             if (g4 == 0 && row < p.T) {
                 float* pr = p.part + (((int64_t) row * p.Hq + hq) * p.ns + split) * (D + 2);
@@ -519,7 +663,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                 const int rl_ = c / (D / 2), piece = c % (D / 2), prow = r0 + w * WROWS + rt * 16 + rl_;
                 if (prow < p.T) {
                     typedef uint32_t u2v __attribute__((ext_vector_type(2)));
-                    const u2v x = *reinterpret_cast<const __attribute__((address_space(3))) u2v*>(L + ob + (uint32_t) rl_ * rowp + (uint32_t) piece * 8);
+                    const u2v x = *reinterpret_cast<const __attribute__((address_space(3))) u2v*>(OB + (uint32_t) rl_ * rowp + (uint32_t) piece * 8);
                     *reinterpret_cast<u2v*>(p.part + (((int64_t) prow * p.Hq + hq) * p.ns + split) * (D + 2) + piece * 2) = x;
                 }
             }
@@ -529,32 +673,31 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     {
         const int esz = p.qt == 0 ? 4 : 2;
         const uint32_t rowb = (uint32_t) (D * esz), rowp = rowb + 16;    // bytes a row, padded in LDS
-        const uint32_t ob = (uint32_t) w * 16 * (D * 4 + 16);       // a wave's own region: one row tile at a time
         const int ppr = (int) rowb / 16;                          // 16-byte pieces a row
         uint8_t* const orow = reinterpret_cast<uint8_t*>(p.out) + (int64_t) hq * rowb;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
             const float lsum = l4[rt][0];
             const float inv = lsum > 0.0f ? 1.0f / lsum : 0.0f;
-            const uint32_t at = ob + (uint32_t) n * rowp + (uint32_t) (g4 * 4 * esz);
+            const uint32_t at = (uint32_t) n * rowp + (uint32_t) (g4 * 4 * esz);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 const f4v v = o[rt][dt] * inv;
                 if (p.qt == 0) {
-                    *reinterpret_cast<__attribute__((address_space(3))) f4v*>(L + at + dt * 64) = v;
+                    *reinterpret_cast<__attribute__((address_space(3))) f4v*>(OB + at + dt * 64) = v;
                 } else {
                     typedef uint16_t us4v __attribute__((ext_vector_type(4)));
                     us4v h;
                     if (p.qt == 1) h = us4v{f32_to_f16(v[0]), f32_to_f16(v[1]), f32_to_f16(v[2]), f32_to_f16(v[3])};
                     else h = us4v{f32_to_bf16(v[0]), f32_to_bf16(v[1]), f32_to_bf16(v[2]), f32_to_bf16(v[3])};
-                    *reinterpret_cast<__attribute__((address_space(3))) us4v*>(L + at + dt * 32) = h;
+                    *reinterpret_cast<__attribute__((address_space(3))) us4v*>(OB + at + dt * 32) = h;
                 }
             }
             // the wave reads back its own block only: no barrier, the LDS queue keeps a wave's accesses in order
             for (int c = lane; c < 16 * ppr; c += 64) {
                 const int rl_ = c / ppr, piece = c % ppr, row = r0 + w * WROWS + rt * 16 + rl_;
                 if (row < p.T) {
-                    const u4v x = *reinterpret_cast<const __attribute__((address_space(3))) u4v*>(L + ob + (uint32_t) rl_ * rowp + (uint32_t) piece * 16);
+                    const u4v x = *reinterpret_cast<const __attribute__((address_space(3))) u4v*>(OB + (uint32_t) rl_ * rowp + (uint32_t) piece * 16);
                     *reinterpret_cast<u4v*>(orow + (int64_t) row * p.Hq * rowb + piece * 16) = x;
                 }
             }
