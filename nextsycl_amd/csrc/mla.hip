@@ -40,10 +40,11 @@ namespace {
 
 constexpr int MTILE = 32, ML = 512;
 // waves a work-group (16 rows each): 8 = 128-row groups; 4 = 64-row groups where a group (the pass's rows, or one row's
-// heads under a selection) has at most 128 rows and the pass at most 40960 cells - a decode step of 128 heads then runs
+// heads under a selection) has at most 128 rows and the pass at most 131072 cells - a decode step of 128 heads then runs
 // two groups over half as many cell splits: half the query loads and half the partials, which outweighs a tile loop
-// twice as long up to about that length (measured: 40.6 against 43.6 us at 32768 cells, 56.9 against 52.6 at 65536)
-constexpr int mla_waves(int64_t group_rows, int64_t cells) { return group_rows <= 128 && cells <= 40960 ? 4 : 8; }
+// twice as long up to about that length (kernel + merge between events, 4 against 8 waves: 35.5 / 42.9 us at 32768
+// cells, 46.3 / 51.9 at 65536, 67.4 / 69.1 at 131072)
+constexpr int mla_waves(int64_t group_rows, int64_t cells) { return group_rows <= 128 && cells <= 131072 ? 4 : 8; }
 // a split's partial of a row: u_s[512] = O_s / l_s as halfs (the split's own normalized result: bounded by the cache's
 // values, so half holds it; a quarter of the float32 form's bytes go to m and l), then m (log2 units), l, 2 of padding
 constexpr int MLA_PASS_MAX = 256;    // rows of a prompt a pass of the latent kernel takes at most

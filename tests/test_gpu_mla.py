@@ -44,6 +44,19 @@ def test_latent_decode_small(ops, T, H, R, pos0, qt):
         _close(orc.mla_decode_u(qf, cache, T, H, pos0, scale), ref, "the restatement itself")
 
 
+@pytest.mark.parametrize("T,H,pos0,qt", [(1, 16, 49999, F32), (2, 32, 100000, F16), (1, 16, 131071, F16), (1, 16, 131072, F32)])
+def test_latent_decode_long_contexts(ops, T, H, pos0, qt):
+    """One or two rows behind long contexts: the passes either side of the cell count at which the kernel's 64-row form
+    gives way to the 128-row one, many tiles a split."""
+    n = pos0 + T
+    cache = orc.f2h(orc.randn(21, (n, 576), 0.5))
+    qa = orc.randn(22, (T, H, 576))
+    scale = 1.0 / np.sqrt(192.0)
+    qd, qf = (qa, qa) if qt == F32 else (orc.f2h(qa), orc.h2f(orc.f2h(qa)))
+    got = _latent(ops, qt, qd, cache, T, H, 64, pos0, scale)
+    _close(got, orc.mla_f64(qf, cache, T, H, pos0, scale, 512, 64), "latent decode vs float64 closed form")
+
+
 def _random_cases(n, seed):
     rng = np.random.default_rng(seed)
     out = []
