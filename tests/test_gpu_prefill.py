@@ -160,6 +160,43 @@ def test_prefill_ring(ops):
     check_close(got, ref, F32, "ring prefill")
 
 
+@pytest.mark.parametrize("T,Hq,Hkv,cap,win,p0,kt,qt", [
+    (150, 4, 2, 512, 300, 900, 0, F32),          # a wrapped ring under a window
+    (260, 2, 1, 640, 350, 1500, 3, BF16),        # the window's first key mid-tile, the ring's seam inside the pass's keys
+    (40, 2, 2, 0, 0, 0, 0, F16),                 # one tile
+    (100, 2, 1, 0, 0, 28, 3, BF16),              # two tiles
+    (130, 2, 1, 0, 0, 62, 0, F32),               # three
+    (200, 2, 1, 0, 0, 56, 0, F16),               # four, a pass that starts mid-tile
+    (256, 2, 1, 0, 0, 1024, 3, F32),             # whole tiles only
+    (257, 2, 1, 0, 100, 777, 0, BF16),           # a row block of one row
+])
+def test_prefill_tiles_sent_straight_to_lds(ops, tune, T, Hq, Hkv, cap, win, p0, kt, qt):
+    """The 8-wave form over 16-bit rows of 128 moves its tiles global -> LDS without registers, three buffers a stream:
+    passes of one to many tiles (every buffer rotation), rings with their seam among the pass's keys, windows whose edge
+    falls inside a tile - against the float64 closed form, and bit for bit against the 4-wave form's register staging."""
+    D = 128
+    n = p0 + T
+    if cap:
+        k = orc.randn(31, (n, Hkv * D))
+        v = orc.randn(32, (n, Hkv * D))
+        kc = np.zeros((Hkv, cap, 2 * D), np.uint8)
+        vc = np.zeros((Hkv, cap, 2 * D), np.uint8)
+        for s0 in range(0, n, 128):
+            e = min(n, s0 + 128)
+            orc.kv_store(kt, k[s0:e], v[s0:e], Hkv, D, cap, s0, kc, vc, ring=True)
+    else:
+        cap = n + 3
+        kc, vc = make_kv(kt, Hkv, D, cap, n, cfg=2)
+    qd, qf = make_q(qt, T, Hq, D, cfg=1)
+    tune(TUNE_PREFILL_WAVES, 8)
+    got8, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    tune(TUNE_PREFILL_WAVES, 4)
+    got4, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got8, ref, qt, "prefill, tiles straight to LDS", kt=kt)
+    assert np.array_equal(got8, got4)
+
+
 def test_prompt_rows_agree_with_decode_rows(ops):
     """The reference's --prompt-decode check (cli/nextsycl/src/main.rs:869-917): a prompt pass's row t against the
     decode pass at position p0 + t - two kernels, one result within the path's tolerance."""
