@@ -148,6 +148,23 @@ int ns_mg_attn(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_
 int64_t ns_mg_attn_block_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win);
 int ns_mg_attn_block(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
                      int64_t win, float* out, float* scratch);
+/* ricursive's attention: rows at positions p0.. against a half cache that is a ring of R rows a head (position p in slot
+ * p % R); a row at position p sees the keys p - W + 1 .. p (W 0: all of 0 .. p); scale 1 / sqrt(D). D 128, 1, 2, 4, 6, 8
+ * or 10 query heads a key head; the keys of a window must still be in the ring (R >= W + T - 1). Replaces:
+ * kernels/llm/ricursive/rc.h:22-32 (rc.cpp:182-225), bound at llm/ricursive/src/ffi.rs:70-71 */
+int ns_rc_kv_store(ns_gpu* g, const float* k, int64_t ks, const float* v, int64_t vs, int64_t T, int64_t Hkv, int64_t D, int64_t R, int64_t p0,
+                   void* kc, void* vc);
+int64_t ns_rc_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t W, int64_t p0);
+int ns_rc_attn(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t R,
+               int64_t W, int64_t p0, float* out, float* scratch);
+/* nemotron-h's attention layers: causal, no positions, scale 1 / sqrt(D), half cache [Hkv][cap][D]; D 128, query heads
+ * a multiple of 8 a key head. Replaces: kernels/llm/nemotronh/nh.h:36-44 (nh.cpp:551-588), bound at
+ * llm/nemotronh/src/ffi.rs:91-92 */
+int ns_nh_kv_store(ns_gpu* g, const float* k, int64_t ks, const float* v, int64_t vs, int64_t T, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
+                   void* kc, void* vc);
+int64_t ns_nh_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0);
+int ns_nh_attn(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap,
+               int64_t p0, float* out, float* scratch);
 /* The weights one decode row q [Hq][D] (float32, normed and rotated) gives the n keys of a head-major cache of form kt,
  * reduced over the heads and ADDED to out [n]: their mean (mode 0) or their largest (mode 1); softmax in float32 with
  * scale 1 / sqrt(D). scratch: 2 Hq floats (each head's largest score and sum). The scores are kept [Hq][n] in memory

@@ -21,6 +21,10 @@ int ns_q35_qk_norm_rope_pos(ns_gpu* g, const float* src, int64_t ss, int64_t hs,
 /* kernels/llm/qwen35/q35.h:58-60, q35.cpp:256-279. As ns_q35_qk_norm_rope without the norm. */
 int ns_q35_rope(ns_gpu* g, const float* src, int64_t ss, int64_t hs, float* dst, int64_t ds, int64_t T, int64_t H, int64_t D, int64_t n_rot,
                 float theta, int64_t p0);
+/* kernels/llm/ricursive/rc.h:17-21, rc.cpp:148-181. As ns_q35_qk_norm_rope with the rotation over all D features
+ * (rope != 0) or none (rope 0). */
+int ns_rc_qk_norm_rope(ns_gpu* g, const float* src, int64_t ss, int64_t hs, float* dst, int64_t ds, int64_t T, int64_t H, int64_t D,
+                       const float* w, float eps, int rope, float theta, int64_t p0);
 /* kernels/llm/museglimmer/mg.h:19-20, mg.cpp:157-190. y[t * ys + h * D ..] = RMS norm of x[t * xs + h * D ..] (weight w,
  * eps), then rotary positions over all D: rope 0 none, 1 adjacent pairs (2i, 2i + 1), 2 halves (i, i + D / 2); angle
  * (p0 + t) * theta^(-2 i / D). y may be x. */

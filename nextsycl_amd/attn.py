@@ -60,6 +60,12 @@ ATTN_H = {
     "ns_mg_attn": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, i32, P, P]),
     "ns_mg_attn_block_scratch": (i64, [i64, i64, i64, i64, i64, i64]),
     "ns_mg_attn_block": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_rc_kv_store": (i32, [P, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_rc_attn_scratch": (i64, [i64, i64, i64, i64, i64, i64]),
+    "ns_rc_attn": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_nh_kv_store": (i32, [P, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_nh_attn_scratch": (i64, [i64, i64, i64, i64, i64]),
+    "ns_nh_attn": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P, P]),
     "ns_q35_attn_probs": (i32, [P, i32, P, P, i64, i64, i64, i64, i64, i32, P, P]),
     "ns_mm3s_attend_supported": (i32, [i64, i64, i64]),
     "ns_mm3s_attend": (i32, [P, P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
@@ -96,6 +102,7 @@ MLA_H = {
 PRE_H = {
     "ns_q35_qk_norm_rope": (i32, [P, P, i64, i64, P, i64, i64, i64, i64, P, f32, i64, f32, i64]),
     "ns_q35_qk_norm_rope_pos": (i32, [P, P, i64, i64, P, i64, i64, i64, i64, P, f32, i64, f32, P, i64, i64, i64]),
+    "ns_rc_qk_norm_rope": (i32, [P, P, i64, i64, P, i64, i64, i64, i64, P, f32, i32, f32, i64]),
     "ns_q35_rope": (i32, [P, P, i64, i64, P, i64, i64, i64, i64, i64, f32, i64]),
     "ns_mg_qk_norm_rope": (i32, [P, P, i64, P, i64, i64, i64, i64, P, f32, i32, f32, i64]),
     "ns_llm_minimaxm3_rope": (i32, [P, P, i64, i64, i64, i64, i64, i64, f32]),
@@ -201,6 +208,23 @@ class Ops:
         _need(vc, self.cache_bytes(0, Hkv, cap, D), "kv_store value cache")
         self.ok(self.k.mg_kv_store(self.raw(), k.ptr, v.ptr, T, Hkv, D, cap, p0, kc.ptr, vc.ptr), "kv_store")
 
+    def rc_kv_store(self, k, ks, v, vs, T, Hkv, D, R, p0, kc, vc):
+        """ns_rc_kv_store: half rows into a ring of R rows a head (position p in slot p % R)."""
+        if T > 0:
+            _need(k, ((T - 1) * ks + Hkv * D) * 4, "kv_store k")
+            _need(v, ((T - 1) * vs + Hkv * D) * 4, "kv_store v")
+        _need(kc, self.cache_bytes(0, Hkv, R, D), "kv_store key cache")
+        _need(vc, self.cache_bytes(0, Hkv, R, D), "kv_store value cache")
+        self.ok(self.k.rc_kv_store(self.raw(), k.ptr, ks, v.ptr, vs, T, Hkv, D, R, p0, kc.ptr, vc.ptr), "kv_store")
+
+    def nh_kv_store(self, k, ks, v, vs, T, Hkv, D, cap, p0, kc, vc):
+        if T > 0:
+            _need(k, ((T - 1) * ks + Hkv * D) * 4, "kv_store k")
+            _need(v, ((T - 1) * vs + Hkv * D) * 4, "kv_store v")
+        _need(kc, self.cache_bytes(0, Hkv, cap, D), "kv_store key cache")
+        _need(vc, self.cache_bytes(0, Hkv, cap, D), "kv_store value cache")
+        self.ok(self.k.nh_kv_store(self.raw(), k.ptr, ks, v.ptr, vs, T, Hkv, D, cap, p0, kc.ptr, vc.ptr), "kv_store")
+
     def kv_dequant(self, kt, rows, n, D, out):
         rb = kv_row_bytes(kt, D)
         _need(rows, n * rb, "kv_dequant rows")
@@ -294,6 +318,30 @@ class Ops:
         if scratch is not None:
             _need(scratch, self.k.mg_attn_scratch(T, Hq, Hkv, D, p0, win, int(causal)) * 4, "attention scratch")
         self.ok(self.k.mg_attn(self.raw(), q.ptr, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, int(causal), out.ptr,
+                               scratch.ptr if scratch is not None else None), "attention")
+
+    def rc_attn(self, q, qs, kc, vc, T, Hq, Hkv, D, R, W, p0, out, scratch):
+        """ns_rc_attn: ricursive's attention over a ring of R rows a head, window W (0: none)."""
+        if T > 0:
+            _need(q, ((T - 1) * qs + Hq * D) * 4, "attention q")
+            _need(out, T * Hq * D * 4, "attention out")
+        _need(kc, self.cache_bytes(0, Hkv, R, D), "attention key cache")
+        _need(vc, self.cache_bytes(0, Hkv, R, D), "attention value cache")
+        if scratch is not None:
+            _need(scratch, self.k.rc_attn_scratch(T, Hq, Hkv, D, W, p0) * 4, "attention scratch")
+        self.ok(self.k.rc_attn(self.raw(), q.ptr, qs, kc.ptr, vc.ptr, T, Hq, Hkv, D, R, W, p0, out.ptr,
+                               scratch.ptr if scratch is not None else None), "attention")
+
+    def nh_attn(self, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, out, scratch):
+        """ns_nh_attn: nemotron-h's attention layers (causal, no window)."""
+        if T > 0:
+            _need(q, ((T - 1) * qs + Hq * D) * 4, "attention q")
+            _need(out, T * Hq * D * 4, "attention out")
+        _need(kc, self.cache_bytes(0, Hkv, cap, D), "attention key cache")
+        _need(vc, self.cache_bytes(0, Hkv, cap, D), "attention value cache")
+        if scratch is not None:
+            _need(scratch, self.k.nh_attn_scratch(T, Hq, Hkv, D, p0) * 4, "attention scratch")
+        self.ok(self.k.nh_attn(self.raw(), q.ptr, qs, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, out.ptr,
                                scratch.ptr if scratch is not None else None), "attention")
 
     def mg_attn_block(self, q, kc, vc, T, Hq, Hkv, D, cap, p0, win, out, scratch):

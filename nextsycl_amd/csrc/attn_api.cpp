@@ -85,6 +85,38 @@ int ns_mg_attn_block(ns_gpu* g, const float* q, const void* kc, const void* vc, 
     return ns_mg_attn(g, q, kc, vc, T, Hq, Hkv, D, cap, p0, win, 0, out, scratch);
 }
 
+// ---- ricursive and nemotron-h: the same two kernels under their engines' names -----------------------------------------
+
+int64_t ns_rc_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t W, int64_t p0) {
+    return T >= 1 && T <= DECODE_ROWS ? ns_attn_decode_scratch(T, Hq, Hkv, D, p0, W) : 0;
+}
+
+int ns_rc_attn(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t R,
+               int64_t W, int64_t p0, float* out, float* scratch) {
+    if (T <= 0) return 0;
+    if (W > 0 && R < W + T - 1 && p0 + T > R) return ns_fail("ns_rc_attn: the ring is smaller than the window and the rows");
+    if (W == 0 && p0 + T > R) return ns_fail("ns_rc_attn: past the cache's capacity");
+    if (D != 128) return ns_fail("ns_rc_attn: heads of 128");
+    const int64_t G = Hkv > 0 && Hq % Hkv == 0 ? Hq / Hkv : 0;
+    if (G != 1 && G != 2 && G != 4 && G != 6 && G != 8 && G != 10) return ns_fail("ns_rc_attn: 1, 2, 4, 6, 8 or 10 query heads a key head");
+    if (T <= DECODE_ROWS) return ns_attn_decode_any(g, "ns_rc_attn", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, R, p0, W, DecodeExtra{}, 0.0f, out, scratch);
+    return ns_attn_prompt_any(g, "ns_rc_attn", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, R, p0, W, 1, -1, 0.0f, out);
+}
+
+int64_t ns_nh_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0) {
+    return T >= 1 && T <= DECODE_ROWS ? ns_attn_decode_scratch(T, Hq, Hkv, D, p0, 0) : 0;
+}
+
+int ns_nh_attn(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap,
+               int64_t p0, float* out, float* scratch) {
+    if (T <= 0) return 0;
+    if (p0 + T > cap) return ns_fail("ns_nh_attn: past the cache's capacity");
+    if (D != 128 || Hkv <= 0 || Hq % 8 != 0 || Hq % Hkv != 0 || (Hq / Hkv) % 8 != 0)
+        return ns_fail("ns_nh_attn: head 128, query heads a multiple of 8 a key head");
+    if (T <= DECODE_ROWS) return ns_attn_decode_any(g, "ns_nh_attn", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, DecodeExtra{}, 0.0f, out, scratch);
+    return ns_attn_prompt_any(g, "ns_nh_attn", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, 1, -1, 0.0f, out);
+}
+
 // ---- MiniMax-M3: position-major cache, explicit scale, no scratch argument ------------------------------------------------
 
 // One body for the dense / block-list passes of every MiniMax entry point. part NULL: the partials of a pass of up to 16

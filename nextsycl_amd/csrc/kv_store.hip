@@ -160,6 +160,20 @@ int ns_mg_kv_store(ns_gpu* g, const float* k, const float* v, int64_t T, int64_t
     return ns_attn_kv_store(g, 0, 1, k, Hkv * D, v, Hkv * D, T, Hkv, D, cap, p0, kc, vc);
 }
 
+int ns_rc_kv_store(ns_gpu* g, const float* k, int64_t ks, const float* v, int64_t vs, int64_t T, int64_t Hkv, int64_t D, int64_t R, int64_t p0,
+                   void* kc, void* vc) {
+    if (T <= 0) return 0;
+    if (T > R) return ns_fail("ns_rc_kv_store: more rows than the ring holds");
+    return ns_attn_kv_store(g, 0, 1, k, ks, v, vs, T, Hkv, D, R, p0, kc, vc);
+}
+
+int ns_nh_kv_store(ns_gpu* g, const float* k, int64_t ks, const float* v, int64_t vs, int64_t T, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
+                   void* kc, void* vc) {
+    if (T <= 0) return 0;
+    if (p0 + T > cap) return ns_fail("ns_nh_kv_store: past the cache's capacity");
+    return ns_attn_kv_store(g, 0, 0, k, ks, v, vs, T, Hkv, D, cap, p0, kc, vc);
+}
+
 int ns_attn_kv_dequant(ns_gpu* g, int kt, const void* rows, int64_t n, int64_t D, int64_t stride, float* out) {
     NS_TRY
     if (n <= 0) return 0;

@@ -436,6 +436,14 @@ int ns_q35_qk_norm_rope(ns_gpu* g, const float* src, int64_t ss, int64_t hs, flo
     NS_CATCH
 }
 
+int ns_rc_qk_norm_rope(ns_gpu* g, const float* src, int64_t ss, int64_t hs, float* dst, int64_t ds, int64_t T, int64_t H, int64_t D,
+                       const float* w, float eps, int rope, float theta, int64_t p0) {
+    if (T <= 0) return 0;
+    if (D % 16 != 0 || D > 512) return ns_fail("ns_rc_qk_norm_rope: D a multiple of 16");
+    // (rotate-half over all D features, or none: the qwen35 form with n_rot = D or 0, the same arithmetic)
+    return ns_q35_qk_norm_rope(g, src, ss, hs, dst, ds, T, H, D, w, eps, rope ? D : 0, theta, p0);
+}
+
 int ns_q35_rope(ns_gpu* g, const float* src, int64_t ss, int64_t hs, float* dst, int64_t ds, int64_t T, int64_t H, int64_t D, int64_t n_rot,
                 float theta, int64_t p0) {
     NS_TRY

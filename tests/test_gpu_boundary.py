@@ -266,3 +266,115 @@ def test_glm_latent_width_256(ops):
     big = DevBuf(g, 100001 * 2 * L)
     with pytest.raises(Error, match="widened in the library's scratch"):
         ops.mla_attend(DevBuf(g, 8 * L * 4), big, DevBuf(g, 8 * L * 4), 1, 8, L, 100000, scale)
+
+
+# ricursive's engine (ns_rc_*: a ring of R rows a head, a window W, 10 query heads a key head among its ratios) and
+# nemotron-h's attention layers (ns_nh_*: plain causal, 8 query heads a key head)
+RC = [
+    # T, Hq, Hkv, R, W, p0
+    (1, 10, 1, 4096, 0, 3000),          # one decode row, all keys, the cache not yet a ring
+    (1, 20, 2, 1024, 1000, 5000),       # a wrapped ring under a window
+    (8, 10, 1, 600, 512, 2047),         # verify rows; the ring's seam inside the window
+    (16, 12, 2, 2048, 0, 100),          # 6 query heads a key head
+    (40, 10, 1, 700, 600, 1500),        # a prompt chunk through the ring
+    (300, 8, 4, 400, 64, 900),          # more rows than the window: R >= W + T - 1
+]
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,R,W,p0", RC)
+def test_ricursive_entry_points(ops, T, Hq, Hkv, R, W, p0):
+    """ns_rc_kv_store writes the ring the oracle's store writes, byte for byte; ns_rc_attn over it against the float64
+    closed form (kernels/llm/ricursive/rc.cpp:182-225)."""
+    D = 128
+    g = ops.gpu
+    n = p0 + T
+    k, v = orc.randn(41, (n, Hkv * D)), orc.randn(42, (n, Hkv * D))
+    kc = np.zeros((Hkv, R, 2 * D), np.uint8)
+    vc = np.zeros((Hkv, R, 2 * D), np.uint8)
+    kcb, vcb = DevBuf.of(g, kc), DevBuf.of(g, vc)
+    step = min(R, 96)
+    for s in range(0, n, step):
+        e = min(n, s + step)
+        orc.kv_store(0, k[s:e], v[s:e], Hkv, D, R, s, kc=kc, vc=vc, ring=True)
+        ops.rc_kv_store(DevBuf.of(g, k[s:e]), Hkv * D, DevBuf.of(g, v[s:e]), Hkv * D, e - s, Hkv, D, R, s, kcb, vcb)
+    assert np.array_equal(kcb.read(np.uint8).reshape(kc.shape), kc) and np.array_equal(vcb.read(np.uint8).reshape(vc.shape), vc)
+    qd, qf = make_q(F32, T, Hq, D)
+    ob = DevBuf(g, T * Hq * D * 4)
+    ob.fill(0xFF)
+    sc = DevBuf(g, max(4, 4 * ops.k.rc_attn_scratch(T, Hq, Hkv, D, W, p0)))
+    ops.rc_attn(DevBuf.of(g, qd), Hq * D, kcb, vcb, T, Hq, Hkv, D, R, W, p0, ob, sc)
+    got = ob.read(np.float32).reshape(T, Hq * D)
+    check_close(got, orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, R, p0, win=W), F32, "ns_rc_attn vs float64 closed form")
+
+
+def test_ricursive_entry_points_refuse_what_the_reference_refuses(ops):
+    g = ops.gpu
+    D, Hkv = 128, 1
+    kcb = DevBuf(g, Hkv * 64 * 2 * D)
+    q, out = DevBuf(g, 16 * 10 * D * 4), DevBuf(g, 16 * 10 * D * 4)
+    sc = DevBuf(g, 1 << 20)
+    with pytest.raises(Error, match="the ring is smaller than the window and the rows"):
+        ops.rc_attn(q, 10 * D, kcb, kcb, 4, 10, Hkv, D, 64, 64, 100, out, sc)
+    with pytest.raises(Error, match="past the cache's capacity"):
+        ops.rc_attn(q, 10 * D, kcb, kcb, 4, 10, Hkv, D, 64, 0, 61, out, sc)
+    with pytest.raises(Error, match="1, 2, 4, 6, 8 or 10 query heads a key head"):
+        ops.rc_attn(q, 5 * D, kcb, kcb, 1, 5, Hkv, D, 64, 0, 10, out, sc)
+    with pytest.raises(Error, match="more rows than the ring holds"):
+        ops.rc_kv_store(DevBuf(g, 65 * D * 4), D, DevBuf(g, 65 * D * 4), D, 65, Hkv, D, 64, 0, kcb, kcb)
+    with pytest.raises(Error, match="query heads a multiple of 8 a key head"):
+        ops.nh_attn(q, 10 * D, kcb, kcb, 1, 10, Hkv, D, 64, 3, out, sc)
+    with pytest.raises(Error, match="past the cache's capacity"):
+        ops.nh_attn(q, 8 * D, kcb, kcb, 2, 8, Hkv, D, 64, 63, out, sc)
+    ops.rc_attn(q, 10 * D, kcb, kcb, 0, 10, Hkv, D, 64, 0, 1000, out, None)      # no rows: nothing is checked
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,p0", [(1, 32, 4, 5000), (4, 16, 2, 2046), (16, 8, 1, 77), (200, 16, 2, 300)])
+def test_nemotronh_entry_points(ops, T, Hq, Hkv, p0):
+    """ns_nh_kv_store / ns_nh_attn (kernels/llm/nemotronh/nh.cpp:551-588): the store byte for byte, the attention against
+    the float64 closed form, and - up to 16 rows - the very bits of ns_q35_attn, whose pass it is."""
+    D = 128
+    g = ops.gpu
+    cap = p0 + T + 3
+    k, v = orc.randn(51, (p0 + T, Hkv * D)), orc.randn(52, (p0 + T, Hkv * D))
+    kc, vc = orc.kv_store(0, k, v, Hkv, D, cap, 0)
+    kcb, vcb = DevBuf(g, kc.nbytes), DevBuf(g, vc.nbytes)
+    kcb.fill(0)
+    vcb.fill(0)
+    # rows of a wider buffer (strides of their own), in two calls
+    wide_k, wide_v = np.zeros((p0 + T, Hkv * D + 32), np.float32), np.zeros((p0 + T, Hkv * D + 64), np.float32)
+    wide_k[:, :Hkv * D], wide_v[:, :Hkv * D] = k, v
+    h = (p0 + T) // 2
+    for s, e in ((0, h), (h, p0 + T)):
+        if e > s:
+            ops.nh_kv_store(DevBuf.of(g, wide_k[s:e]), Hkv * D + 32, DevBuf.of(g, wide_v[s:e]), Hkv * D + 64, e - s, Hkv, D, cap, s, kcb, vcb)
+    assert np.array_equal(kcb.read(np.uint8).reshape(kc.shape), kc) and np.array_equal(vcb.read(np.uint8).reshape(vc.shape), vc)
+    qd, qf = make_q(F32, T, Hq, D)
+    qb, ob = DevBuf.of(g, qd), DevBuf(g, T * Hq * D * 4)
+    ob.fill(0xFF)
+    sc = DevBuf(g, max(4, 4 * ops.k.nh_attn_scratch(T, Hq, Hkv, D, p0)))
+    ops.nh_attn(qb, Hq * D, kcb, vcb, T, Hq, Hkv, D, cap, p0, ob, sc)
+    got = ob.read(np.float32).reshape(T, Hq * D)
+    check_close(got, orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, cap, p0), F32, "ns_nh_attn vs float64 closed form")
+    ob2 = DevBuf(g, T * Hq * D * 4)
+    sc2 = DevBuf(g, max(4, 4 * ops.k.q35_attn_scratch(T, Hq, Hkv, D, p0)))
+    ops.q35_attn(qb, Hq * D, kcb, vcb, T, Hq, Hkv, D, cap, p0, ob2, sc2)
+    assert np.array_equal(ob2.read(np.float32).reshape(T, Hq * D).view(np.uint32), got.view(np.uint32))
+
+
+@pytest.mark.parametrize("rope", [0, 1])
+def test_ricursive_norm_and_rotary(ops, rope):
+    """ns_rc_qk_norm_rope (kernels/llm/ricursive/rc.cpp:148-181) is ns_q35_qk_norm_rope turned over all D features, or
+    over none: the same bits, and the oracle's restatement within the path's tolerance."""
+    T, H, D, p0, theta, eps = 9, 10, 128, 777, 1.0e6, 1.0e-6
+    g = ops.gpu
+    x = orc.randn(61, (T, H * D))
+    w = (1.0 + 0.1 * orc.randn(62, (D,))).astype(np.float32)
+    xb, wb = DevBuf.of(g, x), DevBuf.of(g, w)
+    a, b = DevBuf(g, x.nbytes), DevBuf(g, x.nbytes)
+    ops.ok(ops.k.rc_qk_norm_rope(ops.raw(), xb.ptr, H * D, D, a.ptr, H * D, T, H, D, wb.ptr, eps, rope, theta, p0), "ns_rc_qk_norm_rope")
+    ops.ok(ops.k.q35_qk_norm_rope(ops.raw(), xb.ptr, H * D, D, b.ptr, H * D, T, H, D, wb.ptr, eps, D if rope else 0, theta, p0), "ns_q35_qk_norm_rope")
+    got = a.read(np.float32)
+    assert np.array_equal(got.view(np.uint32), b.read(np.float32).view(np.uint32))
+    ref = orc.q35_norm_rope(x.reshape(T, H, D), T, H, D, w, eps, D if rope else 0, theta, p0)
+    # (the angle's argument reduction: an error of about pos * 2^-23 radians, as for the qwen35 entry points)
+    assert np.abs(got.reshape(ref.shape) - ref).max() <= (4 * (1 + p0 + T) * 2.0 ** -23 + 2e-6) * float(np.abs(ref).max())
