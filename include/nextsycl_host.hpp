@@ -55,8 +55,10 @@ public:
     X(ns_mg_kv_store) X(ns_mg_attn_scratch) X(ns_mg_attn) X(ns_mg_attn_prompt_supported) X(ns_mg_attn_prompt)                            \
     X(ns_mg_attn_decode_supported) X(ns_mg_attn_decode_scratch) X(ns_mg_attn_decode) X(ns_llm_minimaxm3_attend)                          \
     X(ns_rc_kv_store) X(ns_rc_attn_scratch) X(ns_rc_attn) X(ns_nh_kv_store) X(ns_nh_attn_scratch) X(ns_nh_attn)                          \
+    X(ns_nhs_attn_prompt_supported) X(ns_nhs_attn_prompt) X(ns_nhs_attn_decode_supported) X(ns_nhs_attn_decode_scratch)                  \
+    X(ns_nhs_attn_decode)                                                                                                                \
     X(ns_attn_kv_store) X(ns_attn_decode_scratch) X(ns_attn_decode_t) X(ns_attn_prompt_t) X(ns_attn_decode_static)                       \
-    X(ns_ds2_kv_store) X(ns_ds2_mla_decode) X(ns_ds2_mla_decode_q6k) X(ns_mla_decode_latent_scratch) X(ns_mla_decode_latent)             \
+    X(ns_ds2_rope) X(ns_ds2_kv_store) X(ns_ds2_mla_decode) X(ns_ds2_mla_decode_q6k) X(ns_mla_decode_latent_scratch) X(ns_mla_decode_latent)             \
     X(ns_mla_attend) X(ns_mla_attend_sel) X(ns_mla_attend_sel_q8) X(ns_to_q8row) X(ns_gather_q8_h)
 
 class Api {

@@ -131,6 +131,16 @@ int ns_q35_attn_prompt(ns_gpu* g, const float* q, int64_t qs, const void* kc, co
 int ns_q35_attn_prompt_kv(ns_gpu* g, int kt, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv,
                           int64_t D, int64_t cap, int64_t p0, float* out);
 
+/* nemotron-h's silo names of the same two passes (the reference: D 128, 16 query heads a key head, decode rows 1..8).
+ * Replaces: kernels/llm/nemotronh/silo/nhs.h:60-69 (silo/attn.cpp:337-369) */
+int ns_nhs_attn_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);
+int ns_nhs_attn_prompt(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
+                       int64_t cap, int64_t p0, float* out);
+int ns_nhs_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);
+int64_t ns_nhs_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0);
+int ns_nhs_attn_decode(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
+                       int64_t cap, int64_t p0, float* out, float* scratch);
+
 /* ---- the engines' own ("exact") attention entry points, routed to the kernels above ----------------------------- */
 
 /* Replaces: kernels/llm/qwen35/q35.h:61-66 (q35.cpp:590-612) */

@@ -41,6 +41,13 @@ int ns_ds2_mla_decode(ns_gpu* g, const float* q, const uint16_t* kb, const uint1
  * kernels/llm/deepseek2/ds2.h:38-41 (ds2.cpp:117-134,157-173,237-246,272-281) */
 int ns_ds2_mla_decode_q6k(ns_gpu* g, const float* q, const void* kvb, const uint16_t* cache, float* out, int64_t T, int64_t H, int64_t pos0,
                           float scale);
+/* ggml's YaRN rope (adjacent pairs) in place on x: T rows `row` floats apart, H heads `head` floats apart, the rotated
+ * part n_dims values from float `off` of each head, row t at position pos0 + t; out (nullable): the rotated part also
+ * written there (rows out_row, heads out_head floats apart). The decode step's q_pe (and k_pe, where an engine keeps it
+ * apart from the latent cache). Replaces: kernels/llm/deepseek2/ds2.h:20-27 (ds2.cpp:59-83) */
+int ns_ds2_rope(ns_gpu* g, float* x, int64_t T, int64_t H, int64_t row, int64_t head, int64_t off, int64_t n_dims, int64_t pos0,
+                float freq_base, float freq_scale, float ext_factor, float mscale, float corr0, float corr1, float* out, int64_t out_row,
+                int64_t out_head);
 /* The latent cache's rows pos0 .. pos0 + T - 1 from kv [T][L + R] float32: the first L RMS-normed with w (eps), the last
  * R rotated by ggml's YaRN rope on adjacent pairs. Replaces: kernels/llm/deepseek2/ds2.h:28-31 (ds2.cpp:85-112) */
 int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint16_t* cache, int64_t T, int64_t L, int64_t R, int64_t pos0,

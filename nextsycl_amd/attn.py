@@ -54,6 +54,11 @@ ATTN_H = {
     "ns_q35_attn_prompt_supported": (i32, [i64, i64, i64, i64]),
     "ns_q35_attn_prompt": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P]),
     "ns_q35_attn_prompt_kv": (i32, [P, i32, P, i64, P, P, i64, i64, i64, i64, i64, i64, P]),
+    "ns_nhs_attn_prompt_supported": (i32, [i64, i64, i64, i64]),
+    "ns_nhs_attn_prompt": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P]),
+    "ns_nhs_attn_decode_supported": (i32, [i64, i64, i64, i64]),
+    "ns_nhs_attn_decode_scratch": (i64, [i64, i64, i64, i64, i64]),
+    "ns_nhs_attn_decode": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P, P]),
     "ns_q35_attn_scratch": (i64, [i64, i64, i64, i64, i64]),
     "ns_q35_attn": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P, P]),
     "ns_mg_attn_scratch": (i64, [i64, i64, i64, i64, i64, i64, i32]),
@@ -90,6 +95,7 @@ MLA_H = {
     "ns_ds2_mla_decode": (i32, [P, P, P, P, P, P, i64, i64, i64, f32]),
     "ns_ds2_mla_decode_q6k": (i32, [P, P, P, P, P, i64, i64, i64, f32]),
     "ns_ds2_kv_store": (i32, [P, P, P, f32, P, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32]),
+    "ns_ds2_rope": (i32, [P, P, i64, i64, i64, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32, P, i64, i64]),
     "ns_mla_attend_sel": (i32, [P, P, P, P, i64, i64, i64, i64, f32, P, P, i64]),
     "ns_mla_attend_sel_q8": (i32, [P, P, P, P, i64, i64, i64, i64, f32, P, P, i64]),
     "ns_to_q8row": (i32, [P, P, P, i64, i64]),

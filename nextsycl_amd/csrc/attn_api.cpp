@@ -46,6 +46,14 @@ int ns_q35_attn_prompt_kv(ns_gpu* g, int kt, const float* q, int64_t qs, const v
     return ns_attn_prompt_any(g, "ns_q35_attn_prompt_kv", 0, kt, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, 1, -1, 0.0f, out);
 }
 
+int ns_nhs_attn_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) { return ns_mg_attn_prompt_supported(T, Hq, Hkv, D); }
+
+int ns_nhs_attn_prompt(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
+                       int64_t cap, int64_t p0, float* out) {
+    if (!ns_nhs_attn_prompt_supported(T, Hq, Hkv, D)) return ns_fail("ns_nhs_attn_prompt: more than 16 rows, heads of 128 or 256, query heads a multiple of the key heads");
+    return ns_attn_prompt_any(g, "ns_nhs_attn_prompt", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, 1, -1, 0.0f, out);
+}
+
 // ---- the engines' own entry points: decode rows split, prompt rows flash -------------------------------------------------
 
 int64_t ns_q35_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0) {

@@ -996,6 +996,13 @@ int ns_q35_attn_decode_kv(ns_gpu* g, int kt, const float* q, int64_t qs, const v
     return decode_checked(g, "ns_q35_attn_decode_kv", 0, kt, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, DecodeExtra{}, 0.0f, out, scratch);
 }
 
+int ns_nhs_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) { return ns_q35_attn_decode_supported(T, Hq, Hkv, D); }
+int64_t ns_nhs_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0) { return ns_attn_decode_scratch(T, Hq, Hkv, D, p0, 0); }
+int ns_nhs_attn_decode(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
+                       int64_t cap, int64_t p0, float* out, float* scratch) {
+    return decode_checked(g, "ns_nhs_attn_decode", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, 0, DecodeExtra{}, 0.0f, out, scratch);
+}
+
 int ns_mg_attn_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) { return ns_q35_attn_decode_supported(T, Hq, Hkv, D); }
 int64_t ns_mg_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win) {
     return ns_attn_decode_scratch(T, Hq, Hkv, D, p0, win);

@@ -892,6 +892,29 @@ __global__ __launch_bounds__(256) void ds2_kv_store_kernel(const float* __restri
     }
 }
 
+// YaRN rotary positions in place on the rotated part of every head of x (adjacent pairs), a copy of that part to out
+// where given; a thread a (row, head, pair)
+__global__ __launch_bounds__(256) void ds2_rope_kernel(float* __restrict__ x, int64_t T, int64_t H, int64_t row, int64_t head, int64_t off, int64_t n_dims,
+                                                       int64_t pos0, float freq_base, float freq_scale, float ext_factor, float mscale, float corr0,
+                                                       float corr1, float* __restrict__ out, int64_t out_row, int64_t out_head) {
+    const int64_t pairs = n_dims / 2, gi = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (gi >= T * H * pairs) return;
+    const int64_t i = gi % pairs, h = (gi / pairs) % H, t = gi / (pairs * H);
+    const int i0 = (int) (2 * i);
+    float c, s;
+    yarn_cs((float) (pos0 + t), i0, (int) n_dims, freq_base, freq_scale, ext_factor, mscale, corr0, corr1, c, s);
+    float* v = x + t * row + h * head + off + i0;
+    const float x0 = v[0], x1 = v[1];
+    const float y0 = x0 * c - x1 * s, y1 = x0 * s + x1 * c;
+    v[0] = y0;
+    v[1] = y1;
+    if (out) {
+        float* o = out + t * out_row + h * out_head + i0;
+        o[0] = y0;
+        o[1] = y1;
+    }
+}
+
 // GLM's q8 latent rows: a wave a row, a lane... 16 lanes a row, a lane a block of 32: the scale rounded to half BEFORE it
 // divides, clamp to +-127 (kernels/llm/glm5next/glm.cpp:1282-1299)
 __global__ __launch_bounds__(256) void to_q8row_kernel(const float* __restrict__ x, uint8_t* __restrict__ y, int64_t n) {
@@ -1146,6 +1169,21 @@ int ns_ds2_mla_decode_q6k(ns_gpu* g, const float* q, const void* kvb, const uint
     NS_TRY
     if (T > 0 && !kvb) return ns_fail("ns_ds2_mla_decode_q6k: a null buffer");
     return ds2_decode(g, "ns_ds2_mla_decode_q6k", q, nullptr, nullptr, (const uint8_t*) kvb, cache, out, T, H, pos0, scale);
+    NS_CATCH
+}
+
+int ns_ds2_rope(ns_gpu* g, float* x, int64_t T, int64_t H, int64_t row, int64_t head, int64_t off, int64_t n_dims, int64_t pos0,
+                float freq_base, float freq_scale, float ext_factor, float mscale, float corr0, float corr1, float* out, int64_t out_row,
+                int64_t out_head) {
+    NS_TRY
+    if (n_dims % 2 != 0) return ns_fail("ns_ds2_rope: an even rotated width");
+    if (T <= 0 || H <= 0 || n_dims <= 0) return 0;
+    if (!g || !x) return ns_fail("ns_ds2_rope: a null buffer");
+    NS_HIP(hipSetDevice(g->dev));
+    ds2_rope_kernel<<<(unsigned) ((T * H * (n_dims / 2) + 255) / 256), 256, 0, g->q>>>(x, T, H, row, head, off, n_dims, pos0, freq_base, freq_scale, ext_factor,
+                                                                            mscale, corr0, corr1, out, out_row, out_head);
+    NS_LAUNCHED("ds2_rope");
+    return 0;
     NS_CATCH
 }
 

@@ -768,6 +768,31 @@ ORC_API int orc_ds2_kv_store(const float* kv, const float* w, float eps, uint16_
     return 0;
 }
 
+/* ggml's YaRN rope in place on the rotated part of every head, a copy of that part to out where given -
+ * kernels/llm/deepseek2/ds2.cpp:59-83 */
+ORC_API int orc_ds2_rope(float* x, int64_t T, int64_t H, int64_t row, int64_t head, int64_t off, int64_t n_dims, int64_t pos0, float freq_base,
+                         float freq_scale, float ext_factor, float mscale, float corr0, float corr1, float* out, int64_t out_row, int64_t out_head) {
+    if (n_dims % 2) return -1;
+    for (int64_t t = 0; t < T; ++t)
+        for (int64_t h = 0; h < H; ++h)
+            for (int64_t i = 0; i < n_dims / 2; ++i) {
+                const int i0 = (int) (2 * i);
+                float c, s;
+                yarn_cs((float) (pos0 + t), i0, (int) n_dims, freq_base, freq_scale, ext_factor, mscale, corr0, corr1, &c, &s);
+                float* v = x + t * row + h * head + off + i0;
+                const float x0 = v[0], x1 = v[1];
+                const float y0 = x0 * c - x1 * s, y1 = x0 * s + x1 * c;
+                v[0] = y0;
+                v[1] = y1;
+                if (out) {
+                    float* o = out + t * out_row + h * out_head + i0;
+                    o[0] = y0;
+                    o[1] = y1;
+                }
+            }
+    return 0;
+}
+
 /* q~ = k_b q_nope per (row, head): qa [T][H][L + R] = [q~ (L) | q_pe (R)] from q [T][H][nope + R], kb half [H][L][nope] -
  * kernels/llm/deepseek2/ds2.cpp:176-184 (a lane sums 8 products, 16 lanes reduced) */
 ORC_API void orc_mla_absorb(const float* q, const uint16_t* kb, float* qa, int64_t T, int64_t H, int64_t L, int64_t R, int64_t NOPE) {

@@ -55,6 +55,7 @@ def lib():
             "orc_mm3_idx_topk": (None, [P, P, i64, i64, i64, i64]),
             "orc_glm_mla_attend_sel": (None, [P, P, C.c_int, P, i64, i64, i64, i64, f32, P, P, i64]),
             "orc_ds2_kv_store": (C.c_int, [P, P, f32, P, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32]),
+            "orc_ds2_rope": (C.c_int, [P, i64, i64, i64, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32, P, i64, i64]),
             "orc_mla_absorb": (None, [P, P, P, i64, i64, i64, i64, i64]),
             "orc_mla_decode_u": (None, [P, P, P, i64, i64, i64, i64, i64, f32]),
             "orc_mla_vb": (None, [P, P, P, i64, i64, i64, i64]),
@@ -267,6 +268,16 @@ def ds2_kv_store(kv, w, eps, cache, T, L, R, pos0, freq_base, freq_scale, ext_fa
     if rc:
         raise ValueError("orc_ds2_kv_store: bad arguments")
     return cache
+
+
+def ds2_rope(x, T, H, row, head, off, n_dims, pos0, freq_base, freq_scale, ext_factor, mscale, corr0, corr1, out=None, out_row=0, out_head=0):
+    """ns_ds2_rope: x (float32, modified in place and returned); out: an array the rotated part is also written into."""
+    x = _c(x, np.float32)
+    rc = lib().orc_ds2_rope(_p(x), T, H, row, head, off, n_dims, pos0, freq_base, freq_scale, ext_factor, mscale, corr0, corr1,
+                            _p(out) if out is not None else None, out_row, out_head)
+    if rc:
+        raise ValueError("orc_ds2_rope: bad arguments")
+    return x
 
 
 def mla_absorb(q, kb, T, H, L=512, R=64, NOPE=128):

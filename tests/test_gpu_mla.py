@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from helpers import MAX_ABS, REL_L2
-from nextsycl_amd import DevBuf
+from nextsycl_amd import DevBuf, Error
 from nextsycl_amd.attn import F16, F32
 from oracle import orc
 
@@ -197,6 +197,36 @@ def test_ds2_kv_store(ops):
         gr, wr = orc.h2f(got[pos0:, L:]).astype(np.float64), orc.h2f(want[pos0:, L:]).astype(np.float64)
         assert (np.abs(gr - wr) <= np.abs(wr) * 2.0 ** -10 + 1e-6).all()
         assert (got[pos0:, L:] == want[pos0:, L:]).mean() > 0.9
+
+
+@pytest.mark.parametrize("yarn", [(10000.0, 1.0, 0.0, 1.0, 0.0, 0.0), (10000.0, 0.025, 1.0, 1.3, 10.0, 23.0)])
+def test_ds2_rope(ops, yarn):
+    """ns_ds2_rope (kernels/llm/deepseek2/ds2.cpp:59-83): a decode step's q_pe - 64 of each head's 192 floats - turned in
+    place, the copy to `out`, every other float untouched; cos / sin come from another library than the oracle's, so a
+    float may differ by a few ulps of the angle."""
+    T, H, head, off, n, pos0 = 7, 16, 192, 128, 64, 3000
+    row = H * head + 5
+    g = ops.gpu
+    x = orc.randn(7, (T, row))
+    want_out = np.zeros((T, H, n), np.float32)
+    want = orc.ds2_rope(x.copy(), T, H, row, head, off, n, pos0, *yarn, want_out, H * n, n)
+    xb, ob = DevBuf.of(g, x), DevBuf(g, want_out.nbytes)
+    ob.fill(0)
+    ops.ok(ops.k.ds2_rope(ops.raw(), xb.ptr, T, H, row, head, off, n, pos0, *yarn, ob.ptr, H * n, n), "ns_ds2_rope")
+    got, got_out = xb.read(np.float32).reshape(T, row), ob.read(np.float32).reshape(T, H, n)
+    rot = np.zeros((T, row), bool)
+    for h in range(H):
+        rot[:, h * head + off:h * head + off + n] = True
+    assert np.array_equal(got[~rot], x[~rot])
+    tol = (4.0 * (1.0 + pos0 + T) * 2.0 ** -23 + 2e-6) * float(np.abs(x).max()) * max(1.0, yarn[3])
+    assert np.abs(got - want).max() <= tol and np.abs(got_out - want_out).max() <= tol
+    assert np.array_equal(got_out.reshape(T, H * n), got[rot].reshape(T, H * n))
+    # no copy asked for, and the refusal
+    xb2 = DevBuf.of(g, x)
+    ops.ok(ops.k.ds2_rope(ops.raw(), xb2.ptr, T, H, row, head, off, n, pos0, *yarn, None, 0, 0), "ns_ds2_rope")
+    assert np.array_equal(xb2.read(np.float32).reshape(T, row), got)
+    with pytest.raises(Error, match="an even rotated width"):
+        ops.ok(ops.k.ds2_rope(ops.raw(), xb2.ptr, T, H, row, head, off, 63, pos0, *yarn, None, 0, 0), "ns_ds2_rope")
 
 
 def test_full_ds2_mla_decode_at_bench_size(ops):

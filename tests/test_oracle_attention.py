@@ -180,3 +180,46 @@ def test_ds2_kv_store_reduces_to_textbook_rope():
         assert np.abs(got[t, L::2] - (x0 * np.cos(ang) - x1 * np.sin(ang))).max() < 3e-3
         assert np.abs(got[t, L + 1::2] - (x0 * np.sin(ang) + x1 * np.cos(ang))).max() < 3e-3
     assert (cache[:pos0] == 0).all()
+
+
+def test_ds2_rope_is_ggml_yarn_in_closed_form():
+    """orc.ds2_rope (and with it the angle code ds2_kv_store shares) against ggml's rope_yarn written out in float64: the
+    extrapolated angle pos * base^(-i0 / n), the interpolated one freq_scale times it, their mix by the ramp between the
+    correction dims times ext_factor, cos and sin times mscale - with the mix switched on, off, and a plain rope; the
+    rotated slice only, the copy to `out`, every other float untouched."""
+    T, H, row, head, off, n, pos0 = 5, 3, 3 * 40 + 7, 40, 8, 24, 4000
+    for base, fs, ext, ms, c0, c1 in ((10000.0, 1.0, 0.0, 1.0, 0.0, 0.0), (10000.0, 0.025, 1.0, 1.3, 3.0, 9.0), (5.0e5, 0.5, 0.4, 0.8, 2.0, 6.5)):
+        x = orc.randn(3, (T, row))
+        out = np.full((T, H, n), 7.0, np.float32)
+        got = orc.ds2_rope(x.copy(), T, H, row, head, off, n, pos0, base, fs, ext, ms, c0, c1, out, H * n, n)
+        want = x.astype(np.float64)
+        i = np.arange(n // 2)
+        ramp = 1.0 - np.clip((i - c0) / max(0.001, c1 - c0), 0.0, 1.0)
+        for t in range(T):
+            extrap = (pos0 + t) * base ** (-2.0 * i / n)
+            interp = fs * extrap
+            theta = interp * (1 - ramp * ext) + extrap * ramp * ext if ext != 0.0 else interp
+            c, s_ = np.cos(theta) * ms, np.sin(theta) * ms
+            for h in range(H):
+                a = x[t, h * head + off:h * head + off + n].astype(np.float64)
+                want[t, h * head + off:h * head + off + n:2] = a[0::2] * c - a[1::2] * s_
+                want[t, h * head + off + 1:h * head + off + n:2] = a[0::2] * s_ + a[1::2] * c
+        # (float32 angles of a few thousand radians: 2^-12 radians an ulp, a few of them by the repeated products)
+        assert np.abs(got - want).max() < 4e-4 * np.abs(x).max() * max(1.0, ms)
+        rot = np.zeros((T, row), bool)
+        for h in range(H):
+            rot[:, h * head + off:h * head + off + n] = True
+        assert np.array_equal(got[~rot], x[~rot])
+        for h in range(H):
+            assert np.array_equal(out[:, h], got[:, h * head + off:h * head + off + n])
+    # small positions: the float32 chain is then tight against float64
+    x = orc.randn(4, (2, 64))
+    got = orc.ds2_rope(x.copy(), 2, 1, 64, 64, 0, 64, 3, 10000.0, 0.25, 1.0, 1.2, 10.0, 23.0)
+    i = np.arange(32)
+    ramp = 1.0 - np.clip((i - 10.0) / 13.0, 0.0, 1.0)
+    for t in range(2):
+        extrap = (3 + t) * 10000.0 ** (-2.0 * i / 64)
+        theta = 0.25 * extrap * (1 - ramp) + extrap * ramp
+        a = x[t].astype(np.float64)
+        assert np.abs(got[t, 0::2] - (a[0::2] * np.cos(theta) - a[1::2] * np.sin(theta)) * 1.2).max() < 1e-5
+        assert np.abs(got[t, 1::2] - (a[0::2] * np.sin(theta) + a[1::2] * np.cos(theta)) * 1.2).max() < 1e-5
