@@ -69,6 +69,19 @@ int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, in
  * 0 .. pos0 + T - 1 are rounded to half into memory the library keeps per ns_gpu and read from there (-1 when they do not
  * fit beside the partials: ~48K cells). Replaces: kernels/llm/glm5next/glm.h:47 (glm.cpp:782-812) */
 int ns_mla_attend(ns_gpu* g, const float* qa, const float* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale);
+/* GLM's DSA indexer, which fills the lists ns_mla_attend_sel reads (pools of 4 consecutive tokens). Replaces:
+ * kernels/llm/glm5next/glm.h:48-55 (glm.cpp:876-1019), bound at llm/glm5next/src/ffi.rs.
+ * ns_idx_pool: the pools completed by tokens [pos0, pos0 + T): pooled[j][c] = sum_m softmax_m(ig_m[c] + ape[m][c]) ik_m[c]
+ *   over pool j's 4 members (ik, ig [T][D] float32, ape [4][D]); a member before pos0 comes from ring [8][2 D] (ik | ig at
+ *   slot position % 8), which then takes this pass's last (up to 8) tokens.
+ * ns_idx_score: S [T H][n] (iq . pooled^T for pools [j0, j0 + n), the engine's GEMM), w [T][H]: score[r][j0 + jj] =
+ *   sum_h max(S[r H + h][jj], 0) w[r][h], heads in order, for the pools row r sees (j < (pos0 + r + 1) / 4), else -inf;
+ *   score rows ld floats apart.
+ * ns_topk: the K highest of score[r][0, n) into sel[r][0, K) as positions in ascending order, ties at the K-th value to the
+ *   lowest positions; the same list every run. */
+int ns_idx_pool(ns_gpu* g, float* ring, const float* ik, const float* ig, const float* ape, float* pooled, int64_t pos0, int64_t T, int64_t D);
+int ns_idx_score(ns_gpu* g, const float* S, const float* w, float* score, int64_t T, int64_t H, int64_t j0, int64_t n, int64_t ld, int64_t pos0);
+int ns_topk(ns_gpu* g, const float* score, int32_t* sel, int64_t T, int64_t n, int64_t ld, int64_t K);
 /* out [n][512] half = the q8 latent rows idx[i] of src, widened: half(scale x q), one rounding (a prompt pass's gather).
  * Replaces: kernels/llm/glm5next/glm.h:78 (glm.cpp:1301-1325) */
 int ns_gather_q8_h(ns_gpu* g, const void* src, const int32_t* idx, uint16_t* out, int64_t n, int64_t L);

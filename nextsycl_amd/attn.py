@@ -101,6 +101,9 @@ MLA_H = {
     "ns_to_q8row": (i32, [P, P, P, i64, i64]),
     "ns_mla_attend": (i32, [P, P, P, P, i64, i64, i64, i64, f32]),
     "ns_gather_q8_h": (i32, [P, P, P, P, i64, i64]),
+    "ns_idx_pool": (i32, [P, P, P, P, P, P, i64, i64, i64]),
+    "ns_idx_score": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64]),
+    "ns_topk": (i32, [P, P, P, i64, i64, i64, i64]),
 }
 
 

@@ -7,6 +7,7 @@
 // equal scores, -1 once nothing finite is left, picked scores overwritten with -inf).
 #include "ns_internal.hpp"
 #include "ns_attn.h"
+#include "ns_mla.h"
 #include "kv_formats.hpp"
 #include "attn_common.hpp"
 
@@ -125,9 +126,285 @@ __global__ __launch_bounds__(64) void idx_topk_reg_kernel(float* __restrict__ bs
     }
 }
 
+// ---- GLM's DSA indexer (kernels/llm/glm5next/glm.cpp:876-1019): pools of 4 consecutive tokens --------------------------
+
+// the pools completed by this pass: pooled[j][c] = sum_m softmax_m(ig_m[c] + ape[m][c]) ik_m[c] over pool j's 4 members
+// (positions 4 j + m; a member before pos0 comes from the ring: ik | ig at slot position % 8). A thread a (pool, feature)
+__global__ __launch_bounds__(256) void glm_idx_pool_kernel(const float* __restrict__ ring, const float* __restrict__ ik, const float* __restrict__ ig,
+                                                           const float* __restrict__ ape, float* __restrict__ pooled, int64_t pos0, int64_t j_lo, int64_t npool,
+                                                           int64_t D) {
+    const int64_t gi = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (gi >= npool * D) return;
+    const int64_t j = j_lo + gi / D, c = gi % D;
+    float lg[4], kv[4], mx = -INFINITY;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        const int64_t pp = 4 * j + m;
+        const float* k = pp >= pos0 ? ik + (pp - pos0) * D : ring + (pp % 8) * 2 * D;
+        const float* gg = pp >= pos0 ? ig + (pp - pos0) * D : ring + (pp % 8) * 2 * D + D;
+        kv[m] = k[c];
+        lg[m] = gg[c] + ape[m * D + c];
+        mx = fmaxf(mx, lg[m]);
+    }
+    float sum = 0.0f, acc = 0.0f;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        const float e = expf(lg[m] - mx);
+        sum += e;
+        acc += e * kv[m];
+    }
+    pooled[j * D + c] = acc / sum;
+}
+
+// the ring takes the pass's last (up to 8) tokens: ik | ig at slot position % 8
+__global__ __launch_bounds__(256) void glm_idx_ring_kernel(float* __restrict__ ring, const float* __restrict__ ik, const float* __restrict__ ig, int64_t pos0,
+                                                           int64_t first, int64_t rows, int64_t D) {
+    const int64_t gi = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (gi >= rows * D) return;
+    const int64_t pp = first + gi / D, c = gi % D;
+    ring[(pp % 8) * 2 * D + c] = ik[(pp - pos0) * D + c];
+    ring[(pp % 8) * 2 * D + D + c] = ig[(pp - pos0) * D + c];
+}
+
+// score[r][j0 + jj] = sum_h relu(S[r H + h][jj]) w[r][h] in head order for the pools row r sees, -inf for the others
+__global__ __launch_bounds__(256) void glm_idx_score_kernel(const float* __restrict__ S, const float* __restrict__ w, float* __restrict__ score, int64_t T,
+                                                            int64_t H, int64_t j0, int64_t n, int64_t ld, int64_t pos0) {
+    const int64_t gi = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (gi >= T * n) return;
+    const int64_t r = gi / n, jj = gi % n, j = j0 + jj;
+    const int64_t nv = (pos0 + r + 1) / 4;
+    float s = -INFINITY;
+    if (j < nv) {
+        s = 0.0f;
+        for (int64_t h = 0; h < H; ++h) s += fmaxf(S[(r * H + h) * n + jj], 0.0f) * w[r * H + h];
+    }
+    score[r * ld + j] = s;
+}
+
+// the K highest of a row's n scores as positions in ascending order, ties at the K-th value to the lowest positions: a
+// radix select over the floats' order-preserving keys (4 digits of 8 bits, a histogram a digit in LDS), then one ordered
+// compaction - every thread its own run of positions, two scans over the work-group, no atomics in what is written, so
+// the list (and the sums of the attention that reads it) is the same every run. A work-group of 1024 a row.
+constexpr int TOPK_WG = 1024, TOPK_NH = 16;
+__device__ __forceinline__ uint32_t order_key(float f) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);             // a larger float, a larger key
+}
+// exclusive prefix sum of one value a thread over the work-group (the total to every thread through `total`)
+__device__ uint32_t wg_exclusive_scan(uint32_t v, uint32_t* wsum, uint32_t& total) {
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    uint32_t x = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t y = __shfl_up(x, o, 64);
+        if (lane >= o) x += y;
+    }
+    if (lane == 63) wsum[wv] = x;
+    __syncthreads();
+    uint32_t before = 0, all = 0;
+    for (int i = 0; i < TOPK_WG / 64; ++i) {
+        const uint32_t t = wsum[i];
+        if (i < wv) before += t;
+        all += t;
+    }
+    __syncthreads();
+    total = all;
+    return before + x - v;
+}
+__global__ __launch_bounds__(TOPK_WG) void glm_topk_kernel(const float* __restrict__ score, int32_t* __restrict__ sel, int64_t n, int64_t ld, int64_t K) {
+    __shared__ uint32_t hist[TOPK_NH * 256];
+    __shared__ uint32_t st[3];                                     // prefix, mask, still needed
+    __shared__ uint32_t wsum[TOPK_WG / 64];
+    const int64_t r = blockIdx.x;
+    const int lid = threadIdx.x;
+    const float* row = score + r * ld;
+    if (lid == 0) {
+        st[0] = 0;
+        st[1] = 0;
+        st[2] = (uint32_t) K;
+    }
+    uint32_t* mine = hist + (lid % TOPK_NH) * 256;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        for (int b = lid; b < TOPK_NH * 256; b += TOPK_WG) hist[b] = 0;
+        __syncthreads();
+        const uint32_t prefix = st[0], mask = st[1];
+        for (int64_t j = lid; j < n; j += TOPK_WG) {
+            const uint32_t k = order_key(row[j]);
+            if ((k & mask) == prefix) atomicAdd(&mine[(k >> shift) & 255], 1u);
+        }
+        __syncthreads();
+        if (lid < 256) {
+            uint32_t c = 0;
+            for (int m = 0; m < TOPK_NH; ++m) c += hist[m * 256 + lid];
+            hist[lid] = c;
+        }
+        __syncthreads();
+        if (lid == 0) {
+            // the digit, from the top, at which the count of keys at or above it reaches what is still needed
+            const uint32_t need = st[2];
+            uint32_t above = 0;
+            int d = 255;
+            for (; d > 0; --d) {
+                if (above + hist[d] >= need) break;
+                above += hist[d];
+            }
+            st[0] = prefix | ((uint32_t) d << shift);
+            st[1] = mask | (255u << shift);
+            st[2] = need - above;
+        }
+        __syncthreads();
+    }
+    const uint32_t kth = st[0], ties = st[2];
+    const int64_t seg = (n + TOPK_WG - 1) / TOPK_WG, j0 = std::min<int64_t>(n, lid * seg), j1 = std::min<int64_t>(n, j0 + seg);
+    uint32_t gt = 0, eq = 0;
+    for (int64_t j = j0; j < j1; ++j) {
+        const uint32_t k = order_key(row[j]);
+        gt += k > kth;
+        eq += k == kth;
+    }
+    uint32_t total;
+    const uint32_t eq_before = wg_exclusive_scan(eq, wsum, total);
+    const uint32_t eq_take = eq_before >= ties ? 0u : std::min(eq, ties - eq_before);
+    uint32_t at = wg_exclusive_scan(gt + eq_take, wsum, total);
+    uint32_t eq_left = eq_take;
+    for (int64_t j = j0; j < j1; ++j) {
+        const uint32_t k = order_key(row[j]);
+        if (k > kth || (k == kth && eq_left > 0)) {
+            if (k == kth) --eq_left;
+            if (at < (uint32_t) K) sel[r * K + at] = (int32_t) j;
+            ++at;
+        }
+    }
+}
+
+// The same selection for rows of up to PER x 1024 scores, their keys held in registers (score j = i 1024 + lid: loaded
+// once, coalesced, all in flight) - the row is read from memory once instead of five times with a dependent load an
+// iteration. The histogram has a copy a lane (64 copies, 257 words apart: the lanes of a wave never meet in an address or
+// a bank, however few digits the row's scores share - the top digit, sign and exponent, takes a handful of values), the
+// digit is found by a suffix scan over 256 threads instead of one thread's walk, and the ordered compaction is one
+// work-group scan an i: a position's place in the list = the greater keys before it + the equal ones before it that
+// are still taken, both counts riding in one packed scan.
+template <int PER>
+__global__ __launch_bounds__(TOPK_WG) void glm_topk_reg_kernel(const float* __restrict__ score, int32_t* __restrict__ sel, int n, int64_t ld, int K) {
+    constexpr int NC = 64, CS = 257;
+    __shared__ uint32_t hist[NC * CS];
+    __shared__ uint32_t st[3];
+    __shared__ uint32_t wsum[TOPK_WG / 64];
+    const int64_t r = blockIdx.x;
+    const int lid = threadIdx.x, lane = lid & 63, wv = lid >> 6;
+    const float* row = score + r * ld;
+    uint32_t key[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int j = i * TOPK_WG + lid;
+        key[i] = j < n ? order_key(row[j]) : 0u;
+    }
+    if (lid == 0) {
+        st[0] = 0;
+        st[1] = 0;
+        st[2] = (uint32_t) K;
+    }
+    uint32_t* mine = hist + lane * CS;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        for (int b = lid; b < NC * CS; b += TOPK_WG) hist[b] = 0;
+        __syncthreads();
+        const uint32_t prefix = st[0], mask = st[1], need = st[2];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int j = i * TOPK_WG + lid;
+            if (j < n && (key[i] & mask) == prefix) atomicAdd(&mine[(key[i] >> shift) & 255], 1u);
+        }
+        __syncthreads();
+        // thread lid < 256 takes digit d = 255 - lid: its count, then the count of every digit at or above it
+        uint32_t c = 0, incl = 0;
+        const int d = 255 - lid;
+        if (lid < 256) {
+            for (int m = 0; m < NC; ++m) c += hist[m * CS + d];
+            incl = c;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const uint32_t y = __shfl_up(incl, o, 64);
+                if (lane >= o) incl += y;
+            }
+            if (lane == 63) wsum[wv] = incl;
+        }
+        __syncthreads();
+        if (lid < 256) {
+            for (int x = 0; x < wv; ++x) incl += wsum[x];
+            const uint32_t above = incl - c;                       // keys in digits above d
+            if (above < need && (incl >= need || d == 0)) {        // (d = 0 takes what is left, as the walk from the top does)
+                st[0] = prefix | ((uint32_t) d << shift);
+                st[1] = mask | (255u << shift);
+                st[2] = need - above;
+            }
+        }
+        __syncthreads();
+    }
+    const uint32_t kth = st[0], ties = st[2];
+    uint32_t base_gt = 0, base_eq = 0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        if (i * TOPK_WG >= n || base_gt + std::min(base_eq, ties) >= (uint32_t) K) break;      // (uniform)
+        const int j = i * TOPK_WG + lid;
+        const bool valid = j < n, gt = valid && key[i] > kth, eq = valid && key[i] == kth;
+        uint32_t total;
+        const uint32_t before = wg_exclusive_scan((gt ? 1u : 0u) | (eq ? 0x10000u : 0u), wsum, total);
+        const uint32_t eq_before = base_eq + (before >> 16), at = base_gt + (before & 0xFFFFu) + std::min(eq_before, ties);
+        if ((gt || (eq && eq_before < ties)) && at < (uint32_t) K) sel[r * K + at] = j;
+        base_gt += total & 0xFFFFu;
+        base_eq += total >> 16;
+    }
+}
+
 }  // namespace
 
 extern "C" {
+
+int ns_idx_pool(ns_gpu* g, float* ring, const float* ik, const float* ig, const float* ape, float* pooled, int64_t pos0, int64_t T, int64_t D) {
+    NS_TRY
+    if (T <= 0 || D <= 0) return 0;
+    if (pos0 < 0) return ns_fail("ns_idx_pool: a position");
+    if (!g || !ring || !ik || !ig || !ape || !pooled) return ns_fail("ns_idx_pool: a null buffer");
+    NS_HIP(hipSetDevice(g->dev));
+    const int64_t j_lo = pos0 / 4, j_hi = (pos0 + T) / 4;
+    if (j_hi > j_lo) {
+        glm_idx_pool_kernel<<<(unsigned) (((j_hi - j_lo) * D + 255) / 256), 256, 0, g->q>>>(ring, ik, ig, ape, pooled, pos0, j_lo, j_hi - j_lo, D);
+        NS_LAUNCHED("idx_pool");
+    }
+    const int64_t first = std::max<int64_t>(pos0, pos0 + T - 8);
+    glm_idx_ring_kernel<<<(unsigned) (((pos0 + T - first) * D + 255) / 256), 256, 0, g->q>>>(ring, ik, ig, pos0, first, pos0 + T - first, D);
+    NS_LAUNCHED("idx_pool ring");
+    return 0;
+    NS_CATCH
+}
+
+int ns_idx_score(ns_gpu* g, const float* S, const float* w, float* score, int64_t T, int64_t H, int64_t j0, int64_t n, int64_t ld, int64_t pos0) {
+    NS_TRY
+    if (T <= 0 || n <= 0) return 0;
+    if (H < 0 || j0 < 0 || ld < j0 + n || pos0 < 0) return ns_fail("ns_idx_score: heads, a pool range inside a score row, a position");
+    if (!g || !S || !w || !score) return ns_fail("ns_idx_score: a null buffer");
+    NS_HIP(hipSetDevice(g->dev));
+    glm_idx_score_kernel<<<(unsigned) ((T * n + 255) / 256), 256, 0, g->q>>>(S, w, score, T, H, j0, n, ld, pos0);
+    NS_LAUNCHED("idx_score");
+    return 0;
+    NS_CATCH
+}
+
+int ns_topk(ns_gpu* g, const float* score, int32_t* sel, int64_t T, int64_t n, int64_t ld, int64_t K) {
+    NS_TRY
+    if (T <= 0 || K <= 0) return 0;
+    // (fewer scores than K: the reference's select then takes all n, in position order, and leaves the list's rest as it was)
+    if (n < 0 || ld < n || n > (int64_t) 1 << 30 || K > (int64_t) 1 << 30) return ns_fail("ns_topk: score rows at least n apart");
+    if (!g || !score || !sel) return ns_fail("ns_topk: a null buffer");
+    NS_HIP(hipSetDevice(g->dev));
+    if (n <= 8 * TOPK_WG) glm_topk_reg_kernel<8><<<(unsigned) T, TOPK_WG, 0, g->q>>>(score, sel, (int) n, ld, (int) K);
+    else if (n <= 32 * TOPK_WG) glm_topk_reg_kernel<32><<<(unsigned) T, TOPK_WG, 0, g->q>>>(score, sel, (int) n, ld, (int) K);
+    else if (n <= 64 * TOPK_WG) glm_topk_reg_kernel<64><<<(unsigned) T, TOPK_WG, 0, g->q>>>(score, sel, (int) n, ld, (int) K);
+    else glm_topk_kernel<<<(unsigned) T, TOPK_WG, 0, g->q>>>(score, sel, n, ld, K);
+    NS_LAUNCHED("topk");
+    return 0;
+    NS_CATCH
+}
 
 int ns_llm_minimaxm3_idx_scores(ns_gpu* g, const float* iq, const uint16_t* ik, float* bs, int64_t T, int64_t G, int64_t nblk, int64_t pos0, int64_t local) {
     NS_TRY

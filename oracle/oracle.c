@@ -793,6 +793,88 @@ ORC_API int orc_ds2_rope(float* x, int64_t T, int64_t H, int64_t row, int64_t he
     return 0;
 }
 
+/* GLM's DSA indexer - kernels/llm/glm5next/glm.cpp:876-1019 */
+ORC_API void orc_idx_pool(float* ring, const float* ik, const float* ig, const float* ape, float* pooled, int64_t pos0, int64_t T, int64_t D) {
+    const int64_t j_lo = pos0 / 4, j_hi = (pos0 + T) / 4;
+    for (int64_t j = j_lo; j < j_hi; ++j)
+        for (int64_t c = 0; c < D; ++c) {
+            float lg[4], kv[4], mx = -INFINITY;
+            for (int m = 0; m < 4; ++m) {
+                const int64_t p = 4 * j + m;
+                const float* k = p >= pos0 ? ik + (p - pos0) * D : ring + (p % 8) * 2 * D;
+                const float* gg = p >= pos0 ? ig + (p - pos0) * D : ring + (p % 8) * 2 * D + D;
+                kv[m] = k[c];
+                lg[m] = gg[c] + ape[m * D + c];
+                mx = fmaxf(mx, lg[m]);
+            }
+            float s = 0.f, acc = 0.f;
+            for (int m = 0; m < 4; ++m) {
+                const float e = expf(lg[m] - mx);
+                s += e;
+                acc += e * kv[m];
+            }
+            pooled[j * D + c] = acc / s;
+        }
+    const int64_t first = pos0 > pos0 + T - 8 ? pos0 : pos0 + T - 8;
+    for (int64_t p = first; p < pos0 + T; ++p)
+        for (int64_t c = 0; c < D; ++c) {
+            ring[(p % 8) * 2 * D + c] = ik[(p - pos0) * D + c];
+            ring[(p % 8) * 2 * D + D + c] = ig[(p - pos0) * D + c];
+        }
+}
+
+ORC_API void orc_idx_score(const float* S, const float* w, float* score, int64_t T, int64_t H, int64_t j0, int64_t n, int64_t ld, int64_t pos0) {
+    for (int64_t r = 0; r < T; ++r)
+        for (int64_t jj = 0; jj < n; ++jj) {
+            const int64_t j = j0 + jj, nv = (pos0 + r + 1) / 4;
+            float s = -INFINITY;
+            if (j < nv) {
+                s = 0.f;
+                for (int64_t h = 0; h < H; ++h) s += fmaxf(S[(r * H + h) * n + jj], 0.f) * w[r * H + h];
+            }
+            score[r * ld + j] = s;
+        }
+}
+
+/* the K highest of a row as positions in ascending order, ties at the K-th value to the lowest positions (the radix
+ * select of glm.cpp:940-1019 restated as what it selects: count the keys above the K-th, take those and the first
+ * remaining equal ones) */
+ORC_API void orc_topk(const float* score, int32_t* sel, int64_t T, int64_t n, int64_t ld, int64_t K) {
+    for (int64_t r = 0; r < T; ++r) {
+        const float* row = score + r * ld;
+        uint32_t* key = (uint32_t*) malloc((size_t) (n > 0 ? n : 1) * sizeof(uint32_t));
+        for (int64_t j = 0; j < n; ++j) {
+            uint32_t u;
+            memcpy(&u, row + j, 4);
+            key[j] = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+        }
+        /* the K-th largest key, digit by digit from the top */
+        uint32_t prefix = 0, mask = 0, need = (uint32_t) K;
+        for (int shift = 24; shift >= 0; shift -= 8) {
+            uint32_t hist[256] = {0};
+            for (int64_t j = 0; j < n; ++j)
+                if ((key[j] & mask) == prefix) hist[(key[j] >> shift) & 255]++;
+            uint32_t above = 0;
+            int d = 255;
+            for (; d > 0; --d) {
+                if (above + hist[d] >= need) break;
+                above += hist[d];
+            }
+            prefix |= (uint32_t) d << shift;
+            mask |= 255u << shift;
+            need -= above;
+        }
+        int64_t at = 0;
+        uint32_t ties = need;
+        for (int64_t j = 0; j < n && at < K; ++j)
+            if (key[j] > prefix || (key[j] == prefix && ties > 0)) {
+                if (key[j] == prefix) --ties;
+                sel[r * K + at++] = (int32_t) j;
+            }
+        free(key);
+    }
+}
+
 /* q~ = k_b q_nope per (row, head): qa [T][H][L + R] = [q~ (L) | q_pe (R)] from q [T][H][nope + R], kb half [H][L][nope] -
  * kernels/llm/deepseek2/ds2.cpp:176-184 (a lane sums 8 products, 16 lanes reduced) */
 ORC_API void orc_mla_absorb(const float* q, const uint16_t* kb, float* qa, int64_t T, int64_t H, int64_t L, int64_t R, int64_t NOPE) {

@@ -55,6 +55,9 @@ def lib():
             "orc_mm3_idx_topk": (None, [P, P, i64, i64, i64, i64]),
             "orc_glm_mla_attend_sel": (None, [P, P, C.c_int, P, i64, i64, i64, i64, f32, P, P, i64]),
             "orc_ds2_kv_store": (C.c_int, [P, P, f32, P, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32]),
+            "orc_idx_pool": (None, [P, P, P, P, P, i64, i64, i64]),
+            "orc_idx_score": (None, [P, P, P, i64, i64, i64, i64, i64, i64]),
+            "orc_topk": (None, [P, P, i64, i64, i64, i64]),
             "orc_ds2_rope": (C.c_int, [P, i64, i64, i64, i64, i64, i64, i64, f32, f32, f32, f32, f32, f32, P, i64, i64]),
             "orc_mla_absorb": (None, [P, P, P, i64, i64, i64, i64, i64]),
             "orc_mla_decode_u": (None, [P, P, P, i64, i64, i64, i64, i64, f32]),
@@ -278,6 +281,25 @@ def ds2_rope(x, T, H, row, head, off, n_dims, pos0, freq_base, freq_scale, ext_f
     if rc:
         raise ValueError("orc_ds2_rope: bad arguments")
     return x
+
+
+def glm_idx_pool(ring, ik, ig, ape, pooled, pos0, T, D):
+    """ns_idx_pool: ring [8][2 D] and pooled [pools][D] (float32, contiguous) are updated in place."""
+    lib().orc_idx_pool(_p(ring), _p(_c(ik, np.float32)), _p(_c(ig, np.float32)), _p(_c(ape, np.float32)), _p(pooled), pos0, T, D)
+
+
+def glm_idx_score(S, w, score, T, H, j0, n, pos0):
+    """ns_idx_score: score [T][ld] (float32, contiguous) gets columns j0 .. j0 + n - 1."""
+    lib().orc_idx_score(_p(_c(S, np.float32)), _p(_c(w, np.float32)), _p(score), T, H, j0, n, score.shape[1], pos0)
+
+
+def glm_topk(score, n, K):
+    """ns_topk over score [T][ld]: sel [T][K] int32 (entries past a row's n stay -1)."""
+    score = _c(score, np.float32)
+    T, ld = score.shape
+    sel = np.full((T, K), -1, np.int32)
+    lib().orc_topk(_p(score), _p(sel), T, n, ld, K)
+    return sel
 
 
 def mla_absorb(q, kb, T, H, L=512, R=64, NOPE=128):

@@ -4,7 +4,7 @@ selection itself (comparisons only) bit for bit."""
 import numpy as np
 import pytest
 
-from nextsycl_amd import DevBuf
+from nextsycl_amd import DevBuf, Error
 from oracle import orc
 
 pytestmark = pytest.mark.gpu
@@ -129,3 +129,65 @@ def test_glm_dense_row_past_the_selection_bound_is_marked(ops):
     want = orc.glm_mla_attend_sel(qa, rows, False, T, H, L, pos0, 0.05, sel, cnt, K)
     close(got[:1], want.reshape(T, H * L)[:1])
     assert np.isnan(got[1]).all()
+
+
+def test_glm_indexer_pools(ops):
+    """ns_idx_pool over the engine's sequence of passes (a prompt chunk, then decode and verify passes whose pools reach
+    back into the ring): pooled keys within float32 rounding of the oracle's (the exponential comes from another library),
+    the ring byte for byte."""
+    g = ops.gpu
+    D, n_tok = 128, 213
+    ik, ig, ape = orc.randn(5, (n_tok, D)), orc.randn(6, (n_tok, D)), orc.randn(7, (4, D), 0.5)
+    ring = np.zeros((8, 2 * D), np.float32)
+    pooled = np.zeros((n_tok // 4 + 1, D), np.float32)
+    rb, pb, ab = DevBuf.of(g, ring), DevBuf.of(g, pooled), DevBuf.of(g, ape)
+    pos = 0
+    for T in (150, 1, 1, 3, 5, 1, 2, 4, 9, 16, 1, 20):
+        orc.glm_idx_pool(ring, ik[pos:pos + T], ig[pos:pos + T], ape, pooled, pos, T, D)
+        kb, gb = DevBuf.of(g, ik[pos:pos + T]), DevBuf.of(g, ig[pos:pos + T])
+        ops.ok(ops.k.idx_pool(ops.raw(), rb.ptr, kb.ptr, gb.ptr, ab.ptr, pb.ptr, pos, T, D), "ns_idx_pool")
+        pos += T
+        assert np.array_equal(rb.read(np.float32).reshape(ring.shape), ring)
+    assert pos == n_tok
+    got = pb.read(np.float32).reshape(pooled.shape)
+    assert np.abs(got - pooled).max() <= 4e-6 * np.abs(pooled).max()
+    assert (got[n_tok // 4] == 0).all()
+
+
+@pytest.mark.parametrize("T,H,j0,n,ld,pos0", [(1, 32, 0, 2500, 2500, 9999), (5, 32, 128, 300, 700, 1700), (40, 8, 0, 64, 80, 100)])
+def test_glm_indexer_scores(ops, T, H, j0, n, ld, pos0):
+    g = ops.gpu
+    S, w = orc.randn(9, (T * H, n)), orc.randn(10, (T, H))
+    score = np.full((T, ld), 3.0, np.float32)
+    sb = DevBuf.of(g, score)
+    orc.glm_idx_score(S, w, score, T, H, j0, n, pos0)
+    Sb, wb = DevBuf.of(g, S), DevBuf.of(g, w)
+    ops.ok(ops.k.idx_score(ops.raw(), Sb.ptr, wb.ptr, sb.ptr, T, H, j0, n, ld, pos0), "ns_idx_score")
+    got = sb.read(np.float32).reshape(score.shape)
+    fin = np.isfinite(score)
+    assert np.array_equal(np.isneginf(got), np.isneginf(score))
+    # (a head's product may be fused into the sum on one side and not on the other)
+    assert np.abs(got[fin] - score[fin]).max() <= 1e-5 * max(1.0, float(np.abs(score[fin]).max()))
+    with pytest.raises(Error, match="a pool range inside a score row"):
+        ops.ok(ops.k.idx_score(ops.raw(), Sb.ptr, wb.ptr, sb.ptr, T, H, j0, n, j0 + n - 1, pos0), "ns_idx_score")
+
+
+@pytest.mark.parametrize("T,n,K", [(1, 1, 1), (3, 7, 3), (2, 300, 40), (4, 5000, 512), (1, 5000, 4999), (2, 37, 37), (2, 20, 50), (1, 33000, 2048),
+                                   (8, 1024, 1024), (3, 1025, 1), (2, 8192, 100), (2, 8193, 2048), (1, 32768, 2048), (2, 32769, 700), (1, 65536, 2048), (1, 65537, 300)])
+def test_glm_top_k(ops, T, n, K):
+    """ns_topk: the oracle's list bit for bit - on rows with many equal scores (the ties at the K-th value go to the lowest
+    positions), -inf tails, fewer scores than K (the list's rest is left as it was) - and the same list on a second run."""
+    g = ops.gpu
+    rng = np.random.default_rng(n + K)
+    ld = n + 6
+    sc = rng.choice((np.round(rng.standard_normal(max(n // 3, 2)), 1) + 0.05).astype(np.float32), size=(T, ld)).astype(np.float32)
+    if T > 1:
+        sc[1, n // 2:n] = -np.inf
+    if T > 2:
+        sc[2, :n] = rng.standard_normal(n).astype(np.float32)    # all different
+    want = orc.glm_topk(sc, n, K)
+    scb = DevBuf.of(g, sc)
+    for _ in range(2):
+        sb = DevBuf.of(g, np.full((T, K), -1, np.int32))
+        ops.ok(ops.k.topk(ops.raw(), scb.ptr, sb.ptr, T, n, ld, K), "ns_topk")
+        assert np.array_equal(sb.read(np.int32).reshape(T, K), want)

@@ -92,3 +92,60 @@ def test_glm_cell_pools():
                 assert np.abs(got[t, h] - want).max() < 2e-5
             else:
                 assert not got[t, h].any()
+
+
+def _glm_indexer_inputs(seed, n_tok, D):
+    return orc.randn(seed, (n_tok, D)), orc.randn(seed + 1, (n_tok, D)), orc.randn(seed + 2, (4, D), 0.5)
+
+
+def test_glm_indexer_pools_in_closed_form():
+    """orc.glm_idx_pool (kernels/llm/glm5next/glm.cpp:883-916) against the softmax written out in float64, fed as the
+    engine feeds it: a prompt chunk, then passes of 1, 3 and 5 tokens whose pools' earlier members come from the ring;
+    the ring holds the last 8 tokens, ik | ig, at slot position % 8."""
+    D, n_tok = 24, 61
+    ik, ig, ape = _glm_indexer_inputs(5, n_tok, D)
+    ring = np.zeros((8, 2 * D), np.float32)
+    pooled = np.full((n_tok // 4 + 1, D), np.nan, np.float32)
+    pos = 0
+    for T in (18, 1, 3, 5, 1, 1, 1, 2, 4, 9, 16):
+        orc.glm_idx_pool(ring, ik[pos:pos + T], ig[pos:pos + T], ape, pooled, pos, T, D)
+        pos += T
+        for p in range(max(0, pos - 8), pos):
+            assert np.array_equal(ring[p % 8, :D], ik[p]) and np.array_equal(ring[p % 8, D:], ig[p])
+    assert pos == n_tok
+    for j in range(n_tok // 4):
+        lg = ig[4 * j:4 * j + 4].astype(np.float64) + ape
+        wgt = np.exp(lg - lg.max(axis=0))
+        want = (wgt * ik[4 * j:4 * j + 4]).sum(axis=0) / wgt.sum(axis=0)
+        assert np.abs(pooled[j] - want).max() < 1e-5, j
+    assert np.isnan(pooled[n_tok // 4]).all()                # the incomplete pool is not written
+
+
+def test_glm_indexer_scores_and_top_k():
+    """orc.glm_idx_score: the relu-weighted head sum in float64, -inf for the pools a row does not see yet, columns
+    outside [j0, j0 + n) untouched. orc.glm_topk: the K largest as ascending positions, ties at the K-th value to the
+    lowest positions - against a stable sort, on rows with many equal scores, -inf tails and fewer scores than K."""
+    T, H, j0, n, ld, pos0 = 5, 6, 3, 20, 40, 70
+    S = orc.randn(9, (T * H, n))
+    w = orc.randn(10, (T, H))
+    score = np.full((T, ld), 7.0, np.float32)
+    orc.glm_idx_score(S, w, score, T, H, j0, n, pos0)
+    for r in range(T):
+        nv = (pos0 + r + 1) // 4
+        want = (np.maximum(S[r * H:(r + 1) * H].astype(np.float64), 0.0) * w[r].astype(np.float64)[:, None]).sum(axis=0)
+        for jj in range(n):
+            if j0 + jj < nv:
+                assert abs(score[r, j0 + jj] - want[jj]) < 1e-5
+            else:
+                assert score[r, j0 + jj] == -np.inf
+        assert (score[r, :j0] == 7.0).all() and (score[r, j0 + n:] == 7.0).all()
+    rng = np.random.default_rng(3)
+    for n, K in ((1, 1), (7, 3), (300, 40), (5000, 512), (5000, 4999), (37, 37), (20, 50)):
+        sc = rng.choice(np.round(rng.standard_normal(max(n // 3, 2)), 1).astype(np.float32) + 0.05, size=(3, n + 5)).astype(np.float32)
+        sc[1, n // 2:n] = -np.inf                            # the pools a row does not see yet
+        sel = orc.glm_topk(sc, n, K)
+        for r in range(3):
+            order = np.lexsort((np.arange(n), -sc[r, :n].astype(np.float64)))      # by score descending, then position
+            want = np.sort(order[:min(K, n)])
+            assert np.array_equal(sel[r, :min(K, n)], want), (n, K, r)
+            assert (sel[r, min(K, n):] == -1).all()
