@@ -191,3 +191,43 @@ def test_glm_top_k(ops, T, n, K):
         sb = DevBuf.of(g, np.full((T, K), -1, np.int32))
         ops.ok(ops.k.topk(ops.raw(), scb.ptr, sb.ptr, T, n, ld, K), "ns_topk")
         assert np.array_equal(sb.read(np.int32).reshape(T, K), want)
+
+
+def test_glm_indexer_feeds_the_latent_attention(ops):
+    """The engine's sequence for a layer (llm/glm5next/src/engine.rs:1965-2013): pooled keys pass by pass, then for a verify
+    pass the pool scores (the iq . pooled^T product is the engine's GEMM: taken here in numpy), the top pools a row, the
+    counts - and ns_mla_attend_sel over those lists. The lists are the oracle's select of the scores the GPU produced, bit
+    for bit; the attention is the oracle's over the same lists."""
+    g = ops.gpu
+    D, hh, kp, H, L = 128, 4, 16, 16, 512
+    n_tok, T = 301, 3
+    pos0 = n_tok - T
+    ik, ig, ape = orc.randn(21, (n_tok, D)), orc.randn(22, (n_tok, D)), orc.randn(23, (4, D), 0.5)
+    rb, pb, ab = DevBuf(g, 8 * 2 * D * 4), DevBuf(g, (n_tok // 4 + 1) * D * 4), DevBuf.of(g, ape)
+    rb.fill(0)
+    pb.fill(0)
+    pos = 0
+    for t in (200, 60, 38, T):
+        kb, gb = DevBuf.of(g, ik[pos:pos + t]), DevBuf.of(g, ig[pos:pos + t])
+        ops.ok(ops.k.idx_pool(ops.raw(), rb.ptr, kb.ptr, gb.ptr, ab.ptr, pb.ptr, pos, t, D), "ns_idx_pool")
+        pos += t
+    n = (pos0 + T) // 4
+    assert n > kp
+    pooled = pb.read(np.float32).reshape(-1, D)[:n]
+    iq, w = orc.randn(24, (T * hh, D)), orc.randn(25, (T, hh))
+    S = (iq @ pooled.T).astype(np.float32)                                   # [T hh][n]
+    Sb, wb, scb, selb = DevBuf.of(g, S), DevBuf.of(g, w), DevBuf(g, T * n * 4), DevBuf.of(g, np.full((T, kp), -1, np.int32))
+    ops.ok(ops.k.idx_score(ops.raw(), Sb.ptr, wb.ptr, scb.ptr, T, hh, 0, n, n, pos0), "ns_idx_score")
+    ops.ok(ops.k.topk(ops.raw(), scb.ptr, selb.ptr, T, n, n, kp), "ns_topk")
+    score = scb.read(np.float32).reshape(T, n)
+    sel = selb.read(np.int32).reshape(T, kp)
+    assert np.array_equal(sel, orc.glm_topk(score, n, kp))
+    for r in range(T):
+        assert (sel[r] < (pos0 + r + 1) // 4).all() and (np.diff(sel[r]) > 0).all()      # pools the row sees, in position order
+    cnt = np.array([kp if (pos0 + r + 1) // 4 > kp else -1 for r in range(T)], np.int32)
+    qa = orc.randn(26, (T, H * L), 0.3)
+    rows = orc.f2h(orc.randn(27, (n_tok, L))).view(np.uint8).reshape(n_tok, 2 * L)
+    u = DevBuf(g, T * H * L * 4)
+    u.fill(0xFF)
+    ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, 0.044, sel=selb, sel_cnt=DevBuf.of(g, cnt), K=kp)
+    close(u.read(np.float32).reshape(T, H * L), orc.glm_mla_attend_sel(qa, rows, False, T, H, L, pos0, 0.044, sel, cnt, kp))
