@@ -281,9 +281,8 @@ __global__ __launch_bounds__(TOPK_WG) void glm_topk_kernel(const float* __restri
 // once, coalesced, all in flight) - the row is read from memory once instead of five times with a dependent load an
 // iteration. The histogram has a copy a lane (64 copies, 257 words apart: the lanes of a wave never meet in an address or
 // a bank, however few digits the row's scores share - the top digit, sign and exponent, takes a handful of values), the
-// digit is found by a suffix scan over 256 threads instead of one thread's walk, and the ordered compaction is one
-// work-group scan an i: a position's place in the list = the greater keys before it + the equal ones before it that
-// are still taken, both counts riding in one packed scan.
+// digit is found by a suffix scan over 256 threads instead of one thread's walk, and a position's place in the list = the
+// greater keys before it + the equal ones before it that are still taken, both from ballots and one scan (below).
 template <int PER>
 __global__ __launch_bounds__(TOPK_WG) void glm_topk_reg_kernel(const float* __restrict__ score, int32_t* __restrict__ sel, int n, int64_t ld, int K) {
     constexpr int NC = 64, CS = 257;
@@ -340,19 +339,44 @@ __global__ __launch_bounds__(TOPK_WG) void glm_topk_reg_kernel(const float* __re
         }
         __syncthreads();
     }
+    // The list in position order: position j = i 1024 + 64 wv + lane. Every wave counts its greater and its equal keys a
+    // slice i (two ballots), the counts' running sums over (slice, wave) - 16 PER entries in that order - are one
+    // work-group scan each, and a key's place is then its wave's running sum plus the lanes before it in its ballot.
     const uint32_t kth = st[0], ties = st[2];
-    uint32_t base_gt = 0, base_eq = 0;
+    uint32_t* const cg = hist;                                     // [PER][16] greater keys a (slice, wave), then their running sums
+    uint32_t* const ce = hist + PER * 16;                          // the same for the equal keys
+    constexpr int NW = TOPK_WG / 64;
+    static_assert(PER * NW <= TOPK_WG && 2 * PER * NW <= NC * CS, "one scan entry a thread");
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-        if (i * TOPK_WG >= n || base_gt + std::min(base_eq, ties) >= (uint32_t) K) break;      // (uniform)
+        const int j = i * TOPK_WG + lid;
+        const bool valid = j < n;
+        const uint64_t bg = __ballot(valid && key[i] > kth), be = __ballot(valid && key[i] == kth);
+        if (lane == 0) {
+            cg[i * NW + wv] = (uint32_t) __popcll(bg);
+            ce[i * NW + wv] = (uint32_t) __popcll(be);
+        }
+    }
+    __syncthreads();
+    uint32_t total;
+    const uint32_t mg = lid < PER * NW ? cg[lid] : 0u, me = lid < PER * NW ? ce[lid] : 0u;
+    const uint32_t pg = wg_exclusive_scan(mg, wsum, total);
+    const uint32_t pe = wg_exclusive_scan(me, wsum, total);
+    if (lid < PER * NW) {
+        cg[lid] = pg;
+        ce[lid] = pe;
+    }
+    __syncthreads();
+    const uint64_t below = ((uint64_t) 1 << lane) - 1;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
         const int j = i * TOPK_WG + lid;
         const bool valid = j < n, gt = valid && key[i] > kth, eq = valid && key[i] == kth;
-        uint32_t total;
-        const uint32_t before = wg_exclusive_scan((gt ? 1u : 0u) | (eq ? 0x10000u : 0u), wsum, total);
-        const uint32_t eq_before = base_eq + (before >> 16), at = base_gt + (before & 0xFFFFu) + std::min(eq_before, ties);
+        const uint64_t bg = __ballot(gt), be = __ballot(eq);
+        if (!(bg | be)) continue;                                  // (uniform: nothing of this wave's slice is taken)
+        const uint32_t eq_before = ce[i * NW + wv] + (uint32_t) __popcll(be & below);
+        const uint32_t at = cg[i * NW + wv] + (uint32_t) __popcll(bg & below) + std::min(eq_before, ties);
         if ((gt || (eq && eq_before < ties)) && at < (uint32_t) K) sel[r * K + at] = j;
-        base_gt += total & 0xFFFFu;
-        base_eq += total >> 16;
     }
 }
 
