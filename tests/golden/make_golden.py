@@ -15,7 +15,14 @@ Rules restated (their sources are the public formats the reference follows):
                          away from zero, clamp to +-127 (kernels/llm/glm5next/glm.cpp:1282-1299)
   attention              softmax(q K^T scale + causal / window mask) V over the widened cache, float64
   absorbed MLA           softmax(qa C^T scale) C[:, :512] over the half latent cache, float64
-The files are loaded with numpy.load(allow_pickle=False)."""
+  YaRN rope              ggml's rope_yarn on adjacent pairs: the angle pos * base^(-i0 / n) scaled by freq_scale, mixed
+                         with the unscaled one by the ramp between the correction dims times ext_factor; cos and sin
+                         times mscale (kernels/llm/deepseek2/ds2.cpp:15-34, 59-83), float64
+  GLM's indexer          pooled key = the softmax over a pool's 4 members of (gate + ape) applied to their keys; pool score =
+                         sum over heads of max(S, 0) w, -inf for pools a row does not see; the K best as ascending
+                         positions, ties at the K-th value to the lowest positions (kernels/llm/glm5next/glm.cpp:876-1019)
+The files are loaded with numpy.load(allow_pickle=False). A file whose arrays would not change is left as it is (a zip's
+bytes carry its writing time)."""
 import hashlib
 import os
 
@@ -136,10 +143,54 @@ def main():
     rows = glm_q8rows(x)
     files["mla.npz"] = {"shape": np.array([T, H, pos0], np.int64), "cache": cache.view(np.uint16), "qa": qa, "scale": np.array([scale]), "u": u,
                         "glm_x": x, "glm_rows": rows}
+    # ---- the steps either side of the latent attention: YaRN rope on a decode step's q_pe, GLM's indexer
+    r2 = np.random.default_rng(20240612)
+    T, H, head, off, n_dims, pos0 = 3, 4, 192, 128, 64, 1000
+    xr = r2.standard_normal((T, H * head), dtype=np.float32)
+    yarn = np.array([10000.0, 0.025, 1.0, 1.3, 10.0, 23.0])             # base, freq_scale, ext_factor, mscale, corr dims
+    i = np.arange(n_dims // 2)
+    ramp = 1.0 - np.clip((i - yarn[4]) / max(0.001, yarn[5] - yarn[4]), 0.0, 1.0)
+    yr = xr.astype(np.float64)
+    for t in range(T):
+        extrap = (pos0 + t) * yarn[0] ** (-2.0 * i / n_dims)
+        theta = yarn[1] * extrap * (1 - ramp * yarn[2]) + extrap * ramp * yarn[2]
+        c, sn = np.cos(theta) * yarn[3], np.sin(theta) * yarn[3]
+        for h in range(H):
+            a = xr[t, h * head + off:h * head + off + n_dims].astype(np.float64)
+            yr[t, h * head + off:h * head + off + n_dims:2] = a[0::2] * c - a[1::2] * sn
+            yr[t, h * head + off + 1:h * head + off + n_dims:2] = a[0::2] * sn + a[1::2] * c
+    D, n_tok, hh, K = 32, 50, 4, 5
+    ik, ig = r2.standard_normal((n_tok, D), dtype=np.float32), r2.standard_normal((n_tok, D), dtype=np.float32)
+    ape = r2.standard_normal((4, D), dtype=np.float32) * np.float32(0.5)
+    pooled = np.zeros((n_tok // 4, D))
+    for j in range(n_tok // 4):
+        lg = ig[4 * j:4 * j + 4].astype(np.float64) + ape
+        wgt = np.exp(lg - lg.max(axis=0))
+        pooled[j] = (wgt * ik[4 * j:4 * j + 4]).sum(axis=0) / wgt.sum(axis=0)
+    Tq, q0 = 3, n_tok - 3                                                 # a verify pass of 3 rows at positions 47..49
+    npool = n_tok // 4
+    S = r2.standard_normal((Tq * hh, npool), dtype=np.float32)
+    S[:, 5] = S[:, 3]                                                     # equal scores: the tie rule decides
+    w = np.abs(r2.standard_normal((Tq, hh), dtype=np.float32))
+    score = np.full((Tq, npool), -np.inf)
+    for r in range(Tq):
+        nv = (q0 + r + 1) // 4
+        score[r, :nv] = (np.maximum(S[r * hh:(r + 1) * hh, :nv].astype(np.float64), 0.0) * w[r].astype(np.float64)[:, None]).sum(axis=0)
+    score32 = score.astype(np.float32)
+    score32[:, 5] = score32[:, 3]
+    sel = np.stack([np.sort(np.lexsort((np.arange(npool), -score32[r].astype(np.float64)))[:K]) for r in range(Tq)]).astype(np.int32)
+    files["select.npz"] = {"rope_shape": np.array([T, H, head, off, n_dims, pos0], np.int64), "rope_x": xr, "rope_yarn": yarn, "rope_y": yr,
+                           "idx_shape": np.array([D, n_tok, hh, K, Tq, q0], np.int64), "idx_ik": ik, "idx_ig": ig, "idx_ape": ape,
+                           "idx_pooled": pooled, "idx_S": S, "idx_w": w, "idx_score": score, "idx_score32": score32, "idx_sel": sel}
     lines = []
     for fn, arrs in files.items():
         path = os.path.join(HERE, fn)
-        np.savez_compressed(path, **arrs)
+        same = False
+        if os.path.exists(path):
+            with np.load(path, allow_pickle=False) as old:
+                same = set(old.files) == set(arrs) and all(np.array_equal(old[k], arrs[k], equal_nan=True) and old[k].dtype == np.asarray(arrs[k]).dtype for k in arrs)
+        if not same:
+            np.savez_compressed(path, **arrs)
         lines.append("%s  %s" % (hashlib.sha256(open(path, "rb").read()).hexdigest(), fn))
     open(os.path.join(HERE, "MANIFEST.sha256"), "w").write("\n".join(lines) + "\n")
     print("\n".join(lines))

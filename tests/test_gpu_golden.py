@@ -53,3 +53,31 @@ def test_mla_and_glm_rows_on_the_fixtures(ops):
     yb = DevBuf(g, rows.nbytes)
     ops.to_q8row(DevBuf.of(g, z["glm_x"]), yb, rows.shape[0], 512)
     assert np.array_equal(yb.read(np.uint8).reshape(rows.shape), rows)
+
+
+def test_rope_and_indexer_on_the_fixtures(ops):
+    z = np.load(os.path.join(GOLD, "select.npz"), allow_pickle=False)
+    g = ops.gpu
+    T, H, head, off, n_dims, pos0 = (int(x) for x in z["rope_shape"])
+    xb = DevBuf.of(g, z["rope_x"])
+    ops.ok(ops.k.ds2_rope(ops.raw(), xb.ptr, T, H, H * head, head, off, n_dims, pos0, *(float(v) for v in z["rope_yarn"]), None, 0, 0), "ns_ds2_rope")
+    assert np.abs(xb.read(np.float32).reshape(T, H * head) - z["rope_y"]).max() < 1e-4 * np.abs(z["rope_x"]).max() * float(z["rope_yarn"][3])
+    D, n_tok, hh, K, Tq, q0 = (int(x) for x in z["idx_shape"])
+    rb, pb, ab = DevBuf(g, 8 * 2 * D * 4), DevBuf(g, (n_tok // 4) * D * 4), DevBuf.of(g, z["idx_ape"])
+    rb.fill(0)
+    pb.fill(0)
+    pos = 0
+    for t in (30, 1, 2, 5, 12):
+        kb, gb = DevBuf.of(g, z["idx_ik"][pos:pos + t]), DevBuf.of(g, z["idx_ig"][pos:pos + t])
+        ops.ok(ops.k.idx_pool(ops.raw(), rb.ptr, kb.ptr, gb.ptr, ab.ptr, pb.ptr, pos, t, D), "ns_idx_pool")
+        pos += t
+    assert np.abs(pb.read(np.float32).reshape(-1, D) - z["idx_pooled"]).max() < 1e-5
+    npool = n_tok // 4
+    Sb, wb, scb = DevBuf.of(g, z["idx_S"]), DevBuf.of(g, z["idx_w"]), DevBuf(g, Tq * npool * 4)
+    ops.ok(ops.k.idx_score(ops.raw(), Sb.ptr, wb.ptr, scb.ptr, Tq, hh, 0, npool, npool, q0), "ns_idx_score")
+    score, want = scb.read(np.float32).reshape(Tq, npool), z["idx_score"]
+    assert np.array_equal(np.isneginf(score), np.isneginf(want))
+    assert np.abs(score[np.isfinite(want)] - want[np.isfinite(want)]).max() < 1e-5
+    s32, selb = DevBuf.of(g, z["idx_score32"]), DevBuf.of(g, np.full((Tq, K), -1, np.int32))
+    ops.ok(ops.k.topk(ops.raw(), s32.ptr, selb.ptr, Tq, npool, npool, K), "ns_topk")
+    assert np.array_equal(selb.read(np.int32).reshape(Tq, K), z["idx_sel"])

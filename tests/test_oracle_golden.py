@@ -26,7 +26,7 @@ def test_manifest():
         digest, fn = ln.split()
         assert hashlib.sha256(open(os.path.join(GOLD, fn), "rb").read()).hexdigest() == digest, fn
         seen += 1
-    assert seen == 2
+    assert seen == 3
 
 
 @pytest.mark.parametrize("kt", [0, 1, 2, 3])
@@ -52,3 +52,25 @@ def test_mla_and_glm_rows():
     assert np.abs(u64 - z["u"]).max() < 1e-12
     assert orc.compare(orc.mla_decode_u(z["qa"], z["cache"], T, H, pos0, scale), z["u"])[0] < 5e-6
     assert np.array_equal(orc.glm_to_q8row(z["glm_x"], 512), z["glm_rows"])
+
+
+def test_rope_and_indexer():
+    z = load("select.npz")
+    T, H, head, off, n_dims, pos0 = (int(x) for x in z["rope_shape"])
+    y = orc.ds2_rope(z["rope_x"].copy(), T, H, H * head, head, off, n_dims, pos0, *(float(v) for v in z["rope_yarn"]))
+    assert np.abs(y - z["rope_y"]).max() < 1e-4 * np.abs(z["rope_x"]).max() * float(z["rope_yarn"][3])     # float32 angles near 1000 radians
+    D, n_tok, hh, K, Tq, q0 = (int(x) for x in z["idx_shape"])
+    ring = np.zeros((8, 2 * D), np.float32)
+    pooled = np.zeros((n_tok // 4, D), np.float32)
+    pos = 0
+    for t in (30, 1, 2, 5, 12):
+        orc.glm_idx_pool(ring, z["idx_ik"][pos:pos + t], z["idx_ig"][pos:pos + t], z["idx_ape"], pooled, pos, t, D)
+        pos += t
+    assert pos == n_tok and np.abs(pooled - z["idx_pooled"]).max() < 1e-5
+    npool = n_tok // 4
+    score = np.zeros((Tq, npool), np.float32)
+    orc.glm_idx_score(z["idx_S"], z["idx_w"], score, Tq, hh, 0, npool, q0)
+    want = z["idx_score"]
+    assert np.array_equal(np.isneginf(score), np.isneginf(want))
+    assert np.abs(score[np.isfinite(want)] - want[np.isfinite(want)]).max() < 1e-5
+    assert np.array_equal(orc.glm_topk(z["idx_score32"], npool, K), z["idx_sel"])
