@@ -1,5 +1,5 @@
-// attn_prefill.hip: causal GQA flash attention of a prompt pass's rows against the KV cache (half or bfloat16 rows,
-// D = 128) for gfx950.
+// attn_prefill.hip: causal GQA flash attention of a prompt pass's rows against the KV cache (half, bfloat16, q8_0 or q4_0
+// rows; D = 128 or 256) for gfx950.
 //
 // Bound: MFMA. 4 D flops a visible (row, key) pair against 2 x 2 D bytes a key shared by every row that sees it:
 // thousands of flops a byte at prompt lengths.
@@ -8,16 +8,18 @@
 // of one query head (a wave 32 of them: two 16-row MFMA tiles) and streams the keys its rows see in 64-key tiles,
 // heaviest row blocks first (the last block sees the most keys). The G query heads of a key head on one row block are
 // neighbours in the logical order and, through the XCD-aware mapping of work-group ids, share one L2. A tile's K and V
-// rows are fetched by all 512 threads (16-byte chunks): global -> registers two tiles ahead -> LDS one tile ahead, two
-// register sets, two LDS buffers, one barrier a tile.
+// rows are fetched by all 512 threads (16-byte chunks). The 8-wave form over 16-bit rows sends them global -> LDS directly
+// (global_load_lds_dwordx4, two tiles ahead, three unpadded buffers a stream, the bank swizzle applied to the global
+// addresses, one barrier a tile that counts the transfers in flight); the other forms (4 waves, quantized rows, D = 256)
+// go global -> registers two tiles ahead -> LDS one tile ahead: two register sets, two padded LDS buffers.
 //
 // A wave's tile step, in the transposed orientation (a lane owns one query row of each row tile, so the row maximum,
 // the rescale and the normalisation never leave the lane):
-//   S^T[key][row] = K Q^T        K from LDS as the A operand (ds_read_b128, rows padded to 288 bytes), Q^T in registers
+//   S^T[key][row] = K Q^T        K from LDS as the A operand (ds_read_b128; rows padded to 288 bytes, or swizzled), Q^T in registers
 //   base-2 online softmax in float32 (scale folded into the exponent's fma; the accumulators rescaled only when a
 //   row's maximum moved); only 32-key halves crossing a row's causal or window edge are masked
 //   P^T -> 16 bit = the B operand of the second product as it stands
-//   O^T[d][row]  += V^T P^T      V^T from LDS through ds_read_b64_tr_b16 (rows padded to 288 bytes)
+//   O^T[d][row]  += V^T P^T      V^T from LDS through ds_read_b64_tr_b16 (rows padded to 288 bytes, or swizzled)
 //
 // Reference behaviour kept: kernels/llm/museglimmer/silo/attn.cpp:56-267 and kernels/llm/qwen35/silo/attn.cpp:105-313
 // (prompt form: causal from p0, window, ring slots, 16-bit operands with float32 softmax and accumulation, rows past T
