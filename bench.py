@@ -189,6 +189,53 @@ def timed(w, steps, warmup):
     return ms, main, max(0.0, ms * 1e6 - main)
 
 
+def graph_step_ms(w, n=50):
+    """ms a step when `n` steps are captured into a HIP graph on the library's stream and replayed - how a serving loop
+    queues a token's launches (no host call a kernel, the runtime hands the device the whole chain). Only for the
+    workloads of two launches a step; None where the capture does not go through. The library records kernel launches
+    only (no memset, no allocation), so the replay does what the calls did."""
+    import ctypes as C
+    if w.kind == "pre" or w.kind == "prefill" or (w.kind == "mla" and w.T > 16):
+        return None
+    g = w.ops.gpu
+    try:
+        hip = C.CDLL("libamdhip64.so")
+        hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+        hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
+        hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+        hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+        hip.hipGraphDestroy.argtypes = [C.c_void_p]
+        stream = C.cast(C.c_void_p(g.api.gpu_queue(g.raw)), C.POINTER(C.c_void_p))[0]
+        g.sync()
+        graph, ex = C.c_void_p(), C.c_void_p()
+        if hip.hipStreamBeginCapture(stream, 2) != 0:                 # (relaxed mode)
+            return None
+        try:
+            for _ in range(n):
+                w.step()
+        finally:
+            rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+        if rc != 0 or not graph.value or hip.hipGraphInstantiate(C.byref(ex), graph, None, None, 0) != 0:
+            return None
+        try:
+            for _ in range(3):
+                hip.hipGraphLaunch(ex, stream)
+            g.sync()
+            t0 = g.stamp()
+            hip.hipGraphLaunch(ex, stream)
+            hip.hipGraphLaunch(ex, stream)
+            t1 = g.stamp()
+            ns = g.elapsed_ns(t0, t1) / (2 * n)
+        finally:
+            g.sync()
+            hip.hipGraphExecDestroy(ex)
+            hip.hipGraphDestroy(graph)
+        return ns / 1e6
+    except Exception:
+        return None
+
+
 # HBM bytes per launch of each workload's dominant kernel as rocprofv3 counted them (FETCH_SIZE + WRITE_SIZE per dispatch,
 # each scaled by what the same counter reads for a plain copy kernel of known size). A counter run cannot be made from
 # inside this script: the figure is read from the committed summary of that run, profiles/<kernel>_<workload>.md (its line
@@ -324,6 +371,7 @@ def main():
         nbuf = min(nbuf, 40)
         w = Workload(ops, name, nbuf)
         ms, main_ns, merge_ns = timed(w, steps, warmup)
+        w.graph_ms = graph_step_ms(w)
         return w, ms, main_ns, merge_ns
 
     w, ms, main_ns, merge_ns = run(a.workload, a.steps, a.warmup)
@@ -348,6 +396,8 @@ def main():
     }
     if merge_ns:
         line["merge_kernel_us"] = round(merge_ns / 1e3, 2)
+    if w.graph_ms:
+        line["graph_ms_per_step"] = round(w.graph_ms, 5)
     del w
     if not a.no_extra:
         others = {}
@@ -359,6 +409,8 @@ def main():
             others[name] = {"ms_per_step": round(m2, 5), "step_" + ("TFLOP/s" if ww.kind not in ("decode", "pre") else "GB/s"):
                             round((ww.flops / (m2 * 1e-3) / 1e12) if ww.kind not in ("decode", "pre") else (ww.bytes / (m2 * 1e-3) / 1e9), 2), "roofline": r,
                             "merge_kernel_us": round(g2 / 1e3, 2)}
+            if ww.graph_ms:
+                others[name]["graph_ms_per_step"] = round(ww.graph_ms, 5)
             del ww
             if not a.no_cpu:
                 others[name]["cpu_baseline"] = cpu_baseline(name)
