@@ -101,7 +101,11 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // value tile (rows + 32 bytes)
     constexpr int RS = DMA ? D * 2 : D * 2 + 32;
     constexpr int VTILE = TILE * RS;
-    constexpr int STAGE = DMA ? 2 * VTILE : VTILE;
+    // q8_0 rows of 128 values: the tile's raw rows go global -> LDS too (rows of 136 bytes as 9 chunks of 16: the ninth is
+    // the row's last 16 bytes, so the 8 bytes of scales sit in its upper half), one buffer a stream behind the value stage
+    constexpr bool QDMA = KT == 1 && D == 128;
+    constexpr int QROW = 144, QRAW = TILE * QROW;
+    constexpr int STAGE = DMA ? 2 * VTILE : QDMA ? VTILE + 2 * QRAW : VTILE;
     constexpr int OROW = D + 4;                                    // floats a row of a wave's merge buffer
     constexpr int MERGE = RT * 16 * OROW * 4;
     // a wave's own region: its value stage while it streams, its (O, m, l) for the merge afterwards
@@ -258,6 +262,58 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         }
     };
 
+    uint32_t qoff5[QDMA ? 5 : 1];
+    if constexpr (QDMA) {
+#pragma unroll
+        for (int i = 0; i < 5; ++i) {
+            const int u = std::min(i * 64 + lane, TILE * 9 - 1), row = u / 9, c = u % 9;
+            qoff5[i] = (uint32_t) (row * p.row_stride) + (uint32_t) (c < 8 ? c * 16 : 120);
+        }
+    }
+    auto qdma_tile = [&](int64_t ti, int which) __attribute__((always_inline)) {
+        const int j0 = (int) (ti * TILE - jb);
+        const bool plain = !selp && !p.wrap && j0 >= 0 && j0 + TILE - 1 <= span;
+        const uint8_t* base = (which ? vbase : kbase) + (plain ? (jb_slot + j0) * p.row_stride : 0);
+#pragma unroll
+        for (int i = 0; i < 5; ++i) {
+            uint32_t off = qoff5[i];
+            if (!plain) {
+                const int u = std::min(i * 64 + lane, TILE * 9 - 1), row = u / 9, c = u % 9;
+                off = (uint32_t) tile_off(ti, j0, row) + (uint32_t) (c < 8 ? c * 16 : 120);
+            }
+            if (i < 4 || lane < 32) {
+                const uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t) (uintptr_t) (stage + VTILE + which * QRAW + i * 1024));
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+                asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m), "v"(off), "s"(base) : "memory", "m0");
+#pragma clang diagnostic pop
+            }
+        }
+    };
+    // the raw tile out of LDS into the register set the quantized path works on (the same registers a global load fills)
+    auto qread_tile = [&](R& r) __attribute__((always_inline)) {
+        const uint8_t* rk = stage + VTILE;
+        const uint8_t* rv = stage + VTILE + QRAW;
+#pragma unroll
+        for (int kt2 = 0; kt2 < 2; ++kt2) {
+            const uint8_t* kr = rk + (kt2 * 16 + n) * QROW;
+#pragma unroll
+            for (int kb = 0; kb < KB; kb += 2) {
+                const uint4 x = *reinterpret_cast<const uint4*>(kr + kb * 32 + g4 * 16);
+                r.k[kt2][kb][0] = x.x; r.k[kt2][kb][1] = x.y;
+                r.k[kt2][kb + 1][0] = x.z; r.k[kt2][kb + 1][1] = x.w;
+                r.ksc[kt2][kb] = r.ksc[kt2][kb + 1] = *reinterpret_cast<const uint16_t*>(kr + 136 + 2 * (kb + g4 / 2));
+            }
+        }
+        const int cp = lane % R::CPR, kr0 = lane / R::CPR;
+#pragma unroll
+        for (int i = 0; i < R::NLV; ++i) {
+            const uint8_t* vr = rv + (kr0 + R::KPI * i) * QROW;
+            r.v[i] = *reinterpret_cast<const uint4*>(vr + cp * 16);
+            r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + 136 + 2 * (cp / 2));
+        }
+    };
+
     // ---- this wave's tiles: absolute tile index % 4 == w, over [jb, je). The first one is requested before anything
     // else: nothing in it depends on the queries
     const int64_t tb = jb / TILE, te = jb < je ? (je + TILE - 1) / TILE : tb;
@@ -267,6 +323,9 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         if constexpr (DMA) {
             dma_tile(ti, 0);
             dma_tile(ti, 1);
+        } else if constexpr (QDMA) {
+            qdma_tile(ti, 0);
+            qdma_tile(ti, 1);
         } else {
             load_tile(ra, ti);
         }
@@ -535,6 +594,22 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         if constexpr (DMA) {
             for (; ti + WAVES < te; ti += WAVES) process_tile(ra, ti, more);
             process_tile(ra, ti, last);
+        } else if constexpr (QDMA) {
+            // the tile's raw rows have landed (requested a tile ago); once they are in registers the next tile's are
+            // requested into the same two buffers and travel under this tile's arithmetic
+            for (;; ti += WAVES) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                qread_tile(ra);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                const bool has_next = ti + WAVES < te;
+                if (has_next) {
+                    qdma_tile(ti + WAVES, 0);
+                    qdma_tile(ti + WAVES, 1);
+                }
+                process_tile(ra, ti, more);
+                if (!has_next) break;
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         } else {
             while (ti + 2 * WAVES < te) {
                 load_tile(rb, ti + WAVES);
