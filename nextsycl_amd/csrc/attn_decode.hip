@@ -101,10 +101,18 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // value tile (rows + 32 bytes)
     constexpr int RS = DMA ? D * 2 : D * 2 + 32;
     constexpr int VTILE = TILE * RS;
-    // q8_0 rows of 128 values: the tile's raw rows go global -> LDS too (rows of 136 bytes as 9 chunks of 16: the ninth is
-    // the row's last 16 bytes, so the 8 bytes of scales sit in its upper half), one buffer a stream behind the value stage
-    constexpr bool QDMA = KT == 1 && D == 128;
-    constexpr int QROW = 144, QRAW = TILE * QROW;
+    // quantized rows: the tile's raw rows go global -> LDS too, a row as QCH chunks of 16 bytes - the last chunk is the
+    // row's last 16 bytes (rows of 136 or 72 bytes are no whole number of chunks: their last chunk overlaps the one before
+    // and the scales sit in its upper half) - one buffer a stream behind the value stage
+    // (q4_0 rows of 128 values keep the register path: their arithmetic bounds them - 19.7 against 20.7 us for a 4-row
+    // pass over 65536 keys - where q8_0 rows gain 13 % and rows of 256 values 11 - 14 %)
+    constexpr bool QDMA = KT == 1 || (KT == 2 && D == 256);
+    constexpr int QRB = KT == 1 ? D + D / 16 : D / 2 + D / 16;     // bytes a cache row
+    constexpr int QVB = KT == 1 ? D : D / 2;                       // of them values
+    constexpr int QCH = (QRB + 15) / 16, QROW = QCH * 16, QRAW = TILE * QROW;
+    constexpr int QSOFF = (QCH - 1) * 16 + QVB - (QRB - 16);       // where a row's scales sit in its LDS row
+    constexpr int QNI = (TILE * QCH + 63) / 64;                    // transfer instructions a tile and stream
+    static_assert(!QDMA || (TILE * QCH) % 64 == 32 || (TILE * QCH) % 64 == 0, "the last instruction is whole or half");
     constexpr int STAGE = DMA ? 2 * VTILE : QDMA ? VTILE + 2 * QRAW : VTILE;
     constexpr int OROW = D + 4;                                    // floats a row of a wave's merge buffer
     constexpr int MERGE = RT * 16 * OROW * 4;
@@ -218,7 +226,8 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // quantized rows: the tile's keys (MFMA A layout) and values raw into registers
     // (interior tiles of an unwrapped, unlisted cache: a wave-uniform tile address plus a lane's row offset, worked out once)
     const uint32_t qk_lane = (uint32_t) (n * p.row_stride), qv_lane = (uint32_t) ((lane / R::CPR) * p.row_stride);
-    auto load_rows = [&](R& r, auto krow, auto vrow) __attribute__((always_inline)) {
+    // (soff: where a row's scales start - behind its values in the cache, in its last chunk's upper part in LDS)
+    auto load_rows = [&](R& r, auto krow, auto vrow, int soff) __attribute__((always_inline)) {
 #pragma unroll
         for (int kt2 = 0; kt2 < 2; ++kt2) {
             const uint8_t* kr = krow(kt2);
@@ -232,12 +241,12 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                         const u4a8 x = *reinterpret_cast<const u4a8*>(kr + kb * 32 + g4 * 16);
                         r.k[kt2][kb][0] = x[0]; r.k[kt2][kb][1] = x[1];
                         r.k[kt2][kb + 1][0] = x[2]; r.k[kt2][kb + 1][1] = x[3];
-                        r.ksc[kt2][kb] = r.ksc[kt2][kb + 1] = *reinterpret_cast<const uint16_t*>(kr + D + 2 * (kb + g4 / 2));
+                        r.ksc[kt2][kb] = r.ksc[kt2][kb + 1] = *reinterpret_cast<const uint16_t*>(kr + soff + 2 * (kb + g4 / 2));
                     }
                 } else {
                     const uint2 x = *reinterpret_cast<const uint2*>(kr + kb * 16 + (g4 & 1) * 8);
                     r.k[kt2][kb][0] = x.x; r.k[kt2][kb][1] = x.y;
-                    r.ksc[kt2][kb] = *reinterpret_cast<const uint16_t*>(kr + D / 2 + 2 * kb);
+                    r.ksc[kt2][kb] = *reinterpret_cast<const uint16_t*>(kr + soff + 2 * kb);
                 }
             }
         }
@@ -246,8 +255,8 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         for (int i = 0; i < R::NLV; ++i) {
             const uint8_t* vr = vrow(i);
             r.v[i] = *reinterpret_cast<const uint4*>(vr + cp * 16);
-            if constexpr (KT == 1) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D + 2 * (cp / 2));
-            if constexpr (KT == 2) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + D / 2 + 2 * cp);
+            if constexpr (KT == 1) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + soff + 2 * (cp / 2));
+            if constexpr (KT == 2) r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + soff + 2 * cp);
         }
     };
     auto load_tile = [&](R& r, int64_t ti) __attribute__((always_inline)) {
@@ -255,33 +264,39 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         if (!selp && !p.wrap && j0 >= 0 && j0 + TILE - 1 <= span) {
             const uint8_t* kt0 = kbase + (jb_slot + j0) * p.row_stride;
             const uint8_t* vt0 = vbase + (jb_slot + j0) * p.row_stride;
-            load_rows(r, [&](int kt2) { return kt0 + kt2 * 16 * p.row_stride + qk_lane; }, [&](int i) { return vt0 + R::KPI * i * p.row_stride + qv_lane; });
+            load_rows(r, [&](int kt2) { return kt0 + kt2 * 16 * p.row_stride + qk_lane; }, [&](int i) { return vt0 + R::KPI * i * p.row_stride + qv_lane; }, QVB);
         } else {
             const int kr0 = lane / R::CPR;
-            load_rows(r, [&](int kt2) { return kbase + tile_off(ti, j0, kt2 * 16 + n); }, [&](int i) { return vbase + tile_off(ti, j0, kr0 + R::KPI * i); });
+            load_rows(r, [&](int kt2) { return kbase + tile_off(ti, j0, kt2 * 16 + n); }, [&](int i) { return vbase + tile_off(ti, j0, kr0 + R::KPI * i); }, QVB);
         }
     };
 
-    uint32_t qoff5[QDMA ? 5 : 1];
+    uint32_t qoff5[QDMA ? QNI : 1];
     if constexpr (QDMA) {
 #pragma unroll
-        for (int i = 0; i < 5; ++i) {
-            const int u = std::min(i * 64 + lane, TILE * 9 - 1), row = u / 9, c = u % 9;
-            qoff5[i] = (uint32_t) (row * p.row_stride) + (uint32_t) (c < 8 ? c * 16 : 120);
+        for (int i = 0; i < QNI; ++i) {
+            const int u = std::min(i * 64 + lane, TILE * QCH - 1), row = u / QCH, c = u % QCH;
+            qoff5[i] = (uint32_t) (row * p.row_stride) + (uint32_t) (c < QCH - 1 ? c * 16 : QRB - 16);
         }
     }
     auto qdma_tile = [&](int64_t ti, int which) __attribute__((always_inline)) {
         const int j0 = (int) (ti * TILE - jb);
         const bool plain = !selp && !p.wrap && j0 >= 0 && j0 + TILE - 1 <= span;
-        const uint8_t* base = (which ? vbase : kbase) + (plain ? (jb_slot + j0) * p.row_stride : 0);
+        const uint64_t base_v = (uint64_t) (uintptr_t) ((which ? vbase : kbase) + (plain ? (jb_slot + j0) * p.row_stride : 0));
+        // (wave-uniform by construction; said so to the compiler, which wants it in scalar registers)
+        // (the builtin returns a signed int: each half goes through uint32_t, or a low half with its top bit set would
+        // sign-extend over the high one)
+        const uint32_t base_lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) base_v);
+        const uint32_t base_hi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (base_v >> 32));
+        const uint8_t* base = reinterpret_cast<const uint8_t*>((uint64_t) base_lo | ((uint64_t) base_hi << 32));
 #pragma unroll
-        for (int i = 0; i < 5; ++i) {
+        for (int i = 0; i < QNI; ++i) {
             uint32_t off = qoff5[i];
             if (!plain) {
-                const int u = std::min(i * 64 + lane, TILE * 9 - 1), row = u / 9, c = u % 9;
-                off = (uint32_t) tile_off(ti, j0, row) + (uint32_t) (c < 8 ? c * 16 : 120);
+                const int u = std::min(i * 64 + lane, TILE * QCH - 1), row = u / QCH, c = u % QCH;
+                off = (uint32_t) tile_off(ti, j0, row) + (uint32_t) (c < QCH - 1 ? c * 16 : QRB - 16);
             }
-            if (i < 4 || lane < 32) {
+            if (i < QNI - 1 || (TILE * QCH) % 64 == 0 || lane < 32) {
                 const uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t) (uintptr_t) (stage + VTILE + which * QRAW + i * 1024));
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
@@ -294,24 +309,8 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     auto qread_tile = [&](R& r) __attribute__((always_inline)) {
         const uint8_t* rk = stage + VTILE;
         const uint8_t* rv = stage + VTILE + QRAW;
-#pragma unroll
-        for (int kt2 = 0; kt2 < 2; ++kt2) {
-            const uint8_t* kr = rk + (kt2 * 16 + n) * QROW;
-#pragma unroll
-            for (int kb = 0; kb < KB; kb += 2) {
-                const uint4 x = *reinterpret_cast<const uint4*>(kr + kb * 32 + g4 * 16);
-                r.k[kt2][kb][0] = x.x; r.k[kt2][kb][1] = x.y;
-                r.k[kt2][kb + 1][0] = x.z; r.k[kt2][kb + 1][1] = x.w;
-                r.ksc[kt2][kb] = r.ksc[kt2][kb + 1] = *reinterpret_cast<const uint16_t*>(kr + 136 + 2 * (kb + g4 / 2));
-            }
-        }
-        const int cp = lane % R::CPR, kr0 = lane / R::CPR;
-#pragma unroll
-        for (int i = 0; i < R::NLV; ++i) {
-            const uint8_t* vr = rv + (kr0 + R::KPI * i) * QROW;
-            r.v[i] = *reinterpret_cast<const uint4*>(vr + cp * 16);
-            r.vsc[i] = *reinterpret_cast<const uint16_t*>(vr + 136 + 2 * (cp / 2));
-        }
+        const int kr0 = lane / R::CPR;
+        load_rows(r, [&](int kt2) { return rk + (kt2 * 16 + n) * QROW; }, [&](int i) { return rv + (kr0 + R::KPI * i) * QROW; }, QSOFF);
     };
 
     // ---- this wave's tiles: absolute tile index % 4 == w, over [jb, je). The first one is requested before anything
