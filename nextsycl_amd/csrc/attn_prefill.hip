@@ -8,10 +8,12 @@
 // of one query head (a wave 32 of them: two 16-row MFMA tiles) and streams the keys its rows see in 64-key tiles,
 // heaviest row blocks first (the last block sees the most keys). The G query heads of a key head on one row block are
 // neighbours in the logical order and, through the XCD-aware mapping of work-group ids, share one L2. A tile's K and V
-// rows are fetched by all 512 threads (16-byte chunks). The 8-wave form over 16-bit rows sends them global -> LDS directly
-// (global_load_lds_dwordx4, two tiles ahead, three unpadded buffers a stream, the bank swizzle applied to the global
-// addresses, one barrier a tile that counts the transfers in flight); the other forms (4 waves, quantized rows, D = 256)
-// go global -> registers two tiles ahead -> LDS one tile ahead: two register sets, two padded LDS buffers.
+// rows are fetched by all the work-group's threads (16-byte chunks). Over 16-bit rows at D = 128 they go global -> LDS
+// directly (global_load_lds_dwordx4, unpadded buffers, the bank swizzle applied to the global addresses, one barrier a
+// tile that waits on the wave's transfers): the 8-wave form two tiles ahead into three buffers a stream, the barrier
+// leaving the newest tile's transfers in flight; the 4-wave form (two work-groups a CU) one tile ahead into two buffers a
+// stream, requested right behind the barrier that frees them. The other forms (quantized rows, D = 256) go global ->
+// registers two tiles ahead -> LDS one tile ahead: two register sets, two padded LDS buffers.
 //
 // A wave's tile step, in the transposed orientation (a lane owns one query row of each row tile, so the row maximum,
 // the rescale and the normalisation never leave the lane):
@@ -91,16 +93,20 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // c ^ 2 (r % 8)) so that neither the operand reads of 16 keys' same chunk nor the transposing reads meet a bank
     // conflict; three buffers a stream, each an array of its own so that the compiler can tell a transfer's target from
     // the arrays being read (it waits for every transfer in flight before a read it cannot tell apart)
-    constexpr bool DMA = D == 128 && KT == 0 && PW == 8;
+    // The 4-wave form (two work-groups a CU) has LDS for two buffers a stream: a tile is then requested one tile ahead,
+    // right behind the barrier that frees its buffer, and the next barrier waits for every transfer of the wave.
+    constexpr bool DMA = D == 128 && KT == 0 && (PW == 8 || PW == 4);
+    constexpr int NBUF = PW == 8 ? 3 : 2;                         // tile buffers a stream
+    constexpr int NJ = 16 / PW;                                   // transfer instructions a wave, tile and stream
     constexpr int TB = KT_TILE * 256;
     constexpr int TBP = TB + 512;                                 // (two waves' output staging, 8448 B each, go through one array)
     __shared__ __attribute__((aligned(16))) uint8_t lds[DMA ? 16 : 2 * (KBUF + VBUF)];
     __shared__ __attribute__((aligned(1024))) uint8_t dk0[DMA ? TBP : 16];
     __shared__ __attribute__((aligned(1024))) uint8_t dk1[DMA ? TBP : 16];
-    __shared__ __attribute__((aligned(1024))) uint8_t dk2[DMA ? TBP : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t dk2[DMA && NBUF == 3 ? TBP : 16];
     __shared__ __attribute__((aligned(1024))) uint8_t dv0[DMA ? TBP : 16];
     __shared__ __attribute__((aligned(1024))) uint8_t dv1[DMA ? TBP : 16];
-    __shared__ __attribute__((aligned(1024))) uint8_t dv2[DMA ? TBP : 16];
+    __shared__ __attribute__((aligned(1024))) uint8_t dv2[DMA && NBUF == 3 ? TBP : 16];
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -295,11 +301,11 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // lanes a row: lane l position l % 16 of row 4 (2 w + j) + l / 16), so it fetches the chunk that belongs there. Whole
     // tiles of an unwrapped cache: a wave-uniform tile address plus lane offsets worked out once; else the row is clamped
     // into the pass's keys (masked anyway) and a ring's slot worked out, as the register path does
-    uint32_t koff[DMA ? 2 : 1], voff[DMA ? 2 : 1];
+    uint32_t koff[DMA ? NJ : 1], voff[DMA ? NJ : 1];
     if constexpr (DMA) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int r = (w * 2 + j) * 4 + (lane >> 4), cp = lane & 15;
+        for (int j = 0; j < NJ; ++j) {
+            const int r = (w * NJ + j) * 4 + (lane >> 4), cp = lane & 15;
             koff[j] = (uint32_t) (r * p.row_stride) + (uint32_t) ((cp ^ (r & 15)) << 4);
             voff[j] = (uint32_t) (r * p.row_stride) + (uint32_t) ((cp ^ (2 * (r & 7))) << 4);
         }
@@ -319,12 +325,12 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         if (krel >= plain0 && krel <= plain1) {
             const uint8_t* sp = cache + (base + (int64_t) krel * KT_TILE) * p.row_stride;
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                dma16(sp, VAL ? voff[j] : koff[j], dst + (w * 2 + j) * 1024);
+            for (int j = 0; j < NJ; ++j)
+                dma16(sp, VAL ? voff[j] : koff[j], dst + (w * NJ + j) * 1024);
         } else {
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const int r = (w * 2 + j) * 4 + (lane >> 4), cp = lane & 15;
+            for (int j = 0; j < NJ; ++j) {
+                const int r = (w * NJ + j) * 4 + (lane >> 4), cp = lane & 15;
                 const int rel = std::min(std::max(krel * KT_TILE - kbeg32 + r, 0), kspan);
                 int64_t slot = kbeg_slot + rel;
                 if (p.wrap) {
@@ -332,7 +338,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                     slot = slot >= p.cap ? slot - p.cap : slot;
                 }
                 const uint32_t off = (uint32_t) (slot * p.row_stride) + (uint32_t) ((VAL ? cp ^ (2 * (r & 7)) : cp ^ (r & 15)) << 4);
-                dma16(cache, off, dst + (w * 2 + j) * 1024);
+                dma16(cache, off, dst + (w * NJ + j) * 1024);
             }
         }
     };
@@ -342,7 +348,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // transfers still in flight
     auto tile_barrier = [&]() __attribute__((always_inline)) {
         if constexpr (DMA) {
-            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+            if constexpr (NBUF == 3) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         } else {
@@ -553,6 +560,46 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         const std::true_type VALUES;
         lds_u8* const K0 = (lds_u8*) dk0; lds_u8* const K1 = (lds_u8*) dk1; lds_u8* const K2 = (lds_u8*) dk2;
         lds_u8* const W0 = (lds_u8*) dv0; lds_u8* const W1 = (lds_u8*) dv1; lds_u8* const W2 = (lds_u8*) dv2;
+       if constexpr (NBUF == 2) {
+        // ---- two buffers a stream, tile k in buffer k % 2; behind tile k's barrier K(k) and V(k - 1) have been read, so
+        // K(k + 2) and V(k + 1) are requested into their buffers there and have a tile's time to land:
+        //   step 2k   : A reads V(k-1) half 1, B's operands K(k) half 1
+        //   barrier (every transfer of this wave has landed: K(k+1), V(k));  request K(k+2), V(k+1)
+        //   step 2k+1 : A reads V(k) half 0,   B's operands K(k+1) half 0
+        dma(K0, kbase, 0, KEYS);
+        dma(W0, vbase, 0, VALUES);
+        dma(K1, kbase, 1, KEYS);
+        {   // the V buffer step 0 "adds" with zero weights must hold numbers
+            const u4v z = {0u, 0u, 0u, 0u};
+            for (uint32_t at = (uint32_t) tid * 16; at < (uint32_t) TB; at += PW * 64 * 16)
+                *reinterpret_cast<__attribute__((address_space(3))) u4v*>(W1 + at) = z;
+        }
+        tile_barrier();
+        {
+            s8v kpre[KPRE][KB];
+            kread(kpre, K0);
+            scores(sA, K0, kpre);
+        }
+        // kb / vb: the tile's own buffers; kn: the next tile's keys, vp: the tile before's values (the other buffers)
+        auto tile2 = [&](int k, lds_u8* kb, lds_u8* vb, lds_u8* kn, lds_u8* vp) __attribute__((always_inline)) {
+            step(sA, sB, kb + 32 * 256, vp + 32 * 256, 64 * k, !(64 * k >= w_full_beg && 64 * k + 32 <= w_full_end));
+            tile_barrier();
+            dma(kb, kbase, k + 2, KEYS);
+            dma(vp, vbase, k + 1, VALUES);
+            step(sB, sA, kn, vb, 64 * k + 32, !(64 * k + 32 >= w_full_beg && 64 * k + 64 <= w_full_end));
+        };
+        for (int k = 0; k < nt; k += 2) {
+            tile2(k, K0, W0, K1, W1);
+            if (k + 1 >= nt) break;
+            tile2(k + 1, K1, W1, K0, W0);
+        }
+        {
+            s8v vpre[VPRE];
+            lds_u8* const vl = (((nt - 1) & 1) ? W1 : W0) + 32 * 256;
+            vread(vpre, vl);
+            weigh(vl, vpre);
+        }
+       } else {
         dma(K0, kbase, 0, KEYS);
         dma(W0, vbase, 0, VALUES);
         dma(K1, kbase, 1, KEYS);
@@ -591,6 +638,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             vread(vpre, vl);
             weigh(vl, vpre);
         }
+       }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // (transfers past the last tile land in buffers the output goes through)
       } else {
         Stage stk, stv;
@@ -644,7 +692,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // tile buffers, free now) so that it leaves as whole rows, 16 bytes a lane and 4 (float32: 2) rows an instruction
     __syncthreads();                                              // every wave is done with the tiles
     // (DMA: the tile buffers are arrays of their own; two waves' staging regions go through each of the first four)
-    lds_u8* const OB = DMA ? ((w & 3) == 0 ? (lds_u8*) dk0 : (w & 3) == 1 ? (lds_u8*) dk1 : (w & 3) == 2 ? (lds_u8*) dk2 : (lds_u8*) dv0) + (w >> 2) * 16 * (D * 4 + 16)
+    lds_u8* const OB = DMA && NBUF == 2 ? (w == 0 ? (lds_u8*) dk0 : w == 1 ? (lds_u8*) dk1 : w == 2 ? (lds_u8*) dv0 : (lds_u8*) dv1)
+                       : DMA ? ((w & 3) == 0 ? (lds_u8*) dk0 : (w & 3) == 1 ? (lds_u8*) dk1 : (w & 3) == 2 ? (lds_u8*) dk2 : (lds_u8*) dv0) + (w >> 2) * 16 * (D * 4 + 16)
                            : L + w * 16 * (D * 4 + 16);
     if (p.ns > 1) {
         // ---- a key split's partial: the rows' unnormalized sums as float32, then (m, l) - D + 2 floats a (row, head, split),

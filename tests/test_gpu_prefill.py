@@ -171,9 +171,10 @@ def test_prefill_ring(ops):
     (257, 2, 1, 0, 100, 777, 0, BF16),           # a row block of one row
 ])
 def test_prefill_tiles_sent_straight_to_lds(ops, tune, T, Hq, Hkv, cap, win, p0, kt, qt):
-    """The 8-wave form over 16-bit rows of 128 moves its tiles global -> LDS without registers, three buffers a stream:
-    passes of one to many tiles (every buffer rotation), rings with their seam among the pass's keys, windows whose edge
-    falls inside a tile - against the float64 closed form, and bit for bit against the 4-wave form's register staging."""
+    """Over 16-bit rows of 128 both forms move their tiles global -> LDS without registers, the 8-wave form into three
+    buffers a stream, the 4-wave form into two: passes of one to many tiles (every buffer rotation of either), rings
+    with their seam among the pass's keys, windows whose edge falls inside a tile - against the float64 closed form, and
+    the two forms bit for bit against each other."""
     D = 128
     n = p0 + T
     if cap:
