@@ -82,6 +82,15 @@ int ns_mla_attend(ns_gpu* g, const float* qa, const float* c, float* u, int64_t 
 int ns_idx_pool(ns_gpu* g, float* ring, const float* ik, const float* ig, const float* ape, float* pooled, int64_t pos0, int64_t T, int64_t D);
 int ns_idx_score(ns_gpu* g, const float* S, const float* w, float* score, int64_t T, int64_t H, int64_t j0, int64_t n, int64_t ld, int64_t pos0);
 int ns_topk(ns_gpu* g, const float* score, int32_t* sel, int64_t T, int64_t n, int64_t ld, int64_t K);
+/* The pieces of the reference's prompt path around its GEMMs (ns_mla_attend_sel with any T does the whole of that path
+ * in one call; these serve an engine that keeps the reference's chain). Replaces: kernels/llm/glm5next/glm.h:58-60
+ * (glm.cpp:1023-1060), bound at llm/glm5next/src/ffi.rs:117.
+ * ns_mla_cells: each row's cells as a list - idx [T][NC] int32 (0 past the row's cells), n [T] their count, at most NC:
+ *   with lists (sel [T][K], sel_cnt [T]) the 4 tokens of each listed pool, then the row's incomplete pool; sel_cnt null
+ *   or sel_cnt[t] < 0: every cell up to the row's own position pos0 + t.
+ * ns_softmax_masked: S [R H][NC] in place: softmax of scale x S over the first n[r] cells of row r's H heads, 0 behind. */
+int ns_mla_cells(ns_gpu* g, const int32_t* sel, const int32_t* sel_cnt, int64_t T, int64_t K, int64_t pos0, int32_t* idx, int32_t* n, int64_t NC);
+int ns_softmax_masked(ns_gpu* g, float* S, int64_t R, int64_t H, int64_t NC, const int32_t* n, float scale);
 /* out [n][512] half = the q8 latent rows idx[i] of src, widened: half(scale x q), one rounding (a prompt pass's gather).
  * Replaces: kernels/llm/glm5next/glm.h:78 (glm.cpp:1301-1325) */
 int ns_gather_q8_h(ns_gpu* g, const void* src, const int32_t* idx, uint16_t* out, int64_t n, int64_t L);

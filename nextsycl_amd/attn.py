@@ -104,6 +104,8 @@ MLA_H = {
     "ns_idx_pool": (i32, [P, P, P, P, P, P, i64, i64, i64]),
     "ns_idx_score": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64]),
     "ns_topk": (i32, [P, P, P, i64, i64, i64, i64]),
+    "ns_mla_cells": (i32, [P, P, P, i64, i64, i64, P, P, i64]),
+    "ns_softmax_masked": (i32, [P, P, i64, i64, i64, P, f32]),
 }
 
 
@@ -445,6 +447,23 @@ class Ops:
         _need(idx, n * 4, "gather_q8_h indices")
         _need(out, n * L * 2, "gather_q8_h out")
         self.ok(self.k.gather_q8_h(self.raw(), src.ptr, idx.ptr, out.ptr, n, L), "gather_q8_h")
+
+    def mla_cells(self, T, K, pos0, idx, n, NC, sel=None, sel_cnt=None):
+        """ns_mla_cells: each row's cells as a list idx [T][NC] int32 and their count n [T] (sel / sel_cnt None: every
+        cell up to the row's position)."""
+        _need(idx, T * NC * 4, "mla_cells idx")
+        _need(n, T * 4, "mla_cells counts")
+        if sel_cnt is not None:
+            _need(sel, T * K * 4, "mla_cells pools")
+            _need(sel_cnt, T * 4, "mla_cells pool counts")
+        opt = lambda b: b.ptr if b is not None else None
+        self.ok(self.k.mla_cells(self.raw(), opt(sel), opt(sel_cnt), T, K, pos0, idx.ptr, n.ptr, NC), "mla_cells")
+
+    def softmax_masked(self, S, R, H, NC, n, scale):
+        """ns_softmax_masked: S [R H][NC] float32 in place, row r's heads over their first n[r] cells, 0 behind."""
+        _need(S, R * H * NC * 4, "softmax_masked scores")
+        _need(n, R * 4, "softmax_masked counts")
+        self.ok(self.k.softmax_masked(self.raw(), S.ptr, R, H, NC, n.ptr, scale), "softmax_masked")
 
     def to_q8row(self, x, y, n, L):
         _need(x, n * L * 4, "to_q8row x")

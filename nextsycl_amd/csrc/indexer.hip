@@ -380,6 +380,76 @@ __global__ __launch_bounds__(TOPK_WG) void glm_topk_reg_kernel(const float* __re
     }
 }
 
+// A row's latent cells as a list (the prompt path that gathers them): row t of the pass sees, with a selection, the 4
+// tokens of each of its sel_cnt[t] listed pools and then its incomplete pool's tokens 4 ((p + 1) / 4) .. p; without one
+// (no counts, or a negative count) the cells 0 .. p. idx [T][NC] takes the first NC of them (0 past their end), n [T]
+// their count, at most NC (kernels/llm/glm5next/glm.cpp:1023-1039)
+__global__ __launch_bounds__(256) void glm_cells_kernel(const int32_t* __restrict__ sel, const int32_t* __restrict__ sel_cnt, int64_t T, int64_t K,
+                                                        int64_t pos0, int32_t* __restrict__ idx, int32_t* __restrict__ n, int64_t NC) {
+    const int64_t t = blockIdx.y;
+    const int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (i >= NC) return;
+    const int64_t pos = pos0 + t;
+    const int64_t ns = sel_cnt ? sel_cnt[t] : -1;
+    const int64_t tail0 = 4 * ((pos + 1) / 4);
+    const int64_t cnt = ns < 0 ? pos + 1 : 4 * ns + (pos + 1 - tail0);
+    int64_t c = 0;
+    if (i < cnt) c = ns < 0 ? i : i < 4 * ns ? 4 * (int64_t) sel[t * K + i / 4] + i % 4 : tail0 + (i - 4 * ns);
+    idx[t * NC + i] = (int32_t) c;
+    if (i == 0) n[t] = (int32_t) std::min(cnt, NC);
+}
+
+// Row softmax of scores S [R H rows of NC]: row r's heads over its first n[r] cells, scaled; the rest of the row 0
+// (kernels/llm/glm5next/glm.cpp:1041-1060). A work-group a row; rows of up to 256 PER cells stay in registers between
+// the maximum, the sum and the division (one read and one write of the row), longer ones are read three times
+template <int PER>
+__global__ __launch_bounds__(256) void glm_softmax_masked_kernel(float* __restrict__ S, int64_t H, int64_t NC, const int32_t* __restrict__ n, float scale) {
+    __shared__ float red[8];
+    const int64_t rh = blockIdx.x, r = rh / H;
+    float* row = S + rh * NC;
+    const int64_t m = std::min<int64_t>(std::max<int32_t>(n[r], 0), NC);
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    float x[PER > 0 ? PER : 1];
+    float mx = -INFINITY;
+    if constexpr (PER > 0) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int64_t i = tid + 256 * j;
+            x[j] = i < m ? row[i] * scale : -INFINITY;
+            mx = fmaxf(mx, x[j]);
+        }
+    } else {
+        for (int64_t i = tid; i < m; i += 256) mx = fmaxf(mx, row[i] * scale);
+    }
+    mx = wave_max(mx);
+    if (lane == 0) red[wv] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float sum = 0.0f;
+    if constexpr (PER > 0) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            x[j] = x[j] == -INFINITY ? 0.0f : expf(x[j] - mx);
+            sum += x[j];
+        }
+    } else {
+        for (int64_t i = tid; i < m; i += 256) sum += expf(row[i] * scale - mx);
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) red[4 + wv] = sum;
+    __syncthreads();
+    sum = (red[4] + red[5]) + (red[6] + red[7]);
+    if constexpr (PER > 0) {
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int64_t i = tid + 256 * j;
+            if (i < NC) row[i] = i < m ? x[j] / sum : 0.0f;
+        }
+    } else {
+        for (int64_t i = tid; i < NC; i += 256) row[i] = i < m ? expf(row[i] * scale - mx) / sum : 0.0f;
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -426,6 +496,34 @@ int ns_topk(ns_gpu* g, const float* score, int32_t* sel, int64_t T, int64_t n, i
     else if (n <= 64 * TOPK_WG) glm_topk_reg_kernel<64><<<(unsigned) T, TOPK_WG, 0, g->q>>>(score, sel, (int) n, ld, (int) K);
     else glm_topk_kernel<<<(unsigned) T, TOPK_WG, 0, g->q>>>(score, sel, n, ld, K);
     NS_LAUNCHED("topk");
+    return 0;
+    NS_CATCH
+}
+
+int ns_mla_cells(ns_gpu* g, const int32_t* sel, const int32_t* sel_cnt, int64_t T, int64_t K, int64_t pos0, int32_t* idx, int32_t* n, int64_t NC) {
+    NS_TRY
+    if (T <= 0 || NC <= 0) return 0;
+    if (sel_cnt && !sel) return ns_fail("ns_mla_cells: counts, but no lists");
+    if (!g || !idx || !n) return ns_fail("ns_mla_cells: a null buffer");
+    if (pos0 < 0 || K < 0 || pos0 + T > (int64_t) 1 << 31 || T > 65535) return ns_fail("ns_mla_cells: positions below 2^31, at most 65535 rows");
+    NS_HIP(hipSetDevice(g->dev));
+    glm_cells_kernel<<<dim3((unsigned) ((NC + 255) / 256), (unsigned) T), 256, 0, g->q>>>(sel, sel_cnt, T, K, pos0, idx, n, NC);
+    NS_LAUNCHED("mla_cells");
+    return 0;
+    NS_CATCH
+}
+
+int ns_softmax_masked(ns_gpu* g, float* S, int64_t R, int64_t H, int64_t NC, const int32_t* n, float scale) {
+    NS_TRY
+    if (R <= 0 || H <= 0 || NC <= 0) return 0;
+    if (!g || !S || !n) return ns_fail("ns_softmax_masked: a null buffer");
+    if (R * H >= (int64_t) 1 << 31) return ns_fail("ns_softmax_masked: too many rows");
+    NS_HIP(hipSetDevice(g->dev));
+    const unsigned rows = (unsigned) (R * H);
+    if (NC <= 256 * 4) glm_softmax_masked_kernel<4><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+    else if (NC <= 256 * 16) glm_softmax_masked_kernel<16><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+    else glm_softmax_masked_kernel<0><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+    NS_LAUNCHED("softmax_masked");
     return 0;
     NS_CATCH
 }

@@ -1165,6 +1165,35 @@ ORC_API void orc_glm_gather_q8_h(const uint8_t* src, const int32_t* idx, uint16_
     }
 }
 
+/* Each row's cells as a list: idx [T][NC], n [T] - kernels/llm/glm5next/glm.cpp:1023-1039. sel_cnt NULL or sel_cnt[t] < 0:
+ * the cells 0 .. p; else the 4 tokens of each listed pool, then the incomplete pool's tokens 4 ((p + 1) / 4) .. p. */
+ORC_API void orc_glm_mla_cells(const int32_t* sel, const int32_t* sel_cnt, int64_t T, int64_t K, int64_t pos0, int32_t* idx, int32_t* n, int64_t NC) {
+    for (int64_t t = 0; t < T; ++t) {
+        const int64_t p = pos0 + t, ns = sel_cnt ? sel_cnt[t] : -1, tail0 = 4 * ((p + 1) / 4);
+        const int64_t cnt = ns < 0 ? p + 1 : 4 * ns + (p + 1 - tail0);
+        for (int64_t i = 0; i < NC; ++i) {
+            int64_t c = 0;
+            if (i < cnt) c = ns < 0 ? i : i < 4 * ns ? 4 * (int64_t) sel[t * K + i / 4] + i % 4 : tail0 + (i - 4 * ns);
+            idx[t * NC + i] = (int32_t) c;
+        }
+        n[t] = (int32_t) (cnt < NC ? cnt : NC);
+    }
+}
+
+/* Row softmax of S [R H][NC] in place over the first n[r] cells of row r's heads, scaled; 0 behind them -
+ * kernels/llm/glm5next/glm.cpp:1041-1060 (float32 throughout; the reference adds a work-group's terms in tree order,
+ * here in index order) */
+ORC_API void orc_glm_softmax_masked(float* S, int64_t R, int64_t H, int64_t NC, const int32_t* n, float scale) {
+    for (int64_t rh = 0; rh < R * H; ++rh) {
+        float* row = S + rh * NC;
+        const int64_t m = n[rh / H];
+        float mx = -INFINITY, sum = 0.0f;
+        for (int64_t i = 0; i < m; ++i) mx = fmaxf(mx, row[i] * scale);
+        for (int64_t i = 0; i < m; ++i) sum += expf(row[i] * scale - mx);
+        for (int64_t i = 0; i < NC; ++i) row[i] = i < m ? expf(row[i] * scale - mx) / sum : 0.0f;
+    }
+}
+
 /* ------------------------------------------------------------------------------------ norm + rotary positions */
 
 /* kernels/llm/qwen35/q35.cpp:220-254 (w != NULL: RMS norm first), :256-279 (w == NULL: ns_q35_rope), :350-386 (pos3 != NULL:

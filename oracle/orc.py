@@ -48,6 +48,8 @@ def lib():
             "orc_attn_probs": (C.c_int, [C.c_int, P, P, i64, i64, i64, i64, i64, C.c_int, P]),
             "orc_glm_mla_attend_f32": (None, [P, P, P, i64, i64, i64, i64, f32]),
             "orc_glm_gather_q8_h": (None, [P, P, P, i64, i64]),
+            "orc_glm_mla_cells": (None, [P, P, i64, i64, i64, P, P, i64]),
+            "orc_glm_softmax_masked": (None, [P, i64, i64, i64, P, f32]),
             "orc_attn_flash_model": (C.c_int, [P, i64, P, P, C.c_int, C.c_int, i64, i64, i64, i64, i64, i64, i64, i64, P]),
             "orc_mm3_attend": (C.c_int, [P, P, P, P, i64, i64, i64, i64, f32]),
             "orc_mm3_attend_sel": (C.c_int, [P, P, P, P, i64, P, i64, i64, i64, i64, f32]),
@@ -381,6 +383,22 @@ def glm_gather_q8_h(src, idx, L):
     src, idx = np.ascontiguousarray(src, np.uint8), _c(idx, np.int32)
     out = np.empty((idx.size, L), np.uint16)
     lib().orc_glm_gather_q8_h(_p(src), _p(idx), _p(out), idx.size, L)
+    return out
+
+
+def glm_mla_cells(T, K, pos0, NC, sel=None, sel_cnt=None):
+    """ns_mla_cells: (idx [T][NC] int32, n [T] int32) - each row's cells as a list."""
+    idx, n = np.empty((T, NC), np.int32), np.empty(T, np.int32)
+    if sel_cnt is not None:
+        sel, sel_cnt = _c(sel, np.int32), _c(sel_cnt, np.int32)
+    lib().orc_glm_mla_cells(_p(sel) if sel_cnt is not None else None, _p(sel_cnt) if sel_cnt is not None else None, T, K, pos0, _p(idx), _p(n), NC)
+    return idx, n
+
+
+def glm_softmax_masked(S, R, H, NC, n, scale):
+    """ns_softmax_masked: the masked row softmax of S [R H][NC] (a copy)."""
+    out, n = np.array(S, np.float32, order="C").reshape(R * H, NC), _c(n, np.int32)
+    lib().orc_glm_softmax_masked(_p(out), R, H, NC, _p(n), float(scale))
     return out
 
 

@@ -231,3 +231,35 @@ def test_glm_indexer_feeds_the_latent_attention(ops):
     u.fill(0xFF)
     ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, 0.044, sel=selb, sel_cnt=DevBuf.of(g, cnt), K=kp)
     close(u.read(np.float32).reshape(T, H * L), orc.glm_mla_attend_sel(qa, rows, False, T, H, L, pos0, 0.044, sel, cnt, kp))
+
+
+@pytest.mark.gpu
+def test_glm_prompt_path_pieces(ops):
+    """ns_mla_cells bit for bit and ns_softmax_masked within float32 rounding of the oracle: lists with room to spare and
+    cut short, rows without lists, and score rows of every kernel form (kept in registers, and re-read)."""
+    g = ops.gpu
+    T, K, pos0 = 7, 9, 1234
+    rng = np.random.default_rng(5)
+    sel = rng.integers(0, (pos0 + 1) // 4, (T, K)).astype(np.int32)
+    cnt = np.array([9, 0, -1, 4, 1, -1, 9], np.int32)
+    for NC, lists in ((64, True), (17, True), (1280, True), (1280, False), (300, False)):
+        ib, nb = DevBuf(g, T * NC * 4), DevBuf(g, T * 4)
+        ib.fill(0xFF)
+        nb.fill(0xFF)
+        ops.mla_cells(T, K if lists else 0, pos0, ib, nb, NC, DevBuf.of(g, sel) if lists else None, DevBuf.of(g, cnt) if lists else None)
+        want_i, want_n = orc.glm_mla_cells(T, K if lists else 0, pos0, NC, sel if lists else None, cnt if lists else None)
+        assert np.array_equal(nb.read(np.int32), want_n), (NC, lists)
+        assert np.array_equal(ib.read(np.int32).reshape(T, NC), want_i), (NC, lists)
+    for R, H, NC, counts in ((3, 4, 64, (64, 0, 13)), (2, 3, 1024, (1000, 1)), (2, 2, 2112, (2051, 2112)), (2, 2, 5000, (4999, 300)), (1, 5, 257, (200,))):
+        S = orc.randn(R + NC, (R * H, NC), 3.0)
+        n = np.array(counts, np.int32)
+        sb = DevBuf.of(g, S)
+        ops.softmax_masked(sb, R, H, NC, DevBuf.of(g, n), 0.29)
+        got = sb.read(np.float32).reshape(R * H, NC)
+        want = orc.glm_softmax_masked(S, R, H, NC, n, 0.29)
+        assert np.array_equal(got == 0.0, want == 0.0) or np.abs(got - want).max() < 1e-7
+        assert np.abs(got - want).max() <= 2e-6 * max(want.max(), 1e-30) + 1e-9, (R, H, NC)
+        for rh in range(R * H):
+            assert not got[rh, n[rh // H]:].any()
+            if n[rh // H]:
+                assert abs(got[rh].sum() - 1.0) < 1e-5

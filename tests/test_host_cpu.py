@@ -94,6 +94,9 @@ def test_null_buffers_are_refused_before_any_launch(handle):
     refused("ns_to_q8row", [P, P, P, i64, i64], (None, b, None, 1, 512), "null")
     refused("ns_gather_q8_h", [P, P, P, P, i64, i64], (None, b, None, b, 1, 512), "null")
     refused("ns_gather_q8_h", [P, P, P, P, i64, i64], (None, b, b, b, 1, 256), "512")
+    refused("ns_mla_cells", [P, P, P, i64, i64, i64, P, P, i64], (None, None, None, 2, 0, 5, b, None, 64), "null")
+    refused("ns_mla_cells", [P, P, P, i64, i64, i64, P, P, i64], (None, None, b, 2, 4, 5, b, b, 64), "no lists")
+    refused("ns_softmax_masked", [P, P, i64, i64, i64, P, f32], (None, b, 2, 4, 64, None, 1.0), "null")
     refused("ns_attn_tune", [C.c_int, i64], (9, 1), "knob")
     refused("ns_attn_tune", [C.c_int, i64], (0, -1), "knob")
     handle.ns_attn_tune.restype = C.c_int

@@ -149,3 +149,56 @@ def test_glm_indexer_scores_and_top_k():
             want = np.sort(order[:min(K, n)])
             assert np.array_equal(sel[r, :min(K, n)], want), (n, K, r)
             assert (sel[r, min(K, n):] == -1).all()
+
+
+def _cells_of(pos, pools):
+    """A row's cells from the statement of the selection: the 4 tokens of each listed pool, then the tokens of the row's
+    incomplete pool; no list: every cell up to the row's own."""
+    if pools is None:
+        return list(range(pos + 1))
+    return [4 * int(b) + i for b in pools for i in range(4)] + list(range(4 * ((pos + 1) // 4), pos + 1))
+
+
+def test_glm_cells_and_masked_softmax():
+    """ns_mla_cells / ns_softmax_masked (kernels/llm/glm5next/glm.cpp:1023-1060): the lists against the selection spelt out
+    in Python, the softmax against scipy's in float64 - and the chain they belong to (gather, scores, softmax, weighted sum
+    in numpy) against the latent attention over the same lists."""
+    from scipy.special import softmax
+    T, K, pos0 = 5, 6, 41
+    sel = np.array([[9, 2, 5, 0, 1, 3], [1, 0, 7, 4, 9, 8], [3, 3, 3, 3, 3, 3], [0, 1, 2, 3, 4, 5], [8, 6, 4, 2, 0, 1]], np.int32)
+    cnt = np.array([3, 6, 0, -1, 2], np.int32)
+    for NC in (64, 16, 1):                                                   # room for every cell; lists cut short
+        idx, n = orc.glm_mla_cells(T, K, pos0, NC, sel, cnt)
+        for t in range(T):
+            cells = _cells_of(pos0 + t, None if cnt[t] < 0 else sel[t, :cnt[t]])
+            assert n[t] == min(len(cells), NC)
+            assert idx[t].tolist() == (cells + [0] * NC)[:NC]
+    idx, n = orc.glm_mla_cells(T, 0, pos0, 64)                                # no lists at all: dense rows
+    for t in range(T):
+        assert n[t] == pos0 + t + 1 and idx[t, :n[t]].tolist() == list(range(pos0 + t + 1)) and not idx[t, n[t]:].any()
+
+    R, H, NC, scale = 4, 3, 40, 0.37
+    S = orc.randn(3, (R * H, NC), 4.0)
+    S[1] += 300.0                                                            # large scores: the maximum is taken off first
+    m = np.array([40, 17, 0, 1], np.int32)
+    got = orc.glm_softmax_masked(S, R, H, NC, m, scale)
+    for rh in range(R * H):
+        k = m[rh // H]
+        assert not got[rh, k:].any()
+        if k:
+            assert np.abs(got[rh, :k] - softmax(S[rh, :k].astype(np.float64) * scale)).max() < 2e-6
+
+    # the chain of the prompt path: cells -> gathered latents -> scores -> masked softmax -> weighted latents
+    T, Hh, L, K, pos0, scale = 3, 2, 512, 4, 30, 0.05
+    ncell = pos0 + T
+    qa = orc.randn(6, (T, Hh * L), 0.3)
+    cache, cf = orc.randn_f16(7, (ncell, L))
+    sel = np.array([[5, 1, 3, 0], [2, 6, 0, 1], [0, 0, 0, 0]], np.int32)
+    cnt = np.array([4, 2, -1], np.int32)
+    NC = 64
+    idx, n = orc.glm_mla_cells(T, K, pos0, NC, sel, cnt)
+    sc = np.stack([qa[t].reshape(Hh, L) @ cf[idx[t]].T for t in range(T)]).astype(np.float32)      # [T][Hh][NC]
+    pr = orc.glm_softmax_masked(sc.reshape(T * Hh, NC), T, Hh, NC, n, scale).reshape(T, Hh, NC)
+    u = np.stack([pr[t] @ cf[idx[t]] for t in range(T)]).reshape(T, Hh * L)
+    want = orc.glm_mla_attend_sel(qa, cache.view(np.uint8), False, T, Hh, L, pos0, scale, sel, cnt, K)
+    assert np.abs(u - want).max() < 2e-5
