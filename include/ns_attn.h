@@ -141,6 +141,17 @@ int64_t ns_nhs_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D
 int ns_nhs_attn_decode(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D,
                        int64_t cap, int64_t p0, float* out, float* scratch);
 
+/* ricursive's silo names of the same two passes: heads of 128, 10 query heads a key head, ring caches [Hkv][cap][128] half
+ * (slot position % cap), window win (<= 0: every key), rows Hq x 128 floats apart; _prompt more than 16 rows, _decode 1..16.
+ * Replaces: kernels/llm/ricursive/silo/silo.h:38-49 (silo/attn.cpp:282-360), bound at llm/ricursive/src/ffi.rs:138-141 */
+int ns_rc_flash_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);
+int ns_rc_flash_prompt(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
+                       int64_t win, float* out);
+int ns_rc_flash_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D);
+int64_t ns_rc_flash_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win);
+int ns_rc_flash_decode(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
+                       int64_t win, float* out, float* scratch);
+
 /* ---- the engines' own ("exact") attention entry points, routed to the kernels above ----------------------------- */
 
 /* Replaces: kernels/llm/qwen35/q35.h:61-66 (q35.cpp:590-612) */

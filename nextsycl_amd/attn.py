@@ -68,6 +68,11 @@ ATTN_H = {
     "ns_rc_kv_store": (i32, [P, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]),
     "ns_rc_attn_scratch": (i64, [i64, i64, i64, i64, i64, i64]),
     "ns_rc_attn": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_rc_flash_prompt_supported": (i32, [i64, i64, i64, i64]),
+    "ns_rc_flash_prompt": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, P]),
+    "ns_rc_flash_decode_supported": (i32, [i64, i64, i64, i64]),
+    "ns_rc_flash_decode_scratch": (i64, [i64, i64, i64, i64, i64, i64]),
+    "ns_rc_flash_decode": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, P, P]),
     "ns_nh_kv_store": (i32, [P, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]),
     "ns_nh_attn_scratch": (i64, [i64, i64, i64, i64, i64]),
     "ns_nh_attn": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, P, P]),
@@ -342,6 +347,20 @@ class Ops:
             _need(scratch, self.k.rc_attn_scratch(T, Hq, Hkv, D, W, p0) * 4, "attention scratch")
         self.ok(self.k.rc_attn(self.raw(), q.ptr, qs, kc.ptr, vc.ptr, T, Hq, Hkv, D, R, W, p0, out.ptr,
                                scratch.ptr if scratch is not None else None), "attention")
+
+    def rc_flash(self, q, kc, vc, T, Hq, Hkv, D, cap, p0, win, out, scratch=None):
+        """ricursive's silo names: ns_rc_flash_decode (1..16 rows, with scratch) or ns_rc_flash_prompt (more)."""
+        _need(q, T * Hq * D * 4, "attention q")
+        _need(out, T * Hq * D * 4, "attention out")
+        _need(kc, self.cache_bytes(0, Hkv, cap, D), "attention key cache")
+        _need(vc, self.cache_bytes(0, Hkv, cap, D), "attention value cache")
+        if T <= 16:
+            if scratch is not None:
+                _need(scratch, max(0, self.k.rc_flash_decode_scratch(T, Hq, Hkv, D, p0, win)) * 4, "attention scratch")
+            self.ok(self.k.rc_flash_decode(self.raw(), q.ptr, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, out.ptr,
+                                           scratch.ptr if scratch is not None else None), "attention")
+        else:
+            self.ok(self.k.rc_flash_prompt(self.raw(), q.ptr, kc.ptr, vc.ptr, T, Hq, Hkv, D, cap, p0, win, out.ptr), "attention")
 
     def nh_attn(self, q, qs, kc, vc, T, Hq, Hkv, D, cap, p0, out, scratch):
         """ns_nh_attn: nemotron-h's attention layers (causal, no window)."""

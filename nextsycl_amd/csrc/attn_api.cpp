@@ -111,6 +111,31 @@ int ns_rc_attn(ns_gpu* g, const float* q, int64_t qs, const void* kc, const void
     return ns_attn_prompt_any(g, "ns_rc_attn", 0, 0, 0, q, qs, kc, vc, T, Hq, Hkv, D, R, p0, W, 1, -1, 0.0f, out);
 }
 
+// ricursive's silo names (kernels/llm/ricursive/silo/attn.cpp:282-360): heads of 128, 10 query heads a key head, ring
+// caches, a window; rows Hq x 128 floats apart
+int ns_rc_flash_decode_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) { return T >= 1 && T <= DECODE_ROWS && D == 128 && Hkv > 0 && Hq == 10 * Hkv; }
+
+int64_t ns_rc_flash_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win) {
+    return ns_attn_decode_scratch(T, Hq, Hkv, D, p0, win);
+}
+
+int ns_rc_flash_decode(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
+                       int64_t win, float* out, float* scratch) {
+    if (!ns_rc_flash_decode_supported(T, Hq, Hkv, D)) return ns_fail("ns_rc_flash_decode: 1..16 rows, heads of 128, 10 query heads a key head");
+    if (!scratch) return ns_fail("ns_rc_flash_decode: no scratch");
+    return ns_attn_decode_any(g, "ns_rc_flash_decode", 0, 0, 0, q, Hq * D, kc, vc, T, Hq, Hkv, D, cap, p0, win, DecodeExtra{}, 0.0f, out, scratch);
+}
+
+int ns_rc_flash_prompt_supported(int64_t T, int64_t Hq, int64_t Hkv, int64_t D) { return T > DECODE_ROWS && D == 128 && Hkv > 0 && Hq == 10 * Hkv; }
+
+int ns_rc_flash_prompt(ns_gpu* g, const float* q, const void* kc, const void* vc, int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0,
+                       int64_t win, float* out) {
+    if (!ns_rc_flash_prompt_supported(T, Hq, Hkv, D)) return ns_fail("ns_rc_flash_prompt: more than 16 rows, heads of 128, 10 query heads a key head");
+    const int64_t need = win > 0 ? std::min(p0 + T, win + T - 1) : p0 + T;
+    if (need > cap) return ns_fail("ns_rc_flash_prompt: the cache's ring is shorter than the window and the pass");
+    return ns_attn_prompt_any(g, "ns_rc_flash_prompt", 0, 0, 0, q, Hq * D, kc, vc, T, Hq, Hkv, D, cap, p0, win, 1, -1, 0.0f, out);
+}
+
 int64_t ns_nh_attn_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0) {
     return T >= 1 && T <= DECODE_ROWS ? ns_attn_decode_scratch(T, Hq, Hkv, D, p0, 0) : 0;
 }

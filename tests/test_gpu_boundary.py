@@ -307,6 +307,36 @@ def test_ricursive_entry_points(ops, T, Hq, Hkv, R, W, p0):
     check_close(got, orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, R, p0, win=W), F32, "ns_rc_attn vs float64 closed form")
 
 
+@pytest.mark.parametrize("T,Hkv,R,W,p0", [(1, 2, 4096, 0, 3000), (4, 1, 512, 500, 2045), (16, 2, 300, 256, 1000), (40, 1, 700, 512, 5000),
+                                          (300, 2, 900, 0, 600)])
+def test_ricursive_silo_names(ops, T, Hkv, R, W, p0):
+    """ns_rc_flash_decode / ns_rc_flash_prompt (kernels/llm/ricursive/silo/attn.cpp:282-360) over a ring written by
+    ns_rc_kv_store: the float64 closed form, and the very bits of ns_rc_attn, whose passes they are."""
+    D, Hq = 128, 10 * Hkv
+    g = ops.gpu
+    n = p0 + T
+    k, v = orc.randn(43, (n, Hkv * D)), orc.randn(44, (n, Hkv * D))
+    kc = np.zeros((Hkv, R, 2 * D), np.uint8)
+    vc = np.zeros((Hkv, R, 2 * D), np.uint8)
+    for s in range(0, n, R):
+        orc.kv_store(0, k[s:min(n, s + R)], v[s:min(n, s + R)], Hkv, D, R, s, kc=kc, vc=vc, ring=True)
+    kcb, vcb = DevBuf.of(g, kc), DevBuf.of(g, vc)
+    qd, qf = make_q(F32, T, Hq, D)
+    qb = DevBuf.of(g, qd)
+    assert ops.k.rc_flash_decode_supported(T, Hq, Hkv, D) == (T <= 16) and ops.k.rc_flash_prompt_supported(T, Hq, Hkv, D) == (T > 16)
+    assert not ops.k.rc_flash_decode_supported(1, 8 * Hkv, Hkv, D) and not ops.k.rc_flash_prompt_supported(64, Hq, Hkv, 256)
+    ob = DevBuf(g, T * Hq * D * 4)
+    ob.fill(0xFF)
+    sc = DevBuf(g, max(4, 4 * ops.k.rc_flash_decode_scratch(T, Hq, Hkv, D, p0, W))) if T <= 16 else None
+    ops.rc_flash(qb, kcb, vcb, T, Hq, Hkv, D, R, p0, W, ob, sc)
+    got = ob.read(np.float32).reshape(T, Hq * D)
+    check_close(got, orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, R, p0, win=W), F32, "ricursive's silo names vs float64 closed form")
+    ob2 = DevBuf(g, T * Hq * D * 4)
+    sc2 = DevBuf(g, max(4, 4 * ops.k.rc_attn_scratch(T, Hq, Hkv, D, W, p0)))
+    ops.rc_attn(qb, Hq * D, kcb, vcb, T, Hq, Hkv, D, R, W, p0, ob2, sc2)
+    assert np.array_equal(ob2.read(np.float32).view(np.uint32), got.reshape(-1).view(np.uint32))
+
+
 def test_ricursive_entry_points_refuse_what_the_reference_refuses(ops):
     g = ops.gpu
     D, Hkv = 128, 1
@@ -326,6 +356,13 @@ def test_ricursive_entry_points_refuse_what_the_reference_refuses(ops):
     with pytest.raises(Error, match="past the cache's capacity"):
         ops.nh_attn(q, 8 * D, kcb, kcb, 2, 8, Hkv, D, 64, 63, out, sc)
     ops.rc_attn(q, 10 * D, kcb, kcb, 0, 10, Hkv, D, 64, 0, 1000, out, None)      # no rows: nothing is checked
+    with pytest.raises(Error, match="1..16 rows, heads of 128, 10 query heads a key head"):
+        ops.rc_flash(q, kcb, kcb, 4, 8, Hkv, D, 64, 10, 0, out, sc)
+    with pytest.raises(Error, match="ns_rc_flash_decode: no scratch"):
+        ops.rc_flash(q, kcb, kcb, 4, 10, Hkv, D, 64, 10, 0, out, None)
+    big_q, big_out = DevBuf(g, 40 * 10 * D * 4), DevBuf(g, 40 * 10 * D * 4)
+    with pytest.raises(Error, match="the cache's ring is shorter than the window and the pass"):
+        ops.rc_flash(big_q, kcb, kcb, 40, 10, Hkv, D, 64, 100, 32, big_out)
 
 
 @pytest.mark.parametrize("T,Hq,Hkv,p0", [(1, 32, 4, 5000), (4, 16, 2, 2046), (16, 8, 1, 77), (200, 16, 2, 300)])
