@@ -197,40 +197,32 @@ def graph_step_ms(w, n=50):
     import ctypes as C
     if w.kind == "pre" or w.kind == "prefill" or (w.kind == "mla" and w.T > 16):
         return None
-    g = w.ops.gpu
+    g, k = w.ops.gpu, w.ops.k
     try:
-        hip = C.CDLL("libamdhip64.so")
-        hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
-        hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
-        hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
-        hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
-        hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
-        hip.hipGraphDestroy.argtypes = [C.c_void_p]
-        stream = C.cast(C.c_void_p(g.api.gpu_queue(g.raw)), C.POINTER(C.c_void_p))[0]
         g.sync()
-        graph, ex = C.c_void_p(), C.c_void_p()
-        if hip.hipStreamBeginCapture(stream, 2) != 0:                 # (relaxed mode)
+        h = C.c_void_p()
+        if k.q35_graph_begin(g.raw, C.byref(h)) != 0:                 # ns_q35_graph_*: the library's stream capture
             return None
         try:
             for _ in range(n):
                 w.step()
         finally:
-            rc = hip.hipStreamEndCapture(stream, C.byref(graph))
-        if rc != 0 or not graph.value or hip.hipGraphInstantiate(C.byref(ex), graph, None, None, 0) != 0:
+            rc = k.q35_graph_end(g.raw, h)
+        if rc != 0:
+            k.q35_graph_free(h)
             return None
         try:
             for _ in range(3):
-                hip.hipGraphLaunch(ex, stream)
+                k.q35_graph_launch(g.raw, h)
             g.sync()
             t0 = g.stamp()
-            hip.hipGraphLaunch(ex, stream)
-            hip.hipGraphLaunch(ex, stream)
+            k.q35_graph_launch(g.raw, h)
+            k.q35_graph_launch(g.raw, h)
             t1 = g.stamp()
             ns = g.elapsed_ns(t0, t1) / (2 * n)
         finally:
             g.sync()
-            hip.hipGraphExecDestroy(ex)
-            hip.hipGraphDestroy(graph)
+            k.q35_graph_free(h)
         return ns / 1e6
     except Exception:
         return None

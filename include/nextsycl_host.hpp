@@ -55,6 +55,7 @@ public:
     X(ns_mg_kv_store) X(ns_mg_attn_scratch) X(ns_mg_attn) X(ns_mg_attn_prompt_supported) X(ns_mg_attn_prompt)                            \
     X(ns_mg_attn_decode_supported) X(ns_mg_attn_decode_scratch) X(ns_mg_attn_decode) X(ns_llm_minimaxm3_attend)                          \
     X(ns_rc_kv_store) X(ns_rc_attn_scratch) X(ns_rc_attn) X(ns_nh_kv_store) X(ns_nh_attn_scratch) X(ns_nh_attn)                          \
+    X(ns_q35_graph_begin) X(ns_q35_graph_end) X(ns_q35_graph_launch) X(ns_q35_graph_free) \
     X(ns_rc_flash_prompt_supported) X(ns_rc_flash_prompt) X(ns_rc_flash_decode_supported) X(ns_rc_flash_decode_scratch) X(ns_rc_flash_decode) \
     X(ns_nhs_attn_prompt_supported) X(ns_nhs_attn_prompt) X(ns_nhs_attn_decode_supported) X(ns_nhs_attn_decode_scratch)                  \
     X(ns_nhs_attn_decode)                                                                                                                \

@@ -242,6 +242,15 @@ int ns_attn_profile(ns_gpu* g, int on);
  * rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled against. This library's own */
 int ns_attn_copy_probe(ns_gpu* g, void* dst, const void* src, size_t bytes);
 int ns_attn_profile_last(ns_gpu* g, double* main_ns, double* merge_ns);
+/* A stretch of a pass as one submission: what is queued on g's compute stream from begin (*out: the graph) to end is
+ * recorded, not run (a HIP graph by stream capture; every entry point of this library records kernel launches only);
+ * end finishes it, launch replays it on g's stream, free releases it (also one still recording). A decode token recorded
+ * once and replayed saves the launches' host cost and the gaps between dependent kernels.
+ * Replaces: kernels/llm/qwen35/q35.h:47-52 (q35.cpp:505-549: SYCL command graphs), bound at llm/qwen35/src/ffi.rs:114-117 */
+int ns_q35_graph_begin(ns_gpu* g, void** out);
+int ns_q35_graph_end(ns_gpu* g, void* h);
+int ns_q35_graph_launch(ns_gpu* g, void* h);
+void ns_q35_graph_free(void* h);
 /* Tuning knobs for sweeps and tests (this library's own): knob 0 work-groups a decode pass aims for, 1 key splits and
  * 2 waves a work-group (4 or 8) of a prompt pass, 3 work-groups an MLA pass aims for, 4 heads a wave of the
  * pre-attention kernel; value 0 = the library's own choice. Each knob starts from its environment variable (NS_DEC_WGS,

@@ -68,6 +68,10 @@ ATTN_H = {
     "ns_rc_kv_store": (i32, [P, P, i64, P, i64, i64, i64, i64, i64, i64, P, P]),
     "ns_rc_attn_scratch": (i64, [i64, i64, i64, i64, i64, i64]),
     "ns_rc_attn": (i32, [P, P, i64, P, P, i64, i64, i64, i64, i64, i64, i64, P, P]),
+    "ns_q35_graph_begin": (i32, [P, C.POINTER(P)]),
+    "ns_q35_graph_end": (i32, [P, P]),
+    "ns_q35_graph_launch": (i32, [P, P]),
+    "ns_q35_graph_free": (None, [P]),
     "ns_rc_flash_prompt_supported": (i32, [i64, i64, i64, i64]),
     "ns_rc_flash_prompt": (i32, [P, P, P, P, i64, i64, i64, i64, i64, i64, i64, P]),
     "ns_rc_flash_decode_supported": (i32, [i64, i64, i64, i64]),

@@ -154,6 +154,76 @@ void ns_gpu_close(ns_gpu* g) {
 
 void* ns_gpu_queue(ns_gpu* g) { return &g->q; }
 
+// ---- a stretch of a pass as one submission: what is queued on the handle's compute stream between begin and end is
+// recorded into a HIP graph instead of run (stream capture: kernel launches only - no entry point of this library
+// records a memset or allocates), instantiated at end, replayed by launch (kernels/llm/qwen35/q35.cpp:505-549: the same
+// four calls over a SYCL command graph)
+namespace {
+struct NsGraph {
+    int dev = 0;
+    hipStream_t q = nullptr;          // the stream that records; null once recording has ended
+    hipGraphExec_t exec = nullptr;
+};
+}  // namespace
+
+int ns_q35_graph_begin(ns_gpu* g, void** out) {
+    NS_TRY
+    if (!g || !out) return ns_fail("ns_q35_graph_begin: a null argument");
+    NS_HIP(hipSetDevice(g->dev));
+    // (relaxed: other threads of the engine may be allocating or copying on their own streams meanwhile)
+    NS_HIP(hipStreamBeginCapture(g->q, hipStreamCaptureModeRelaxed));
+    NsGraph* gr = new NsGraph;
+    gr->dev = g->dev;
+    gr->q = g->q;
+    *out = gr;
+    return 0;
+    NS_CATCH
+}
+
+int ns_q35_graph_end(ns_gpu* g, void* h) {
+    NS_TRY
+    NsGraph* gr = static_cast<NsGraph*>(h);
+    if (!g || !gr) return ns_fail("ns_q35_graph_end: a null argument");
+    if (!gr->q || gr->q != g->q) return ns_fail("ns_q35_graph_end: not the graph this GPU is recording");
+    NS_HIP(hipSetDevice(g->dev));
+    gr->q = nullptr;
+    hipGraph_t graph = nullptr;
+    NS_HIP(hipStreamEndCapture(g->q, &graph));
+    if (!graph) return ns_fail("ns_q35_graph_end: the recording was dropped (a call that cannot be recorded was made on the stream)");
+    const hipError_t e = hipGraphInstantiate(&gr->exec, graph, nullptr, nullptr, 0);
+    (void) hipGraphDestroy(graph);
+    NS_HIP(e);
+    return 0;
+    NS_CATCH
+}
+
+int ns_q35_graph_launch(ns_gpu* g, void* h) {
+    NS_TRY
+    NsGraph* gr = static_cast<NsGraph*>(h);
+    if (!g || !gr) return ns_fail("ns_q35_graph_launch: a null argument");
+    if (!gr->exec) return ns_fail("ns_q35_graph_launch: a graph not finished");
+    if (gr->dev != g->dev) return ns_fail("ns_q35_graph_launch: a graph of another GPU");
+    NS_HIP(hipSetDevice(g->dev));
+    NS_HIP(hipGraphLaunch(gr->exec, g->q));
+    return 0;
+    NS_CATCH
+}
+
+void ns_q35_graph_free(void* h) {
+    NsGraph* gr = static_cast<NsGraph*>(h);
+    if (!gr) return;
+    if (gr->q) {                      // freed while still recording: the recording ends here, and is dropped
+        hipGraph_t graph = nullptr;
+        (void) hipSetDevice(gr->dev);
+        if (hipStreamEndCapture(gr->q, &graph) == hipSuccess && graph) (void) hipGraphDestroy(graph);
+    }
+    if (gr->exec) {
+        (void) hipSetDevice(gr->dev);
+        (void) hipGraphExecDestroy(gr->exec);
+    }
+    delete gr;
+}
+
 int ns_gpu_memory(ns_gpu* g, uint64_t* total, int64_t* free_bytes) {
     NS_TRY
     NS_HIP(hipSetDevice(g->dev));

@@ -75,3 +75,58 @@ def test_decode_token_in_a_graph():
         hip.hipGraphExecDestroy(ex)
         hip.hipGraphDestroy(graph)
         g.close()
+
+
+def test_decode_token_through_the_library_graph_calls():
+    """The same token recorded and replayed through ns_q35_graph_begin / _end / _launch / _free (the reference's four
+    calls, here over HIP stream capture): nothing runs while recording, every replay equals the eager calls bit for bit,
+    a graph still recording cannot be launched, and one freed while recording leaves the stream usable."""
+    g = Gpu.open(0)
+    ops = Ops(g)
+    T, Hq, Hkv, D, p0, kt, qt = 2, 16, 2, 128, 3000, 0, F16
+    cap = p0 + T
+    kc, vc = make_kv(kt, Hkv, D, cap, p0)
+    kcb, vcb = DevBuf.of(g, kc), DevBuf.of(g, vc)
+    kb, vb = DevBuf(g, T * Hkv * D * 4), DevBuf(g, T * Hkv * D * 4)
+    qb, ob = DevBuf(g, T * Hq * D * 2), DevBuf(g, T * Hq * D * 2)
+
+    def token():
+        ops.kv_store(kt, kb, Hkv * D, vb, Hkv * D, T, Hkv, D, cap, p0, kcb, vcb)
+        ops.decode_static(qt, kt, qb, Hq * D, kcb, vcb, T, Hq, Hkv, D, cap, p0, ob)
+
+    try:
+        # a recording that is dropped: freed before it ended
+        h = C.c_void_p()
+        ops.ok(ops.k.q35_graph_begin(ops.raw(), C.byref(h)), "graph begin")
+        token()
+        assert ops.k.q35_graph_launch(ops.raw(), h) == -1 and "not finished" in g.api.error()
+        ops.k.q35_graph_free(h)
+        g.sync()
+        # the recording that is kept
+        ob.fill(0xFF)
+        g.sync()
+        h = C.c_void_p()
+        ops.ok(ops.k.q35_graph_begin(ops.raw(), C.byref(h)), "graph begin")
+        try:
+            token()
+        finally:
+            ops.ok(ops.k.q35_graph_end(ops.raw(), h), "graph end")
+        g.sync()
+        assert (ob.read(np.uint16) == 0xFFFF).all()                  # recorded, not run
+        for rep in range(3):
+            k, v = orc.randn(170 + rep, (T, Hkv * D)), orc.randn(180 + rep, (T, Hkv * D))
+            qd, _ = make_q(qt, T, Hq, D, cfg=rep)
+            kb.write(k)
+            vb.write(v)
+            qb.write(qd)
+            ob.fill(0xFF)
+            g.sync()
+            ops.ok(ops.k.q35_graph_launch(ops.raw(), h), "graph launch")
+            g.sync()
+            got = ob.read(np.uint16)
+            ob.fill(0xFF)
+            token()
+            assert np.array_equal(got, ob.read(np.uint16)), rep
+        ops.k.q35_graph_free(h)
+    finally:
+        g.close()
