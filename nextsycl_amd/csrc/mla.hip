@@ -9,7 +9,8 @@
 // Work split: grid (cell split, row group). A work-group of 8 waves owns 128 (row, head) pairs - one decode row's 128
 // heads - a wave 16 of them (one 16-row MFMA tile: 72 registers of queries, 128 of accumulators), and a split of the
 // cells in 32-cell tiles; short passes of at most 128 rows run 4 waves = 64 pairs a work-group (mla_waves). Half rows go
-// global -> LDS directly two tiles ahead into three LDS buffers, one barrier a tile; GLM's q8 rows are fetched through
+// global -> LDS directly two tiles ahead into three LDS buffers (the 4-wave form: three ahead into four), one barrier a
+// tile; GLM's q8 rows are fetched through
 // registers and widened to half on the way. The tile is shared by the work-group's waves. LDS
 // rows are 74 chunks of 16 bytes (72 of data, 2 of padding): rows 32 bytes apart modulo 256 spread both access patterns
 // over the banks - 16 rows x 16 bytes of one column (the score product's operand) and 8 rows x 32 bytes (the
@@ -88,15 +89,21 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
     constexpr int CPR = Q8 ? ML / 16 : DK / 8;           // 16-byte loads a cache row
     constexpr int NCH = MTILE * CPR;                     // loads a tile
     constexpr int NLD = (NCH + MW * 64 - 1) / (MW * 64); // loads a thread per tile (the last may be idle)
-    // three tile buffers, three separate arrays: reads of one are then known not to touch a buffer a transfer is
-    // still writing
+    // three tile buffers (four under the pipelined step of the 4-wave form), separate arrays: reads of one are then
+    // known not to touch a buffer a transfer is still writing
     __shared__ __attribute__((aligned(16))) uint8_t lds0[TILEB];
     __shared__ __attribute__((aligned(16))) uint8_t lds1[TILEB];
     __shared__ __attribute__((aligned(16))) uint8_t lds2[TILEB];
+    // (the pipelined step works on two tiles at once - it scores tile it + 1 while it weighs tile it - so with three
+    // buffers the tile it requests is the one its own end waits for, and a step lasts one memory latency; the fourth
+    // buffer lets a request travel a step longer: the tile loop without its products 12.1 -> 9.3 us at 32768 cells)
+    constexpr bool FOUR = MW == 4 && !Q8;
+    __shared__ __attribute__((aligned(16))) uint8_t lds3[FOUR ? TILEB : 16];
     typedef __attribute__((address_space(3))) uint8_t lds_u8;
     lds_u8* const B0 = (lds_u8*) lds0;
     lds_u8* const B1 = (lds_u8*) lds1;
     lds_u8* const B2 = (lds_u8*) lds2;
+    lds_u8* const B3 = (lds_u8*) lds3;
 
     const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -402,7 +409,8 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
     // pipe fed while the vector unit works - a tile's step is two straight-line blocks,
     //   1: S^T of tile it + 1 (its buffer landed a step ago)   ||   weights of tile it = exp2(arguments), sum, rounding
     //   2: O^T += C^T P^T of tile it                           ||   exponent arguments of tile it + 1 and their largest
-    // then (rarely) the move of the reference, the wait for tile it + 2's transfers and the barrier. Past the split's last
+    // then (rarely) the move of the reference, the wait for tile it + 2's transfers (tile it + 3's, requested at the
+    // step's head, stay in flight) and the barrier. Past the split's last
     // tile block 1 scores whatever the next buffer holds: every such cell is masked.
     float a_cur[8];
     auto args_of = [&](const f4v (&s)[2], int it, float (&a)[8]) -> float {
@@ -481,8 +489,8 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         }
     };
-    auto pstep = [&](lds_u8* rd, lds_u8* nx1, lds_u8* nx2, int it) {
-        if (it + 2 < nt) dma(nx2, it + 2);
+    auto pstep = [&](lds_u8* rd, lds_u8* nx1, lds_u8* nx3, int it) {
+        if (it + 3 < nt) dma(nx3, it + 3);
         // ---- block 1
         f4v s[2];
         scores_of(nx1, s);
@@ -501,9 +509,9 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
         weigh_of(rd, pb);
         const float amax = args_of(s, it + 1, a_cur);
         regrow(amax, a_cur);
-        // (the next step's first block reads tile it + 2, requested at the head of this one: every transfer of this wave
-        // has to have landed. A fourth buffer with requests three tiles ahead measured the same, 20.4 us at 32768 cells)
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // (the next step's first block reads tile it + 2, requested a step ago: only this step's request may stay out)
+        if (it + 3 < nt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
@@ -540,11 +548,13 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
             step(B2, B0, B1, it + 2);
         }
     } else {
-        // the first two tiles are on their way before the queries are loaded
+        // the first two tiles are on their way before the queries are loaded, the third behind them
         if (nt > 0) dma(B0, 0);
         if (nt > 1) dma(B1, 1);
         load_queries();
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (nt > 2) dma(B2, 2);
+        if (nt > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (nt > 0) {
@@ -553,12 +563,16 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
             const float amax = args_of(s, 0, a_cur);
             regrow(amax, a_cur);
         }
-        for (int it = 0; it < nt; it += 3) {
-            pstep(B0, B1, B2, it);
-            if (it + 1 >= nt) break;
-            pstep(B1, B2, B0, it + 1);
-            if (it + 2 >= nt) break;
-            pstep(B2, B0, B1, it + 2);
+        if constexpr (FOUR) {
+            for (int it = 0; it < nt; it += 4) {
+                pstep(B0, B1, B3, it);
+                if (it + 1 >= nt) break;
+                pstep(B1, B2, B0, it + 1);
+                if (it + 2 >= nt) break;
+                pstep(B2, B3, B1, it + 2);
+                if (it + 3 >= nt) break;
+                pstep(B3, B0, B2, it + 3);
+            }
         }
     }
 
