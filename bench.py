@@ -7,8 +7,9 @@ A step is one pass of the hot path over one batch of synthetic input, inputs res
 starts. The default workload is BASELINE.json's configs[1] - causal GQA flash-attention prefill, batch 1, 8192 rows, 40
 query heads / 8 key heads, head 128, bfloat16 Q / K / V / output - and `value` is its TFLOP/s counted on the causal
 flops 4 D Hq S (S + 1) / 2. The line also carries:
-  roofline      the dominant kernel's algorithmic flops (or bytes) per launch over its device time, measured with HIP
-                events on the library's own compute stream (ns_attn_profile), against MI355X's published peak;
+  roofline      the step's algorithmic flops (or bytes) over its device time - the median of 10 runs of steps between HIP
+                event stamps on the library's own compute stream, every launch of a step included (a decode step's merge
+                kernel too) - against MI355X's published peak; the dominant kernel alone from the committed kernel trace;
   cpu_baseline  the CPU oracle (a port of the reference's exact kernel, OpenMP) timed on this host on a bounded sample;
   others        the decode-side workloads of the same metric (GB/s of algorithmic KV bytes, % of 8 TB/s): the 32K GQA
                 decode target, BASELINE configs 1, 3, 5 - unless --no-extra.
@@ -147,10 +148,12 @@ class Workload:
 
 
 SETTLE_MS = 100.0
+GROUPS = 10
 
 
 def timed(w, steps, warmup):
-    """(ms per step over exactly `steps` steps, average device ns of the dominant kernel, of the merge kernel)."""
+    """(ms per step over exactly `steps` steps by the host's clock around two syncs; the step's device time in ns: the
+    median over GROUPS runs of steps queued back to back between two HIP event stamps on the library's compute stream)."""
     g = w.ops.gpu
     # untimed: the W warmup steps, and then more of the same until the GPU has been under load for SETTLE_MS - an idle
     # MI355X takes tens of milliseconds of work to reach its steady clocks (the first MFMA-bound launches after a pause
@@ -168,25 +171,18 @@ def timed(w, steps, warmup):
         w.step()
     g.sync()
     ms = (time.perf_counter() - t0) * 1e3 / steps
-    # the dominant kernel alone: the same steps with the library told to queue its main kernel only (no merge launch),
-    # back to back between two HIP event stamps on the library's compute stream - the kernel's own launch duration on a
-    # busy queue, what rocprofv3's kernel trace reports. (Events around every single launch open gaps and read ~3 us long
-    # for kernels of 20 us.) The merge kernel's share is the rest of the step.
-    if w.kind == "pre" or w.kind == "prefill" or (w.kind == "mla" and w.T > 16):
-        # one launch a step / several passes a step: the step itself, launched back to back, is the figure
-        return ms, ms * 1e6, 0.0
-    w.ops.profile(2)
-    for _ in range(8):
-        w.step()
-    g.sync()
-    n = max(steps, 50)
-    t0 = g.stamp()
-    for _ in range(n):
-        w.step()
-    t1 = g.stamp()
-    main = g.elapsed_ns(t0, t1) / n
-    w.ops.profile(0)
-    return ms, main, max(0.0, ms * 1e6 - main)
+    # the same steps on the device's clock: every launch of a step (main kernel, merge, a cache's widening) and the gaps
+    # between dependent launches are inside; the median of GROUPS runs of `per` steps each
+    per = max(10, steps // GROUPS)
+    runs = []
+    for _ in range(GROUPS):
+        a = g.stamp()
+        for _ in range(per):
+            w.step()
+        b = g.stamp()
+        runs.append((a, b))
+    dev = sorted(g.elapsed_ns(a, b) / per for a, b in runs)
+    return ms, 0.5 * (dev[(GROUPS - 1) // 2] + dev[GROUPS // 2])
 
 
 def graph_step_ms(w, n=50):
@@ -228,42 +224,42 @@ def graph_step_ms(w, n=50):
         return None
 
 
-# HBM bytes per launch of each workload's dominant kernel as rocprofv3 counted them (FETCH_SIZE + WRITE_SIZE per dispatch,
-# each scaled by what the same counter reads for a plain copy kernel of known size). A counter run cannot be made from
-# inside this script: the figure is read from the committed summary of that run, profiles/<kernel>_<workload>.md (its line
-# "traffic_bytes_per_launch: N"), and is null where no such summary exists.
-def measured_traffic(kernel, workload):
+# What a profiler run says about each workload's dominant kernel: rocprofv3 cannot be driven from inside this script, so
+# the figures are read from the committed summary of such a run of this script, profiles/<kernel>_<workload>.md - its
+# lines "traffic_bytes_per_launch: N" (FETCH_SIZE + WRITE_SIZE per dispatch, each scaled by what the same counter reads
+# for a plain copy kernel of known size) and "kernel_avg_us: T" (the kernel trace's average duration of that kernel) -
+# and are null where no such summary exists.
+def from_profile(kernel, workload, key):
     import re
     path = os.path.join(ROOT, "profiles", "%s_%s.md" % (kernel, workload))
     try:
-        m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), re.M)
+        m = re.search(r"^%s:\s*([0-9.eE+]+)" % key, open(path).read(), re.M)
     except OSError:
         return None
     return float(m.group(1)) if m else None
 
 
-def roofline(w, main_ns):
-    r = _roofline(w, main_ns)
-    r["traffic"] = measured_traffic(r["kernel"], w.name)
-    return r
+KERNEL = {"pre": "pre_attn_kernel", "mla": "mla_decode_kernel", "prefill": "attn_prefill_kernel", "decode": "attn_decode_kernel"}
 
 
-def _roofline(w, main_ns):
-    if w.kind == "pre":
-        ach = w.bytes / main_ns
-        return {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
-                "kernel": "pre_attn_kernel", "kernel_us": round(main_ns / 1e3, 2)}
+def roofline(w, step_ns):
+    """The step against the roofline that bounds its dominant kernel. `achieved` / `frac`: algorithmic flops (or bytes) of
+    the step over the step's device time, every launch of the step included (a decode step's merge kernel, a bfloat16
+    cache's widening in front of the prompt kernel). `kernel_us` / `frac_kernel`: the dominant kernel alone, from the
+    committed kernel trace of this script."""
+    kernel = KERNEL[w.kind]
+    hbm = w.kind in ("pre", "decode")
+    ach = w.bytes / step_ns if hbm else w.flops / step_ns / 1e3
+    peak = PEAK_HBM_GBS if hbm else PEAK_TFLOPS_BF16
+    r = {"bound": "hbm" if hbm else "mfma", "achieved": round(ach, 2), "peak": peak, "unit": "GB/s" if hbm else "TFLOP/s", "frac": round(ach / peak, 4),
+         "traffic": from_profile(kernel, w.name, "traffic_bytes_per_launch"), "kernel": kernel, "step_us": round(step_ns / 1e3, 2)}
     if w.kind == "mla":
-        ach = w.flops / main_ns / 1e3
-        return {"bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_TFLOPS_BF16, "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS_BF16, 4),
-                "traffic": None, "kernel": "mla_decode_kernel", "kernel_us": round(main_ns / 1e3, 2), "hbm_GB/s": round(w.bytes / main_ns, 1)}
-    if w.kind == "prefill":
-        ach = w.flops / main_ns / 1e3
-        return {"bound": "mfma", "achieved": round(ach, 2), "peak": PEAK_TFLOPS_BF16, "unit": "TFLOP/s", "frac": round(ach / PEAK_TFLOPS_BF16, 4),
-                "traffic": None, "kernel": "attn_prefill_kernel", "kernel_us": round(main_ns / 1e3, 2)}
-    ach = w.bytes / main_ns
-    return {"bound": "hbm", "achieved": round(ach, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ach / PEAK_HBM_GBS, 4), "traffic": None,
-            "kernel": "attn_decode_kernel", "kernel_us": round(main_ns / 1e3, 2)}
+        r["hbm_GB/s"] = round(w.bytes / step_ns, 1)
+    kus = from_profile(kernel, w.name, "kernel_avg_us")
+    if kus:
+        r["kernel_us"] = kus
+        r["frac_kernel"] = round((w.bytes / kus / 1e3 if hbm else w.flops / kus / 1e6) / peak, 4)
+    return r
 
 
 def cpu_baseline(name):
@@ -324,7 +320,7 @@ def cpu_baseline(name):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="prefill8k", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -362,11 +358,11 @@ def main():
         nbuf = 1 if kind == "prefill" else 16 if kind == "mla" else 4 if kind == "pre" else max(4, int(np.ceil(600e6 / (2 * WORKLOADS[name][3] * WORKLOADS[name][5] * kv_bytes(WORKLOADS[name][6], WORKLOADS[name][4])))))
         nbuf = min(nbuf, 40)
         w = Workload(ops, name, nbuf)
-        ms, main_ns, merge_ns = timed(w, steps, warmup)
+        ms, step_ns = timed(w, steps, warmup)
         w.graph_ms = graph_step_ms(w)
-        return w, ms, main_ns, merge_ns
+        return w, ms, step_ns
 
-    w, ms, main_ns, merge_ns = run(a.workload, a.steps, a.warmup)
+    w, ms, step_ns = run(a.workload, a.steps, a.warmup)
     if w.kind == "pre":
         metric, unit, value = "pre-attention step HBM GB/s (algorithmic bytes), 1 MI355X", "GB/s", w.bytes / (ms * 1e-3) / 1e9
     elif w.kind == "mla":
@@ -384,10 +380,8 @@ def main():
                    "kv_form": {0: "f16", 1: "q8_0", 2: "q4_0", 3: "bf16"}[w.kt], "flops_per_step": w.flops, "bytes_per_step": w.bytes,
                    "untimed_settle_ms": SETTLE_MS},
         "tokens_per_s": round(w.T / (ms * 1e-3), 1),
-        "roofline": roofline(w, main_ns),
+        "roofline": roofline(w, step_ns),
     }
-    if merge_ns:
-        line["merge_kernel_us"] = round(merge_ns / 1e3, 2)
     if w.graph_ms:
         line["graph_ms_per_step"] = round(w.graph_ms, 5)
     del w
@@ -396,11 +390,10 @@ def main():
         for name in ("decode32k", "decode4k", "decode128k_q8", "verify64k", "mla32k", "prefill8k", "mla_prompt8k", "pre_store8k"):
             if name == a.workload:
                 continue
-            ww, m2, k2, g2 = run(name, max(10, a.steps), a.warmup)
+            ww, m2, k2 = run(name, max(10, a.steps), a.warmup)
             r = roofline(ww, k2)
             others[name] = {"ms_per_step": round(m2, 5), "step_" + ("TFLOP/s" if ww.kind not in ("decode", "pre") else "GB/s"):
-                            round((ww.flops / (m2 * 1e-3) / 1e12) if ww.kind not in ("decode", "pre") else (ww.bytes / (m2 * 1e-3) / 1e9), 2), "roofline": r,
-                            "merge_kernel_us": round(g2 / 1e3, 2)}
+                            round((ww.flops / (m2 * 1e-3) / 1e12) if ww.kind not in ("decode", "pre") else (ww.bytes / (m2 * 1e-3) / 1e9), 2), "roofline": r}
             if ww.graph_ms:
                 others[name]["graph_ms_per_step"] = round(ww.graph_ms, 5)
             del ww

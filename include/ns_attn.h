@@ -234,9 +234,8 @@ int ns_llm_minimaxm3_idx_topk(ns_gpu* g, float* bs, int32_t* sel, int64_t T, int
  * attention call records HIP events on the compute stream before its main kernel, between it and the merge kernel, and
  * after; ns_attn_profile_last waits for the last call's and returns the two kernels' device times in nanoseconds
  * (merge_ns 0 for a call without a merge). The events open gaps between the launches and read a few microseconds long
- * for kernels this short, so: on = 2: attention calls queue their main kernel ONLY - no merge launch, the output is NOT
- * written - and a run of such calls between two ns_stamp's divided by its length is that kernel's own launch duration
- * on a busy queue. on = 0 (the default): neither */
+ * for kernels this short: a kernel's own launch duration is what a kernel trace reports. on = 0 (the default): no
+ * events. Every call writes its output whatever the setting; other values of `on` are refused */
 int ns_attn_profile(ns_gpu* g, int on);
 /* a plain device-to-device copy kernel (16 bytes a thread, reads `bytes`, writes `bytes`): the kernel of known size that
  * rocprofv3's FETCH_SIZE / WRITE_SIZE counters are scaled against. This library's own */
@@ -253,8 +252,9 @@ int ns_q35_graph_launch(ns_gpu* g, void* h);
 void ns_q35_graph_free(void* h);
 /* Tuning knobs for sweeps and tests (this library's own): knob 0 work-groups a decode pass aims for, 1 key splits and
  * 2 waves a work-group (4 or 8) of a prompt pass, 3 work-groups an MLA pass aims for, 4 heads a wave of the
- * pre-attention kernel; value 0 = the library's own choice. Each knob starts from its environment variable (NS_DEC_WGS,
- * NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW), read once a process */
+ * pre-attention kernel, 5 = 1: a prompt pass over a bfloat16 cache keeps bfloat16 operands instead of widening the
+ * cache's rows to half first; value 0 = the library's own choice. Each knob starts from its environment variable
+ * (NS_DEC_WGS, NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW, NS_PREFILL_BF16), read once a process */
 int ns_attn_tune(int knob, int64_t value);
 
 #ifdef __cplusplus

@@ -230,7 +230,7 @@ int ns_mm3s_attend_block(ns_gpu* g, const float* q, const uint16_t* kc, const ui
 // ---- tuning knobs (tests and sweeps): read from the environment once, then only changed through ns_attn_tune
 
 namespace {
-const char* const TUNE_ENV[NS_TUNE_KNOBS] = {"NS_DEC_WGS", "NS_PREFILL_SPLITS", "NS_PREFILL_WAVES", "NS_MLA_WGS", "NS_PRE_HPW"};
+const char* const TUNE_ENV[NS_TUNE_KNOBS] = {"NS_DEC_WGS", "NS_PREFILL_SPLITS", "NS_PREFILL_WAVES", "NS_MLA_WGS", "NS_PRE_HPW", "NS_PREFILL_BF16"};
 std::atomic<int64_t>* tune_table() {
     static std::atomic<int64_t> t[NS_TUNE_KNOBS];
     static const bool once = [] {
@@ -250,7 +250,7 @@ int64_t ns_tune_get(int knob) { return knob >= 0 && knob < NS_TUNE_KNOBS ? tune_
 extern "C" {
 
 int ns_attn_tune(int knob, int64_t value) {
-    if (knob < 0 || knob >= NS_TUNE_KNOBS || value < 0) return ns_fail("ns_attn_tune: a knob 0..4 and a value of 0 (the default) or more");
+    if (knob < 0 || knob >= NS_TUNE_KNOBS || value < 0) return ns_fail("ns_attn_tune: a knob 0..5 and a value of 0 (the default) or more");
     tune_table()[knob].store(value, std::memory_order_relaxed);
     return 0;
 }

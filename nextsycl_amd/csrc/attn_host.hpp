@@ -31,7 +31,10 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
                        void* out);
 
 // Tuning knobs, 0 = the library's own choice: work-groups a decode pass aims for, key splits and waves of a prompt pass,
-// work-groups an MLA pass aims for, heads a wave of the pre-attention kernel. Each starts from its environment variable
-// (NS_DEC_WGS, NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW), read once, and changes only through ns_attn_tune
-enum { NS_TUNE_DEC_WGS = 0, NS_TUNE_PREFILL_SPLITS = 1, NS_TUNE_PREFILL_WAVES = 2, NS_TUNE_MLA_WGS = 3, NS_TUNE_PRE_HPW = 4, NS_TUNE_KNOBS = 5 };
+// work-groups an MLA pass aims for, heads a wave of the pre-attention kernel, and whether a prompt pass over a bfloat16
+// cache keeps bfloat16 operands (1) instead of widening its rows to half first. Each starts from its environment variable
+// (NS_DEC_WGS, NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW, NS_PREFILL_BF16), read once, and changes only
+// through ns_attn_tune
+enum { NS_TUNE_DEC_WGS = 0, NS_TUNE_PREFILL_SPLITS = 1, NS_TUNE_PREFILL_WAVES = 2, NS_TUNE_MLA_WGS = 3, NS_TUNE_PRE_HPW = 4, NS_TUNE_PREFILL_BF16 = 5,
+       NS_TUNE_KNOBS = 6 };
 int64_t ns_tune_get(int knob);

@@ -1082,7 +1082,7 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     }
     NS_LAUNCHED("mla_decode");
     if (ns_profile_mark(g, 1)) return -1;
-    if (ns > 1 && !g->main_only) {
+    if (ns > 1) {
         if (ot == 0) mla_merge_kernel<0><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
         else mla_merge_kernel<1><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
         NS_LAUNCHED("mla_merge");

@@ -46,8 +46,8 @@ int ns_profile_mark(ns_gpu* g, int i) {
 extern "C" {
 
 int ns_attn_profile(ns_gpu* g, int on) {
+    if (on != 0 && on != 1) return ns_fail("ns_attn_profile: 0 (off) or 1 (events around the kernels of every attention call)");
     g->profile = on == 1;
-    g->main_only = on == 2;
     g->pev_used = 0;
     return 0;
 }

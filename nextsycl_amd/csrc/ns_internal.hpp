@@ -22,9 +22,6 @@ struct ns_gpu {
     size_t own_scratch_floats = 0;
     // ns_attn_profile: events around the kernels of the last attention call (measurement only; off by default)
     bool profile = false;
-    // ns_attn_profile(g, 2): attention calls queue their main kernel only (no merge launch; the output is not written), so
-    // that back-to-back calls between two stamps time that kernel alone (measurement only)
-    bool main_only = false;
     hipEvent_t pev[3] = {nullptr, nullptr, nullptr};
     int pev_used = 0;
 };

@@ -1,6 +1,7 @@
 """Shared by the parity tests: seeded inputs from the oracle's generator, caches packed by the oracle's stores, the
 HIP path called through the C ABI wrappers, and the comparison measures (max-abs, relative L2) with the tolerances of
-the path: max-abs 2e-3 and relative L2 1e-3 against the float64 closed form for float32 / half outputs."""
+the path: max-abs 2e-3 and relative L2 1e-3 against the float64 closed form (`tolerances` states the one rule by which
+the absolute bound grows with the output's size and a bfloat16 rounding widens both)."""
 import numpy as np
 
 from nextsycl_amd import DevBuf
@@ -76,17 +77,47 @@ def gpu_prompt(ops, qt, kt, q_dev_arr, kc, vc, T, Hq, Hkv, D, cap, p0, win=0, pm
     return out_to_f32(qt, raw).reshape(T, Hq * D), raw
 
 
-def check_close(got, ref64, qt=F32, what="", kt=0):
-    """The path's bar against the float64 closed form: max-abs 2e-3, relative L2 1e-3. Where bfloat16 enters - output
-    rows of that type, or a bfloat16 cache (the kernel's MFMA operands are then bfloat16: the query and the softmax
-    weights are rounded to 8 significant bits) - the bound of that rounding, 2^-9 relative, is added: a correctly
-    rounded bfloat16 copy of the exact result already sits at ~1.6e-3 relative L2."""
+U_HALF, U_BF16 = 2.0 ** -11, 2.0 ** -8      # unit roundoffs: half carries 11 significant bits, bfloat16 8
+
+
+def tolerances(ref64, qt=F32, kt=0, bf16_weights=False, bf16_queries=False):
+    """The path's bar against the float64 closed form, as ONE rule for every cache form and row type.
+
+    relative L2 <= 1e-3 and max-abs <= max(2e-3, sum of u |ref|max over the 16-bit roundings between the stored values
+    and the output), u the unit roundoff of the rounded type (half 2^-11, bfloat16 2^-8). The roundings of a pass:
+      - the softmax weights, rounded for the second product: half (the reference: qwen35/silo/attn.cpp:225-227) - also
+        over a bfloat16 cache, whose values are widened to half for it (prompt passes) or whose weights are split into two
+        bfloat16 numbers (decode passes). bf16_weights: the one path that keeps a single bfloat16 weight, a prompt pass over
+        a bfloat16 cache too long for the library's scratch (or forced by knob 5);
+      - q8_0 / q4_0 values, staged as halfs before the products as the reference stages them (silo/attn.cpp:56-76), where
+        the closed form multiplies the unrounded int x scale;
+      - a 16-bit output row.
+    Why max-abs scales with |ref|max: an output that is the mean of two values v1, v2 under weights rounded with unit
+    roundoff u moves by up to u |v1 - v2| / 2 <= u |v|max, so the absolute bound 2e-3 can hold only while |out| < 4 (half).
+    A bfloat16 rounding is 8 times coarser: each adds 2^-9 to the relative bound as well (a correctly rounded bfloat16
+    copy of the exact result sits at ~1.6e-3 relative L2). bf16_queries: float32 / half query rows against a bfloat16
+    cache on a path that multiplies them as bfloat16 (they are rounded once to 8 bits for the first product)."""
+    n_half = (0 if bf16_weights else 1) + (kt in (1, 2)) + (qt == F16)
+    n_bf16 = (1 if bf16_weights else 0) + (qt == BF16) + (1 if bf16_queries else 0)
+    big = float(np.abs(ref64).max())
+    return max(MAX_ABS, (n_half * U_HALF + n_bf16 * U_BF16) * big), REL_L2 + n_bf16 * BF16_ROUND
+
+
+def check_close(got, ref64, qt=F32, what="", kt=0, bf16_weights=False, bf16_queries=False):
+    """got against the float64 closed form under `tolerances`; returns (max-abs, relative L2)."""
     mx, rel, cos = orc.compare(got, ref64)
-    tol_abs, tol_rel = MAX_ABS, REL_L2
-    if qt == BF16 or kt == 3:
-        # one rounding for the weights, one for an output of that type: each at most 2^-9 of the largest value
-        tol_abs = MAX_ABS + ((qt == BF16) + (kt == 3)) * BF16_ROUND * float(np.abs(ref64).max())
-        tol_rel = REL_L2 + BF16_ROUND
+    tol_abs, tol_rel = tolerances(ref64, qt, kt, bf16_weights, bf16_queries)
     assert np.isfinite(got).all(), "%s: non-finite output" % what
     assert mx <= tol_abs and rel <= tol_rel, "%s: max-abs %.3g (<= %.3g), rel-L2 %.3g (<= %.3g), cosine %.6f" % (what, mx, tol_abs, rel, tol_rel, cos)
     return mx, rel
+
+
+def assert_bf16_rows_follow(raw16, got32, what=""):
+    """A pass's bfloat16 output rows against the same pass's float32 output rows: each the rounding of the other's value up
+    to the one bfloat16 step by which two roundings of nearly the same number may differ (bfloat16 query rows enter the
+    first product as bfloat16, float32 ones as half: the same exact products, summed by two different matrix instructions),
+    and the same number in all but a few per thousand."""
+    want = orc.f2bf(np.ascontiguousarray(got32, np.float32)).ravel().astype(np.int32)
+    have = np.asarray(raw16).ravel().astype(np.int32)
+    step = np.abs(want - have)
+    assert step.max() <= 1 and np.count_nonzero(step) <= 5e-3 * step.size, "%s: up to %d steps apart, %d of %d differ" % (what, step.max(), np.count_nonzero(step), step.size)

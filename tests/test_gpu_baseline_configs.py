@@ -4,7 +4,7 @@ whole 256-row blocks against the closed form plus size-independent properties ov
 import numpy as np
 import pytest
 
-from helpers import SEED_K, SEED_Q, SEED_V, check_close, gpu_decode, gpu_prompt, make_kv, make_q
+from helpers import SEED_K, SEED_Q, SEED_V, assert_bf16_rows_follow, check_close, gpu_decode, gpu_prompt, make_kv, make_q
 from nextsycl_amd import DevBuf
 from nextsycl_amd.attn import BF16, F16, F32
 from oracle import orc
@@ -69,12 +69,6 @@ def test_config5_mtp_verify_64k(ops):
         assert np.array_equal(one, raw[t]), t
 
 
-# The float32-output variant of the bf16 prefill kernel is held to a fixed bound: relative L2 2.0e-3 against the float64
-# closed form on whole 256-row blocks. What is left in it is the rounding of the softmax weights to bfloat16 for the second
-# product (~1.5e-3 on its own); the queries enter the first product exactly as given.
-CONFIG2_F32_REL_L2 = 2.0e-3
-
-
 def test_config2_prefill_8k(ops, record_property):
     """configs[1]: seq 8192, 40 / 8 heads (G = 5), head 128, bf16 Q / K / V and output, causal. Three whole 256-row blocks
     (the first, a middle one, the last: every wave and row tile of a work-group, every head) against the float64 closed
@@ -86,10 +80,11 @@ def test_config2_prefill_8k(ops, record_property):
     bufs = (DevBuf.of(g, kc), DevBuf.of(g, vc))
     got, raw = gpu_prompt(ops, BF16, 3, qd, kc, vc, T, Hq, Hkv, D, T, 0, bufs=bufs)
     assert np.isfinite(got).all() and raw.shape == (T * Hq * D,)
-    # the float32-output variant of the same kernel: the kernel's own error without the output's bfloat16 rounding; the
-    # bfloat16 output is exactly its rounding
+    # the float32-output variant of the same pass: the kernel's own error without the output's bfloat16 rounding, held to
+    # the path's plain bar - max-abs 2e-3, relative L2 1e-3 (the cache's values are widened to half, exactly, and the
+    # softmax weights are half); the bfloat16 output is its rounding
     got32, _ = gpu_prompt(ops, F32, 3, qf, kc, vc, T, Hq, Hkv, D, T, 0, bufs=bufs)
-    assert np.array_equal(orc.f2bf(got32).ravel(), raw)
+    assert_bf16_rows_follow(raw, got32, "config 2")
     worst = [0.0, 0.0]
     for r0 in (0, 4096, 7936):
         ref = orc.attn_f64(qf[r0:r0 + 256], kc, vc, 3, 256, Hq, Hkv, D, T, r0)
@@ -97,7 +92,7 @@ def test_config2_prefill_8k(ops, record_property):
         mx, rel, _ = orc.compare(got32[r0:r0 + 256], ref)
         print("config 2, float32 output, rows %d..%d: max-abs %.3e, relative L2 %.3e" % (r0, r0 + 255, mx, rel))
         worst = [max(worst[0], mx), max(worst[1], rel)]
-        assert rel <= CONFIG2_F32_REL_L2 and mx <= 2e-3 + 2.0 ** -9 * np.abs(ref).max(), (r0, mx, rel)
+        assert rel <= 1e-3 and mx <= 2e-3, (r0, mx, rel)
     record_property("config2_f32_max_abs", worst[0])
     record_property("config2_f32_rel_l2", worst[1])
     # row 0 sees one key: its output is that key's value row, exactly
@@ -106,4 +101,4 @@ def test_config2_prefill_8k(ops, record_property):
     # V = 1 everywhere: every one of the 8192 x 40 x 128 outputs is 1 (each row's weights sum to one)
     ones = np.ascontiguousarray(np.broadcast_to(np.array([0x3F80], np.uint16).view(np.uint8), (Hkv, T, D, 2)).reshape(Hkv, T, 2 * D))
     g1, _ = gpu_prompt(ops, F32, 3, qf, kc, ones, T, Hq, Hkv, D, T, 0, bufs=(bufs[0], DevBuf.of(g, ones)))
-    assert np.abs(g1 - 1.0).max() < 4e-3         # the weights are rounded to bfloat16 for the product, their sum is not
+    assert np.abs(g1 - 1.0).max() < 1e-6         # numerator and denominator carry the very same rounded weights
