@@ -17,9 +17,11 @@
 //
 // A wave's tile step, in the transposed orientation (a lane owns one query row of each row tile, so the row maximum,
 // the rescale and the normalisation never leave the lane):
-//   S^T[key][row] = K Q^T        K from LDS as the A operand (ds_read_b128; rows padded to 288 bytes, or swizzled), Q^T in registers
-//   base-2 online softmax in float32 (scale folded into the exponent's fma; the accumulators rescaled only when a
-//   row's maximum moved); only 32-key halves crossing a row's causal or window edge are masked
+//   S^T[key][row] = K Q^T        K from LDS as the A operand (ds_read_b128; rows padded to 288 bytes, or swizzled), Q^T in registers.
+//                                Half operands: Q carries the softmax scale x log2 e and the product starts from minus the
+//                                softmax reference, so a score leaves the matrix unit as the argument of its exponential
+//   base-2 online softmax in float32 (the accumulators rescaled only when a row's maximum moved); only 32-key halves
+//   crossing a row's causal or window edge are masked
 //   P^T -> 16 bit = the B operand of the second product as it stands
 //   O^T[d][row]  += V^T P^T      V^T from LDS through ds_read_b64_tr_b16 (rows padded to 288 bytes, or swizzled)
 //
@@ -54,10 +56,6 @@ struct PrefillParams {
     const uint8_t* vc;
     int64_t head_stride, row_stride, cap;
     int wrap;
-    // the value cache's geometry when it is not the key cache's (a bfloat16 cache's values widened to half into a
-    // buffer of the library's: position order, never wrapped)
-    int64_t v_head_stride, v_row_stride;
-    int v_wrap;
     int T, Hq, G;
     int64_t p0, win;
     int causal;                 // 0: every row sees to the pass's last key (a draft block)
@@ -76,20 +74,20 @@ typedef uint32_t u4v __attribute__((ext_vector_type(4)));
 // the same at an address that is only 8-byte aligned (q8_0 / q4_0 rows of 128 values are 136 / 72 bytes long)
 typedef uint32_t u4a8 __attribute__((ext_vector_type(4), aligned(8)));
 
-// The queries enter the first product as they are given (16-bit rows bit for bit, float32 rows rounded once) and the
-// softmax scale (x log2 e) rides in one fused multiply-add a score. Folding the scale into the 16-bit query operand
-// instead saves that instruction but rounds 16-bit queries a second time (bfloat16 at 8192 rows: relative L2 against
-// the closed form 2.3e-3 instead of 1.5e-3)
-// BF: queries and keys are bfloat16 operands of the first product (else half); BFV: weights and values are bfloat16
-// operands of the second (else half). A bfloat16 cache runs <BF, !BFV> over values the host side has widened to half.
-template <int D, bool BF, bool BFV, int KT, int PW>
+// BF: bfloat16 operands (a bfloat16 cache too long to be widened to half first), else half.
+template <int D, bool BF, int KT, int PW>
 __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_prefill_kernel(const PrefillParams p) {
     static_assert(D == 128 || D == 256, "head size 128 or 256");
     static_assert(KT == 0 || !BF, "quantized rows are widened to half");
-    static_assert(BF || !BFV, "bfloat16 weights only over a bfloat16 cache");
     // a wave owns RT row tiles of 16: 32 rows at D = 128; 16 at D = 256, whose accumulators are twice as wide
     constexpr int RT = D == 128 ? 2 : 1, WROWS = RT * 16, ROWS = PW * WROWS;
     constexpr int KB = D / 32, DT = D / 16;
+    // Half operands: the query enters the first product scaled by the softmax scale x log2 e and rounded once to half - what
+    // the reference's kernels do (qwen35/silo/attn.cpp:112,147: qh = half(q x qscale)) - and the product starts from minus
+    // the softmax reference (ntile), so a score leaves the matrix unit as the argument of its exponential: no vector
+    // instruction a score between the two. bfloat16 operands (8 bits: a second rounding would show) keep the scale in a
+    // fused multiply-add a score.
+    constexpr bool PRESCALE = !BF;
     // bytes a staged key row / value row: rows 32 bytes apart modulo 256, so that the 16-byte operand reads of 16 keys (and
     // the transposing reads of the values) meet no bank conflict - 16 bytes apart the key reads would, two ways
     constexpr int KS = D * 2 + 32, VS = D * 2 + 32;
@@ -164,7 +162,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             for (int kb = 0; kb < KB; ++kb) {
                 const float f[8] = {raw[kb][0].x, raw[kb][0].y, raw[kb][0].z, raw[kb][0].w, raw[kb][1].x, raw[kb][1].y, raw[kb][1].z, raw[kb][1].w};
 #pragma unroll
-                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = to16<BF>(f[i]);
+                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = to16<BF>(PRESCALE ? f[i] * p.sl2 : f[i]);
             }
         } else {
             uint4 raw[KB];
@@ -176,14 +174,16 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
                     const uint16_t b16 = (uint16_t) (ww[i >> 1] >> (16 * (i & 1)));
-                    // rows of the operand type pass through bit for bit; the other 16-bit type is rounded once
-                    qreg[rt][kb][i] = (p.qt == 2) == BF ? (short) b16 : to16<BF>(p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16));
+                    // bfloat16 operands: rows of that type pass through bit for bit, others are rounded once; half operands:
+                    // the row x the scale, rounded once
+                    if constexpr (PRESCALE) qreg[rt][kb][i] = to16<BF>((p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16)) * p.sl2);
+                    else qreg[rt][kb][i] = (p.qt == 2) == BF ? (short) b16 : to16<BF>(p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16));
                 }
             }
         }
     }
     const uint8_t* kbase = p.kc + (int64_t) hk * p.head_stride;
-    const uint8_t* vbase = p.vc + (int64_t) hk * p.v_head_stride;
+    const uint8_t* vbase = p.vc + (int64_t) hk * p.head_stride;
     const int64_t t0 = kbeg / KT_TILE, t1 = (kend + KT_TILE - 1) / KT_TILE;
     const int nt = kend > kbeg ? (int) (t1 - t0) : 0;             // (a split past the block's last key: nothing to do)
     // From here on keys are counted from the first tile's first key (32-bit): tile k holds keys 64 k .. 64 k + 63, step
@@ -215,11 +215,13 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         thr[rt] = -INFINITY;
         l4[rt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
     }
-    f4v o[RT][DT];
+    f4v o[RT][DT], ntile[RT];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+    for (int rt = 0; rt < RT; ++rt) {
+        ntile[rt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) o[rt][dt] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+    }
 
     // ---- global -> registers -> LDS. A cache row is fetched in 16-byte raw chunks: 16-bit rows D / 8 of them, each one
     // LDS piece; q8_0 rows D / 16 (16 int8 -> 2 pieces of 8 halfs, the block's half scale fetched beside it); q4_0 rows
@@ -237,33 +239,30 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         u4v raw[NST];
         uint16_t sc[KT == 0 ? 1 : NST];
     };
-    const int64_t kbeg_slot = p.wrap ? kbeg % p.cap : kbeg, vbeg_slot = p.v_wrap ? kbeg % p.cap : kbeg;
+    const int64_t kbeg_slot = p.wrap ? kbeg % p.cap : kbeg;
     const int kspan = (int) (kend - kbeg) - 1;
     const int kbeg32 = (int) (kbeg - base);
     const int key0 = tid / CPR, rc = tid % CPR;                   // chunk i of this thread: key key0 + KPI i, raw chunk rc
     const uint32_t lane_off = (uint32_t) (key0 * p.row_stride) + (uint32_t) rc * 16;
-    const uint32_t lane_off_v = (uint32_t) (key0 * p.v_row_stride) + (uint32_t) rc * 16;
     // where a chunk's scale sits in its row: q8_0 a half a block of 32 behind D values, q4_0 behind D / 2 bytes
     // (as a distance from the chunk itself)
     const uint32_t sc_rel = (KT == 1 ? (uint32_t) (D + 2 * (rc / 2)) : (uint32_t) (D / 2 + 2 * rc)) - (uint32_t) rc * 16;
     const int plain0 = kbeg32 > 0 ? 1 : 0, plain1 = p.wrap ? -1 : (int) ((kend - base) / KT_TILE) - 1;
-    const int plain1_v = p.v_wrap ? -1 : (int) ((kend - base) / KT_TILE) - 1;
-    auto fetch = [&](Stage& st, const uint8_t* cache, int krel, auto which_c) {
-        constexpr bool VAL = decltype(which_c)::value;
-        const int64_t rs = VAL ? p.v_row_stride : p.row_stride;
-        const bool wrap = VAL ? p.v_wrap : p.wrap;
+    auto fetch = [&](Stage& st, const uint8_t* cache, int krel) {
+        const int64_t rs = p.row_stride;
+        const bool wrap = p.wrap;
         const uint8_t* sp = cache;
         uint32_t off[NST];                                        // of the raw chunk
-        if (krel >= plain0 && krel <= (VAL ? plain1_v : plain1)) {
+        if (krel >= plain0 && krel <= plain1) {
             sp += (base + (int64_t) krel * KT_TILE) * rs;
 #pragma unroll
-            for (int i = 0; i < NST; ++i) off[i] = (VAL ? lane_off_v : lane_off) + (uint32_t) (i * KPI * rs);
+            for (int i = 0; i < NST; ++i) off[i] = lane_off + (uint32_t) (i * KPI * rs);
         } else {
             const int rel0 = krel * KT_TILE - kbeg32 + key0;
 #pragma unroll
             for (int i = 0; i < NST; ++i) {
                 const int rel = std::min(std::max(rel0 + KPI * i, 0), kspan);
-                int64_t slot = (VAL ? vbeg_slot : kbeg_slot) + rel;
+                int64_t slot = kbeg_slot + rel;
                 if (wrap) {
                     slot = slot >= p.cap ? slot - p.cap : slot;
                     slot = slot >= p.cap ? slot - p.cap : slot;
@@ -319,7 +318,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         for (int j = 0; j < NJ; ++j) {
             const int r = (w * NJ + j) * 4 + (lane >> 4), cp = lane & 15;
             koff[j] = (uint32_t) (r * p.row_stride) + (uint32_t) ((cp ^ (r & 15)) << 4);
-            voff[j] = (uint32_t) (r * p.v_row_stride) + (uint32_t) ((cp ^ (2 * (r & 7))) << 4);
+            voff[j] = (uint32_t) (r * p.row_stride) + (uint32_t) ((cp ^ (2 * (r & 7))) << 4);
         }
     }
     // (one transfer instruction: 64 lanes x 16 bytes from base + the lane's offset to 1 KiB of LDS at dst, wave-uniform.
@@ -334,9 +333,9 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     };
     auto dma = [&](lds_u8* dst, const uint8_t* cache, int krel, auto which_c) __attribute__((always_inline)) {
         constexpr bool VAL = decltype(which_c)::value;
-        const int64_t rs = VAL ? p.v_row_stride : p.row_stride;
-        const bool wrap = VAL ? p.v_wrap : p.wrap;
-        if (krel >= plain0 && krel <= (VAL ? plain1_v : plain1)) {
+        const int64_t rs = p.row_stride;
+        const bool wrap = p.wrap;
+        if (krel >= plain0 && krel <= plain1) {
             const uint8_t* sp = cache + (base + (int64_t) krel * KT_TILE) * rs;
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
@@ -346,7 +345,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             for (int j = 0; j < NJ; ++j) {
                 const int r = (w * NJ + j) * 4 + (lane >> 4), cp = lane & 15;
                 const int rel = std::min(std::max(krel * KT_TILE - kbeg32 + r, 0), kspan);
-                int64_t slot = (VAL ? vbeg_slot : kbeg_slot) + rel;
+                int64_t slot = kbeg_slot + rel;
                 if (wrap) {
                     slot = slot >= p.cap ? slot - p.cap : slot;
                     slot = slot >= p.cap ? slot - p.cap : slot;
@@ -423,7 +422,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                 for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt)
-                        s[rt][kt2] = mfma16<BF>(kpre[kt2][kb], qreg[rt][kb], kb == 0 ? f4v{0.0f, 0.0f, 0.0f, 0.0f} : s[rt][kt2]);
+                        s[rt][kt2] = mfma16<BF>(kpre[kt2][kb], qreg[rt][kb], kb == 0 ? ntile[rt] : s[rt][kt2]);
         } else {
 #pragma unroll
             for (int kt2 = 0; kt2 < 2; ++kt2) {
@@ -433,7 +432,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                     ka[kb] = kt2 == 0 ? kpre[0][kb] : *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(kl + k_rd + kt2 * 16 * KS + kb * 64);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
-                    f4v acc = mfma16<BF>(ka[0], qreg[rt][0], f4v{0.0f, 0.0f, 0.0f, 0.0f});
+                    f4v acc = mfma16<BF>(ka[0], qreg[rt][0], ntile[rt]);
 #pragma unroll
                     for (int kb = 1; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
                     s[rt][kt2] = acc;
@@ -442,16 +441,16 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         }
     };
     // O^T += V^T P^T of one 32-key half (LDS byte offset vl) with the weights in pb
-    constexpr short ONE16 = BFV ? (short) 0x3F80 : (short) 0x3C00;
+    constexpr short ONE16 = BF ? (short) 0x3F80 : (short) 0x3C00;
     const s8v ones = {ONE16, ONE16, ONE16, ONE16, ONE16, ONE16, ONE16, ONE16};
     auto weigh = [&](const lds_u8* vl, const s8v (&vpre)[VPRE]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) l4[rt] = mfma16<BFV>(ones, pb[rt], l4[rt]);
+        for (int rt = 0; rt < RT; ++rt) l4[rt] = mfma16<BF>(ones, pb[rt], l4[rt]);
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const s8v va = dt < VPRE ? vpre[dt] : vread1(vl, dt);
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) o[rt][dt] = mfma16<BFV>(va, pb[rt], o[rt][dt]);
+            for (int rt = 0; rt < RT; ++rt) o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
         }
     };
     // One step of the wave's software pipeline. Step s holds the scores of its own half in sc (computed a step earlier)
@@ -491,7 +490,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) a[rt][e] = __builtin_fmaf(sc[rt][e >> 2][e & 3], p.sl2, nbr[rt]);
+            for (int e = 0; e < 8; ++e) a[rt][e] = PRESCALE ? sc[rt][e >> 2][e & 3] : __builtin_fmaf(sc[rt][e >> 2][e & 3], p.sl2, nbr[rt]);
         weigh(vl_prev, vpre);
         bool grow = false;
 #pragma unroll
@@ -504,7 +503,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
             for (int i = 0; i < RT * DT + RT; ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, PRESCALE ? 1 : 2, 0);
             }
         }
         if (bar_mid) tile_barrier();
@@ -520,6 +519,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) o[rt][dt] *= c;
                 nbr[rt] -= delta;
+                if constexpr (PRESCALE) ntile[rt] = f4v{nbr[rt], nbr[rt], nbr[rt], nbr[rt]};
 #pragma unroll
                 for (int e = 0; e < 8; ++e) a[rt][e] -= delta;
                 thr[rt] = (fresh && nokey) ? -INFINITY : 8.0f;
@@ -529,7 +529,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) pb[rt][e] = to16<BFV>(fast_exp2(a[rt][e]));     // -inf -> 0
+            for (int e = 0; e < 8; ++e) pb[rt][e] = to16<BF>(fast_exp2(a[rt][e]));     // -inf -> 0
         }
         if constexpr (D == 128) {
             // a matrix instruction, an exponential, and a conversion after every other
@@ -656,10 +656,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");           // (transfers past the last tile land in buffers the output goes through)
       } else {
         Stage stk, stv;
-        const std::false_type KEYS;
-        const std::true_type VALUES;
-        fetch(stk, kbase, 0, KEYS);
-        fetch(stv, vbase, 0, VALUES);
+        fetch(stk, kbase, 0);
+        fetch(stv, vbase, 0);
         {   // the V buffer step 0 "adds" with zero weights must hold numbers
             const u4v z = {0u, 0u, 0u, 0u};
             for (uint32_t at = (uint32_t) tid * 16; at < (uint32_t) VBUF; at += PW * 64 * 16)
@@ -667,8 +665,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         }
         stash_k(stk, 0);
         stash_v(stv, 0);
-        fetch(stk, kbase, 1, KEYS);
-        fetch(stv, vbase, 1, VALUES);
+        fetch(stk, kbase, 1);
+        fetch(stv, vbase, 1);
         __syncthreads();
         {
             s8v kpre[KPRE][KB];
@@ -678,20 +676,20 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         for (int k = 0; k < nt; k += 2) {
             // tile k: buffers 0
             stash_k(stk, 1);
-            fetch(stk, kbase, k + 2, KEYS);
+            fetch(stk, kbase, k + 2);
             step(sA, sB, L + 32 * KS, L + V0 + VBUF + 32 * VS, 64 * k, !(64 * k >= w_full_beg && 64 * k + 32 <= w_full_end), upper);
             if (!upper) __syncthreads();
             stash_v(stv, 1);
-            fetch(stv, vbase, k + 2, VALUES);
+            fetch(stv, vbase, k + 2);
             step(sB, sA, L + KBUF, L + V0, 64 * k + 32, !(64 * k + 32 >= w_full_beg && 64 * k + 64 <= w_full_end));
             if (k + 1 >= nt) break;
             // tile k + 1: buffers 1
             stash_k(stk, 0);
-            fetch(stk, kbase, k + 3, KEYS);
+            fetch(stk, kbase, k + 3);
             step(sA, sB, L + KBUF + 32 * KS, L + V0 + 32 * VS, 64 * k + 64, !(64 * k + 64 >= w_full_beg && 64 * k + 96 <= w_full_end), upper);
             if (!upper) __syncthreads();
             stash_v(stv, 0);
-            fetch(stv, vbase, k + 3, VALUES);
+            fetch(stv, vbase, k + 3);
             step(sB, sA, L, L + V0 + VBUF, 64 * k + 96, !(64 * k + 96 >= w_full_beg && 64 * k + 128 <= w_full_end));
         }
         // the last step's product
@@ -799,19 +797,17 @@ __global__ __launch_bounds__(256) void kv_bf16_to_half_kernel(const WidenParams 
     *reinterpret_cast<u4v*>(p.dst[z] + (((int64_t) h * p.n + j) * CPR + c) * 16) = y;
 }
 
-// vhalf: a bfloat16 cache whose values the caller has widened to half (the weights are then half as well)
 template <int D, int PW>
-int launch_prefill(ns_gpu* g, int kt, bool vhalf, const PrefillParams& p, dim3 grid) {
+int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
     constexpr int TH = PW * 64;
     if (kt == 0) {
-        attn_prefill_kernel<D, false, false, 0, PW><<<grid, TH, 0, g->q>>>(p);
+        attn_prefill_kernel<D, false, 0, PW><<<grid, TH, 0, g->q>>>(p);
     } else if (kt == 3) {
-        if (vhalf) attn_prefill_kernel<D, true, false, 0, PW><<<grid, TH, 0, g->q>>>(p);
-        else attn_prefill_kernel<D, true, true, 0, PW><<<grid, TH, 0, g->q>>>(p);
+        attn_prefill_kernel<D, true, 0, PW><<<grid, TH, 0, g->q>>>(p);
     } else if (kt == 1) {
-        attn_prefill_kernel<D, false, false, 1, PW><<<grid, TH, 0, g->q>>>(p);
+        attn_prefill_kernel<D, false, 1, PW><<<grid, TH, 0, g->q>>>(p);
     } else if constexpr (D == 256 || PW == 4) {
-        attn_prefill_kernel<D, false, false, 2, PW><<<grid, TH, 0, g->q>>>(p);
+        attn_prefill_kernel<D, false, 2, PW><<<grid, TH, 0, g->q>>>(p);
     } else {
         // (a q4_0 tile of 128-value rows is 256 chunks: fewer than 8 waves have threads - the caller takes 4 waves)
         return ns_fail("ns_attn_prompt: internal: q4_0 rows of 128 values take 4 waves");
@@ -895,28 +891,22 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     p.kbs = skbs;
     p.k0 = sk0;
     p.part = g->own_scratch;
-    p.v_head_stride = p.head_stride;
-    p.v_row_stride = p.row_stride;
-    p.v_wrap = p.wrap;
-    // A bfloat16 cache. The second product's weights would be bfloat16 too - 8 significant bits, a relative L2 error of
-    // ~1.6e-3 in the output on its own - so the pass's value rows are first widened to half (exactly: see
-    // kv_bf16_to_half_kernel) into the library's scratch, behind the key splits' partials, and the weights are half, as
-    // in the reference's kernels. The first product takes bfloat16 queries and the keys as they are (both exact); rows of
-    // another type would be rounded to 8 bits for it, so for them the keys are widened as well and the pass runs as one
-    // over a half cache. A pass whose rows do not fit the scratch keeps bfloat16 operands throughout (so does knob 5 = 1).
-    bool vhalf = false;
+    // A bfloat16 cache. As bfloat16 operands the softmax weights would carry 8 significant bits - a relative L2 error of
+    // ~1.6e-3 in the output on its own - and the query could not take the scale (a second rounding at 8 bits shows). So the
+    // pass's key and value rows are first widened to half (exactly: see kv_bf16_to_half_kernel) into the library's scratch,
+    // behind the key splits' partials, and the pass runs as one over a half cache: half weights and a scaled half query, as
+    // in the reference's kernels. A pass whose rows do not fit the scratch keeps bfloat16 operands (so does knob 5 = 1).
     int kt_run = kt;
     if (kt == 3 && ns_tune_get(NS_TUNE_PREFILL_BF16) != 1) {
         const int64_t kf = kfirst >= 0 ? kfirst : win > 0 ? std::max<int64_t>(0, p0 + 1 - win) : 0, n = p0 + T - kf;
-        const int both = qt != 2;
         const size_t part_bytes = sns > 1 ? ((size_t) (T * Hq * sns * (D + 2)) * 4 + 255) / 256 * 256 : 0;
         const size_t one = (size_t) (Hkv * n * D * 2);
-        if (part_bytes + (both ? 2 : 1) * one <= g->own_scratch_floats * 4 && n * D * 2 < (int64_t) 1 << 32) {
+        if (part_bytes + 2 * one <= g->own_scratch_floats * 4 && n * D * 2 < (int64_t) 1 << 32) {
             uint8_t* const buf = (uint8_t*) g->own_scratch + part_bytes;
             WidenParams wp{};
-            wp.src[0] = (const uint8_t*) vc;
+            wp.src[0] = (const uint8_t*) kc;
             wp.dst[0] = buf;
-            wp.src[1] = (const uint8_t*) kc;
+            wp.src[1] = (const uint8_t*) vc;
             wp.dst[1] = buf + one;
             wp.head_stride = p.head_stride;
             wp.row_stride = p.row_stride;
@@ -924,30 +914,24 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
             wp.kf = kf;
             wp.n = n;
             wp.wrap = p.wrap;
-            const dim3 wgrid((unsigned) ((n * (D / 8) + 255) / 256), (unsigned) Hkv, both ? 2u : 1u);
+            const dim3 wgrid((unsigned) ((n * (D / 8) + 255) / 256), (unsigned) Hkv, 2u);
             if (D == 128) kv_bf16_to_half_kernel<16><<<wgrid, 256, 0, g->q>>>(wp);
             else kv_bf16_to_half_kernel<32><<<wgrid, 256, 0, g->q>>>(wp);
             NS_LAUNCHED("kv_bf16_to_half");
             // (position j of head h at buf + (h n + j - kf) 2 D: the kernel is given the address position 0 would have)
-            p.vc = buf - kf * D * 2;
-            p.v_head_stride = n * D * 2;
-            p.v_row_stride = D * 2;
-            p.v_wrap = 0;
-            vhalf = true;
-            if (both) {
-                p.kc = buf + one - kf * D * 2;
-                p.head_stride = p.v_head_stride;
-                p.row_stride = p.v_row_stride;
-                p.wrap = 0;
-                kt_run = 0;
-            }
+            p.kc = buf - kf * D * 2;
+            p.vc = buf + one - kf * D * 2;
+            p.head_stride = n * D * 2;
+            p.row_stride = D * 2;
+            p.wrap = 0;
+            kt_run = 0;
         }
     }
     const int64_t units = ((T + ROWS - 1) / ROWS) * Hkv;               // (row block, key head); padded to the 8 XCDs
     dim3 grid((unsigned) ((units + 7) / 8 * 8 * (Hq / Hkv)), (unsigned) p.ns);
     if (ns_profile_mark(g, 0)) return -1;
-    if ((D == 256 ? (PWs == 8 ? launch_prefill<256, 8>(g, kt_run, vhalf, p, grid) : launch_prefill<256, 4>(g, kt_run, vhalf, p, grid))
-                  : PWs == 8 ? launch_prefill<128, 8>(g, kt_run, vhalf, p, grid) : launch_prefill<128, 4>(g, kt_run, vhalf, p, grid)) != 0)
+    if ((D == 256 ? (PWs == 8 ? launch_prefill<256, 8>(g, kt_run, p, grid) : launch_prefill<256, 4>(g, kt_run, p, grid))
+                  : PWs == 8 ? launch_prefill<128, 8>(g, kt_run, p, grid) : launch_prefill<128, 4>(g, kt_run, p, grid)) != 0)
         return -1;
     NS_LAUNCHED("attn_prefill");
     if (ns_profile_mark(g, 1)) return -1;
