@@ -397,10 +397,11 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
             if (more) stash(nx1, H1, NLD);
             __syncthreads();
         } else {
-            // this wave's transfers of tile it + 1 are done when at most tile it + 2's are still in flight; a bare
-            // barrier then (the fence of __syncthreads would wait for tile it + 2 as well)
-            if (it + 2 < nt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
-            else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            // this wave's transfers of tile it + 1 are done when at most tile it + 2's are still in flight, and every LDS read
+            // it has issued has returned (a wave past the barrier requests a transfer into the buffer this step read); a
+            // bare barrier then (the fence of __syncthreads would wait for tile it + 2 as well)
+            if (it + 2 < nt) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(NDMA) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         }
@@ -510,8 +511,8 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
         const float amax = args_of(s, it + 1, a_cur);
         regrow(amax, a_cur);
         // (the next step's first block reads tile it + 2, requested a step ago: only this step's request may stay out)
-        if (it + 3 < nt) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (it + 3 < nt) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(NDMA) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
@@ -536,8 +537,8 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
         if (nt > 0) dma(B0, 0);
         if (nt > 1) dma(B1, 1);
         load_queries();
-        if (nt > 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (nt > 1) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(NDMA) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         for (int it = 0; it < nt; it += 3) {
@@ -553,8 +554,8 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
         if (nt > 1) dma(B1, 1);
         load_queries();
         if (nt > 2) dma(B2, 2);
-        if (nt > 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NDMA) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (nt > 2) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(NDMA) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (nt > 0) {

@@ -55,6 +55,7 @@ int ns_attn_profile(ns_gpu* g, int on) {
 int ns_attn_profile_last(ns_gpu* g, double* main_ns, double* merge_ns) {
     NS_TRY
     *main_ns = *merge_ns = 0.0;
+    if (g->recording) return ns_fail("ns_attn_profile_last: the compute stream is recording a graph (ns_q35_graph_end first)");
     if (g->pev_used < 2) return ns_fail("ns_attn_profile_last: no profiled attention call yet");
     NS_HIP(hipSetDevice(g->dev));
     NS_HIP(hipEventSynchronize(g->pev[g->pev_used - 1]));
@@ -138,6 +139,7 @@ int ns_gpu_open(int index, ns_gpu** out) {
 void ns_gpu_close(ns_gpu* g) {
     if (!g) return;
     (void) hipSetDevice(g->dev);
+    if (g->recording) ns_graph_drop(g->recording);                // (a recording still open ends here; its handle stays the caller's to free)
     if (g->q) (void) hipStreamSynchronize(g->q);
     if (g->cq) (void) hipStreamSynchronize(g->cq);
     if (g->cq2) (void) hipStreamSynchronize(g->cq2);
@@ -162,19 +164,38 @@ namespace {
 struct NsGraph {
     int dev = 0;
     hipStream_t q = nullptr;          // the stream that records; null once recording has ended
+    ns_gpu* owner = nullptr;          // the handle that records (null once recording has ended, or the handle has been closed)
     hipGraphExec_t exec = nullptr;
 };
+// ends a recording that is still open and drops what it recorded
+void drop_recording(NsGraph* gr) {
+    if (!gr->q) return;
+    hipGraph_t graph = nullptr;
+    (void) hipSetDevice(gr->dev);
+    if (hipStreamEndCapture(gr->q, &graph) == hipSuccess && graph) (void) hipGraphDestroy(graph);
+    gr->q = nullptr;
+    if (gr->owner) gr->owner->recording = nullptr;
+    gr->owner = nullptr;
+}
 }  // namespace
+
+void ns_graph_drop(void* h) { drop_recording(static_cast<NsGraph*>(h)); }
 
 int ns_q35_graph_begin(ns_gpu* g, void** out) {
     NS_TRY
     if (!g || !out) return ns_fail("ns_q35_graph_begin: a null argument");
+    if (g->recording) return ns_fail("ns_q35_graph_begin: this GPU is recording a graph already");
     NS_HIP(hipSetDevice(g->dev));
-    // (relaxed: other threads of the engine may be allocating or copying on their own streams meanwhile)
-    NS_HIP(hipStreamBeginCapture(g->q, hipStreamCaptureModeRelaxed));
-    NsGraph* gr = new NsGraph;
+    NsGraph* gr = new NsGraph;        // (before the capture begins: a failure here leaves the stream as it was)
     gr->dev = g->dev;
     gr->q = g->q;
+    gr->owner = g;
+    // (relaxed: other threads of the engine may be allocating or copying on their own streams meanwhile)
+    if (ns_hip_check(hipStreamBeginCapture(g->q, hipStreamCaptureModeRelaxed), "hipStreamBeginCapture") != 0) {
+        delete gr;
+        return -1;
+    }
+    g->recording = gr;
     *out = gr;
     return 0;
     NS_CATCH
@@ -187,6 +208,8 @@ int ns_q35_graph_end(ns_gpu* g, void* h) {
     if (!gr->q || gr->q != g->q) return ns_fail("ns_q35_graph_end: not the graph this GPU is recording");
     NS_HIP(hipSetDevice(g->dev));
     gr->q = nullptr;
+    gr->owner = nullptr;
+    g->recording = nullptr;
     hipGraph_t graph = nullptr;
     NS_HIP(hipStreamEndCapture(g->q, &graph));
     if (!graph) return ns_fail("ns_q35_graph_end: the recording was dropped (a call that cannot be recorded was made on the stream)");
@@ -212,11 +235,7 @@ int ns_q35_graph_launch(ns_gpu* g, void* h) {
 void ns_q35_graph_free(void* h) {
     NsGraph* gr = static_cast<NsGraph*>(h);
     if (!gr) return;
-    if (gr->q) {                      // freed while still recording: the recording ends here, and is dropped
-        hipGraph_t graph = nullptr;
-        (void) hipSetDevice(gr->dev);
-        if (hipStreamEndCapture(gr->q, &graph) == hipSuccess && graph) (void) hipGraphDestroy(graph);
-    }
+    drop_recording(gr);               // (freed while still recording: the recording ends here, and is dropped)
     if (gr->exec) {
         (void) hipSetDevice(gr->dev);
         (void) hipGraphExecDestroy(gr->exec);
@@ -357,6 +376,7 @@ int ns_stamp(ns_gpu* g, int64_t* ticket) { return ns_mark(g, ticket); }
 
 int ns_elapsed(ns_gpu* g, int64_t t0, int64_t t1, double* ns) {
     NS_TRY
+    if (g->recording) return ns_fail("ns_elapsed: the compute stream is recording a graph (ns_q35_graph_end first)");
     NS_HIP(hipSetDevice(g->dev));
     hipEvent_t a = ticket_event(g, t0), b = ticket_event(g, t1);
     if (!a || !b) return ns_fail("ns_elapsed: a ticket that was never issued");
@@ -371,6 +391,7 @@ int ns_elapsed(ns_gpu* g, int64_t t0, int64_t t1, double* ns) {
 
 int ns_sync(ns_gpu* g) {
     NS_TRY
+    if (g->recording) return ns_fail("ns_sync: the compute stream is recording a graph (ns_q35_graph_end first)");
     NS_HIP(hipSetDevice(g->dev));
     NS_HIP(hipStreamSynchronize(g->q));
     return 0;

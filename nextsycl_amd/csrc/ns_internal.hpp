@@ -24,6 +24,9 @@ struct ns_gpu {
     bool profile = false;
     hipEvent_t pev[3] = {nullptr, nullptr, nullptr};
     int pev_used = 0;
+    // the graph this handle's compute stream is recording into (ns_q35_graph_begin .. _end), or null: while it is set, calls
+    // that wait for the stream (ns_sync, ns_elapsed, ns_attn_profile_last) are refused, and ns_gpu_close drops the recording
+    void* recording = nullptr;
 };
 
 // records profile event i on the compute stream when profiling is on (creates it on first use); 0 or -1
@@ -32,6 +35,9 @@ int ns_profile_mark(ns_gpu* g, int i);
 // attn_decode.hip: looks up, once a device and with that device current, the address of the device-resident scratch
 // array that ns_attn_decode_static uses (called by ns_gpu_open); 0 or -1
 int ns_attn_static_scratch_init(int dev);
+
+// ns_hip.cpp: ends the recording of a graph handle (ns_q35_graph_begin) that is still open and drops what it recorded
+extern "C" void ns_graph_drop(void* h);
 
 // sets the calling thread's error text (ns_last_error) and returns -1
 int ns_fail(const std::string& what);

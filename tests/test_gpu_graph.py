@@ -100,7 +100,13 @@ def test_decode_token_through_the_library_graph_calls():
         ops.ok(ops.k.q35_graph_begin(ops.raw(), C.byref(h)), "graph begin")
         token()
         assert ops.k.q35_graph_launch(ops.raw(), h) == -1 and "not finished" in g.api.error()
+        # while the stream records, calls that would wait for it are refused (and the recording survives them), and a
+        # second recording cannot begin
+        assert g.api.sync(g.raw) == -1 and "recording" in g.api.error()
+        h2 = C.c_void_p()
+        assert ops.k.q35_graph_begin(ops.raw(), C.byref(h2)) == -1 and "recording" in g.api.error()
         ops.k.q35_graph_free(h)
+        g.sync()                                        # (the stream runs again)
         g.sync()
         # the recording that is kept
         ob.fill(0xFF)

@@ -46,3 +46,54 @@ def test_static_scratch_decode_rejects_what_does_not_fit(ops):
     assert rc == -1 and "the array holds" in ops.k.api.error()
     with pytest.raises(Error):
         ops.decode_static(F32, 0, b, Hq * D, b, b, 17, Hq, Hkv, D, 64, 0, b)
+
+
+def test_static_scratch_decode_allocates_nothing(ops):
+    """A run of calls leaves the device's free memory where it was (ns_gpu_memory around 50 calls whose buffers all exist
+    beforehand), and a call goes through a stream capture that forbids allocation (mode "global": any hipMalloc on any
+    thread fails the capture) - kernel launches are all it queues."""
+    import ctypes as C
+
+    g = ops.gpu
+    T, Hq, Hkv, D, p0 = 2, 16, 2, 128, 3000
+    cap = p0 + T
+    kc, vc = make_kv(0, Hkv, D, cap, cap)
+    qd, _ = make_q(F16, T, Hq, D)
+    kcb, vcb, qb, ob = DevBuf.of(g, kc), DevBuf.of(g, vc), DevBuf.of(g, qd), DevBuf(g, T * Hq * D * 2)
+    ops.decode_static(F16, 0, qb, Hq * D, kcb, vcb, T, Hq, Hkv, D, cap, p0, ob)      # (first call: anything lazy has happened)
+    g.sync()
+    want = ob.read(np.uint16)
+    total, free0 = C.c_uint64(), C.c_int64()
+    assert g.api.gpu_memory(g.raw, C.byref(total), C.byref(free0)) == 0
+    for _ in range(50):
+        ops.decode_static(F16, 0, qb, Hq * D, kcb, vcb, T, Hq, Hkv, D, cap, p0, ob)
+    g.sync()
+    free1 = C.c_int64()
+    assert g.api.gpu_memory(g.raw, C.byref(total), C.byref(free1)) == 0
+    assert free1.value == free0.value
+    # under a capture that refuses allocation
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    stream = C.cast(C.c_void_p(g.api.gpu_queue(g.raw)), C.POINTER(C.c_void_p))[0]
+    graph, ex = C.c_void_p(), C.c_void_p()
+    ob.fill(0)
+    g.sync()
+    assert hip.hipStreamBeginCapture(stream, 0) == 0                                   # hipStreamCaptureModeGlobal
+    try:
+        ops.decode_static(F16, 0, qb, Hq * D, kcb, vcb, T, Hq, Hkv, D, cap, p0, ob)
+    finally:
+        rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+    assert rc == 0 and graph.value
+    assert hip.hipGraphInstantiate(C.byref(ex), graph, None, None, 0) == 0
+    try:
+        assert hip.hipGraphLaunch(ex, stream) == 0
+        g.sync()
+        assert np.array_equal(ob.read(np.uint16), want)
+    finally:
+        hip.hipGraphExecDestroy(ex)
+        hip.hipGraphDestroy(graph)
