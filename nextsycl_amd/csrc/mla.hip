@@ -78,13 +78,22 @@ struct MlaParams {
 
 typedef uint32_t u4v __attribute__((ext_vector_type(4)));   // a 16-byte chunk in flight (a plain vector: stays in registers)
 
-// R: rope features (64: DeepSeek's [512 | 64] rows; 0: GLM's latent-only rows); Q8: GLM's q8 rows
-template <int R, bool Q8, int MW>
+// floats of a split's partial of a row of LW latents: {half u_s[LW], float m, l, -, -}
+constexpr int pstride_of(int LW) { return LW / 2 + 4; }
+
+// LW: latent width (512; 256: GLM's other width, latent-only half rows); R: rope features (64: DeepSeek's [512 | 64] rows;
+// 0: GLM's latent-only rows); Q8: GLM's q8 rows
+template <int LW, int R, bool Q8, int MW>
 __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(const MlaParams p) {
+    static_assert(LW == 512 || (LW == 256 && R == 0 && !Q8), "latent rows of 512, or latent-only half rows of 256");
+    constexpr int ML = LW, PSTRIDE = pstride_of(LW);     // (inside this kernel the latent width is the template's)
     constexpr int MROWS = MW * 16;
     constexpr int DK = ML + R, KB = DK / 32, DT = ML / 16;
-    constexpr int RCH = 74, RSTRIDE = RCH * 16;          // chunks / bytes a staged row (whatever DK)
-    constexpr int TILEB = MTILE * RSTRIDE;
+    // chunks / bytes a staged row: the data's chunks + 2 of padding at width 512 (whatever R), so that rows lie an odd
+    // multiple of 32 bytes apart modulo 256
+    constexpr int RCH = LW == 512 ? 74 : LW / 8 + 2, RSTRIDE = RCH * 16;
+    // (a buffer also stages four waves' output rows: 16 rows of 528 bytes each)
+    constexpr int TILEB = MTILE * RSTRIDE > 4 * 16 * 528 ? MTILE * RSTRIDE : 4 * 16 * 528;
     constexpr int64_t CROW = Q8 ? ML / 32 * 2 + ML : DK * 2;   // bytes a cache row
     constexpr int CPR = Q8 ? ML / 16 : DK / 8;           // 16-byte loads a cache row
     constexpr int NCH = MTILE * CPR;                     // loads a tile
@@ -591,11 +600,11 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
         lds_u8* const ob = (w < 4 ? B0 : B1) + (w & 3) * 16 * OROW;
         typedef _Float16 h4v __attribute__((ext_vector_type(4)));
         const float sc = n_all > p.kbs ? __builtin_nanf("") : inv_l;
-        const int passes = p.ot == 0 ? 4 : 2, dpp = DT / passes;      // passes over the latents, 16-latent tiles a pass
         const int64_t rowb = p.ot == 0 ? ML * 4 : ML * 2;
+        const int passes = (int) (rowb / 512), dpp = DT / passes;     // passes of 512 bytes over a row's latents, 16-latent tiles a pass
         for (int hp = 0; hp < passes; ++hp) {
 #pragma unroll
-            for (int d2 = 0; d2 < DT / 2; ++d2) {
+            for (int d2 = 0; d2 < 16; ++d2) {
                 if (d2 < dpp) {
                     // (o indexed through a constant-trip loop: the accumulators stay in registers)
                     f4v v = o[0];
@@ -629,10 +638,10 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
         typedef _Float16 h4v __attribute__((ext_vector_type(4)));
         float* const prow = p.part + (int64_t) split * PSTRIDE;
 #pragma unroll
-        for (int hp = 0; hp < 2; ++hp) {
+        for (int hp = 0; hp < ML / 256; ++hp) {
 #pragma unroll
-            for (int d2 = 0; d2 < DT / 2; ++d2) {
-                const f4v v = o[hp * (DT / 2) + d2] * inv_l;
+            for (int d2 = 0; d2 < 16; ++d2) {
+                const f4v v = o[hp * 16 + d2] * inv_l;
                 const h4v h = {(_Float16) v[0], (_Float16) v[1], (_Float16) v[2], (_Float16) v[3]};
                 *reinterpret_cast<__attribute__((address_space(3))) h4v*>(ob + n * OROW + (d2 * 16 + g4 * 4) * 2) = h;
             }
@@ -661,8 +670,9 @@ __global__ __launch_bounds__(MW * 64, MW == 4 ? 1 : 2) void mla_decode_kernel(co
 // 256 latents each: a thread sums 4 latents (one 8-byte load a split) over every fourth split, then the four phases are
 // added in a fixed order. A thread's first 32 loads are requested before anything else, so that they travel while the
 // splits' (m, l) are fetched and turned into weights: one memory latency a row instead of three.
-template <int QT>
+template <int LW, int QT>
 __global__ __launch_bounds__(256) void mla_merge_kernel(const float* __restrict__ part, int ns, void* __restrict__ u) {
+    constexpr int ML = LW, PSTRIDE = pstride_of(LW);     // (two work-groups a row at width 512, one at 256)
     __shared__ float wsh[1024];
     __shared__ float red[8];
     __shared__ f4v ph[256];
@@ -969,25 +979,6 @@ __global__ __launch_bounds__(256) void to_half_kernel(const float* __restrict__ 
     reinterpret_cast<us8v*>(y)[i] = h;
 }
 
-// rows of Ls values into rows of Ld: the first min(Ls, Ld) copied (float32 -> half rounds), the rest zeros. A latent cache
-// of width 256 and its absorbed rows are widened to the kernel's 512 this way (a zero latent adds nothing to a score or
-// to a sum) and the results' first 256 values taken back out
-__device__ __forceinline__ void put_as(float* d, float v) { *d = v; }
-__device__ __forceinline__ void put_as(uint16_t* d, float v) { *d = f32_to_f16(v); }
-__device__ __forceinline__ void put_as(uint16_t* d, uint16_t v) { *d = v; }
-template <class S, class Dt>
-__global__ __launch_bounds__(256) void widen_rows_kernel(const S* __restrict__ src, Dt* __restrict__ dst, int64_t rows, int Ls, int Ld) {
-    const int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x, per = Ld / 4, r = i / per;
-    if (r >= rows) return;
-    const int c0 = (int) (i % per) * 4;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        const int f = c0 + k;
-        if (f < Ls) put_as(dst + r * Ld + f, src[r * Ls + f]);
-        else put_as(dst + r * Ld + f, S(0));
-    }
-}
-
 // out [n][512] half = the q8 latent rows idx[i] of src widened: half(scale x q), one rounding (the product is exact in
 // float32); a thread 8 values (kernels/llm/glm5next/glm.cpp:1301-1325)
 __global__ __launch_bounds__(256) void gather_q8_h_kernel(const uint8_t* __restrict__ src, const int32_t* __restrict__ idx, uint16_t* __restrict__ out,
@@ -1020,9 +1011,11 @@ int64_t mla_kbs(int64_t cells, int64_t groups) {
 
 int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const void* qa, const void* cache, void* u, int64_t T, int64_t H,
                int64_t pos0, float scale, float* scratch, size_t scratch_floats, const int32_t* sel = nullptr, const int32_t* sel_cnt = nullptr,
-               int64_t K = 0) {
+               int64_t K = 0, int LW = 512) {
     const std::string w(who);
     if (T <= 0) return 0;
+    if (LW != 512 && (LW != 256 || R != 0 || q8)) return ns_fail(w + ": latent rows of 512, or latent-only half rows of 256");
+    const int64_t PSTRIDE = pstride_of(LW);
     if (H <= 0 || pos0 < 0) return ns_fail(w + ": heads and a position");
     if (T > MLA_PASS_MAX) return ns_fail(w + ": more rows than a pass holds");
     if (!qa || !cache || !u || !scratch) return ns_fail(w + ": a null buffer");
@@ -1036,7 +1029,7 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     // row beyond it comes out as NaNs (the kernel marks it), not as a plausible wrong answer.
     const bool per_t = sel_cnt != nullptr;
     if (per_t && (!sel || K < 0 || K > (int64_t) 1 << 24)) return ns_fail(w + ": a selection has cell pools and their count");
-    if ((pos0 + T) * (int64_t) (q8 ? 544 : (512 + R) * 2) >= (int64_t) 1 << 32 && per_t) return ns_fail(w + ": a selection over a cache past 4 GiB");
+    if ((pos0 + T) * (int64_t) (q8 ? 544 : (LW + R) * 2) >= (int64_t) 1 << 32 && per_t) return ns_fail(w + ": a selection over a cache past 4 GiB");
     const int64_t rows = T * H;
     const int MW = mla_waves(per_t ? H : rows, pos0 + T), MROWS = MW * 16;
     const int64_t nz = per_t ? T * ((H + MROWS - 1) / MROWS) : (rows + MROWS - 1) / MROWS;
@@ -1073,19 +1066,26 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     dim3 grid((unsigned) (p.flat ? ns * nz : (ns + 7) / 8 * 8 * nz));
     if (ns_profile_mark(g, 0)) return -1;
     if (MW == 4) {
-        if (q8) mla_decode_kernel<0, true, 4><<<grid, 256, 0, g->q>>>(p);
-        else if (R == 64) mla_decode_kernel<64, false, 4><<<grid, 256, 0, g->q>>>(p);
-        else mla_decode_kernel<0, false, 4><<<grid, 256, 0, g->q>>>(p);
+        if (LW == 256) mla_decode_kernel<256, 0, false, 4><<<grid, 256, 0, g->q>>>(p);
+        else if (q8) mla_decode_kernel<512, 0, true, 4><<<grid, 256, 0, g->q>>>(p);
+        else if (R == 64) mla_decode_kernel<512, 64, false, 4><<<grid, 256, 0, g->q>>>(p);
+        else mla_decode_kernel<512, 0, false, 4><<<grid, 256, 0, g->q>>>(p);
     } else {
-        if (q8) mla_decode_kernel<0, true, 8><<<grid, 512, 0, g->q>>>(p);
-        else if (R == 64) mla_decode_kernel<64, false, 8><<<grid, 512, 0, g->q>>>(p);
-        else mla_decode_kernel<0, false, 8><<<grid, 512, 0, g->q>>>(p);
+        if (LW == 256) mla_decode_kernel<256, 0, false, 8><<<grid, 512, 0, g->q>>>(p);
+        else if (q8) mla_decode_kernel<512, 0, true, 8><<<grid, 512, 0, g->q>>>(p);
+        else if (R == 64) mla_decode_kernel<512, 64, false, 8><<<grid, 512, 0, g->q>>>(p);
+        else mla_decode_kernel<512, 0, false, 8><<<grid, 512, 0, g->q>>>(p);
     }
     NS_LAUNCHED("mla_decode");
     if (ns_profile_mark(g, 1)) return -1;
     if (ns > 1) {
-        if (ot == 0) mla_merge_kernel<0><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
-        else mla_merge_kernel<1><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
+        if (LW == 256) {
+            if (ot == 0) mla_merge_kernel<256, 0><<<dim3((unsigned) rows, 1), 256, 0, g->q>>>(scratch, (int) ns, u);
+            else mla_merge_kernel<256, 1><<<dim3((unsigned) rows, 1), 256, 0, g->q>>>(scratch, (int) ns, u);
+        } else {
+            if (ot == 0) mla_merge_kernel<512, 0><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
+            else mla_merge_kernel<512, 1><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
+        }
         NS_LAUNCHED("mla_merge");
     }
     return ns_profile_mark(g, 2);
@@ -1218,54 +1218,25 @@ int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint1
 // GLM's latent-only MLA through the library's own scratch, any number of rows: rows with cell lists of their own go 16 a
 // pass (a row group holds one row's heads, so wider passes gain nothing), dense rows as a prompt's do
 static int mla_sel_rows(ns_gpu* g, const char* who, bool q8, const float* qa, const void* c, float* u, int64_t T, int64_t H, int64_t pos0,
-                        float scale, const int32_t* sel, const int32_t* sel_cnt, int64_t K, float* scratch, size_t scratch_floats) {
+                        float scale, const int32_t* sel, const int32_t* sel_cnt, int64_t K, float* scratch, size_t scratch_floats, int LW = 512) {
     if (H <= 0 || pos0 < 0) return ns_fail(std::string(who) + ": heads and a position");
     if (!qa || !u) return ns_fail(std::string(who) + ": a null buffer");
     for (int64_t t0 = 0, n; t0 < T; t0 += n) {
         n = T <= 16 ? T : sel_cnt ? std::min<int64_t>(16, T - t0) : mla_pass_rows(pos0 + t0, T - t0);
-        if (mla_latent(g, who, 0, 0, 0, q8, qa + t0 * H * ML, c, u + t0 * H * ML, n, H, pos0 + t0, scale, scratch, scratch_floats,
-                       sel_cnt ? sel + t0 * K : nullptr, sel_cnt ? sel_cnt + t0 : nullptr, K))
+        if (mla_latent(g, who, 0, 0, 0, q8, qa + t0 * H * LW, c, u + t0 * H * LW, n, H, pos0 + t0, scale, scratch, scratch_floats,
+                       sel_cnt ? sel + t0 * K : nullptr, sel_cnt ? sel_cnt + t0 : nullptr, K, LW))
             return -1;
     }
     return 0;
 }
 
-// A latent width of 256 (the reference's other width, kernels/llm/glm5next/glm.cpp:1257) rides on the 512-wide kernel: the
-// cache's rows 0 .. pos0 + T - 1 (half, or float32 rounded to half: CT), the absorbed rows and the results pass through
-// the library's scratch, widened with zeros / narrowed again. What the scratch does not hold is refused.
-extern "C++" {
-template <class CT>
-static int mla_narrow(ns_gpu* g, const char* who, const float* qa, const CT* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
-                      const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
-    const std::string w(who);
-    if (H <= 0 || pos0 < 0) return ns_fail(w + ": heads and a position");
-    if (!qa || !c || !u) return ns_fail(w + ": a null buffer");
-    const int64_t cells = pos0 + T, rows = T * H;
-    const size_t c_f = (size_t) cells * ML / 2, q_f = (size_t) rows * ML, u_f = q_f;        // floats of scratch each takes
-    if (c_f + q_f + u_f + (size_t) (16 * H) * PSTRIDE > g->own_scratch_floats)
-        return ns_fail(w + ": a latent width of 256 is widened in the library's scratch, which does not hold " + std::to_string(cells) + " cells and " +
-                       std::to_string(rows) + " rows");
-    NS_HIP(hipSetDevice(g->dev));
-    uint16_t* cw = (uint16_t*) g->own_scratch;
-    float* qw = g->own_scratch + c_f;
-    float* uw = qw + q_f;
-    widen_rows_kernel<CT, uint16_t><<<(unsigned) ((cells * (ML / 4) + 255) / 256), 256, 0, g->q>>>(c, cw, cells, (int) L, ML);
-    widen_rows_kernel<float, float><<<(unsigned) ((rows * (ML / 4) + 255) / 256), 256, 0, g->q>>>(qa, qw, rows, (int) L, ML);
-    NS_LAUNCHED("widen_rows");
-    if (mla_sel_rows(g, who, false, qw, cw, uw, T, H, pos0, scale, sel, sel_cnt, K, uw + u_f, g->own_scratch_floats - (c_f + q_f + u_f))) return -1;
-    widen_rows_kernel<float, float><<<(unsigned) ((rows * (L / 4) + 255) / 256), 256, 0, g->q>>>(uw, u, rows, ML, (int) L);
-    NS_LAUNCHED("narrow_rows");
-    return 0;
-}
-}  // extern "C++"
-
 int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                       const int32_t* sel, const int32_t* sel_cnt, int64_t K) {
     NS_TRY
     if (T <= 0) return 0;
-    if (L == 256) return mla_narrow<uint16_t>(g, "ns_mla_attend_sel", qa, c, u, T, H, L, pos0, scale, sel, sel_cnt, K);
-    if (L != 512) return ns_fail("ns_mla_attend_sel: latent width 256 or 512");
-    return mla_sel_rows(g, "ns_mla_attend_sel", false, qa, c, u, T, H, pos0, scale, sel, sel_cnt, K, g->own_scratch, g->own_scratch_floats);
+    // (both of the reference's widths, kernels/llm/glm5next/glm.cpp:1254-1266, each an instance of the latent kernel)
+    if (L != 256 && L != 512) return ns_fail("ns_mla_attend_sel: latent width 256 or 512");
+    return mla_sel_rows(g, "ns_mla_attend_sel", false, qa, c, u, T, H, pos0, scale, sel, sel_cnt, K, g->own_scratch, g->own_scratch_floats, (int) L);
     NS_CATCH
 }
 
@@ -1283,19 +1254,18 @@ int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, in
 int ns_mla_attend(ns_gpu* g, const float* qa, const float* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale) {
     NS_TRY
     if (T <= 0) return 0;
-    if (L == 256) return mla_narrow<float>(g, "ns_mla_attend", qa, c, u, T, H, L, pos0, scale, nullptr, nullptr, 0);
-    if (L != 512) return ns_fail("ns_mla_attend: latent width 256 or 512");
+    if (L != 256 && L != 512) return ns_fail("ns_mla_attend: latent width 256 or 512");
     if (pos0 < 0 || !c) return ns_fail("ns_mla_attend: a position and a cache");
     if ((uintptr_t) c % 16) return ns_fail("ns_mla_attend: the cache 16-byte aligned");
-    const int64_t cells = pos0 + T, ch_floats = (cells * ML / 2 + 3) / 4 * 4;     // the half rows, counted in floats
+    const int64_t cells = pos0 + T, ch_floats = (cells * L / 2 + 3) / 4 * 4;      // the half rows, counted in floats
     if ((size_t) ch_floats + (size_t) (H > 0 ? 16 * H * PSTRIDE : 0) > g->own_scratch_floats)
         return ns_fail("ns_mla_attend: more cells than the library's scratch holds as half rows (use a half cache and ns_mla_attend_sel)");
     NS_HIP(hipSetDevice(g->dev));
     uint16_t* ch = (uint16_t*) g->own_scratch;
-    to_half_kernel<<<(unsigned) ((cells * ML / 8 + 255) / 256), 256, 0, g->q>>>(c, ch, cells * ML / 8);
+    to_half_kernel<<<(unsigned) ((cells * L / 8 + 255) / 256), 256, 0, g->q>>>(c, ch, cells * L / 8);
     NS_LAUNCHED("to_half");
     return mla_sel_rows(g, "ns_mla_attend", false, qa, ch, u, T, H, pos0, scale, nullptr, nullptr, 0, g->own_scratch + ch_floats,
-                        g->own_scratch_floats - (size_t) ch_floats);
+                        g->own_scratch_floats - (size_t) ch_floats, (int) L);
     NS_CATCH
 }
 

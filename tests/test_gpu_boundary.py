@@ -238,8 +238,8 @@ def test_ds2_mla_decode_with_q6k_weights(ops, T, H, pos0):
 
 def test_glm_latent_width_256(ops):
     """The reference's other latent width (kernels/llm/glm5next/glm.cpp:1257): a half cache dense and with cell pools, a
-    float32 cache dense - against the reference-order restatement at L = 256; and the refusal, with its reason, of a
-    cache the widening does not hold."""
+    float32 cache dense - against the reference-order restatement at L = 256 (an instance of the latent kernel of its own
+    width: no length is refused)."""
     g = ops.gpu
     L, scale = 256, 0.0625
     for T, H, pos0, K in ((1, 64, 2000, 0), (5, 16, 300, 0), (20, 8, 3000, 24), (3, 32, 20000, 128)):
@@ -262,10 +262,19 @@ def test_glm_latent_width_256(ops):
             ops.mla_attend_f32(DevBuf.of(g, qa), DevBuf.of(g, x), u, T, H, L, pos0, scale)
             want = orc.glm_mla_attend_f32(qa, x, T, H, L, pos0, scale).reshape(T, H * L)
             check_close(u.read(np.float32).reshape(T, H * L), want.astype(np.float64), F32, "ns_mla_attend at L = 256")
-    # 100K cells widened to 512 halfs each are 100 MB: more than the library's scratch
-    big = DevBuf(g, 100001 * 2 * L)
-    with pytest.raises(Error, match="widened in the library's scratch"):
-        ops.mla_attend(DevBuf(g, 8 * L * 4), big, DevBuf(g, 8 * L * 4), 1, 8, L, 100000, scale)
+    # a length no scratch bounds: 100,000 cells, a row with cell pools (what the engine passes past 2,560 tokens) against the
+    # float64 closed form over the row's listed cells
+    T, H, pos0, K = 2, 16, 100000, 64
+    n = pos0 + T
+    qa, x = orc.randn(97, (T, H * L), 0.3), orc.randn(98, (n, L), 0.5)
+    rows = orc.f2h(x).view(np.uint8).reshape(n, 2 * L)
+    rng = np.random.default_rng(12)
+    sel = np.stack([np.sort(rng.permutation((pos0 + 1) // 4)[:K]) for _ in range(T)]).astype(np.int32)
+    cnt = np.array([K, K // 2], np.int32)
+    u = DevBuf(g, T * H * L * 4); u.fill(0xFF)
+    ops.mla_attend(DevBuf.of(g, qa), DevBuf.of(g, rows), u, T, H, L, pos0, scale, sel=DevBuf.of(g, sel), sel_cnt=DevBuf.of(g, cnt), K=K)
+    want = orc.glm_mla_attend_sel(qa, rows, False, T, H, L, pos0, scale, sel, cnt, K)
+    check_close(u.read(np.float32).reshape(T, H * L), want.reshape(T, H * L).astype(np.float64), F32, "ns_mla_attend_sel at L = 256, 100,000 cells")
 
 
 # ricursive's engine (ns_rc_*: a ring of R rows a head, a window W, 10 query heads a key head among its ratios) and
