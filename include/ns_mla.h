@@ -57,9 +57,8 @@ int ns_ds2_kv_store(ns_gpu* g, const float* kv, const float* w, float eps, uint1
  * every row sees every earlier cell. Else row t's cells are the pools sel[t K ..][0, sel_cnt[t]) of 4 cells each (cells
  * 4 b .. 4 b + 3) followed by its incomplete pool 4 ((p + 1) / 4) .. p, p = pos0 + t; a negative sel_cnt[t] is a dense
  * row. Any number of rows: rows with lists go 16 a pass on the queue, dense
- * rows as a prompt's. L = 512, or 256 (cache [n][256], qa and u [T][H][256]): the narrow cache's cells 0 .. pos0 + T - 1, the
- * rows and the results are widened with zeros into memory the library keeps per ns_gpu for the call (-1 when they do not
- * fit: ~60,000 cells). Replaces: kernels/llm/glm5next/glm.h:65-66 (glm.cpp:1062-1067,1095-1102,1252-1264) */
+ * rows as a prompt's. L = 512, or 256 (cache [n][256], qa and u [T][H][256]: the same kernel built for rows half as wide).
+ * Replaces: kernels/llm/glm5next/glm.h:65-66 (glm.cpp:1062-1067,1095-1102,1252-1264) */
 int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale,
                       const int32_t* sel, const int32_t* sel_cnt, int64_t K);
 /* the same over q8 latent rows. Replaces: kernels/llm/glm5next/glm.h:79-80 (glm.cpp:1267-1276; the reference: at most 8 rows) */
@@ -97,6 +96,17 @@ int ns_gather_q8_h(ns_gpu* g, const void* src, const int32_t* idx, uint16_t* out
 /* rows x [n][512] float32 -> q8 latent rows y [n][544]: a block's scale amax / 127 rounded to half BEFORE the values are
  * divided by it, round half away from zero, clamp to +-127. Replaces: kernels/llm/glm5next/glm.h:77 (glm.cpp:1282-1299) */
 int ns_to_q8row(ns_gpu* g, const float* x, void* y, int64_t n, int64_t L);
+/* The half products of that chain (the reference: oneMKL). y [T, N] (+)= x [T, K] . w [N, K]^T, x and w half, y and the
+ * sums float32; rows of x ldx, of y ldy elements apart, accumulate != 0 adds to y. ns_gemm_batch_h: `batch` such
+ * products, operand b at x + b sx, w + b sw, y + b sy (elements); op(w) = w^T (w [N, K], rows ldw apart) with trans_w,
+ * else w ([K, N]). Any sizes and strides; 16-byte aligned operands with strides in multiples of 8 load fastest.
+ * ns_to_f16: y[i] = half(x[i]), round to nearest even. Replaces: kernels/llm/glm5next/glm.h:81-82 (glm.cpp:217-225),
+ * glm.h:63-64 (glm.cpp:265-276), glm.h:73 (glm.cpp:208-214), bound at llm/glm5next/src/ffi.rs */
+int ns_gemm_f16(ns_gpu* g, int64_t T, int64_t N, int64_t K, const uint16_t* x, int64_t ldx, const uint16_t* w, float* y, int64_t ldy,
+                int accumulate);
+int ns_gemm_batch_h(ns_gpu* g, int64_t batch, int trans_w, int64_t T, int64_t N, int64_t K, const uint16_t* x, int64_t ldx, int64_t sx,
+                    const uint16_t* w, int64_t ldw, int64_t sw, float* y, int64_t ldy, int64_t sy, int accumulate);
+int ns_to_f16(ns_gpu* g, const float* x, uint16_t* y, int64_t n);
 
 #ifdef __cplusplus
 }

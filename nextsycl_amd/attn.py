@@ -115,6 +115,9 @@ MLA_H = {
     "ns_topk": (i32, [P, P, P, i64, i64, i64, i64]),
     "ns_mla_cells": (i32, [P, P, P, i64, i64, i64, P, P, i64]),
     "ns_softmax_masked": (i32, [P, P, i64, i64, i64, P, f32]),
+    "ns_gemm_f16": (i32, [P, i64, i64, i64, P, i64, P, P, i64, i32]),
+    "ns_gemm_batch_h": (i32, [P, i64, i32, i64, i64, i64, P, i64, i64, P, i64, i64, P, i64, i64, i32]),
+    "ns_to_f16": (i32, [P, P, P, i64]),
 }
 
 
@@ -487,6 +490,29 @@ class Ops:
         _need(S, R * H * NC * 4, "softmax_masked scores")
         _need(n, R * 4, "softmax_masked counts")
         self.ok(self.k.softmax_masked(self.raw(), S.ptr, R, H, NC, n.ptr, scale), "softmax_masked")
+
+    def to_f16(self, x, y, n):
+        """ns_to_f16: y [n] half = x [n] float32."""
+        _need(x, n * 4, "to_f16 x")
+        _need(y, n * 2, "to_f16 y")
+        self.ok(self.k.to_f16(self.raw(), x.ptr, y.ptr, n), "to_f16")
+
+    def gemm_f16(self, T, N, K, x, ldx, w, y, ldy, accumulate=False):
+        """ns_gemm_f16: y [T, N] float32 (+)= x [T, K] half . w [N, K]^T half (kernels/llm/glm5next/glm.cpp:217-225)."""
+        self.gemm_batch_h(1, True, T, N, K, x, ldx, 0, w, K, 0, y, ldy, 0, accumulate, _one=True)
+
+    def gemm_batch_h(self, batch, trans_w, T, N, K, x, ldx, sx, w, ldw, sw, y, ldy, sy, accumulate=False, _one=False):
+        """ns_gemm_batch_h: `batch` products y_b [T, N] float32 (+)= x_b [T, K] . op(w_b), half operands; op(w) = w^T (w
+        [N, K]) with trans_w, else w ([K, N]); strides in elements (kernels/llm/glm5next/glm.cpp:265-276)."""
+        if batch > 0 and T > 0 and N > 0:
+            _need(x, ((batch - 1) * sx + (T - 1) * ldx + K) * 2, "gemm x")
+            _need(w, ((batch - 1) * sw + ((N if trans_w else K) - 1) * ldw + (K if trans_w else N)) * 2, "gemm w")
+            _need(y, ((batch - 1) * sy + (T - 1) * ldy + N) * 4, "gemm y")
+        if _one:
+            self.ok(self.k.gemm_f16(self.raw(), T, N, K, x.ptr, ldx, w.ptr, y.ptr, ldy, int(accumulate)), "gemm_f16")
+        else:
+            self.ok(self.k.gemm_batch_h(self.raw(), batch, int(trans_w), T, N, K, x.ptr, ldx, sx, w.ptr, ldw, sw, y.ptr, ldy, sy,
+                                        int(accumulate)), "gemm_batch_h")
 
     def to_q8row(self, x, y, n, L):
         _need(x, n * L * 4, "to_q8row x")

@@ -30,6 +30,7 @@ SOURCES = {
     "attn_probs.hip": [],
     "attn_api.cpp": [],
     "mla.hip": [],
+    "gemm_h.hip": [],
 }
 
 

@@ -1,0 +1,158 @@
+"""The half products an engine's MLA prompt chain calls - ns_to_f16, ns_gemm_f16, ns_gemm_batch_h (the reference: oneMKL,
+kernels/llm/glm5next/glm.cpp:208-276) - through the C ABI.
+
+What pins them: numpy's float64 product of the same half operands (a float32 sum of exact half x half products may differ
+from it by the sum's own roundings only: at most K 2^-23 sum |x| |w| here), numpy's own float32 -> float16 rounding bit for
+bit, and the chain itself - scores, masked softmax, weighted sum - against ns_mla_attend_sel on the same rows."""
+import numpy as np
+import pytest
+
+from nextsycl_amd import DevBuf, Error
+from oracle import orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _half(seed, shape, s=1.0):
+    return (orc.randn(seed, shape) * s).astype(np.float16)
+
+
+def _bound(x, w_t, K):
+    """the float32 sum's worst case against the exact product: every partial sum rounded once"""
+    return (K + 2) * 2.0 ** -23 * (np.abs(x.astype(np.float64)) @ np.abs(w_t.astype(np.float64))) + 1e-30
+
+
+def test_to_f16_is_numpys_rounding(ops):
+    g = ops.gpu
+    x = orc.randn(3, (100003,)).astype(np.float32) * 37.0
+    # ties, the subnormal range, the overflow edge, signed zeros and infinities
+    x[:12] = [0.0, -0.0, 65504.0, 65519.9, 65520.0, -70000.0, 6e-8, 2.98e-8, 2.9802322e-8, 1.0009765625, 1.00146484375, np.inf]
+    x[12:2012] = (np.arange(2000, dtype=np.float32) + 0.5) * 2.0 ** -25           # halfway between subnormals
+    for n, off in ((x.size, 0), (x.size - 1, 1), (3, 2), (1, 0), (0, 0)):
+        xb = DevBuf.of(g, x)
+        yb = DevBuf(g, max(2 * x.size, 2))
+        yb.fill(0xEE)
+        ops.to_f16(xb.view(4 * off, 4 * n) if n else xb, yb.view(2 * off, 2 * n) if n else yb, n)
+        got = yb.read(np.uint16)
+        with np.errstate(over="ignore"):
+            want = x[off:off + n].astype(np.float16).view(np.uint16)
+        assert np.array_equal(got[off:off + n], want), (n, off)
+        assert (got[:off] == 0xEEEE).all() and (got[off + n:] == 0xEEEE).all()
+
+
+# T, N, K, ldx extra, ldy extra: whole blocks, ragged edges in every dimension, a K below one step, strides that break the
+# 16-byte loads, a single row and column
+SHAPES = [(64, 64, 64, 0, 0), (128, 192, 512, 0, 0), (1, 1, 1, 0, 0), (7, 5, 3, 0, 0), (65, 63, 33, 0, 0), (100, 130, 260, 4, 3),
+          (16, 512, 576, 8, 0), (333, 17, 1000, 1, 7), (2, 700, 8, 0, 0), (130, 64, 40, 24, 64)]
+
+
+@pytest.mark.parametrize("T,N,K,px,py", SHAPES)
+def test_gemm_f16_against_the_exact_product(ops, T, N, K, px, py):
+    g = ops.gpu
+    ldx, ldy = K + px, N + py
+    x, w = _half(T + N, (T, ldx)), _half(K + 7, (N, K), 0.5)
+    y0 = orc.randn(9, (T, ldy)).astype(np.float32)
+    want = x[:, :K].astype(np.float64) @ w.astype(np.float64).T
+    bound = _bound(x[:, :K], w.T, K)
+    xb, wb = DevBuf.of(g, x), DevBuf.of(g, w)
+    for acc in (False, True):
+        yb = DevBuf.of(g, y0)
+        ops.gemm_f16(T, N, K, xb, ldx, wb, yb, ldy, acc)
+        got = yb.read(np.float32).reshape(T, ldy)
+        assert np.array_equal(got[:, N:], y0[:, N:])                                # nothing beside the N columns is written
+        ref = want + (y0[:, :N] if acc else 0.0)
+        err = np.abs(got[:, :N] - ref)
+        assert (err <= bound + (2.0 ** -23 * np.abs(ref) if acc else 0.0)).all(), (T, N, K, acc, err.max())
+
+
+# batch, trans_w, T, N, K, pads of ldx / ldw / ldy, gaps of sx / sw / sy
+BATCHES = [(4, 1, 16, 300, 512, 0, 0, 0, 0, 0, 0), (3, 0, 16, 512, 300, 0, 0, 0, 0, 0, 0), (5, 0, 33, 70, 45, 3, 5, 1, 7, 9, 11),
+           (5, 1, 33, 70, 45, 3, 5, 1, 7, 9, 11), (64, 0, 8, 512, 64, 0, 0, 0, 0, 0, 0), (2, 0, 1, 1, 1, 0, 0, 0, 0, 0, 0),
+           (1, 0, 200, 129, 31, 0, 8, 0, 0, 0, 0), (2, 0, 64, 64, 96, 8, 16, 0, 8, 16, 0)]
+
+
+@pytest.mark.parametrize("B,tw,T,N,K,px,pw,py,gx,gw,gy", BATCHES)
+def test_gemm_batch_h_both_forms(ops, B, tw, T, N, K, px, pw, py, gx, gw, gy):
+    g = ops.gpu
+    ldx, ldy = K + px, N + py
+    wr, wc = (N, K) if tw else (K, N)
+    ldw = wc + pw
+    sx, sw, sy = T * ldx + gx, wr * ldw + gw, T * ldy + gy
+    x, w = _half(B + T, (B * sx,)), _half(B + N, (B * sw,), 0.5)
+    y0 = orc.randn(11, (B * sy,)).astype(np.float32)
+    xb, wb = DevBuf.of(g, x), DevBuf.of(g, w)
+    for acc in (False, True):
+        yb = DevBuf.of(g, y0)
+        ops.gemm_batch_h(B, tw, T, N, K, xb, ldx, sx, wb, ldw, sw, yb, ldy, sy, acc)
+        got = yb.read(np.float32)
+        written = np.zeros(B * sy, bool)
+        for b in range(B):
+            xm = x[b * sx:b * sx + T * ldx].reshape(T, ldx)[:, :K]
+            wm = w[b * sw:b * sw + wr * ldw].reshape(wr, ldw)[:, :wc]
+            wt = wm.T if tw else wm
+            ym = got[b * sy:b * sy + T * ldy].reshape(T, ldy)[:, :N]
+            y0m = y0[b * sy:b * sy + T * ldy].reshape(T, ldy)[:, :N]
+            ref = xm.astype(np.float64) @ wt.astype(np.float64) + (y0m if acc else 0.0)
+            err = np.abs(ym - ref)
+            assert (err <= _bound(xm, wt, K) + (2.0 ** -23 * np.abs(ref) if acc else 0.0)).all(), (b, acc, err.max())
+            written[b * sy:b * sy + T * ldy].reshape(T, ldy)[:, :N] = True
+        assert np.array_equal(got[~written], y0[~written])
+
+
+def test_gemm_refusals_and_empty_products(ops):
+    g = ops.gpu
+    x, w = DevBuf.of(g, _half(1, (64, 64))), DevBuf.of(g, _half(2, (64, 64)))
+    y0 = orc.randn(3, (64, 64)).astype(np.float32)
+    y = DevBuf.of(g, y0)
+    for T, N in ((0, 64), (64, 0)):
+        ops.gemm_f16(T, N, 64, x, 64, w, y, 64)
+        assert np.array_equal(y.read(np.float32).reshape(64, 64), y0)
+    ops.gemm_batch_h(0, 1, 64, 64, 64, x, 64, 0, w, 64, 0, y, 64, 0)
+    assert np.array_equal(y.read(np.float32).reshape(64, 64), y0)
+    # K = 0: an empty sum - zeros, or y as it was
+    ops.gemm_batch_h(1, 0, 64, 64, 0, x, 64, 0, w, 64, 0, y, 64, 0, True)
+    assert np.array_equal(y.read(np.float32).reshape(64, 64), y0)
+    ops.gemm_batch_h(1, 0, 64, 64, 0, x, 64, 0, w, 64, 0, y, 64, 0, False)
+    assert not y.read(np.float32).any()
+    k = ops.k
+    with pytest.raises(Error, match="apart"):
+        ops.ok(k.gemm_f16(ops.raw(), 64, 64, 64, x.ptr, 32, w.ptr, y.ptr, 64, 0), "gemm_f16")
+    with pytest.raises(Error, match="apart"):
+        ops.ok(k.gemm_batch_h(ops.raw(), 1, 0, 64, 64, 32, x.ptr, 64, 0, w.ptr, 32, 0, y.ptr, 64, 0, 0), "gemm_batch_h")
+    with pytest.raises(Error, match="null"):
+        ops.ok(k.gemm_f16(ops.raw(), 64, 64, 64, None, 64, w.ptr, y.ptr, 64, 0), "gemm_f16")
+
+
+@pytest.mark.parametrize("T,H,pos0", [(16, 8, 1000), (40, 4, 0), (5, 64, 2300)])
+def test_the_prompt_chain_agrees_with_the_fused_pass(ops, T, H, pos0):
+    """An engine's prompt branch as the reference runs it (llm/glm5next: cells, half scores, masked softmax, half weighted
+    sum) on this library's pieces, against ns_mla_attend_sel over the same rows."""
+    g = ops.gpu
+    L, n_cells, scale = 512, pos0 + T, 0.0442
+    NC = (n_cells + 63) // 64 * 64
+    qa = orc.randn(T * H + pos0, (T * H, L)).astype(np.float32)
+    cache = np.zeros((NC, L), np.float16)
+    cache[:n_cells] = _half(77 + pos0, (n_cells, L), 0.7)
+    qb, cb = DevBuf.of(g, qa), DevBuf.of(g, cache)
+    # the fused pass
+    uf = DevBuf(g, T * H * L * 4)
+    ops.mla_attend(qb, cb, uf, T, H, L, pos0, scale)
+    fused = uf.read(np.float32).reshape(T * H, L)
+    # the chain
+    idx, cnt = DevBuf(g, T * NC * 4), DevBuf(g, T * 4)
+    ops.mla_cells(T, 0, pos0, idx, cnt, NC)
+    assert np.array_equal(cnt.read(np.int32), pos0 + 1 + np.arange(T))
+    qh = DevBuf(g, T * H * L * 2)
+    ops.to_f16(qb, qh, T * H * L)
+    S = DevBuf(g, T * H * NC * 4)
+    ops.gemm_batch_h(1, 1, T * H, NC, L, qh, L, 0, cb, L, 0, S, NC, 0)
+    ops.softmax_masked(S, T, H, NC, cnt, scale)
+    ph = DevBuf(g, T * H * NC * 2)
+    ops.to_f16(S, ph, T * H * NC)
+    uc = DevBuf(g, T * H * L * 4)
+    uc.fill(0xFF)
+    ops.gemm_batch_h(1, 0, T * H, L, NC, ph, NC, 0, cb, L, 0, uc, L, 0)
+    chain = uc.read(np.float32).reshape(T * H, L)
+    # both round the softmax weights to half once and sum in float32
+    assert np.abs(chain - fused).max() <= 2e-3
+    assert np.linalg.norm(chain - fused) <= 1e-3 * np.linalg.norm(fused)

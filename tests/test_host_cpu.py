@@ -97,6 +97,13 @@ def test_null_buffers_are_refused_before_any_launch(handle):
     refused("ns_mla_cells", [P, P, P, i64, i64, i64, P, P, i64], (None, None, None, 2, 0, 5, b, None, 64), "null")
     refused("ns_mla_cells", [P, P, P, i64, i64, i64, P, P, i64], (None, None, b, 2, 4, 5, b, b, 64), "no lists")
     refused("ns_softmax_masked", [P, P, i64, i64, i64, P, f32], (None, b, 2, 4, 64, None, 1.0), "null")
+    gm = [P, i64, i64, i64, P, i64, P, P, i64, C.c_int]
+    refused("ns_gemm_f16", gm, (None, 4, 4, 64, b, 64, None, b, 4, 0), "null")
+    refused("ns_gemm_f16", gm, (None, 4, 4, 64, b, 32, b, b, 4, 0), "apart")
+    gb = [P, i64, C.c_int, i64, i64, i64, P, i64, i64, P, i64, i64, P, i64, i64, C.c_int]
+    refused("ns_gemm_batch_h", gb, (None, 2, 0, 4, 8, 64, b, 64, 0, b, 4, 0, b, 8, 0, 0), "apart")
+    refused("ns_gemm_batch_h", gb, (None, 2, 1, 4, 8, 64, b, 64, 0, b, 64, 0, None, 8, 0, 0), "null")
+    refused("ns_to_f16", [P, P, P, i64], (None, b, None, 5), "null")
     refused("ns_attn_tune", [C.c_int, i64], (9, 1), "knob")
     refused("ns_attn_tune", [C.c_int, i64], (0, -1), "knob")
     handle.ns_attn_tune.restype = C.c_int
