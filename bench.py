@@ -185,6 +185,28 @@ def timed(w, steps, warmup):
     return ms, 0.5 * (dev[(GROUPS - 1) // 2] + dev[GROUPS // 2])
 
 
+def kernel_events_us(w, n=30):
+    """(dominant kernel, merge kernel) device time in us, each between two HIP events of its own on the compute stream
+    (ns_attn_profile): the median of `n` steps. An event pair around one launch also spans the launch's start-up on the
+    queue, so this reads a little longer than the kernel trace's duration of the same kernel. None for the workloads
+    whose entry point sets no marks."""
+    if w.kind == "pre" or (w.kind == "mla" and w.T > 256):         # (no marks; a longer prompt's passes would each overwrite them)
+        return None
+    ops = w.ops
+    ops.profile(1)
+    try:
+        got = []
+        for _ in range(n):
+            w.step()
+            got.append(ops.profile_last())
+    except Exception:
+        return None
+    finally:
+        ops.profile(0)
+    med = lambda v: sorted(v)[len(v) // 2]
+    return round(med([a for a, _ in got]) / 1e3, 2), round(med([b for _, b in got]) / 1e3, 2)
+
+
 def graph_step_ms(w, n=50):
     """ms a step when `n` steps are captured into a HIP graph on the library's stream and replayed - how a serving loop
     queues a token's launches (no host call a kernel, the runtime hands the device the whole chain). Only for the
@@ -245,8 +267,9 @@ KERNEL = {"pre": "pre_attn_kernel", "mla": "mla_decode_kernel", "prefill": "attn
 def roofline(w, step_ns):
     """The step against the roofline that bounds its dominant kernel. `achieved` / `frac`: algorithmic flops (or bytes) of
     the step over the step's device time, every launch of the step included (a decode step's merge kernel, a bfloat16
-    cache's widening in front of the prompt kernel). `kernel_us` / `frac_kernel`: the dominant kernel alone, from the
-    committed kernel trace of this script."""
+    cache's widening in front of the prompt kernel). `kernel_us` / `frac_kernel`: the dominant kernel alone between two
+    HIP events of its own, measured in this run (`merge_us`: the merge kernel likewise); `kernel_us_trace`: the same
+    kernel's average duration in the committed kernel trace of this script."""
     kernel = KERNEL[w.kind]
     hbm = w.kind in ("pre", "decode")
     ach = w.bytes / step_ns if hbm else w.flops / step_ns / 1e3
@@ -255,10 +278,15 @@ def roofline(w, step_ns):
          "traffic": from_profile(kernel, w.name, "traffic_bytes_per_launch"), "kernel": kernel, "step_us": round(step_ns / 1e3, 2)}
     if w.kind == "mla":
         r["hbm_GB/s"] = round(w.bytes / step_ns, 1)
+    kev = getattr(w, "kev", None)
+    if kev:
+        r["kernel_us"] = kev[0]
+        r["frac_kernel"] = round((w.bytes / kev[0] / 1e3 if hbm else w.flops / kev[0] / 1e6) / peak, 4)
+        if kev[1]:
+            r["merge_us"] = kev[1]
     kus = from_profile(kernel, w.name, "kernel_avg_us")
     if kus:
-        r["kernel_us"] = kus
-        r["frac_kernel"] = round((w.bytes / kus / 1e3 if hbm else w.flops / kus / 1e6) / peak, 4)
+        r["kernel_us_trace"] = kus
     return r
 
 
@@ -359,6 +387,7 @@ def main():
         nbuf = min(nbuf, 40)
         w = Workload(ops, name, nbuf)
         ms, step_ns = timed(w, steps, warmup)
+        w.kev = kernel_events_us(w)
         w.graph_ms = graph_step_ms(w)
         return w, ms, step_ns
 

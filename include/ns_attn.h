@@ -197,7 +197,7 @@ int ns_q35_attn_probs(ns_gpu* g, int kt, const float* q, const void* kc, int64_t
 /* GQA over a position-major half cache [position][G][128], q [T][H][128], explicit scale. sel NULL: dense; else
  * sel [T][G][K] names K blocks of 128 keys a (row, key head) (-1: none), cut at the row's own position (a row is a launch).
  * Replaces: kernels/llm/minimaxm3/mm3.h:33-37 (mm3.cpp:118-190). Needs scratch: this library keeps
- * ns_attn_decode_scratch(T, H, G, 128, pos0, 0) floats per ns_gpu for it (allocated at ns_gpu_open, 64 MiB) */
+ * ns_attn_decode_scratch(T, H, G, 128, pos0, 0) floats per ns_gpu for it (allocated at ns_gpu_open, 256 MiB) */
 int ns_llm_minimaxm3_attend(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
                             int64_t H, int64_t G, int64_t pos0, float scale);
 

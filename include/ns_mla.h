@@ -32,7 +32,7 @@ int ns_mla_decode_latent(ns_gpu* g, int qt, const void* qa, const uint16_t* cach
 
 /* MLA at decode widths in one call: q [T][H][128 nope + 64 rope] (rope part rotated), k_b [H][512][128] and v_b
  * [H][128][512] half, cache [n][576] half -> out [T][H][128] = v_b u. Runs absorb, the latent decode and the value
- * up-projection; its scratch is the library's own (kept per ns_gpu, 64 MiB). Replaces:
+ * up-projection; its scratch is the library's own (kept per ns_gpu, 256 MiB). Replaces:
  * kernels/llm/deepseek2/ds2.h:32-37 (ds2.cpp:139-258, 262-270) */
 int ns_ds2_mla_decode(ns_gpu* g, const float* q, const uint16_t* kb, const uint16_t* vb, const uint16_t* cache, float* out, int64_t T, int64_t H,
                       int64_t pos0, float scale);
@@ -66,7 +66,7 @@ int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, in
                          const int32_t* sel, const int32_t* sel_cnt, int64_t K);
 /* The dense form over a float32 latent cache c [n][L], L = 512 or 256 (every row sees every earlier cell): the cells
  * 0 .. pos0 + T - 1 are rounded to half into memory the library keeps per ns_gpu and read from there (-1 when they do not
- * fit beside the partials: ~48K cells). Replaces: kernels/llm/glm5next/glm.h:47 (glm.cpp:782-812) */
+ * fit beside the partials: ~200,000 cells of 512). Replaces: kernels/llm/glm5next/glm.h:47 (glm.cpp:782-812) */
 int ns_mla_attend(ns_gpu* g, const float* qa, const float* c, float* u, int64_t T, int64_t H, int64_t L, int64_t pos0, float scale);
 /* GLM's DSA indexer, which fills the lists ns_mla_attend_sel reads (pools of 4 consecutive tokens). Replaces:
  * kernels/llm/glm5next/glm.h:48-55 (glm.cpp:876-1019), bound at llm/glm5next/src/ffi.rs.
