@@ -156,3 +156,69 @@ def test_the_prompt_chain_agrees_with_the_fused_pass(ops, T, H, pos0):
     # both round the softmax weights to half once and sum in float32
     assert np.abs(chain - fused).max() <= 2e-3
     assert np.linalg.norm(chain - fused) <= 1e-3 * np.linalg.norm(fused)
+
+
+@pytest.mark.parametrize("T,H,pos0", [(3, 16, 700), (24, 16, 1000), (40, 128, 90)])
+def test_deepseek_prompt_branch_call_for_call(ops, T, H, pos0):
+    """The DeepSeek engine's prompt / long-context branch as it calls the library (llm/deepseek2/src/engine.rs:1165-1253):
+    queries to half, absorbed by k_b (a batch a row at decode widths, a product a head beyond), scores against the cache,
+    masked softmax, the weights to half, the weighted sum over the cache's latent columns (rows 576 apart, 512 read), u to
+    half, v_b - against the float64 chain, and against ns_ds2_mla_decode over the same inputs."""
+    g = ops.gpu
+    nope, rope, lat, vl = 128, 64, 512, 128
+    kl, cr = nope + rope, lat + rope
+    n = pos0 + T
+    nc = (n + 63) // 64 * 64
+    scale = 1.0 / np.sqrt(192.0)
+    cache = np.zeros((nc, cr), np.uint16)
+    cache[:n] = orc.f2h(orc.randn(31 + T, (n, cr), 0.5))
+    q = orc.randn(32 + T, (T, H, kl))
+    kb = orc.f2h(orc.randn(33, (H, lat, nope), 0.09))
+    vb = orc.f2h(orc.randn(34, (H, vl, lat), 0.05))
+    qd, kbd, vbd, cd = DevBuf.of(g, q), DevBuf.of(g, kb), DevBuf.of(g, vb), DevBuf.of(g, cache)
+    # the rotated part sits in qf already (the engine's rope writes it there)
+    qf_host = np.zeros((T, H, cr), np.float32)
+    qf_host[:, :, lat:] = q[:, :, nope:]
+    qf = DevBuf.of(g, qf_host)
+    q16 = DevBuf(g, T * H * kl * 2)
+    ops.to_f16(qd, q16, T * H * kl)
+    sub = lambda b, at, esz: b.view(at * esz, b.len - at * esz)
+    if T <= 8:
+        for r in range(T):
+            ops.gemm_batch_h(H, True, 1, lat, nope, sub(q16, r * H * kl, 2), kl, kl, kbd, nope, lat * nope, sub(qf, r * H * cr, 4), cr, cr)
+    else:
+        for hh in range(H):
+            ops.gemm_f16(T, lat, nope, sub(q16, hh * kl, 2), H * kl, sub(kbd, hh * lat * nope, 2), sub(qf, hh * cr, 4), H * cr)
+    qh = DevBuf(g, T * H * cr * 2)
+    ops.to_f16(qf, qh, T * H * cr)
+    sc = DevBuf(g, T * H * nc * 4)
+    ops.gemm_f16(T * H, nc, cr, qh, cr, cd, sc, nc)
+    cnt = DevBuf.of(g, (pos0 + 1 + np.arange(T)).astype(np.int32))
+    ops.softmax_masked(sc, T, H, nc, cnt, scale)
+    ph = DevBuf(g, T * H * nc * 2)
+    ops.to_f16(sc, ph, T * H * nc)
+    u = DevBuf(g, T * H * lat * 4)
+    u.fill(0xFF)
+    ops.gemm_batch_h(1, False, T * H, lat, nc, ph, nc, T * H * nc, cd, cr, nc * cr, u, lat, T * H * lat)
+    uh = DevBuf(g, T * H * lat * 2)
+    ops.to_f16(u, uh, T * H * lat)
+    oh = DevBuf(g, T * H * vl * 4)
+    oh.fill(0xFF)
+    if T <= 8:
+        for r in range(T):
+            ops.gemm_batch_h(H, True, 1, vl, lat, sub(uh, r * H * lat, 2), lat, lat, vbd, lat, vl * lat, sub(oh, r * H * vl, 4), vl, vl)
+    else:
+        for hh in range(H):
+            ops.gemm_f16(T, vl, lat, sub(uh, hh * lat, 2), H * lat, sub(vbd, hh * vl * lat, 2), sub(oh, hh * vl, 4), H * vl)
+    chain = oh.read(np.float32).reshape(T, H * vl)
+    # the float64 chain over the same stored values
+    qa64 = np.concatenate([np.einsum("hrc,thc->thr", orc.h2f(kb).astype(np.float64), orc.h2f(orc.f2h(q[:, :, :nope])).astype(np.float64)), q[:, :, nope:]], axis=2)
+    u64 = orc.mla_f64(qa64.astype(np.float32), cache[:n], T, H, pos0, scale)
+    want = np.einsum("hvl,thl->thv", orc.h2f(vb).astype(np.float64), u64).reshape(T, H * vl)
+    assert np.abs(chain - want).max() <= 2e-3 and np.linalg.norm(chain - want) <= 1e-3 * np.linalg.norm(want)
+    # and the decode-width entry point over the same inputs (any row count: passes of 16 rows)
+    fused = DevBuf(g, T * H * vl * 4)
+    fused.fill(0xFF)
+    ops.mla_decode(qd, kbd, vbd, DevBuf.of(g, cache[:n]), fused, T, H, pos0, scale)
+    f = fused.read(np.float32).reshape(T, H * vl)
+    assert np.abs(chain - f).max() <= 2e-3 and np.linalg.norm(chain - f) <= 1.5e-3 * np.linalg.norm(f)

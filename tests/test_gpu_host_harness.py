@@ -22,7 +22,7 @@ def harness(*args, timeout=300):
 def test_cpp_host_binds_every_entry_point():
     r = harness("--symbols")
     assert r.returncode == 0, r.stdout + r.stderr
-    assert "87 entry points bound" in r.stdout, r.stdout
+    assert "90 entry points bound" in r.stdout, r.stdout
 
 
 def test_cpp_host_reports_a_missing_library():
