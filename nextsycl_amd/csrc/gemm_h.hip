@@ -10,6 +10,12 @@
 // 16-byte load, no LDS. Where op(w) = w, w [K, N], a step's 32 x 64 block of w goes through LDS and comes back transposed
 // (ds_read_b64_tr_b16). Rows and columns past the edge are clamped on the way in and not written; a K that is no multiple of
 // 8, or operands that are not 16-byte aligned, take the loads element by element.
+//
+// Products large enough to fill the chip (a prompt chunk's scores and weighted sums: tens of thousands of rows) take the
+// tiled form instead: 256 x 128 of y a work-group of 8 waves (a wave 64 x 64: 4 x 4 tiles, two waves a SIMD), K in stages
+// of 64 that travel global -> LDS directly (global_load_lds_dwordx4), two stages ahead into three buffers, one barrier a
+// stage; the 16-byte chunks of a row are XOR-swizzled on the global side so that the operand reads (ds_read_b128 of 16
+// rows' same chunk; the transposing read where op(w) = w) meet no bank conflict. 87 flop a byte staged.
 #include "ns_internal.hpp"
 #include "ns_mla.h"
 #include "attn_common.hpp"
@@ -128,6 +134,129 @@ __global__ __launch_bounds__(256) void gemm_h_kernel(const GemmParams p) {
         }
 }
 
+// ---- the tiled form
+constexpr int TM = 256, TN = 128, TK = 64, TWAVES = 8;
+constexpr int TA_BYTES = TM * TK * 2, TB_BYTES = TN * TK * 2, TSTAGE = TA_BYTES + TB_BYTES;      // 32 KiB + 16 KiB
+constexpr int TDMA_A = TA_BYTES / 1024 / TWAVES, TDMA_B = TB_BYTES / 1024 / TWAVES;             // transfers a wave and stage: 4 + 2
+
+template <bool TRANS_W>
+__global__ __launch_bounds__(TWAVES * 64, 1) void gemm_h_tiled_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[3 * TSTAGE];
+    typedef __attribute__((address_space(3))) uint8_t lds_u8;
+    lds_u8* const L = (lds_u8*) lds;
+    const int tid = threadIdx.x, lane = tid & 63, n = lane & 15, g4 = lane >> 4;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6), wm = w >> 1, wn = w & 1;
+    const int64_t b = blockIdx.z, r0 = (int64_t) blockIdx.y * TM, c0 = (int64_t) blockIdx.x * TN;
+    const uint8_t* const xb = reinterpret_cast<const uint8_t*>(p.x + b * p.sx);
+    const uint8_t* const wb = reinterpret_cast<const uint8_t*>(p.w + b * p.sw);
+    float* const y = p.y + b * p.sy;
+
+    // ---- a stage's transfers. x rows (and w rows where op(w) = w^T) are 128 bytes of the stage = 8 chunks: unit 8 r + pos of the
+    // buffer holds chunk pos ^ ((r / 2) % 8) of row r; rows past the edge are clamped to the last (never written).
+    // op(w) = w: a stage holds 64 k-rows of 128 columns = 16 chunks: unit 16 k + pos holds chunk pos ^ 2 (k % 8); chunks past the
+    // last column are clamped to the last whole one.
+    uint32_t offa[TDMA_A], offb[TDMA_B];
+#pragma unroll
+    for (int j = 0; j < TDMA_A; ++j) {
+        const int u = (w * TDMA_A + j) * 64 + lane, r = u >> 3, kc = (u & 7) ^ ((r >> 1) & 7);
+        offa[j] = (uint32_t) ((std::min<int64_t>(r0 + r, p.T - 1) - r0) * p.ldx * 2 + kc * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < TDMA_B; ++j) {
+        const int u = (w * TDMA_B + j) * 64 + lane;
+        if constexpr (TRANS_W) {
+            const int r = u >> 3, kc = (u & 7) ^ ((r >> 1) & 7);
+            offb[j] = (uint32_t) ((std::min<int64_t>(c0 + r, p.N - 1) - c0) * p.ldw * 2 + kc * 16);
+        } else {
+            const int k = u >> 4, c = (u & 15) ^ (2 * (k & 7));
+            offb[j] = (uint32_t) ((int64_t) k * p.ldw * 2 + (std::min<int64_t>(c0 + 8 * c, p.N - 8) - c0) * 2);
+        }
+    }
+    auto dma16 = [&](const uint8_t* base_, uint32_t off, lds_u8* dst) __attribute__((always_inline)) {
+        const uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t) (uintptr_t) dst);
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"                   // (m0 is reserved: nothing of the compiler's lives in it across this)
+        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m), "v"(off), "s"(base_) : "memory", "m0");
+#pragma clang diagnostic pop
+    };
+    auto dma = [&](int stage, int64_t kt) __attribute__((always_inline)) {
+        lds_u8* const sa = L + stage * TSTAGE;
+        lds_u8* const sb = sa + TA_BYTES;
+        // (lane offsets are relative to the block's first row / column: they stay within 32 bits whatever the matrix)
+        const uint8_t* const xa = xb + (r0 * p.ldx + kt * TK) * 2;
+        const uint8_t* const wa = TRANS_W ? wb + (c0 * p.ldw + kt * TK) * 2 : wb + (kt * TK * p.ldw + c0) * 2;
+#pragma unroll
+        for (int j = 0; j < TDMA_A; ++j) dma16(xa, offa[j], sa + (w * TDMA_A + j) * 1024);
+#pragma unroll
+        for (int j = 0; j < TDMA_B; ++j) dma16(wa, offb[j], sb + (w * TDMA_B + j) * 1024);
+    };
+
+    // ---- this lane's operand addresses within a stage: x rows wm 64 + 16 i + n, chunk 4 kk + g4 (swizzle (n / 2) % 8: the rows'
+    // other terms are multiples of 16); w^T rows likewise; w: rows 32 kk + 8 g4 + n / 4 (+ 4), columns wn 64 + 16 j + 4 (n % 4)
+    const uint32_t a_rd = (uint32_t) ((wm * 64 + n) * 128), swz = (uint32_t) ((n >> 1) & 7);
+    const uint32_t b_rd = (uint32_t) (TA_BYTES + (wn * 64 + n) * 128);
+    const uint32_t bt_rd = (uint32_t) (TA_BYTES + (8 * g4 + (n >> 2)) * 256 + (n & 1) * 8);
+
+    f4v acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
+
+    const int64_t nk = p.K / TK;
+    dma(0, 0);
+    if (nk > 1) dma(1, 1);
+    int stage = 0;
+    for (int64_t kt = 0; kt < nk; ++kt) {
+        // this wave's transfers of stage kt have landed when at most stage kt + 1's are still out, and its reads of the stage
+        // about to be refilled have returned; the barrier makes both everybody's
+        if (kt + 1 < nk) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(TDMA_A + TDMA_B) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (kt + 2 < nk) dma(stage >= 1 ? stage - 1 : 2, kt + 2);
+        lds_u8* const S = L + stage * TSTAGE;
+#pragma unroll
+        for (int kk = 0; kk < TK / 32; ++kk) {
+            s8v a[4], bb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                a[i] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(S + a_rd + i * 16 * 128 + (((uint32_t) (kk * 4 + g4) ^ swz) << 4));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (TRANS_W) {
+                    bb[j] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(S + b_rd + j * 16 * 128 + (((uint32_t) (kk * 4 + g4) ^ swz) << 4));
+                } else {
+                    const uint32_t c = (uint32_t) (wn * 8 + 2 * j + ((n & 3) >> 1));
+                    const uint32_t sl = (uint32_t) (2 * (n >> 2));
+                    const s4v lo = lds_read_tr16((void*) (S + bt_rd + kk * 32 * 256 + ((c ^ sl) << 4)));
+                    const s4v hi = lds_read_tr16((void*) (S + bt_rd + kk * 32 * 256 + 4 * 256 + ((c ^ (sl + 8)) << 4)));
+                    bb[j] = s8v{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = mfma16<false>(a[i], bb[j], acc[i][j]);
+        }
+        stage = stage == 2 ? 0 : stage + 1;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t col = c0 + wn * 64 + 16 * j + n;
+            if (col >= p.N) continue;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int64_t row = r0 + wm * 64 + 16 * i + 4 * g4 + e;
+                if (row >= p.T) continue;
+                float* d = y + row * p.ldy + col;
+                *d = p.accumulate ? *d + acc[i][j][e] : acc[i][j][e];
+            }
+        }
+}
+
 __global__ __launch_bounds__(256) void to_f16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y, int64_t n) {
     const int64_t i = ((int64_t) blockIdx.x * 256 + threadIdx.x) * 4;
     if (i + 4 <= n && ((uintptr_t) x % 16 == 0) && ((uintptr_t) y % 8 == 0)) {
@@ -150,6 +279,16 @@ int gemm_h(ns_gpu* g, const char* who, int64_t batch, int trans_w, int64_t T, in
     GemmParams p{x, w, y, T, N, K, ldx, sx, ldw, sw, ldy, sy, accumulate, 0, 0};
     p.vec_x = (uintptr_t) x % 16 == 0 && ldx % 8 == 0 && sx % 8 == 0;
     p.vec_w = (uintptr_t) w % 16 == 0 && ldw % 8 == 0 && sw % 8 == 0;
+    // the tiled form: aligned operands, whole stages of K, enough of y to be worth 256 x 128 blocks, lane offsets within 32 bits
+    const bool tiled = p.vec_x && p.vec_w && K > 0 && K % TK == 0 && T > 128 && N >= 64 && (trans_w || N % 8 == 0) && (T + TM - 1) / TM <= 65535 &&
+                       ldx < ((int64_t) 1 << 22) && ldw < ((int64_t) 1 << 22);
+    if (tiled) {
+        const dim3 grid((unsigned) ((N + TN - 1) / TN), (unsigned) ((T + TM - 1) / TM), (unsigned) batch);
+        if (trans_w) gemm_h_tiled_kernel<true><<<grid, TWAVES * 64, 0, g->q>>>(p);
+        else gemm_h_tiled_kernel<false><<<grid, TWAVES * 64, 0, g->q>>>(p);
+        NS_LAUNCHED("gemm_h_tiled");
+        return 0;
+    }
     const dim3 grid((unsigned) ((N + 63) / 64), (unsigned) ((T + 63) / 64), (unsigned) batch);
     if (trans_w) gemm_h_kernel<true><<<grid, 256, 0, g->q>>>(p);
     else gemm_h_kernel<false><<<grid, 256, 0, g->q>>>(p);

@@ -43,7 +43,9 @@ def test_to_f16_is_numpys_rounding(ops):
 # T, N, K, ldx extra, ldy extra: whole blocks, ragged edges in every dimension, a K below one step, strides that break the
 # 16-byte loads, a single row and column
 SHAPES = [(64, 64, 64, 0, 0), (128, 192, 512, 0, 0), (1, 1, 1, 0, 0), (7, 5, 3, 0, 0), (65, 63, 33, 0, 0), (100, 130, 260, 4, 3),
-          (16, 512, 576, 8, 0), (333, 17, 1000, 1, 7), (2, 700, 8, 0, 0), (130, 64, 40, 24, 64)]
+          (16, 512, 576, 8, 0), (333, 17, 1000, 1, 7), (2, 700, 8, 0, 0), (130, 64, 40, 24, 64),
+          # the tiled form (whole stages of 64 in K, more than 128 rows): one block and many, ragged rows and columns, padded rows
+          (129, 64, 64, 0, 0), (256, 128, 128, 0, 0), (300, 200, 192, 8, 5), (1000, 129, 576, 0, 0), (2048, 520, 512, 16, 8)]
 
 
 @pytest.mark.parametrize("T,N,K,px,py", SHAPES)
@@ -68,7 +70,10 @@ def test_gemm_f16_against_the_exact_product(ops, T, N, K, px, py):
 # batch, trans_w, T, N, K, pads of ldx / ldw / ldy, gaps of sx / sw / sy
 BATCHES = [(4, 1, 16, 300, 512, 0, 0, 0, 0, 0, 0), (3, 0, 16, 512, 300, 0, 0, 0, 0, 0, 0), (5, 0, 33, 70, 45, 3, 5, 1, 7, 9, 11),
            (5, 1, 33, 70, 45, 3, 5, 1, 7, 9, 11), (64, 0, 8, 512, 64, 0, 0, 0, 0, 0, 0), (2, 0, 1, 1, 1, 0, 0, 0, 0, 0, 0),
-           (1, 0, 200, 129, 31, 0, 8, 0, 0, 0, 0), (2, 0, 64, 64, 96, 8, 16, 0, 8, 16, 0)]
+           (1, 0, 200, 129, 31, 0, 8, 0, 0, 0, 0), (2, 0, 64, 64, 96, 8, 16, 0, 8, 16, 0),
+           # the tiled form in both orientations: ragged blocks, columns that end inside a chunk's block, padded strides
+           (2, 0, 300, 200, 192, 8, 8, 3, 8, 16, 5), (2, 1, 300, 200, 192, 8, 8, 3, 8, 16, 5), (1, 0, 1030, 512, 640, 0, 64, 0, 0, 0, 0),
+           (3, 0, 257, 72, 64, 0, 0, 0, 0, 0, 0), (1, 1, 4100, 1088, 576, 0, 0, 0, 0, 0, 0)]
 
 
 @pytest.mark.parametrize("B,tw,T,N,K,px,pw,py,gx,gw,gy", BATCHES)
