@@ -227,3 +227,41 @@ def test_deepseek_prompt_branch_call_for_call(ops, T, H, pos0):
     ops.mla_decode(qd, kbd, vbd, DevBuf.of(g, cache[:n]), fused, T, H, pos0, scale)
     f = fused.read(np.float32).reshape(T, H * vl)
     assert np.abs(chain - f).max() <= 2e-3 and np.linalg.norm(chain - f) <= 1.5e-3 * np.linalg.norm(f)
+
+
+def test_gemm_sweep(ops):
+    """A hundred seeded products over what the two kernel forms branch on - rows, columns, depth, both forms of w, padded
+    rows and gaps between the batch's matrices, aligned or not, adding to y or not - against the exact product; nothing
+    beside the T x N results may change."""
+    g = ops.gpu
+    rng = np.random.default_rng(20250304)
+    for it in range(100):
+        tiled = rng.random() < 0.7
+        B, tw = int(rng.choice([1, 1, 2, 3])), int(rng.integers(0, 2))
+        T = int(rng.integers(129, 900)) if tiled else int(rng.integers(1, 300))
+        N = int(rng.integers(8, 70)) * 8 if tiled else int(rng.integers(1, 300))
+        K = int(rng.integers(1, 12)) * 64 if tiled else int(rng.integers(0, 300))
+        if tiled and tw and rng.random() < 0.5:
+            N = int(rng.integers(64, 500))
+        al = 8 if tiled else 1
+        ldx, ldy = K + int(rng.integers(0, 4)) * al, N + int(rng.integers(0, 9))
+        wr, wc = (N, K) if tw else (K, N)
+        ldw = wc + int(rng.integers(0, 4)) * al
+        sx, sw, sy = T * ldx + int(rng.integers(0, 3)) * al, wr * ldw + int(rng.integers(0, 3)) * al, T * ldy + int(rng.integers(0, 5))
+        x, w = rng.standard_normal(B * sx + 8).astype(np.float16), (rng.standard_normal(B * sw + 8) * 0.5).astype(np.float16)
+        y0 = rng.standard_normal(B * sy).astype(np.float32)
+        acc = bool(rng.integers(0, 2))
+        yb = DevBuf.of(g, y0)
+        ops.gemm_batch_h(B, tw, T, N, K, DevBuf.of(g, x), ldx, sx, DevBuf.of(g, w), ldw, sw, yb, ldy, sy, acc)
+        got = yb.read(np.float32)
+        written = np.zeros(B * sy, bool)
+        what = "product %d: batch %d, w%s, %d x %d x %d, rows %d / %d / %d apart, adding %d" % (it, B, "^T" if tw else "", T, N, K, ldx, ldw, ldy, acc)
+        for b in range(B):
+            xm = x[b * sx:b * sx + T * ldx].reshape(T, ldx)[:, :K]
+            wm = w[b * sw:b * sw + wr * ldw].reshape(wr, ldw)[:, :wc]
+            wt = wm.T if tw else wm
+            ym = got[b * sy:b * sy + T * ldy].reshape(T, ldy)[:, :N]
+            ref = xm.astype(np.float64) @ wt.astype(np.float64) + (y0[b * sy:b * sy + T * ldy].reshape(T, ldy)[:, :N] if acc else 0.0)
+            assert (np.abs(ym - ref) <= _bound(xm, wt, K) + 2.0 ** -23 * np.abs(ref)).all(), what
+            written[b * sy:b * sy + T * ldy].reshape(T, ldy)[:, :N] = True
+        assert np.array_equal(got[~written], y0[~written]), what
