@@ -283,3 +283,22 @@ def test_q35_prompt_kv_entry_point(ops, T, Hq, Hkv, D, p0):
         rc = ops.k.q35_attn_prompt_kv(g.raw, kt, qb.ptr, Hq * D, kb.ptr, vb.ptr, T, Hq, Hkv, D, cap, p0, ob.ptr)
         assert rc == 0, ops.k.api.error()
         check_close(ob.read(np.float32).reshape(T, -1), orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0), F32, "ns_q35_attn_prompt_kv kt %d" % kt)
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0,win,kt,qt", [
+    (200, 8, 2, 128, 300, 0, 0, F32),
+    (200, 8, 2, 128, 300, 0, 3, BF16),           # the bfloat16 rows are widened out of a position-major cache
+    (333, 10, 2, 128, 1000, 150, 3, F32),        # under a window: the widened copy starts at the window's first key
+    (90, 4, 4, 256, 40, 0, 3, F16),
+    (300, 6, 2, 128, 200, 0, 1, F16),
+])
+def test_prompt_over_a_position_major_cache(ops, T, Hq, Hkv, D, p0, win, kt, qt):
+    """Prompt passes over caches laid out [position][key head][row] (MiniMax-M3's layout: kernels/llm/minimaxm3/mm3.h:33-37),
+    every cache form the typed entry point takes - a bfloat16 cache's rows are widened to half from that layout too."""
+    n = p0 + T
+    cap = n + 5
+    kc, vc = make_kv(kt, Hkv, D, cap, n, cfg=1, pm=True)
+    qd, qf = make_q(qt, T, Hq, D, cfg=2)
+    got, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win, pm=True)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win, pm=True)
+    check_close(got, ref, qt, "prompt over a position-major cache", kt=kt)
