@@ -62,7 +62,7 @@ public:
     X(ns_attn_kv_store) X(ns_attn_decode_scratch) X(ns_attn_decode_t) X(ns_attn_prompt_t) X(ns_attn_decode_static)                       \
     X(ns_ds2_rope) X(ns_ds2_kv_store) X(ns_ds2_mla_decode) X(ns_ds2_mla_decode_q6k) X(ns_mla_decode_latent_scratch) X(ns_mla_decode_latent)             \
     X(ns_mla_attend) X(ns_mla_attend_sel) X(ns_mla_attend_sel_q8) X(ns_to_q8row) X(ns_gather_q8_h)                                     \
-    X(ns_idx_pool) X(ns_idx_score) X(ns_topk) X(ns_mla_cells) X(ns_softmax_masked) X(ns_gemm_f16) X(ns_gemm_batch_h) X(ns_to_f16)
+    X(ns_idx_pool) X(ns_idx_score) X(ns_topk) X(ns_mla_cells) X(ns_softmax_masked) X(ns_gemm_f16) X(ns_gemm_batch_h) X(ns_to_f16) X(ns_gather_h)
 
 class Api {
 public:

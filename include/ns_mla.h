@@ -107,6 +107,10 @@ int ns_gemm_f16(ns_gpu* g, int64_t T, int64_t N, int64_t K, const uint16_t* x, i
 int ns_gemm_batch_h(ns_gpu* g, int64_t batch, int trans_w, int64_t T, int64_t N, int64_t K, const uint16_t* x, int64_t ldx, int64_t sx,
                     const uint16_t* w, int64_t ldw, int64_t sw, float* y, int64_t ldy, int64_t sy, int accumulate);
 int ns_to_f16(ns_gpu* g, const float* x, uint16_t* y, int64_t n);
+/* out [n][C] half = the rows idx[i] of src (rows of C halfs, C a multiple of 8): the cells of a prompt pass's rows gathered
+ * out of a half latent cache, as ns_gather_q8_h does out of a q8 one. Replaces: kernels/llm/glm5next/glm.h:75
+ * (glm.cpp:842-853), called at llm/glm5next/src/engine.rs:106-108,1925 */
+int ns_gather_h(ns_gpu* g, const uint16_t* src, const int32_t* idx, uint16_t* out, int64_t n, int64_t C);
 
 #ifdef __cplusplus
 }

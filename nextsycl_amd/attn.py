@@ -118,6 +118,7 @@ MLA_H = {
     "ns_gemm_f16": (i32, [P, i64, i64, i64, P, i64, P, P, i64, i32]),
     "ns_gemm_batch_h": (i32, [P, i64, i32, i64, i64, i64, P, i64, i64, P, i64, i64, P, i64, i64, i32]),
     "ns_to_f16": (i32, [P, P, P, i64]),
+    "ns_gather_h": (i32, [P, P, P, P, i64, i64]),
 }
 
 
@@ -490,6 +491,13 @@ class Ops:
         _need(S, R * H * NC * 4, "softmax_masked scores")
         _need(n, R * 4, "softmax_masked counts")
         self.ok(self.k.softmax_masked(self.raw(), S.ptr, R, H, NC, n.ptr, scale), "softmax_masked")
+
+    def gather_h(self, src, rows, idx, out, n, C):
+        """ns_gather_h: out [n][C] half = the rows idx[i] of src (`rows` of them)."""
+        _need(src, rows * C * 2, "gather_h rows")
+        _need(idx, n * 4, "gather_h indices")
+        _need(out, n * C * 2, "gather_h out")
+        self.ok(self.k.gather_h(self.raw(), src.ptr, idx.ptr, out.ptr, n, C), "gather_h")
 
     def to_f16(self, x, y, n):
         """ns_to_f16: y [n] half = x [n] float32."""

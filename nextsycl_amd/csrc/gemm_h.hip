@@ -1,4 +1,5 @@
-// gemm_h.hip: the half products of the engines' MLA prompt chain - ns_to_f16, ns_gemm_f16, ns_gemm_batch_h - for gfx950.
+// gemm_h.hip: the half products of the engines' MLA prompt chain - ns_to_f16, ns_gemm_f16, ns_gemm_batch_h - and its gather of
+// half cache rows, ns_gather_h, for gfx950.
 //
 // The reference hands these to oneMKL (kernels/llm/glm5next/glm.cpp:208-276); an engine's prompt branch calls them around
 // its masked softmax (llm/deepseek2/src/engine.rs:1170-1244). The fused route through ns_mla_decode_latent is the fast
@@ -135,12 +136,14 @@ __global__ __launch_bounds__(256) void gemm_h_kernel(const GemmParams p) {
 }
 
 // ---- the tiled form
-constexpr int TM = 256, TN = 128, TK = 64, TWAVES = 8;
-constexpr int TA_BYTES = TM * TK * 2, TB_BYTES = TN * TK * 2, TSTAGE = TA_BYTES + TB_BYTES;      // 32 KiB + 16 KiB
-constexpr int TDMA_A = TA_BYTES / 1024 / TWAVES, TDMA_B = TB_BYTES / 1024 / TWAVES;             // transfers a wave and stage: 4 + 2
+constexpr int TN = 128, TK = 64, TWAVES = 8;
 
-template <bool TRANS_W>
+// TM: rows of y a work-group (256; 128 where x has too few rows for that: a wave then 32 x 64)
+template <bool TRANS_W, int TM>
 __global__ __launch_bounds__(TWAVES * 64, 1) void gemm_h_tiled_kernel(const GemmParams p) {
+    constexpr int TA_BYTES = TM * TK * 2, TB_BYTES = TN * TK * 2, TSTAGE = TA_BYTES + TB_BYTES;      // 32 (16) KiB + 16 KiB
+    constexpr int TDMA_A = TA_BYTES / 1024 / TWAVES, TDMA_B = TB_BYTES / 1024 / TWAVES;             // transfers a wave and stage: 4 (2) + 2
+    constexpr int RW = TM / 4, IT = RW / 16;                                                        // rows a wave, its row tiles
     __shared__ __attribute__((aligned(1024))) uint8_t lds[3 * TSTAGE];
     typedef __attribute__((address_space(3))) uint8_t lds_u8;
     lds_u8* const L = (lds_u8*) lds;
@@ -193,13 +196,13 @@ __global__ __launch_bounds__(TWAVES * 64, 1) void gemm_h_tiled_kernel(const Gemm
 
     // ---- this lane's operand addresses within a stage: x rows wm 64 + 16 i + n, chunk 4 kk + g4 (swizzle (n / 2) % 8: the rows'
     // other terms are multiples of 16); w^T rows likewise; w: rows 32 kk + 8 g4 + n / 4 (+ 4), columns wn 64 + 16 j + 4 (n % 4)
-    const uint32_t a_rd = (uint32_t) ((wm * 64 + n) * 128), swz = (uint32_t) ((n >> 1) & 7);
+    const uint32_t a_rd = (uint32_t) ((wm * RW + n) * 128), swz = (uint32_t) ((n >> 1) & 7);
     const uint32_t b_rd = (uint32_t) (TA_BYTES + (wn * 64 + n) * 128);
     const uint32_t bt_rd = (uint32_t) (TA_BYTES + (8 * g4 + (n >> 2)) * 256 + (n & 1) * 8);
 
-    f4v acc[4][4];
+    f4v acc[IT][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < IT; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[i][j] = f4v{0.0f, 0.0f, 0.0f, 0.0f};
 
@@ -218,9 +221,9 @@ __global__ __launch_bounds__(TWAVES * 64, 1) void gemm_h_tiled_kernel(const Gemm
         lds_u8* const S = L + stage * TSTAGE;
 #pragma unroll
         for (int kk = 0; kk < TK / 32; ++kk) {
-            s8v a[4], bb[4];
+            s8v a[IT], bb[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < IT; ++i)
                 a[i] = *reinterpret_cast<const __attribute__((address_space(3))) s8v*>(S + a_rd + i * 16 * 128 + (((uint32_t) (kk * 4 + g4) ^ swz) << 4));
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -235,21 +238,21 @@ __global__ __launch_bounds__(TWAVES * 64, 1) void gemm_h_tiled_kernel(const Gemm
                 }
             }
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < IT; ++i)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) acc[i][j] = mfma16<false>(a[i], bb[j], acc[i][j]);
         }
         stage = stage == 2 ? 0 : stage + 1;
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < IT; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int64_t col = c0 + wn * 64 + 16 * j + n;
             if (col >= p.N) continue;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int64_t row = r0 + wm * 64 + 16 * i + 4 * g4 + e;
+                const int64_t row = r0 + wm * RW + 16 * i + 4 * g4 + e;
                 if (row >= p.T) continue;
                 float* d = y + row * p.ldy + col;
                 *d = p.accumulate ? *d + acc[i][j][e] : acc[i][j][e];
@@ -268,6 +271,14 @@ __global__ __launch_bounds__(256) void to_f16_kernel(const float* __restrict__ x
     }
 }
 
+// out [n][C] = the rows idx[i] of src, 16 bytes a thread
+__global__ __launch_bounds__(256) void gather_h_kernel(const u4v* __restrict__ src, const int32_t* __restrict__ idx, u4v* __restrict__ out, int64_t n, int cv) {
+    const int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    if (i >= n * cv) return;
+    const int64_t r = i / cv, c = i - r * cv;
+    out[i] = src[(int64_t) idx[r] * cv + c];
+}
+
 int gemm_h(ns_gpu* g, const char* who, int64_t batch, int trans_w, int64_t T, int64_t N, int64_t K, const uint16_t* x, int64_t ldx, int64_t sx,
            const uint16_t* w, int64_t ldw, int64_t sw, float* y, int64_t ldy, int64_t sy, int accumulate) {
     const std::string s(who);
@@ -280,12 +291,19 @@ int gemm_h(ns_gpu* g, const char* who, int64_t batch, int trans_w, int64_t T, in
     p.vec_x = (uintptr_t) x % 16 == 0 && ldx % 8 == 0 && sx % 8 == 0;
     p.vec_w = (uintptr_t) w % 16 == 0 && ldw % 8 == 0 && sw % 8 == 0;
     // the tiled form: aligned operands, whole stages of K, enough of y to be worth 256 x 128 blocks, lane offsets within 32 bits
-    const bool tiled = p.vec_x && p.vec_w && K > 0 && K % TK == 0 && T > 128 && N >= 64 && (trans_w || N % 8 == 0) && (T + TM - 1) / TM <= 65535 &&
-                       ldx < ((int64_t) 1 << 22) && ldw < ((int64_t) 1 << 22);
+    // (256-row blocks from 192 rows on, 128-row blocks from 64: a batch of a row's heads against its cells is 64 - 128 rows a product)
+    const bool tiled = p.vec_x && p.vec_w && K > 0 && K % TK == 0 && T >= 64 && N >= 64 && (trans_w || N % 8 == 0) && ldx < ((int64_t) 1 << 22) &&
+                       ldw < ((int64_t) 1 << 22);
     if (tiled) {
-        const dim3 grid((unsigned) ((N + TN - 1) / TN), (unsigned) ((T + TM - 1) / TM), (unsigned) batch);
-        if (trans_w) gemm_h_tiled_kernel<true><<<grid, TWAVES * 64, 0, g->q>>>(p);
-        else gemm_h_tiled_kernel<false><<<grid, TWAVES * 64, 0, g->q>>>(p);
+        const int64_t tm = T >= 192 ? 256 : 128;
+        const dim3 grid((unsigned) ((N + TN - 1) / TN), (unsigned) ((T + tm - 1) / tm), (unsigned) batch);
+        if (tm == 256) {
+            if (trans_w) gemm_h_tiled_kernel<true, 256><<<grid, TWAVES * 64, 0, g->q>>>(p);
+            else gemm_h_tiled_kernel<false, 256><<<grid, TWAVES * 64, 0, g->q>>>(p);
+        } else {
+            if (trans_w) gemm_h_tiled_kernel<true, 128><<<grid, TWAVES * 64, 0, g->q>>>(p);
+            else gemm_h_tiled_kernel<false, 128><<<grid, TWAVES * 64, 0, g->q>>>(p);
+        }
         NS_LAUNCHED("gemm_h_tiled");
         return 0;
     }
@@ -307,6 +325,20 @@ int ns_to_f16(ns_gpu* g, const float* x, uint16_t* y, int64_t n) {
     NS_HIP(hipSetDevice(g->dev));
     to_f16_kernel<<<(unsigned) ((n + 1023) / 1024), 256, 0, g->q>>>(x, y, n);
     NS_LAUNCHED("to_f16");
+    return 0;
+    NS_CATCH
+}
+
+int ns_gather_h(ns_gpu* g, const uint16_t* src, const int32_t* idx, uint16_t* out, int64_t n, int64_t C) {
+    NS_TRY
+    if (n <= 0 || C <= 0) return 0;
+    if (C % 8 != 0) return ns_fail("ns_gather_h: row width not a multiple of 8");
+    if (!g || !src || !idx || !out) return ns_fail("ns_gather_h: a null buffer");
+    if ((uintptr_t) src % 16 || (uintptr_t) out % 16) return ns_fail("ns_gather_h: rows 16-byte aligned");
+    if ((n * (C / 8) + 255) / 256 >= (int64_t) 1 << 31) return ns_fail("ns_gather_h: too many rows");
+    NS_HIP(hipSetDevice(g->dev));
+    gather_h_kernel<<<(unsigned) ((n * (C / 8) + 255) / 256), 256, 0, g->q>>>(reinterpret_cast<const u4v*>(src), idx, reinterpret_cast<u4v*>(out), n, (int) (C / 8));
+    NS_LAUNCHED("gather_h");
     return 0;
     NS_CATCH
 }

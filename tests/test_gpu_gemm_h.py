@@ -45,7 +45,7 @@ def test_to_f16_is_numpys_rounding(ops):
 SHAPES = [(64, 64, 64, 0, 0), (128, 192, 512, 0, 0), (1, 1, 1, 0, 0), (7, 5, 3, 0, 0), (65, 63, 33, 0, 0), (100, 130, 260, 4, 3),
           (16, 512, 576, 8, 0), (333, 17, 1000, 1, 7), (2, 700, 8, 0, 0), (130, 64, 40, 24, 64),
           # the tiled form (whole stages of 64 in K, more than 128 rows): one block and many, ragged rows and columns, padded rows
-          (129, 64, 64, 0, 0), (256, 128, 128, 0, 0), (300, 200, 192, 8, 5), (1000, 129, 576, 0, 0), (2048, 520, 512, 16, 8)]
+          (100, 64, 64, 0, 0), (191, 200, 64, 8, 1), (192, 200, 64, 0, 0), (129, 64, 64, 0, 0), (256, 128, 128, 0, 0), (300, 200, 192, 8, 5), (1000, 129, 576, 0, 0), (2048, 520, 512, 16, 8)]
 
 
 @pytest.mark.parametrize("T,N,K,px,py", SHAPES)
@@ -73,7 +73,9 @@ BATCHES = [(4, 1, 16, 300, 512, 0, 0, 0, 0, 0, 0), (3, 0, 16, 512, 300, 0, 0, 0,
            (1, 0, 200, 129, 31, 0, 8, 0, 0, 0, 0), (2, 0, 64, 64, 96, 8, 16, 0, 8, 16, 0),
            # the tiled form in both orientations: ragged blocks, columns that end inside a chunk's block, padded strides
            (2, 0, 300, 200, 192, 8, 8, 3, 8, 16, 5), (2, 1, 300, 200, 192, 8, 8, 3, 8, 16, 5), (1, 0, 1030, 512, 640, 0, 64, 0, 0, 0, 0),
-           (3, 0, 257, 72, 64, 0, 0, 0, 0, 0, 0), (1, 1, 4100, 1088, 576, 0, 0, 0, 0, 0, 0)]
+           (3, 0, 257, 72, 64, 0, 0, 0, 0, 0, 0), (1, 1, 4100, 1088, 576, 0, 0, 0, 0, 0, 0),
+           # a batch of rows, a product a row's heads (GLM's chain): 128-row blocks
+           (5, 1, 64, 320, 512, 0, 0, 0, 0, 0, 0), (5, 0, 64, 512, 320, 0, 0, 0, 0, 0, 0), (3, 1, 96, 200, 256, 8, 8, 8, 8, 8, 8)]
 
 
 @pytest.mark.parametrize("B,tw,T,N,K,px,pw,py,gx,gw,gy", BATCHES)
@@ -265,3 +267,58 @@ def test_gemm_sweep(ops):
             assert (np.abs(ym - ref) <= _bound(xm, wt, K) + 2.0 ** -23 * np.abs(ref)).all(), what
             written[b * sy:b * sy + T * ldy].reshape(T, ldy)[:, :N] = True
         assert np.array_equal(got[~written], y0[~written]), what
+
+
+@pytest.mark.parametrize("T,H,pos0,K", [(40, 64, 3000, 16), (33, 16, 500, 8), (70, 128, 12000, 64)])
+def test_glm_prompt_chain_call_for_call(ops, T, H, pos0, K):
+    """GLM's prompt branch as its engine calls the library (llm/glm5next/src/engine.rs:1906-1940): each row's cells as a list,
+    the cells gathered out of the half cache 32 rows at a time, queries to half, a batch of products a row's heads against
+    its own cells, the masked softmax, the weights to half, the batch of weighted sums - against ns_mla_attend_sel over
+    the same lists."""
+    g = ops.gpu
+    lat, scale = 512, 1.0 / np.sqrt(192.0)
+    n = pos0 + T
+    rng = np.random.default_rng(T + K)
+    cache = _half(41 + T, (n, lat), 0.6)
+    qa = orc.randn(42 + T, (T * H, lat)).astype(np.float32)
+    sel = np.stack([np.sort(rng.choice((pos0 + t + 1) // 4, K, replace=False)) for t in range(T)]).astype(np.int32)
+    cnt = np.full(T, K, np.int32)
+    cnt[::7] = -1 if pos0 + T <= 2560 else K // 2               # dense rows where the pass allows them, shorter lists else
+    cd, qd, seld, cntd = DevBuf.of(g, cache), DevBuf.of(g, qa), DevBuf.of(g, sel), DevBuf.of(g, cnt)
+    fused = DevBuf(g, T * H * lat * 4)
+    ops.mla_attend(qd, cd, fused, T, H, lat, pos0, scale, sel=seld, sel_cnt=cntd, K=K)
+    want = fused.read(np.float32).reshape(T * H, lat)
+    dense = bool((cnt < 0).any())
+    nc = ((pos0 + T if dense else 4 * K + 3) + 63) // 64 * 64
+    idx, cb = DevBuf(g, T * nc * 4), DevBuf(g, T * 4)
+    ops.mla_cells(T, K, pos0, idx, cb, nc, seld, cntd)
+    RB = 32
+    gh, qh = DevBuf(g, RB * nc * lat * 2), DevBuf(g, RB * H * lat * 2)
+    sb, ph = DevBuf(g, RB * H * nc * 4), DevBuf(g, RB * H * nc * 2)
+    u = DevBuf(g, T * H * lat * 4)
+    u.fill(0xFF)
+    for r0 in range(0, T, RB):
+        tr = min(RB, T - r0)
+        ops.gather_h(cd, n, idx.view(r0 * nc * 4, tr * nc * 4), gh, tr * nc, lat)
+        ops.to_f16(qd.view(r0 * H * lat * 4, tr * H * lat * 4), qh, tr * H * lat)
+        ops.gemm_batch_h(tr, True, H, nc, lat, qh, lat, H * lat, gh, lat, nc * lat, sb, nc, H * nc)
+        ops.softmax_masked(sb, tr, H, nc, cb.view(r0 * 4, tr * 4), scale)
+        ops.to_f16(sb, ph, tr * H * nc)
+        ops.gemm_batch_h(tr, False, H, lat, nc, ph, nc, H * nc, gh, lat, nc * lat, u.view(r0 * H * lat * 4, tr * H * lat * 4), lat, H * lat)
+    chain = u.read(np.float32).reshape(T * H, lat)
+    assert np.abs(chain - want).max() <= 2e-3
+    assert np.linalg.norm(chain - want) <= 1e-3 * np.linalg.norm(want)
+
+
+def test_gather_h_rows(ops):
+    g = ops.gpu
+    rows, C, n = 5000, 512, 3333
+    src = np.arange(rows * C, dtype=np.uint32).astype(np.uint16).reshape(rows, C)
+    idx = np.random.default_rng(9).integers(0, rows, n).astype(np.int32)
+    out = DevBuf(g, n * C * 2 + 64)
+    out.fill(0xEE)
+    ops.gather_h(DevBuf.of(g, src), rows, DevBuf.of(g, idx), out, n, C)
+    got = out.read(np.uint16)
+    assert np.array_equal(got[:n * C].reshape(n, C), src[idx]) and (got[n * C:] == 0xEEEE).all()
+    with pytest.raises(Error, match="multiple of 8"):
+        ops.gather_h(DevBuf.of(g, src), rows, DevBuf.of(g, idx), out, 4, 100)

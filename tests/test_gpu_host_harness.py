@@ -13,8 +13,8 @@ EXE = os.path.join(HERE, "host", "host_harness")
 
 
 def harness(*args, timeout=300):
-    if not os.path.exists(EXE):
-        subprocess.run(["make", "-C", os.path.join(HERE, "host")], check=True, capture_output=True)
+    # (make rebuilds the harness only where the host header, the oracle or its own source is newer than it)
+    subprocess.run(["make", "-C", os.path.join(HERE, "host")], check=True, capture_output=True)
     env = dict(os.environ, NEXTSYCL_LIB=os.environ.get("NEXTSYCL_LIB") or nextsycl_amd.library_path())
     return subprocess.run([EXE] + list(args), env=env, capture_output=True, text=True, timeout=timeout)
 
@@ -22,7 +22,7 @@ def harness(*args, timeout=300):
 def test_cpp_host_binds_every_entry_point():
     r = harness("--symbols")
     assert r.returncode == 0, r.stdout + r.stderr
-    assert "90 entry points bound" in r.stdout, r.stdout
+    assert "91 entry points bound" in r.stdout, r.stdout
 
 
 def test_cpp_host_reports_a_missing_library():

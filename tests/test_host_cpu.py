@@ -104,6 +104,8 @@ def test_null_buffers_are_refused_before_any_launch(handle):
     refused("ns_gemm_batch_h", gb, (None, 2, 0, 4, 8, 64, b, 64, 0, b, 4, 0, b, 8, 0, 0), "apart")
     refused("ns_gemm_batch_h", gb, (None, 2, 1, 4, 8, 64, b, 64, 0, b, 64, 0, None, 8, 0, 0), "null")
     refused("ns_to_f16", [P, P, P, i64], (None, b, None, 5), "null")
+    refused("ns_gather_h", [P, P, P, P, i64, i64], (None, b, None, b, 4, 512), "null")
+    refused("ns_gather_h", [P, P, P, P, i64, i64], (None, b, b, b, 4, 100), "multiple of 8")
     refused("ns_attn_tune", [C.c_int, i64], (9, 1), "knob")
     refused("ns_attn_tune", [C.c_int, i64], (0, -1), "knob")
     handle.ns_attn_tune.restype = C.c_int
