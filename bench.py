@@ -45,9 +45,48 @@ WORKLOADS = {
 }
 
 
+GEN_SRC, GEN_LIB = os.path.join(ROOT, "bench_inputs.c"), os.path.join(ROOT, "bench_inputs.so")
+_gen = None
+
+
+def build_inputs(force=False):
+    """Compile bench_inputs.c (gcc) into bench_inputs.so beside this script."""
+    import subprocess
+    if force or not os.path.exists(GEN_LIB) or os.path.getmtime(GEN_LIB) < os.path.getmtime(GEN_SRC):
+        subprocess.run(["gcc", "-O3", "-ffp-contract=off", "-std=gnu11", "-shared", "-fPIC", GEN_SRC, "-o", GEN_LIB, "-lm"],
+                       check=True, capture_output=True)
+    return GEN_LIB
+
+
+def _stream(seed, sigma, out):
+    import ctypes as C
+    global _gen
+    if _gen is None:
+        _gen = C.CDLL(build_inputs())
+        _gen.bench_randn_f32.restype, _gen.bench_randn_f32.argtypes = None, [C.c_uint64, C.c_double, C.c_void_p, C.c_int64]
+    _gen.bench_randn_f32(int(seed), float(sigma), out.ctypes.data, out.size)
+
+
+GEN_ROWS = 1024
+
+
 def randn(seed, shape, sigma=1.0):
-    """Seeded N(0, sigma) float32 (numpy's PCG64): the bench's own input generator."""
-    return (np.random.default_rng(seed).standard_normal(shape, dtype=np.float32) * np.float32(sigma)).astype(np.float32)
+    """Seeded N(0, sigma) float32: xorshift64* -> Box-Muller in float64 (bench_inputs.c), the generator the tests' inputs
+    come from as well (there through the oracle's own statement of it). A vector is one stream in memory order; a matrix
+    is a stream every GEN_ROWS rows, seeded seed + the block's first row (the streams are sequential: this is what lets
+    the host's cores draw a few hundred million values in seconds)."""
+    shape = tuple(int(d) for d in shape)
+    out = np.empty(shape, np.float32)
+    if len(shape) < 2 or shape[0] <= GEN_ROWS:
+        _stream(seed, sigma, out.reshape(-1))
+        return out
+    from concurrent.futures import ThreadPoolExecutor
+    rows = shape[0]
+    flat = out.reshape(rows, -1)
+    _stream(seed, sigma, flat[:min(GEN_ROWS, rows)].reshape(-1))          # (loads the generator before the threads start)
+    with ThreadPoolExecutor(max_workers=min(16, os.cpu_count() or 1)) as ex:
+        list(ex.map(lambda s0: _stream(seed + s0, sigma, flat[s0:min(rows, s0 + GEN_ROWS)].reshape(-1)), range(GEN_ROWS, rows, GEN_ROWS)))
+    return out
 
 
 def f2h(x):
@@ -404,7 +443,7 @@ def main():
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {0: "f32", 1: "f16", 2: "bf16"}[w.qt] if w.kt in (0, 3) else "q8_0/f16",
-        "data": "synthetic (seeded numpy PCG64 N(0,1))",
+        "data": "synthetic (seeded xorshift64* + Box-Muller N(0,1))",
         "config": {"workload": w.desc, "name": a.workload, "rows": w.T, "q_heads": w.Hq, "kv_heads": w.Hkv, "head_dim": w.D, "kv_len": w.kv,
                    "kv_form": {0: "f16", 1: "q8_0", 2: "q4_0", 3: "bf16"}[w.kt], "flops_per_step": w.flops, "bytes_per_step": w.bytes,
                    "untimed_settle_ms": SETTLE_MS},

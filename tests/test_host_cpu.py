@@ -147,3 +147,19 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".cpp", ".hpp", ".h")):
                 src = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in src and "liboracle" not in src, os.path.join(dirpath, f)
+
+
+def test_bench_draws_its_inputs_from_the_fixed_generator():
+    """bench.py's inputs come from the generator the tests use - xorshift64* -> Box-Muller, stated once in the oracle and
+    once, independently, in bench_inputs.c: the same bits. A matrix is a stream every 1024 rows, seeded seed + first row."""
+    import numpy as np
+
+    import bench
+    from oracle import orc
+
+    for seed, n, sigma in ((1, 7, 1.0), (0xA11CE, 100001, 0.5), (0xC0FFEE + 8192, 4096, 1.0)):
+        assert np.array_equal(bench.randn(seed, (n,), sigma), orc.randn(seed, (n,), sigma))
+    x = bench.randn(0xB0B, (2500, 96), 0.5)
+    for s0 in (0, 1024, 2048):
+        rows = min(1024, 2500 - s0)
+        assert np.array_equal(x[s0:s0 + rows].ravel(), orc.randn(0xB0B + s0, (rows * 96,), 0.5))
