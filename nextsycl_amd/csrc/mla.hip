@@ -1087,8 +1087,9 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
             else mla_merge_kernel<512, 1><<<dim3((unsigned) rows, 2), 256, 0, g->q>>>(scratch, (int) ns, u);
         }
         NS_LAUNCHED("mla_merge");
+        return ns_profile_mark(g, 2);
     }
-    return ns_profile_mark(g, 2);
+    return 0;
 }
 
 }  // namespace
