@@ -163,3 +163,13 @@ def test_bench_draws_its_inputs_from_the_fixed_generator():
     for s0 in (0, 1024, 2048):
         rows = min(1024, 2500 - s0)
         assert np.array_equal(x[s0:s0 + rows].ravel(), orc.randn(0xB0B + s0, (rows * 96,), 0.5))
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU is what this build runs on: `bench.py --gpus N` with N above 1 exits with a message that says so, before it
+    touches the library or a device."""
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "one GPU" in r.stderr and not r.stdout.strip()
