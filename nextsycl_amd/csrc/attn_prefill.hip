@@ -380,9 +380,13 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) v_rd8[dt] = (uint32_t) (kkv * 256 + ((dt ^ (kkv & 7)) << 5) + (((n & 3) >> 1) << 4) + (n & 1) * 8);
     }
-    s8v pb[RT];
+    // (bfloat16 operands: a weight enters the second product as two bfloat16 numbers, the rounded weight pb and the rounded
+    // rest pl - 16 significant bits between them, where one alone would carry 8 and cost the output ~1.6e-3 of relative L2)
+    s8v pb[RT], pl[BF ? RT : 1];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) pb[rt] = s8v{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int rt = 0; rt < (BF ? RT : 1); ++rt) pl[rt] = s8v{0, 0, 0, 0, 0, 0, 0, 0};
     // S^T of one 32-key half (LDS byte offset kl) against the wave's 32 rows: the raw dot products
     // (the operands of a block's first matrix instructions are read a block earlier - kread / vread - so that their LDS
     // latency passes under the other block's work instead of at the head of this one)
@@ -445,12 +449,18 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     const s8v ones = {ONE16, ONE16, ONE16, ONE16, ONE16, ONE16, ONE16, ONE16};
     auto weigh = [&](const lds_u8* vl, const s8v (&vpre)[VPRE]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) l4[rt] = mfma16<BF>(ones, pb[rt], l4[rt]);
+        for (int rt = 0; rt < RT; ++rt) {
+            l4[rt] = mfma16<BF>(ones, pb[rt], l4[rt]);
+            if constexpr (BF) l4[rt] = mfma16<BF>(ones, pl[rt], l4[rt]);
+        }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const s8v va = dt < VPRE ? vpre[dt] : vread1(vl, dt);
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt) o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
+            for (int rt = 0; rt < RT; ++rt) {
+                o[rt][dt] = mfma16<BF>(va, pb[rt], o[rt][dt]);
+                if constexpr (BF) o[rt][dt] = mfma16<BF>(va, pl[rt], o[rt][dt]);
+            }
         }
     };
     // One step of the wave's software pipeline. Step s holds the scores of its own half in sc (computed a step earlier)
@@ -501,7 +511,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         if constexpr (D == 128) {
             // the matrix instructions of this block with two vector instructions between each
 #pragma unroll
-            for (int i = 0; i < RT * DT + RT; ++i) {
+            for (int i = 0; i < (BF ? 2 : 1) * (RT * DT + RT); ++i) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 __builtin_amdgcn_sched_group_barrier(0x002, PRESCALE ? 1 : 2, 0);
             }
@@ -529,7 +539,11 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) pb[rt][e] = to16<BF>(fast_exp2(a[rt][e]));     // -inf -> 0
+            for (int e = 0; e < 8; ++e) {
+                const float pv = fast_exp2(a[rt][e]);                                   // -inf -> 0
+                pb[rt][e] = to16<BF>(pv);
+                if constexpr (BF) pl[rt][e] = to16<BF>(pv - __builtin_bit_cast(float, (uint32_t) (uint16_t) pb[rt][e] << 16));
+            }
         }
         if constexpr (D == 128) {
             // a matrix instruction, an exponential, and a conversion after every other
@@ -543,6 +557,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         // the step's results are complete here, in program order: nothing of it drifts past the next barrier or branch
         if constexpr (RT == 2) asm volatile("" : "+v"(pb[0]), "+v"(pb[1]));
         else asm volatile("" : "+v"(pb[0]));
+        if constexpr (BF && RT == 2) asm volatile("" : "+v"(pl[0]), "+v"(pl[1]));
+        else if constexpr (BF) asm volatile("" : "+v"(pl[0]));
         __builtin_amdgcn_s_setprio(0);
     };
 
@@ -891,8 +907,9 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     p.kbs = skbs;
     p.k0 = sk0;
     p.part = g->own_scratch;
-    // A bfloat16 cache. As bfloat16 operands the softmax weights would carry 8 significant bits - a relative L2 error of
-    // ~1.6e-3 in the output on its own - and the query could not take the scale (a second rounding at 8 bits shows). So the
+    // A bfloat16 cache. As bfloat16 operands the softmax weights carry 8 significant bits each - the kernel then enters them
+    // as two numbers, twice the second product's matrix instructions - query rows of another type are rounded to 8 bits,
+    // and the query cannot take the scale (a second rounding at 8 bits shows). So the
     // pass's key and value rows are first widened to half (exactly: see kv_bf16_to_half_kernel) into the library's scratch,
     // behind the key splits' partials, and the pass runs as one over a half cache: half weights and a scaled half query, as
     // in the reference's kernels. A pass whose rows do not fit the scratch keeps bfloat16 operands (so does knob 5 = 1).

@@ -80,15 +80,15 @@ def gpu_prompt(ops, qt, kt, q_dev_arr, kc, vc, T, Hq, Hkv, D, cap, p0, win=0, pm
 U_HALF, U_BF16 = 2.0 ** -11, 2.0 ** -8      # unit roundoffs: half carries 11 significant bits, bfloat16 8
 
 
-def tolerances(ref64, qt=F32, kt=0, bf16_weights=False, bf16_queries=False):
+def tolerances(ref64, qt=F32, kt=0, bf16_queries=False):
     """The path's bar against the float64 closed form, as ONE rule for every cache form and row type.
 
     relative L2 <= 1e-3 and max-abs <= max(2e-3, sum of u |ref|max over the 16-bit roundings between the stored values
     and the output), u the unit roundoff of the rounded type (half 2^-11, bfloat16 2^-8). The roundings of a pass:
       - the softmax weights, rounded for the second product: half (the reference: qwen35/silo/attn.cpp:225-227) - also
         over a bfloat16 cache, whose values are widened to half for it (prompt passes) or whose weights are split into two
-        bfloat16 numbers (decode passes). bf16_weights: the one path that keeps a single bfloat16 weight, a prompt pass over
-        a bfloat16 cache too long for the library's scratch (or forced by knob 5);
+        bfloat16 numbers, 16 significant bits between them (decode passes, and prompt passes over a cache too long for the
+        library's scratch to hold widened);
       - q8_0 / q4_0 values, staged as halfs before the products as the reference stages them (silo/attn.cpp:56-76), where
         the closed form multiplies the unrounded int x scale;
       - a 16-bit output row.
@@ -97,16 +97,16 @@ def tolerances(ref64, qt=F32, kt=0, bf16_weights=False, bf16_queries=False):
     A bfloat16 rounding is 8 times coarser: each adds 2^-9 to the relative bound as well (a correctly rounded bfloat16
     copy of the exact result sits at ~1.6e-3 relative L2). bf16_queries: float32 / half query rows against a bfloat16
     cache on a path that multiplies them as bfloat16 (they are rounded once to 8 bits for the first product)."""
-    n_half = (0 if bf16_weights else 1) + (kt in (1, 2)) + (qt == F16)
-    n_bf16 = (1 if bf16_weights else 0) + (qt == BF16) + (1 if bf16_queries else 0)
+    n_half = 1 + (kt in (1, 2)) + (qt == F16)
+    n_bf16 = (qt == BF16) + (1 if bf16_queries else 0)
     big = float(np.abs(ref64).max())
     return max(MAX_ABS, (n_half * U_HALF + n_bf16 * U_BF16) * big), REL_L2 + n_bf16 * BF16_ROUND
 
 
-def check_close(got, ref64, qt=F32, what="", kt=0, bf16_weights=False, bf16_queries=False):
+def check_close(got, ref64, qt=F32, what="", kt=0, bf16_queries=False):
     """got against the float64 closed form under `tolerances`; returns (max-abs, relative L2)."""
     mx, rel, cos = orc.compare(got, ref64)
-    tol_abs, tol_rel = tolerances(ref64, qt, kt, bf16_weights, bf16_queries)
+    tol_abs, tol_rel = tolerances(ref64, qt, kt, bf16_queries)
     assert np.isfinite(got).all(), "%s: non-finite output" % what
     assert mx <= tol_abs and rel <= tol_rel, "%s: max-abs %.3g (<= %.3g), rel-L2 %.3g (<= %.3g), cosine %.6f" % (what, mx, tol_abs, rel, tol_rel, cos)
     return mx, rel
