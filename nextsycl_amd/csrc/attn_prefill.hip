@@ -877,7 +877,10 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     }
     // head size 256, 16-bit rows: a wave owns one 16-row tile, so 8 waves (two a SIMD, 128-row blocks) run the job 1.5 x
     // as fast as 4 (one a SIMD) whenever there are blocks enough for half the CUs
-    int PWs = D == 128 ? (((T + 255) / 256) * Hq * sns >= 512 ? 8 : 4) : (T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
+    // (heads of 128: 256-row blocks pay only where whole ones fill the chip twice over; a pass cut into key splits has few rows -
+    // 64 rows x 64 heads behind 32768 keys: 476 us in 256-row blocks that are three quarters empty, 267 us in 128-row ones;
+    // 256 rows: 518 against 308)
+    int PWs = D == 128 ? (sns == 1 && ((T + 255) / 256) * Hq >= 512 ? 8 : 4) : (T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
     if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_WAVES); forced == 4 || forced == 8) PWs = (int) forced;
     if (kt == 2 && D == 128) PWs = 4;                                 // (a q4_0 tile of 128-value rows has chunks for 256 threads)
     const int64_t ROWS = rows_of((int) D, PWs);
