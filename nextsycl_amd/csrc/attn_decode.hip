@@ -759,6 +759,47 @@ __global__ __launch_bounds__(MERGE_W * 64) void attn_merge_kernel(const float* _
     }
 }
 
+// The same merge for passes of many rows and few splits - a prompt pass cut into key splits leaves tens of thousands of
+// (row, head) pairs of 2 - 64 partials each, and a work-group a pair is then mostly launch: 16 lanes a pair, 16 pairs a
+// work-group, a lane D / 16 features as 8-byte pieces (a partial of D + 2 floats is 8-byte aligned), the splits in ascending
+// order with fused multiply-adds. out = sum O_s 2^(m_s - M) / sum l_s 2^(m_s - M), 0 where the row saw no key.
+template <int D>
+__global__ __launch_bounds__(256) void attn_merge_rows_kernel(const float* __restrict__ part, int ns, int qt, int64_t rows, void* __restrict__ out) {
+    constexpr int PS = D + 2, NP = D / 32;                       // 8-byte pieces a lane
+    const int64_t rh = (int64_t) blockIdx.x * 16 + (threadIdx.x >> 4);
+    if (rh >= rows) return;
+    const int li = threadIdx.x & 15;
+    const float* pr = part + rh * ns * PS;
+    float mx = -INFINITY;
+    for (int s = 0; s < ns; ++s) mx = fmaxf(mx, pr[(int64_t) s * PS + D]);
+    float2 acc[NP];
+#pragma unroll
+    for (int j = 0; j < NP; ++j) acc[j] = float2{0.0f, 0.0f};
+    float ls = 0.0f;
+    for (int s = 0; s < ns; ++s) {
+        const float* ps = pr + (int64_t) s * PS;
+        float2 x[NP];
+#pragma unroll
+        for (int j = 0; j < NP; ++j) x[j] = *reinterpret_cast<const float2*>(ps + 2 * (li + 16 * j));
+        const float2 mlv = *reinterpret_cast<const float2*>(ps + D);
+        const float wgt = mlv.x == -INFINITY ? 0.0f : fast_exp2(mlv.x - mx);
+        ls = fmaf(mlv.y, wgt, ls);
+#pragma unroll
+        for (int j = 0; j < NP; ++j) {
+            acc[j].x = fmaf(x[j].x, wgt, acc[j].x);
+            acc[j].y = fmaf(x[j].y, wgt, acc[j].y);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+        const float a = ls > 0.0f ? acc[j].x / ls : 0.0f, b = ls > 0.0f ? acc[j].y / ls : 0.0f;
+        const int64_t i = rh * D + 2 * (li + 16 * j);
+        if (qt == 0) *reinterpret_cast<float2*>(reinterpret_cast<float*>(out) + i) = float2{a, b};
+        else if (qt == 1) *reinterpret_cast<uint32_t*>(reinterpret_cast<uint16_t*>(out) + i) = (uint32_t) (uint16_t) to16<false>(a) | (uint32_t) (uint16_t) to16<false>(b) << 16;
+        else *reinterpret_cast<uint32_t*>(reinterpret_cast<uint16_t*>(out) + i) = (uint32_t) (uint16_t) to16<true>(a) | (uint32_t) (uint16_t) to16<true>(b) << 16;
+    }
+}
+
 // ---- host side ----------------------------------------------------------------------------------------------------
 
 // work-groups the key splits aim for (key heads x splits): two a CU at head size 128, one at 256 (its LDS footprint admits
@@ -982,6 +1023,15 @@ int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_
 // the merge of [rows][ns][D + 2] partials for the prompt kernel's key splits (the same kernel, the same layout)
 int ns_attn_merge_partials(ns_gpu* g, int64_t D, const float* part, int64_t ns, int qt, int64_t rows, void* out) {
     if (ns > MERGE_MAX_NS) return ns_fail("ns_attn_prompt: more key splits than the merge holds");
+    // (a prompt pass: many (row, head) pairs of few partials each - 16 pairs a work-group; the choice depends on the pass's
+    // shape alone, so a pass is always merged the same way)
+    if (ns <= 64 && rows >= 64) {
+        const unsigned wgs = (unsigned) ((rows + 15) / 16);
+        if (D == 128) attn_merge_rows_kernel<128><<<wgs, 256, 0, g->q>>>(part, (int) ns, qt, rows, out);
+        else attn_merge_rows_kernel<256><<<wgs, 256, 0, g->q>>>(part, (int) ns, qt, rows, out);
+        NS_LAUNCHED("attn_merge_rows");
+        return 0;
+    }
     return D == 128 ? launch_merge<128>(g, part, (int) ns, qt, rows, out) : launch_merge<256>(g, part, (int) ns, qt, rows, out);
 }
 
