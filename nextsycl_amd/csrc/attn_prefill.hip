@@ -123,15 +123,18 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     const int pid = blockIdx.x, xcd = pid % 8, xi = pid / 8;
     const int nblk = (p.T + ROWS - 1) / ROWS;
     const int Hkv = p.Hq / p.G;
-    const int unit = (xi / p.G) * 8 + xcd;
-    if (unit >= nblk * Hkv) return;
+    // (with key splits a split is one more factor of the units, the slowest: a pass of fewer than 8 units still puts work on
+    // every XCD, and a unit's splits - different keys - go to different ones)
+    const int nun = nblk * Hkv, u2 = (xi / p.G) * 8 + xcd;
+    if (u2 >= nun * p.ns) return;
+    const int unit = u2 % nun;
     const int hk = unit % Hkv;
     const int hq = hk * p.G + xi % p.G;
     const int blk = nblk - 1 - unit / Hkv;
     const int r0 = blk * ROWS;
     const int rl = std::min(r0 + ROWS, p.T) - 1;                  // the block's last row
     // keys [kbeg, kend) cover every row of the block; with key splits, the part of them in this work-group's split
-    const int split = blockIdx.y;
+    const int split = u2 / nun;
     int64_t kend = p.causal ? p.p0 + rl + 1 : p.p0 + p.T;
     int64_t kbeg = p.kfirst >= 0 ? p.kfirst : p.win > 0 ? std::max<int64_t>(0, p.p0 + r0 + 1 - p.win) : 0;
     if (p.ns > 1) {
@@ -867,6 +870,15 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
         const int64_t pairs = ((T + 127) / 128) * Hq;
         int64_t ns = std::min<int64_t>({(512 + pairs - 1) / pairs, keys / 1024, 64,
                                         (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
+        // (a pass the context dominates - equal work-groups - whose count would fill the chip's 512 places unevenly, say 640:
+        // cut further, to about two and a half rounds. 1024 rows x 40 heads behind 32768 keys: 740 -> 652 us; 2048 rows: 1467 -> 1280)
+        if (p0 >= T && keys / 1024 >= 2) {
+            const int64_t n0 = std::max<int64_t>(ns, 1), wg = pairs * n0;
+            if ((double) wg / (double) ((wg + 511) / 512 * 512) < 0.85) {
+                const int64_t cap_ns = std::min<int64_t>({keys / 1024, 64, (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
+                ns = std::max(ns, std::min<int64_t>((1280 + pairs - 1) / pairs, cap_ns));
+            }
+        }
         // (a forced count - tests - stays within what the scratch and the merge kernel hold)
         if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_SPLITS)) ns = std::min<int64_t>({forced, 2048, (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
         if (ns >= 2) {
@@ -947,8 +959,9 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
             kt_run = 0;
         }
     }
-    const int64_t units = ((T + ROWS - 1) / ROWS) * Hkv;               // (row block, key head); padded to the 8 XCDs
-    dim3 grid((unsigned) ((units + 7) / 8 * 8 * (Hq / Hkv)), (unsigned) p.ns);
+    const int64_t units = ((T + ROWS - 1) / ROWS) * Hkv * p.ns;        // (split, row block, key head); padded to the 8 XCDs
+    if ((units + 7) / 8 * 8 * (Hq / Hkv) >= (int64_t) 1 << 31) return ns_fail(w + ": too many work-groups");
+    dim3 grid((unsigned) ((units + 7) / 8 * 8 * (Hq / Hkv)));
     if (ns_profile_mark(g, 0)) return -1;
     if ((D == 256 ? (PWs == 8 ? launch_prefill<256, 8>(g, kt_run, p, grid) : launch_prefill<256, 4>(g, kt_run, p, grid))
                   : PWs == 8 ? launch_prefill<128, 8>(g, kt_run, p, grid) : launch_prefill<128, 4>(g, kt_run, p, grid)) != 0)
