@@ -252,8 +252,8 @@ int ns_q35_graph_launch(ns_gpu* g, void* h);
 void ns_q35_graph_free(void* h);
 /* Tuning knobs for sweeps and tests (this library's own): knob 0 work-groups a decode pass aims for, 1 key splits and
  * 2 waves a work-group (4 or 8) of a prompt pass, 3 work-groups an MLA pass aims for, 4 heads a wave of the
- * pre-attention kernel, 5 = 1: a prompt pass over a bfloat16 cache keeps bfloat16 operands instead of widening the
- * cache's rows to half first; value 0 = the library's own choice. Each knob starts from its environment variable
+ * pre-attention kernel, 5 = 1: a prompt pass over a bfloat16, q8_0 or q4_0 cache keeps the rows' own form in the kernel
+ * instead of widening them to half rows first, 5 = 2: it widens them whenever they fit; value 0 = the library's own choice. Each knob starts from its environment variable
  * (NS_DEC_WGS, NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW, NS_PREFILL_BF16), read once a process */
 int ns_attn_tune(int knob, int64_t value);
 

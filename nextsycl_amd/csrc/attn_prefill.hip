@@ -816,6 +816,29 @@ __global__ __launch_bounds__(256) void kv_bf16_to_half_kernel(const WidenParams 
     *reinterpret_cast<u4v*>(p.dst[z] + (((int64_t) h * p.n + j) * CPR + c) * 16) = y;
 }
 
+// The same for q8_0 (KT = 1) and q4_0 (KT = 2) rows: a thread takes 8 values of a 32-value block - 8 bytes, or one nibble
+// of each of 8 bytes - and writes the 8 halfs the kernels' own staging makes of them (half(q x d), one rounding: dq8x8 /
+// dq4x8), so the pass over the widened rows sees the operands the pass over the raw rows would have built.
+template <int KT, int CPR>   // 8-value chunks a row: D / 8
+__global__ __launch_bounds__(256) void kv_quant_to_half_kernel(const WidenParams p) {
+    constexpr int D = CPR * 8;
+    const int64_t j = (int64_t) blockIdx.x * (256 / CPR) + threadIdx.x / CPR;
+    const int c = threadIdx.x % CPR, h = blockIdx.y, z = blockIdx.z;
+    if (j >= p.n) return;
+    const int64_t pos = p.kf + j, slot = p.wrap ? pos % p.cap : pos;
+    const uint8_t* const row = p.src[z] + h * p.head_stride + slot * p.row_stride;
+    const int b = c / 4, cc = c % 4;
+    dq_s8v y;
+    if constexpr (KT == 1) {
+        const uint2 x = *reinterpret_cast<const uint2*>(row + c * 8);
+        y = dq8x8(x.x, x.y, __builtin_bit_cast(_Float16, *reinterpret_cast<const uint16_t*>(row + D + 2 * b)));
+    } else {
+        const uint2 x = *reinterpret_cast<const uint2*>(row + b * 16 + (cc & 1) * 8);
+        y = dq4x8(x.x, x.y, cc >= 2 ? 4 : 0, __builtin_bit_cast(_Float16, *reinterpret_cast<const uint16_t*>(row + D / 2 + 2 * b)));
+    }
+    *reinterpret_cast<dq_s8v*>(p.dst[z] + (((int64_t) h * p.n + j) * CPR + c) * 16) = y;
+}
+
 template <int D, int PW>
 int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
     constexpr int TH = PW * 64;
@@ -892,9 +915,22 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // (heads of 128: 256-row blocks pay only where whole ones fill the chip twice over; a pass cut into key splits has few rows -
     // 64 rows x 64 heads behind 32768 keys: 476 us in 256-row blocks that are three quarters empty, 267 us in 128-row ones;
     // 256 rows: 518 against 308)
+    // A cache that is not half is widened first when its rows fit the library's scratch behind the partials (below)
+    const int64_t wkf = kfirst >= 0 ? kfirst : win > 0 ? std::max<int64_t>(0, p0 + 1 - win) : 0, wn = p0 + T - wkf;
+    const size_t part_bytes = sns > 1 ? ((size_t) (T * Hq * sns * (D + 2)) * 4 + 255) / 256 * 256 : 0;
+    const size_t wone = (size_t) (Hkv * wn * D * 2);
+    // (what widening costs is read once a key; a pass of few rows reads a key only once a row block and query head of its
+    // group: up to 128 rows x 4 heads over bfloat16 rows of 128 - 8 heads over rows of 256 - and up to 256 x 4 over q4_0
+    // rows of 128 the kernel's own staging is the shorter way - 32768 keys behind 64 rows, 8 key heads: 108 against 121 us,
+    // q4_0 86 against 106; q8_0 rows are widened always: 123 against 112. Query rows that are not bfloat16 would be rounded
+    // to it for a bfloat16 first product: their passes widen. Knob 5: 1 keeps the rows' form, 2 widens.)
+    const int64_t key_reads = ((T + 127) / 128) * (Hq / Hkv);
+    const bool own_form = ns_tune_get(NS_TUNE_PREFILL_BF16) == 1 ||
+                          (ns_tune_get(NS_TUNE_PREFILL_BF16) == 0 && (kt == 3 ? qt == 2 && key_reads <= D / 32 : kt == 2 && D == 128 && key_reads <= 8));
+    const bool widen = kt != 0 && !own_form && part_bytes + 2 * wone <= g->own_scratch_floats * 4 && wn * D * 2 < (int64_t) 1 << 32;
     int PWs = D == 128 ? (sns == 1 && ((T + 255) / 256) * Hq >= 512 ? 8 : 4) : (T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
     if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_WAVES); forced == 4 || forced == 8) PWs = (int) forced;
-    if (kt == 2 && D == 128) PWs = 4;                                 // (a q4_0 tile of 128-value rows has chunks for 256 threads)
+    if (kt == 2 && D == 128 && !widen) PWs = 4;                              // (a q4_0 tile of 128-value rows has chunks for 256 threads)
     const int64_t ROWS = rows_of((int) D, PWs);
     if (T > (int64_t) 1 << 30 || ((T + ROWS - 1) / ROWS + 1) * Hq > (int64_t) 1 << 30) return ns_fail(w + ": too many rows or heads");
     if ((pm ? cap * Hkv : cap) * rb >= (int64_t) 1 << 32) return ns_fail(w + ": a key head's cache spans 4 GiB or more");
@@ -922,18 +958,19 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     p.kbs = skbs;
     p.k0 = sk0;
     p.part = g->own_scratch;
-    // A bfloat16 cache. As bfloat16 operands the softmax weights carry 8 significant bits each - the kernel then enters them
-    // as two numbers, twice the second product's matrix instructions - query rows of another type are rounded to 8 bits,
-    // and the query cannot take the scale (a second rounding at 8 bits shows). So the
-    // pass's key and value rows are first widened to half (exactly: see kv_bf16_to_half_kernel) into the library's scratch,
-    // behind the key splits' partials, and the pass runs as one over a half cache: half weights and a scaled half query, as
-    // in the reference's kernels. A pass whose rows do not fit the scratch keeps bfloat16 operands (so does knob 5 = 1).
+    // A cache that is not half. As bfloat16 operands the softmax weights carry 8 significant bits each - the kernel then
+    // enters them as two numbers, twice the second product's matrix instructions - query rows of another type are rounded
+    // to 8 bits, and the query cannot take the scale (a second rounding at 8 bits shows); q8_0 / q4_0 rows are staged as
+    // halfs by every work-group that reads them, once a row block and query head. So the pass's key and value rows are
+    // first widened to half (bfloat16 exactly, quantized rows to the halfs the kernel's own staging builds) into the
+    // library's scratch, behind the key splits' partials, and the pass runs as one over a half cache: half weights and a
+    // scaled half query, as in the reference's kernels (8192 rows behind 32768 keys, rows of 256: q8_0 7062 -> 4827 us,
+    // q4_0 5288 -> 4742, bfloat16 5963 -> 4666). A pass whose rows do not fit the scratch keeps the rows' own form.
     int kt_run = kt;
-    if (kt == 3 && ns_tune_get(NS_TUNE_PREFILL_BF16) != 1) {
-        const int64_t kf = kfirst >= 0 ? kfirst : win > 0 ? std::max<int64_t>(0, p0 + 1 - win) : 0, n = p0 + T - kf;
-        const size_t part_bytes = sns > 1 ? ((size_t) (T * Hq * sns * (D + 2)) * 4 + 255) / 256 * 256 : 0;
-        const size_t one = (size_t) (Hkv * n * D * 2);
-        if (part_bytes + 2 * one <= g->own_scratch_floats * 4 && n * D * 2 < (int64_t) 1 << 32) {
+    if (widen) {
+        {
+            const int64_t kf = wkf, n = wn;
+            const size_t one = wone;
             uint8_t* const buf = (uint8_t*) g->own_scratch + part_bytes;
             WidenParams wp{};
             wp.src[0] = (const uint8_t*) kc;
@@ -947,9 +984,17 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
             wp.n = n;
             wp.wrap = p.wrap;
             const dim3 wgrid((unsigned) ((n * (D / 8) + 255) / 256), (unsigned) Hkv, 2u);
-            if (D == 128) kv_bf16_to_half_kernel<16><<<wgrid, 256, 0, g->q>>>(wp);
-            else kv_bf16_to_half_kernel<32><<<wgrid, 256, 0, g->q>>>(wp);
-            NS_LAUNCHED("kv_bf16_to_half");
+            if (kt == 3) {
+                if (D == 128) kv_bf16_to_half_kernel<16><<<wgrid, 256, 0, g->q>>>(wp);
+                else kv_bf16_to_half_kernel<32><<<wgrid, 256, 0, g->q>>>(wp);
+            } else if (kt == 1) {
+                if (D == 128) kv_quant_to_half_kernel<1, 16><<<wgrid, 256, 0, g->q>>>(wp);
+                else kv_quant_to_half_kernel<1, 32><<<wgrid, 256, 0, g->q>>>(wp);
+            } else {
+                if (D == 128) kv_quant_to_half_kernel<2, 16><<<wgrid, 256, 0, g->q>>>(wp);
+                else kv_quant_to_half_kernel<2, 32><<<wgrid, 256, 0, g->q>>>(wp);
+            }
+            NS_LAUNCHED("kv_to_half");
             // (position j of head h at buf + (h n + j - kf) 2 D: the kernel is given the address position 0 would have)
             p.kc = buf - kf * D * 2;
             p.vc = buf + one - kf * D * 2;

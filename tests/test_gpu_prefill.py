@@ -302,3 +302,32 @@ def test_prompt_over_a_position_major_cache(ops, T, Hq, Hkv, D, p0, win, kt, qt)
     got, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win, pm=True)
     ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win, pm=True)
     check_close(got, ref, qt, "prompt over a position-major cache", kt=kt)
+
+
+def _own_form_cases():
+    """Every case of the tables above over a cache that is not half, as (T, Hq, Hkv, D, p0, win, kt, qt)."""
+    out = [(T, Hq, Hkv, 128, p0, win, kt, qt) for T, Hq, Hkv, p0, win, kt, qt in SMALL + QROWS128]
+    out += [(T, Hq, Hkv, 256, p0, win, kt, qt) for T, Hq, Hkv, p0, win, kt, qt in WIDE]
+    out += SPLIT + _random_cases(32, 20240608)
+    return [c for c in out if c[6] != 0]
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0,win,kt,qt", _own_form_cases())
+def test_prefill_over_the_caches_own_form(ops, tune, T, Hq, Hkv, D, p0, win, kt, qt):
+    """A pass over bfloat16, q8_0 or q4_0 rows first widens them to half rows in the library's scratch and runs as a
+    pass over a half cache (knob 5 = 2 here: always); a pass of few rows, or one whose context is too long for the scratch
+    (knob 5 = 1 here), keeps the rows' own form in the kernel. Both meet the bound; over quantized rows both stage the same halfs (half(q x d), one rounding) and walk the
+    keys in the same order, so they agree bit for bit."""
+    cap = p0 + T + 7
+    kc, vc = make_kv(kt, Hkv, D, cap, p0 + T, cfg=2)
+    qd, qf = make_q(qt, T, Hq, D, cfg=1)
+    tune(5, 2)
+    wide, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    tune(5, 1)
+    own, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(wide, ref, qt, "prefill, rows widened first", kt=kt)
+    # (bfloat16 operands: query rows of another type are rounded to bfloat16 on their way into the first product)
+    check_close(own, ref, qt, "prefill, the cache's own form in the kernel", kt=kt, bf16_queries=kt == 3 and qt != BF16)
+    if kt in (1, 2) and not (kt == 2 and D == 128):
+        assert np.array_equal(np.asarray(wide).view(np.uint8), np.asarray(own).view(np.uint8))
