@@ -81,20 +81,26 @@ __device__ __forceinline__ Rot rope_cs(const PreParams& p, int i, int t) {
             pos = (float) p.pos3[t * 3 + c];
         }
         const float a = pos * powf(p.theta, -2.0f * (float) k / (float) p.n_rot);
-        return Rot{cosf(a), sinf(a), true};
+        float sn, cs;
+        sincosf(a, &sn, &cs);          // (one argument reduction for both)
+        return Rot{cs, sn, true};
     }
     if (p.mode == ROPE_MG_PAIRS || p.mode == ROPE_MG_HALVES) {
         const bool halves = p.mode == ROPE_MG_HALVES;
         const int pr = halves ? (i < D / 2 ? i : i - D / 2) : i / 2;
         const float a = (float) (p.p0 + t) * powf(p.theta, -2.0f * (float) pr / (float) D);
-        return Rot{cosf(a), sinf(a), true};
+        float sn, cs;
+        sincosf(a, &sn, &cs);          // (one argument reduction for both)
+        return Rot{cs, sn, true};
     }
     // ROPE_MM3
     if (i >= p.n_rot) return r;
     const int hr = p.n_rot / 2, k = i % hr;
     float th = (float) (p.p0 + t);
     for (int j = 0; j < k; ++j) th *= p.ts;
-    return Rot{cosf(th), sinf(th), true};
+    float sn, cs;
+    sincosf(th, &sn, &cs);
+    return Rot{cs, sn, true};
 }
 
 // output feature i of a head row: v(j) = x[j] * inv * w[j] (or x[j]), rotated as the mode says by r = rope_cs(p, i, t)
@@ -123,13 +129,20 @@ __device__ __forceinline__ float rope_feature(const PreParams& p, const float* x
 }
 
 // VEC: whole 4-feature groups pair up under the rotation (see below); MAXG: 4-feature groups a lane (1: D up to 256)
-template <bool VEC, int MAXG>
-__global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
+// DC: the head size when it is 128 or 256 - a head row then fills its lanes exactly (no lane idles, no feature past the row)
+// and the reduction over a row's lanes has no branch - else 0: any size, read from the arguments.
+// 4 waves a SIMD (128 registers) for the form that serves the engines' sizes: measured best - 76 against 82 us at 8192 rows x
+// 56 heads with the allocation left alone (138 registers, 3 waves); the other forms keep at least 2
+template <bool VEC, int MAXG, int DC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(VEC && MAXG == 1 ? 4 : 2, 4))) void pre_attn_kernel(const PreParams p) {
     const int lane = threadIdx.x & 63;
-    const int D = p.D;
+    const int D = DC ? DC : p.D;
+    // (DC: every lane holds 4 features of a row; a row past the last loads the last row again and stores nothing - its sums
+    // stay among its own lanes - so nothing has to be zeroed)
+    constexpr bool EXACT = DC != 0;
     // a head row of 64 or 128 features takes 16 or 32 lanes: the wave then carries 4 or 2 consecutive rows t of the same
     // head at once (same group, same weights; the rotation is a lane's own anyway), and no lane idles
-    const int lph = MAXG == 1 && D == 64 ? 16 : MAXG == 1 && D == 128 ? 32 : 64;
+    const int lph = DC == 128 ? 32 : DC == 256 ? 64 : MAXG == 1 && D == 64 ? 16 : MAXG == 1 && D == 128 ? 32 : 64;
     const int rpw = 64 / lph, sub = lane / lph, li = lane - sub * lph;
     // the wave's index as a scalar: the row, the head and its group's descriptor then live in scalar registers
     const int64_t wid = (int64_t) blockIdx.x * 4 + __builtin_amdgcn_readfirstlane((int) (threadIdx.x >> 6));
@@ -226,17 +239,13 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
     constexpr int DTK = decltype(dt_c)::value;
     constexpr bool HASW = decltype(w_c)::value;
     constexpr int kt = DTK - DST_CACHE;
-    HeadIn cur, nxt;
-    fetch(ha, cur);
-    fetch(ha + 1 < hb ? ha + 1 : ha, nxt);
-  for (int h = ha; h < hb; ++h) {
-    HeadIn nx2;
-    fetch(h + 2 < hb ? h + 2 : hb - 1, nx2);          // two heads ahead; the last heads read the last again rather than branch
+    // one head: its row's scale, its features, its stores
+    auto head = [&](int h, const HeadIn& cur) __attribute__((always_inline)) {
     const float* x = cur.x;
     // ---- the row's scale
     float4 xo[MAXG];
 #pragma unroll
-    for (int c = 0; c < MAXG; ++c) xo[c] = li * 4 + c * 256 < D && row_live ? cur.xo[c] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int c = 0; c < MAXG; ++c) xo[c] = EXACT || (li * 4 + c * 256 < D && row_live) ? cur.xo[c] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     float inv = 1.0f;
     if constexpr (HASW) {
         float s = 0.0f;
@@ -269,7 +278,7 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
 #pragma unroll
         for (int c = 0; c < MAXG; ++c) {
             const int i = li * 4 + c * 256;
-            if (i >= D || !row_live) {
+            if (!EXACT && (i >= D || !row_live)) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) y[c][j] = 0.0f;
                 continue;
@@ -349,9 +358,24 @@ __global__ __launch_bounds__(256) void pre_attn_kernel(const PreParams p) {
             }
         }
     }
-    cur = nxt;
-    nxt = nx2;
-  }   // the group's next head
+    };
+    // The group's heads, the loads two heads ahead of the arithmetic: three register sets taken in turn by name (a set
+    // handed on by copy would wait for the newest load - the copy reads it - and nothing would be in flight under the
+    // arithmetic). The last heads read the last again rather than branch
+    HeadIn in0, in1, in2;
+    fetch(ha, in0);
+    fetch(ha + 1 < hb ? ha + 1 : ha, in1);
+    for (int h = ha;;) {
+        fetch(h + 2 < hb ? h + 2 : hb - 1, in2);
+        head(h, in0);
+        if (++h >= hb) break;
+        fetch(h + 2 < hb ? h + 2 : hb - 1, in0);
+        head(h, in1);
+        if (++h >= hb) break;
+        fetch(h + 2 < hb ? h + 2 : hb - 1, in1);
+        head(h, in2);
+        if (++h >= hb) break;
+    }
     };
     auto walk_w = [&](auto w_c) __attribute__((always_inline)) {
         switch (G.dt) {
@@ -376,10 +400,13 @@ int launch_pre(ns_gpu* g, const PreParams& p, const char* who) {
     if (per_t <= 0 || p.T <= 0) return 0;
     // a wave a (row group, head) while that leaves the chip short of waves (a decode step); a prompt's rows have waves to
     // spare, and each then walks several heads of its rows on one evaluation of the rotation (most of a wave's
-    // arithmetic): about 4096 waves a launch measured best, the heads of a row group shared evenly among its waves
+    // arithmetic, as much as some 16 heads). The waves' arithmetic is what a pass of some hundred rows and more waits for, so
+    // fewer, longer waves win until too few are left to keep memory busy: about 2048 waves a launch measured best (512 rows
+    // x 56 heads: 1 / 4 / 7 / 14 / 28 heads a wave 27.2 / 11.6 / 9.9 / 11.2 / 14.7 us; 2048 rows: 7 / 14 / 28 heads 23.3 /
+    // 19.9 / 19.3; 8192 rows: 14 / 28 / 56 heads 76.7 / 73.7 / 74.7), the heads of a row group shared evenly among its waves
     PreParams q = p;
     const int64_t rpw = p.D == 64 ? 4 : p.D == 128 ? 2 : 1, tg = (p.T + rpw - 1) / rpw;
-    q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, tg * per_t / 4096));
+    q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, (tg * per_t + 2047) / 2048));
     q.hpw = (int) ((per_t + (per_t + q.hpw - 1) / q.hpw - 1) / ((per_t + q.hpw - 1) / q.hpw));
     if (const int64_t forced = ns_tune_get(NS_TUNE_PRE_HPW)) q.hpw = (int) std::max<int64_t>(1, std::min<int64_t>(per_t, forced));   // sweeps
     const int64_t waves = tg * ((per_t + q.hpw - 1) / q.hpw);
@@ -388,11 +415,13 @@ int launch_pre(ns_gpu* g, const PreParams& p, const char* who) {
     const bool vec = p.mode == ROPE_NONE || p.mode == ROPE_MG_PAIRS || (p.mode == ROPE_MG_HALVES ? p.D % 8 == 0 : p.n_rot % 8 == 0);
     const dim3 grid((unsigned) ((waves + 3) / 4));
     if (p.D <= 256) {
-        if (vec) pre_attn_kernel<true, 1><<<grid, 256, 0, g->q>>>(q);
-        else pre_attn_kernel<false, 1><<<grid, 256, 0, g->q>>>(q);
+        if (vec && p.D == 128) pre_attn_kernel<true, 1, 128><<<grid, 256, 0, g->q>>>(q);
+        else if (vec && p.D == 256) pre_attn_kernel<true, 1, 256><<<grid, 256, 0, g->q>>>(q);
+        else if (vec) pre_attn_kernel<true, 1, 0><<<grid, 256, 0, g->q>>>(q);
+        else pre_attn_kernel<false, 1, 0><<<grid, 256, 0, g->q>>>(q);
     } else {
-        if (vec) pre_attn_kernel<true, 2><<<grid, 256, 0, g->q>>>(q);
-        else pre_attn_kernel<false, 2><<<grid, 256, 0, g->q>>>(q);
+        if (vec) pre_attn_kernel<true, 2, 0><<<grid, 256, 0, g->q>>>(q);
+        else pre_attn_kernel<false, 2, 0><<<grid, 256, 0, g->q>>>(q);
     }
     NS_LAUNCHED(who);
     return 0;
