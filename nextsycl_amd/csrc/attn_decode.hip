@@ -824,20 +824,16 @@ inline int64_t row_first(int64_t pos, int64_t win) { return win > 0 ? std::max<i
 // rows than 32 re-read the keys once per chunk)
 template <int D, int KT>
 int launch_rt(ns_gpu* g, const DecodeParams& p, int rows, dim3 grid_xy) {
-    // (quantized rows of 256: two row tiles and the staging registers do not fit the register file - one tile a chunk)
-    constexpr bool ONE = D == 256 && (KT == 1 || KT == 2);
-    const int RT = rows <= 16 || ONE ? 1 : 2;
+    // (quantized rows of 256 as two row tiles take the whole register file - 512 with a few spilled - and still beat two
+    // chunks that each lift and widen the tile: 24 / 4 heads x 4 rows behind 131072 q8_0 keys 110.8 -> 76.4 us, q4_0 106.4 -> 72.7)
+    const int RT = rows <= 16 ? 1 : 2;
     DecodeParams c = p;
     c.nz = (rows + RT * 16 - 1) / (RT * 16);
     const int64_t pairs = (int64_t) grid_xy.x * grid_xy.y, wgs = (pairs + 7) / 8 * 8 * c.nz;
     if (wgs >= (int64_t) 1 << 31) return ns_fail("ns_attn_decode: too many work-groups");
     const dim3 grid((unsigned) wgs);
-    if constexpr (ONE) {
-        attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(c);
-    } else {
-        if (RT == 1) attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(c);
-        else attn_decode_kernel<D, 2, KT><<<grid, WAVES * 64, 0, g->q>>>(c);
-    }
+    if (RT == 1) attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(c);
+    else attn_decode_kernel<D, 2, KT><<<grid, WAVES * 64, 0, g->q>>>(c);
     NS_LAUNCHED("attn_decode");
     return 0;
 }

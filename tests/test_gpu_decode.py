@@ -26,7 +26,9 @@ SMALL = [
     (1, 12, 2, 256, 1500, 0, 0, F32),      # qwen35's head size, G 6
     (2, 12, 2, 256, 900, 0, 1, F32),       # ... with a q8_0 cache
     (2, 8, 2, 256, 700, 0, 2, F32),        # ... with a q4_0 cache
-    (4, 12, 2, 256, 800, 0, 1, F32),       # ... q8_0 and 24 rows a key head: chunks of one row tile
+    (4, 12, 2, 256, 800, 0, 1, F32),       # ... q8_0 and 24 rows a key head: two row tiles, the whole register file
+    (5, 12, 2, 256, 5000, 0, 2, F16),      # ... q4_0 and 30 rows
+    (8, 12, 2, 256, 2100, 0, 1, F32),      # ... 48 rows: two chunks of two row tiles
     (4, 16, 2, 128, 1200, 0, 1, F16),      # q8_0, 32 rows a key head: two row tiles
     (1, 8, 2, 128, 5000, 1024, 0, F32),    # a window
     (5, 8, 2, 128, 130, 100, 0, F32),      # a window shorter than a split
@@ -112,7 +114,7 @@ def test_decode_position_major(ops):
     assert np.array_equal(ob.read(np.float32).reshape(T, -1), got)
 
 
-@pytest.mark.parametrize("kt,G,D", [(0, 8, 128), (1, 16, 128), (2, 4, 128), (3, 5, 128), (0, 6, 256)])
+@pytest.mark.parametrize("kt,G,D", [(0, 8, 128), (1, 16, 128), (2, 4, 128), (3, 5, 128), (0, 6, 256), (1, 6, 256), (2, 6, 256)])
 def test_verify_rows_equal_their_one_row_pass(ops, kt, G, D):
     """The reference's spec-check invariant (cli/nextsycl/src/main.rs:967-989): a row's result is the same whatever
     rows share its pass - bit for bit - here across passes of 1, 2, 4 and 8 rows at the same positions."""
