@@ -14,7 +14,6 @@
 #include <cstdlib>
 
 namespace {
-constexpr int64_t DECODE_ROWS = 16;   // passes up to this many rows take the decode kernel
 }
 
 extern "C" {

@@ -970,10 +970,21 @@ int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_
     if ((uintptr_t) q % 16 || ((uintptr_t) kc | (uintptr_t) vc) % 16) return ns_fail(w + ": rows 16-byte aligned");
     NS_HIP(hipSetDevice(g->dev));
     if (K == 0) return ns_fill(g, out, 0, (size_t) (T * Hq * D) * sizeof(float));     // nothing listed: zeros (l = 0)
-    const int64_t keys = K * 128, kbs = dec_kbs(keys, Hkv, D, Hq / Hkv, 0), ns = (keys + kbs - 1) / kbs;
+    // A (row, key head) with its own list is a unit of the launch. A decode or verify pass (up to 16 rows) cuts a row's
+    // listed keys by the row's own count, whatever rows share the pass (a row's bits do not depend on them). A prompt
+    // pass has units enough: its rows' keys are cut only while rows x key heads leave the chip short of work-groups -
+    // from 128 rows on not at all - and the rows go as many to a launch as the scratch holds partials for (a launch a row,
+    // the first form: 2048 rows x 64 / 4 heads with 16 blocks each 34.8 ms)
+    const int64_t keys = K * 128;
+    int64_t kbs = dec_kbs(keys, Hkv, D, Hq / Hkv, 0);
+    if (T > DECODE_ROWS) {
+        const int64_t want = std::max<int64_t>(1, std::min((keys + kbs - 1) / kbs, (512 + T * Hkv - 1) / (T * Hkv)));
+        kbs = ((keys + want - 1) / want + 127) / 128 * 128;
+    }
+    const int64_t ns = (keys + kbs - 1) / kbs;
     if ((size_t) (Hq * ns * (D + 2)) > scratch_floats) return ns_fail(w + ": the pass needs more scratch than the library keeps");
-    // every row in one launch and one merge where the partials of all rows fit the scratch; else a launch a row
-    const bool batched = (size_t) (T * Hq * ns * (D + 2)) <= scratch_floats && T * Hkv <= 65535;
+    const int64_t rows_a_launch = std::min<int64_t>({T, (int64_t) (scratch_floats / (size_t) (Hq * ns * (D + 2))), 65535 / Hkv});
+    if (rows_a_launch < 1) return ns_fail(w + ": too many key heads");
     DecodeParams p{};
     p.qt = 0;
     p.qs = Hq * D;
@@ -997,20 +1008,17 @@ int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_
     p.part = scratch;
     p.selK = (int) K;
     p.selT = 1;
-    if (batched) {
-        p.q = q;
-        p.sel = sel;
-        p.sel_pos = pos0;
-        p.selT = (int) T;
-        if (launch_kt<D>(g, 0, p, p.G, dim3((unsigned) ns, (unsigned) (Hkv * T)))) return -1;
-        return launch_merge<D>(g, scratch, (int) ns, 0, T * Hq, out);
-    }
-    for (int64_t t = 0; t < T; ++t) {
-        p.q = q + t * Hq * D;
-        p.sel = sel + t * Hkv * K;
-        p.sel_pos = pos0 + t;
-        if (launch_kt<D>(g, 0, p, p.G, dim3((unsigned) ns, (unsigned) Hkv))) return -1;
-        if (launch_merge<D>(g, scratch, (int) ns, 0, Hq, out + t * Hq * D)) return -1;
+    for (int64_t t0 = 0; t0 < T; t0 += rows_a_launch) {
+        const int64_t nr = std::min(rows_a_launch, T - t0);
+        p.q = q + t0 * Hq * D;
+        p.sel = sel + t0 * Hkv * K;
+        p.sel_pos = pos0 + t0;
+        p.selT = (int) nr;
+        if (launch_kt<D>(g, 0, p, p.G, dim3((unsigned) ns, (unsigned) (Hkv * nr)))) return -1;
+        // (a verify pass's rows are merged as a decode pass's are; a prompt's many rows of few partials 16 pairs a work-group)
+        if (T <= DECODE_ROWS ? launch_merge<D>(g, scratch, (int) ns, 0, nr * Hq, out + t0 * Hq * D)
+                             : ns_attn_merge_partials(g, D, scratch, ns, 0, nr * Hq, out + t0 * Hq * D))
+            return -1;
     }
     return 0;
     NS_CATCH

@@ -20,6 +20,7 @@ struct DecodeExtra {
 int ns_attn_decode_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const void* q, int64_t qs, const void* kc, const void* vc, int64_t T,
                        int64_t Hq, int64_t Hkv, int64_t D, int64_t cap, int64_t p0, int64_t win, const DecodeExtra& x, float scale, void* out,
                        float* scratch);
+constexpr int64_t DECODE_ROWS = 16;   // passes up to this many rows take the decode kernel
 // attn_decode.hip: block-sparse decode over a position-major half cache (rows with block lists of their own)
 int ns_attn_decode_sel(ns_gpu* g, const char* who, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K,
                        float* out, int64_t T, int64_t Hq, int64_t Hkv, int64_t pos0, float scale, float* scratch, size_t scratch_floats);
@@ -31,8 +32,8 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
                        void* out);
 
 // Tuning knobs, 0 = the library's own choice: work-groups a decode pass aims for, key splits and waves of a prompt pass,
-// work-groups an MLA pass aims for, heads a wave of the pre-attention kernel, and whether a prompt pass over a bfloat16
-// cache keeps bfloat16 operands (1) instead of widening its rows to half first. Each starts from its environment variable
+// work-groups an MLA pass aims for, heads a wave of the pre-attention kernel, and whether a prompt pass over a bfloat16,
+// q8_0 or q4_0 cache keeps the rows' own form in the kernel (1) or widens them to half first whenever they fit (2). Each starts from its environment variable
 // (NS_DEC_WGS, NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW, NS_PREFILL_BF16), read once, and changes only
 // through ns_attn_tune
 enum { NS_TUNE_DEC_WGS = 0, NS_TUNE_PREFILL_SPLITS = 1, NS_TUNE_PREFILL_WAVES = 2, NS_TUNE_MLA_WGS = 3, NS_TUNE_PRE_HPW = 4, NS_TUNE_PREFILL_BF16 = 5,

@@ -44,6 +44,33 @@ def test_minimaxm3_block_lists(ops, T, H, G, pos0, K):
     assert not out2.read(np.float32).any()
 
 
+@pytest.mark.parametrize("T,H,G,pos0,K", [(40, 32, 2, 3000, 5), (300, 64, 4, 700, 16), (8200, 64, 4, 1000, 2)])
+def test_minimaxm3_block_lists_of_a_prompt(ops, T, H, G, pos0, K):
+    """A prompt pass with block lists: every (row, key group) is a unit of one launch, the rows' keys are cut only while
+    the units are few, and a pass whose partials outgrow the library's scratch (the last case: 8200 rows x 64 heads) goes
+    in several launches. Sampled rows against the oracle's one-row pass at their positions."""
+    g = ops.gpu
+    n = pos0 + T
+    q = orc.randn(51, (T, H * 128))
+    kc, _ = orc.randn_f16(52, (n, G, 128)); vc, _ = orc.randn_f16(53, (n, G, 128))
+    rng = np.random.default_rng(9)
+    sel = np.full((T, G, K), -1, np.int32)
+    for t in range(T):
+        nb = (pos0 + t) // 128 + 1                                    # blocks the row can see, its own included
+        for gi in range(G):
+            pick = rng.permutation(nb)[:K]
+            sel[t, gi, :len(pick)] = pick
+    sel[T // 2, 0, 0] = -1                                            # a hole
+    out = DevBuf(g, T * H * 128 * 4); out.fill(0xFF)
+    ops.minimaxm3_attend(DevBuf.of(g, q), DevBuf.of(g, kc), DevBuf.of(g, vc), out, T, H, G, pos0, 0.0884, sel=DevBuf.of(g, sel), K=K)
+    got = out.read(np.float32).reshape(T, H * 128)
+    assert np.isfinite(got).all()
+    rows = sorted(set([0, 1, T // 2, T - 2, T - 1] + [int(t) for t in rng.integers(0, T, 12)]))
+    for t in rows:
+        want = orc.mm3_attend(q[t:t + 1], kc[:pos0 + t + 1], vc[:pos0 + t + 1], 1, H, G, pos0 + t, 0.0884, sel=sel[t:t + 1], K=K)
+        close(got[t:t + 1], want)
+
+
 def test_minimaxm3_indexer(ops):
     g = ops.gpu
     T, G, pos0, local, K = 3, 2, 3000, 2, 8
