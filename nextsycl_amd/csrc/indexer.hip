@@ -400,26 +400,46 @@ __global__ __launch_bounds__(256) void glm_cells_kernel(const int32_t* __restric
 }
 
 // Row softmax of scores S [R H rows of NC]: row r's heads over its first n[r] cells, scaled; the rest of the row 0
-// (kernels/llm/glm5next/glm.cpp:1041-1060). A work-group a row; rows of up to 256 PER cells stay in registers between
-// the maximum, the sum and the division (one read and one write of the row), longer ones are read three times
-template <int PER>
+// (kernels/llm/glm5next/glm.cpp:1041-1060). A work-group a row. VEC: 16-byte accesses (rows of a multiple of 4 cells at
+// 16-byte aligned addresses), else one cell an access. Rows of up to 256 PER accesses stay in registers between the
+// maximum, the sum and the division - one read and one write of the row, up to 32768 cells: the long rows of a prompt's
+// chain are this kernel's everyday case - longer ones are read three times (PER = 0)
+template <int PER, bool VEC>
 __global__ __launch_bounds__(256) void glm_softmax_masked_kernel(float* __restrict__ S, int64_t H, int64_t NC, const int32_t* __restrict__ n, float scale) {
+    constexpr int W = VEC ? 4 : 1;
+    typedef float fw __attribute__((ext_vector_type(W)));
     __shared__ float red[8];
     const int64_t rh = blockIdx.x, r = rh / H;
     float* row = S + rh * NC;
     const int64_t m = std::min<int64_t>(std::max<int32_t>(n[r], 0), NC);
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
-    float x[PER > 0 ? PER : 1];
+    // access j of this thread: cells i0 .. i0 + W - 1, i0 = (tid + 256 j) W
+    auto load = [&](int64_t i0) {
+        fw v;
+        if constexpr (VEC) {
+            v = i0 < m ? *reinterpret_cast<const fw*>(row + i0) : fw{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int e = 0; e < W; ++e) v[e] = i0 + e < m ? v[e] * scale : -INFINITY;
+        } else {
+            v[0] = i0 < m ? row[i0] * scale : -INFINITY;
+        }
+        return v;
+    };
+    fw x[PER > 0 ? PER : 1];
     float mx = -INFINITY;
     if constexpr (PER > 0) {
 #pragma unroll
         for (int j = 0; j < PER; ++j) {
-            const int64_t i = tid + 256 * j;
-            x[j] = i < m ? row[i] * scale : -INFINITY;
-            mx = fmaxf(mx, x[j]);
+            x[j] = load((int64_t) (tid + 256 * j) * W);
+#pragma unroll
+            for (int e = 0; e < W; ++e) mx = fmaxf(mx, x[j][e]);
         }
     } else {
-        for (int64_t i = tid; i < m; i += 256) mx = fmaxf(mx, row[i] * scale);
+        for (int64_t i0 = (int64_t) tid * W; i0 < m; i0 += 256 * W) {
+            const fw v = load(i0);
+#pragma unroll
+            for (int e = 0; e < W; ++e) mx = fmaxf(mx, v[e]);
+        }
     }
     mx = wave_max(mx);
     if (lane == 0) red[wv] = mx;
@@ -428,25 +448,40 @@ __global__ __launch_bounds__(256) void glm_softmax_masked_kernel(float* __restri
     float sum = 0.0f;
     if constexpr (PER > 0) {
 #pragma unroll
-        for (int j = 0; j < PER; ++j) {
-            x[j] = x[j] == -INFINITY ? 0.0f : expf(x[j] - mx);
-            sum += x[j];
-        }
+        for (int j = 0; j < PER; ++j)
+#pragma unroll
+            for (int e = 0; e < W; ++e) {
+                x[j][e] = x[j][e] == -INFINITY ? 0.0f : expf(x[j][e] - mx);
+                sum += x[j][e];
+            }
     } else {
-        for (int64_t i = tid; i < m; i += 256) sum += expf(row[i] * scale - mx);
+        for (int64_t i0 = (int64_t) tid * W; i0 < m; i0 += 256 * W) {
+            const fw v = load(i0);
+#pragma unroll
+            for (int e = 0; e < W; ++e) sum += v[e] == -INFINITY ? 0.0f : expf(v[e] - mx);
+        }
     }
     sum = wave_sum(sum);
     if (lane == 0) red[4 + wv] = sum;
     __syncthreads();
     sum = (red[4] + red[5]) + (red[6] + red[7]);
+    auto store = [&](int64_t i0, fw v) {
+        if (i0 >= NC) return;
+#pragma unroll
+        for (int e = 0; e < W; ++e) v[e] = i0 + e < m ? v[e] / sum : 0.0f;
+        if constexpr (VEC) *reinterpret_cast<fw*>(row + i0) = v;
+        else row[i0] = v[0];
+    };
     if constexpr (PER > 0) {
 #pragma unroll
-        for (int j = 0; j < PER; ++j) {
-            const int64_t i = tid + 256 * j;
-            if (i < NC) row[i] = i < m ? x[j] / sum : 0.0f;
-        }
+        for (int j = 0; j < PER; ++j) store((int64_t) (tid + 256 * j) * W, x[j]);
     } else {
-        for (int64_t i = tid; i < NC; i += 256) row[i] = i < m ? expf(row[i] * scale - mx) / sum : 0.0f;
+        for (int64_t i0 = (int64_t) tid * W; i0 < NC; i0 += 256 * W) {
+            fw v = load(i0);
+#pragma unroll
+            for (int e = 0; e < W; ++e) v[e] = v[e] == -INFINITY ? 0.0f : expf(v[e] - mx);
+            store(i0, v);
+        }
     }
 }
 
@@ -520,9 +555,17 @@ int ns_softmax_masked(ns_gpu* g, float* S, int64_t R, int64_t H, int64_t NC, con
     if (R * H >= (int64_t) 1 << 31) return ns_fail("ns_softmax_masked: too many rows");
     NS_HIP(hipSetDevice(g->dev));
     const unsigned rows = (unsigned) (R * H);
-    if (NC <= 256 * 4) glm_softmax_masked_kernel<4><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
-    else if (NC <= 256 * 16) glm_softmax_masked_kernel<16><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
-    else glm_softmax_masked_kernel<0><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+    if (NC % 4 == 0 && (uintptr_t) S % 16 == 0) {
+        if (NC <= 1024) glm_softmax_masked_kernel<1, true><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+        else if (NC <= 4096) glm_softmax_masked_kernel<4, true><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+        else if (NC <= 16384) glm_softmax_masked_kernel<16, true><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+        else if (NC <= 32768) glm_softmax_masked_kernel<32, true><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+        else glm_softmax_masked_kernel<0, true><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+    } else {
+        if (NC <= 256 * 4) glm_softmax_masked_kernel<4, false><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+        else if (NC <= 256 * 16) glm_softmax_masked_kernel<16, false><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+        else glm_softmax_masked_kernel<0, false><<<rows, 256, 0, g->q>>>(S, H, NC, n, scale);
+    }
     NS_LAUNCHED("softmax_masked");
     return 0;
     NS_CATCH
