@@ -67,6 +67,10 @@ struct PrefillParams {
     int ns;
     int64_t kbs, k0;
     float* part;                // [T][Hq][ns][D + 2]
+    // a pass of few rows: a work-group holds `pack` query heads of its key head - wave w rows (w / pack) x (a wave's rows)
+    // .. of head w % pack - so the heads share every key and value tile the work-group stages. 1: one head, every wave rows
+    // of its own. gw = G / pack: work-groups a (row block, key head)
+    int pack, gw;
 };
 
 // a 16-byte chunk of a K or V row on its way from global memory to LDS (a plain vector type: arrays of it stay in registers)
@@ -121,18 +125,20 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // row block sees the most keys), so every XCD gets the same mix of heavy and light units, heaviest first. The grid is
     // padded to a multiple of 8 units; the work-groups of the padding leave at once.
     const int pid = blockIdx.x, xcd = pid % 8, xi = pid / 8;
-    const int nblk = (p.T + ROWS - 1) / ROWS;
+    const int pk = p.pack, wh = w % pk, wr = w / pk;              // (scalars: this wave's head of the work-group's, its rows' place)
+    const int RB = ROWS / pk;                                     // rows of a head a work-group holds
+    const int nblk = (p.T + RB - 1) / RB;
     const int Hkv = p.Hq / p.G;
     // (with key splits a split is one more factor of the units, the slowest: a pass of fewer than 8 units still puts work on
     // every XCD, and a unit's splits - different keys - go to different ones)
-    const int nun = nblk * Hkv, u2 = (xi / p.G) * 8 + xcd;
+    const int nun = nblk * Hkv, u2 = (xi / p.gw) * 8 + xcd;
     if (u2 >= nun * p.ns) return;
     const int unit = u2 % nun;
     const int hk = unit % Hkv;
-    const int hq = hk * p.G + xi % p.G;
+    const int hq = hk * p.G + (xi % p.gw) * pk + wh;
     const int blk = nblk - 1 - unit / Hkv;
-    const int r0 = blk * ROWS;
-    const int rl = std::min(r0 + ROWS, p.T) - 1;                  // the block's last row
+    const int r0 = blk * RB;
+    const int rl = std::min(r0 + RB, p.T) - 1;                    // the block's last row
     // keys [kbeg, kend) cover every row of the block; with key splits, the part of them in this work-group's split
     const int split = u2 / nun;
     int64_t kend = p.causal ? p.p0 + rl + 1 : p.p0 + p.T;
@@ -147,7 +153,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     s8v qreg[RT][KB];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        const int row = r0 + w * WROWS + rt * 16 + n;
+        const int row = r0 + wr * WROWS + rt * 16 + n;
         const bool live = row < p.T;
         const int rr = live ? row : p.T - 1;
         const int64_t pos = p.p0 + rr;
@@ -195,13 +201,13 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     int lo32[RT], hi32[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        const bool live = r0 + w * WROWS + rt * 16 + n < p.T;
+        const bool live = r0 + wr * WROWS + rt * 16 + n < p.T;
         lo32[rt] = live ? (int) (lo_r[rt] - base) : 1;
         hi32[rt] = live ? (int) (hi_r[rt] - base) : 0;
     }
     // the wave's own steps: from its first row's first key to its last row's last; steps in between that no row's edge
     // crosses need no mask
-    const int wrow0 = r0 + w * WROWS, wrow1 = std::min(wrow0 + WROWS - 1, p.T - 1);
+    const int wrow0 = r0 + wr * WROWS, wrow1 = std::min(wrow0 + WROWS - 1, p.T - 1);
     const int w_full_end = (int) ((p.causal ? p.p0 + wrow0 + 1 : p.p0 + p.T) - base);
     const int w_full_beg = p.kfirst >= 0 ? (int) (p.kfirst - base) : p.win > 0 ? (int) (std::max<int64_t>(0, p.p0 + wrow1 + 1 - p.win) - base) : 0;
 
@@ -738,13 +744,13 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             const uint32_t at = (uint32_t) n * rowp + (uint32_t) (g4 * 16);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<__attribute__((address_space(3))) f4v*>(OB + at + dt * 64) = o[rt][dt];
-            const int row = r0 + w * WROWS + rt * 16 + n;
+            const int row = r0 + wr * WROWS + rt * 16 + n;
             if (g4 == 0 && row < p.T) {
                 float* pr = p.part + (((int64_t) row * p.Hq + hq) * p.ns + split) * (D + 2);
                 *reinterpret_cast<float2*>(pr + D) = float2{thr[rt] < 0.0f ? -INFINITY : -nbr[rt], lsum};
             }
             for (int c = lane; c < 16 * (D / 2); c += 64) {
-                const int rl_ = c / (D / 2), piece = c % (D / 2), prow = r0 + w * WROWS + rt * 16 + rl_;
+                const int rl_ = c / (D / 2), piece = c % (D / 2), prow = r0 + wr * WROWS + rt * 16 + rl_;
                 if (prow < p.T) {
                     typedef uint32_t u2v __attribute__((ext_vector_type(2)));
                     const u2v x = *reinterpret_cast<const __attribute__((address_space(3))) u2v*>(OB + (uint32_t) rl_ * rowp + (uint32_t) piece * 8);
@@ -779,7 +785,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             }
             // the wave reads back its own block only: no barrier, the LDS queue keeps a wave's accesses in order
             for (int c = lane; c < 16 * ppr; c += 64) {
-                const int rl_ = c / ppr, piece = c % ppr, row = r0 + w * WROWS + rt * 16 + rl_;
+                const int rl_ = c / ppr, piece = c % ppr, row = r0 + wr * WROWS + rt * 16 + rl_;
                 if (row < p.T) {
                     const u4v x = *reinterpret_cast<const __attribute__((address_space(3))) u4v*>(OB + (uint32_t) rl_ * rowp + (uint32_t) piece * 16);
                     *reinterpret_cast<u4v*>(orow + (int64_t) row * p.Hq * rowb + piece * 16) = x;
@@ -839,6 +845,17 @@ __global__ __launch_bounds__(256) void kv_quant_to_half_kernel(const WidenParams
     *reinterpret_cast<dq_s8v*>(p.dst[z] + (((int64_t) h * p.n + j) * CPR + c) * 16) = y;
 }
 
+// Query heads a work-group holds (PrefillParams::pack): a pass of so few rows that they fill only some of a work-group's
+// waves gives the other waves further heads of the same key head - 32 rows and fewer: 4 heads to 4 waves - and every
+// staged tile then serves them all (17 rows x 32 / 8 heads behind 32768 keys: each head's work-group re-staged the keys
+// for one live wave). A power of two that divides the group.
+int64_t pack_of(int64_t T, int64_t G, int64_t D, int64_t PW) {
+    const int64_t need = (T + (D == 128 ? 32 : 16) - 1) / (D == 128 ? 32 : 16);       // waves the rows of one head fill
+    int64_t pack = 1;
+    while (pack * 2 * need <= PW && G % (pack * 2) == 0) pack *= 2;
+    return pack;
+}
+
 template <int D, int PW>
 int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
     constexpr int TH = PW * 64;
@@ -890,7 +907,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // scratch (the prompt entry points have no scratch argument): what fits bounds ns.
     {
         const int64_t kf = kfirst >= 0 ? kfirst : win > 0 ? std::max<int64_t>(0, p0 + 1 - win) : 0, keys = p0 + T - kf;
-        const int64_t pairs = ((T + 127) / 128) * Hq;
+        const int64_t pairs = ((T + 127) / 128) * Hq / pack_of(T, Hq / Hkv, D, 4);
         int64_t ns = std::min<int64_t>({(512 + pairs - 1) / pairs, keys / 1024, 64,
                                         (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
         // (a pass the context dominates - equal work-groups - whose count would fill the chip's 512 places unevenly, say 640:
@@ -1004,9 +1021,12 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
             kt_run = 0;
         }
     }
-    const int64_t units = ((T + ROWS - 1) / ROWS) * Hkv * p.ns;        // (split, row block, key head); padded to the 8 XCDs
-    if ((units + 7) / 8 * 8 * (Hq / Hkv) >= (int64_t) 1 << 31) return ns_fail(w + ": too many work-groups");
-    dim3 grid((unsigned) ((units + 7) / 8 * 8 * (Hq / Hkv)));
+    p.pack = (int) pack_of(T, Hq / Hkv, D, PWs);
+    p.gw = (int) (Hq / Hkv) / p.pack;
+    const int64_t RB = ROWS / p.pack;
+    const int64_t units = ((T + RB - 1) / RB) * Hkv * p.ns;            // (split, row block, key head); padded to the 8 XCDs
+    if ((units + 7) / 8 * 8 * p.gw >= (int64_t) 1 << 31) return ns_fail(w + ": too many work-groups");
+    dim3 grid((unsigned) ((units + 7) / 8 * 8 * p.gw));
     if (ns_profile_mark(g, 0)) return -1;
     if ((D == 256 ? (PWs == 8 ? launch_prefill<256, 8>(g, kt_run, p, grid) : launch_prefill<256, 4>(g, kt_run, p, grid))
                   : PWs == 8 ? launch_prefill<128, 8>(g, kt_run, p, grid) : launch_prefill<128, 4>(g, kt_run, p, grid)) != 0)

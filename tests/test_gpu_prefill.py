@@ -304,6 +304,30 @@ def test_prompt_over_a_position_major_cache(ops, T, Hq, Hkv, D, p0, win, kt, qt)
     check_close(got, ref, qt, "prompt over a position-major cache", kt=kt)
 
 
+PACKED = [
+    # T, Hq, Hkv, D, p0, win, kt, qt: passes of so few rows that a work-group holds 2 or 4 query heads of its key head
+    (17, 8, 2, 128, 5000, 0, 0, F16),           # 4 heads a work-group, key splits
+    (32, 16, 2, 128, 300, 0, 0, F32),           # G 8: two work-groups of 4 heads a key head
+    (33, 8, 2, 128, 9000, 0, 3, BF16),          # 2 heads a work-group; bfloat16 operands (few rows: not widened)
+    (20, 12, 2, 128, 700, 256, 1, F16),         # G 6: 2 heads; a window; q8_0 rows widened
+    (64, 6, 1, 128, 2000, 0, 2, F32),           # q4_0 rows of 128 in the kernel's own staging, 2 heads
+    (17, 12, 2, 256, 4000, 0, 0, F32),          # heads of 256: 17 rows fill two of four waves
+    (5, 8, 2, 256, 1000, 0, 1, F16),            # ... 5 rows: 4 heads a work-group
+    (16, 10, 2, 128, 100, 0, 0, F32),           # G 5 has no power of two to share: one head a work-group
+    (40, 4, 1, 128, 0, 0, 0, F16),              # no context: the last rows' blocks see few keys
+]
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0,win,kt,qt", PACKED)
+def test_prefill_work_groups_holding_several_heads(ops, T, Hq, Hkv, D, p0, win, kt, qt):
+    cap = p0 + T + 3
+    kc, vc = make_kv(kt, Hkv, D, cap, p0 + T, cfg=4)
+    qd, qf = make_q(qt, T, Hq, D, cfg=2)
+    got, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
+    ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
+    check_close(got, ref, qt, "prefill, several heads a work-group", kt=kt)
+
+
 def _own_form_cases():
     """Every case of the tables above over a cache that is not half, as (T, Hq, Hkv, D, p0, win, kt, qt)."""
     out = [(T, Hq, Hkv, 128, p0, win, kt, qt) for T, Hq, Hkv, p0, win, kt, qt in SMALL + QROWS128]
