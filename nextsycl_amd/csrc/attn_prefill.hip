@@ -902,13 +902,25 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // Key splits. A pass of few rows over a long context - a chunk of a prompt behind 32K tokens, a long draft block - has
     // too few (row block, head) pairs to fill the chip, each walking every key: its keys are cut into ns splits of whole
     // tiles, a work-group a (row block, head, split), the partials merged by the decode path's merge kernel. ns is
-    // decided from the pass alone (128-row blocks x heads against ~512 work-groups; splits of at least 1024 keys), not
+    // decided from the pass alone (128-row blocks x heads against ~512 work-groups; splits no shorter than the context's length warrants), not
     // from the work-group size, so both sizes sum a row in the same order. The partials live in the library's own
     // scratch (the prompt entry points have no scratch argument): what fits bounds ns.
     {
         const int64_t kf = kfirst >= 0 ? kfirst : win > 0 ? std::max<int64_t>(0, p0 + 1 - win) : 0, keys = p0 + T - kf;
         const int64_t pairs = ((T + 127) / 128) * Hq / pack_of(T, Hq / Hkv, D, 4);
-        int64_t ns = std::min<int64_t>({(512 + pairs - 1) / pairs, keys / 1024, 64,
+        // (how far a context is worth cutting grows with its root where the (row block, head) pairs are few - under 32:
+        // splits of about 256 keys at 2048, 512 at 8192, 1024 at 32768, 2048 at 131072; shorter ones cost more in partials
+        // and their merge than they save, longer ones leave a work-group a long chain of tiles; under 512 keys none. Up to
+        // 64 pairs: twice that; more: 1024 keys and more. 17 rows x 32 / 8 heads behind 1024 keys 25.3 -> 17.5 us, behind 2048
+        // 28.1 -> 20.2, behind 8192 32.8 -> 29.7; 128 rows behind 2048 keys 30.8 -> 26.1.
+        // A pass about as long as its context is mostly diagonal - its row blocks see different key counts, and equal cuts
+        // of the keys leave them unequal work - and is cut as a long pass is, by 1024 keys; so is a pass whose work-groups
+        // hold one head's few rows, three waves of four idle: 17 rows x 40 / 8 heads behind 8192 keys 42 us in 8 splits, 49 in 13)
+        const bool filled = pack_of(T, Hq / Hkv, D, 4) > 1 || T >= 96;
+        const int64_t root = keys < 512 ? 1 : (int64_t) (0.177 * std::sqrt((double) keys));
+        const int64_t by_keys = p0 < 2 * T || !filled || pairs > 64 ? keys / 1024 : pairs < 32 ? root : std::max(keys / 1024, root / 2);
+        const int64_t aim = 512;
+        int64_t ns = std::min<int64_t>({(aim + pairs - 1) / pairs, by_keys, 64,
                                         (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
         // (a pass the context dominates - equal work-groups - whose count would fill the chip's 512 places unevenly, say 640:
         // cut further, to about two and a half rounds. 1024 rows x 40 heads behind 32768 keys: 740 -> 652 us; 2048 rows: 1467 -> 1280)
