@@ -102,3 +102,22 @@ def test_config2_prefill_8k(ops, record_property):
     ones = np.ascontiguousarray(np.broadcast_to(np.array([0x3F80], np.uint16).view(np.uint8), (Hkv, T, D, 2)).reshape(Hkv, T, 2 * D))
     g1, _ = gpu_prompt(ops, F32, 3, qf, kc, ones, T, Hq, Hkv, D, T, 0, bufs=(bufs[0], DevBuf.of(g, ones)))
     assert np.abs(g1 - 1.0).max() < 1e-5         # numerator and denominator carry the very same rounded weights
+
+
+def test_decode_and_prompt_at_256k_context(ops):
+    """The reference's long-context target (docs/256k-context.md): 262144 tokens in a q8_0 cache of 272-byte rows (heads
+    of 256). A two-row verify pass and a 17-row prompt chunk at the cache's end against the float64 closed form; the
+    prompt pass keeps the rows' own form (the widened rows of a context this long do not fit the library's scratch)."""
+    Hq, Hkv, D, n = 8, 2, 256, 262144
+    kc, vc = make_kv(1, Hkv, D, n, n, cfg=1)
+    assert kc.nbytes == Hkv * n * 272 and Hkv * n * 272 < 2 ** 32 and 2 * Hkv * n * D * 2 > 256 << 20
+    g = ops.gpu
+    bufs = (DevBuf.of(g, kc), DevBuf.of(g, vc))
+    T = 2
+    qd, qf = make_q(F16, T, Hq, D, cfg=4)
+    got, _ = gpu_decode(ops, F16, 1, qd, kc, vc, T, Hq, Hkv, D, n, n - T, bufs=bufs)
+    check_close(got, orc.attn_f64(qf, kc, vc, 1, T, Hq, Hkv, D, n, n - T), F16, "verify pass at 262144 keys", kt=1)
+    T = 17
+    qd, qf = make_q(F32, T, Hq, D, cfg=5)
+    got, _ = gpu_prompt(ops, F32, 1, qd, kc, vc, T, Hq, Hkv, D, n, n - T, bufs=bufs)
+    check_close(got, orc.attn_f64(qf, kc, vc, 1, T, Hq, Hkv, D, n, n - T), F32, "prompt chunk at 262144 keys", kt=1)
