@@ -197,7 +197,7 @@ int ns_q35_attn_probs(ns_gpu* g, int kt, const float* q, const void* kc, int64_t
 /* GQA over a position-major half cache [position][G][128], q [T][H][128], explicit scale. sel NULL: dense; else
  * sel [T][G][K] names K blocks of 128 keys a (row, key head) (-1: none), cut at the row's own position (a row is a launch).
  * Replaces: kernels/llm/minimaxm3/mm3.h:33-37 (mm3.cpp:118-190). Needs scratch: this library keeps
- * ns_attn_decode_scratch(T, H, G, 128, pos0, 0) floats per ns_gpu for it (allocated at ns_gpu_open, 256 MiB) */
+ * ns_attn_decode_scratch(T, H, G, 128, pos0, 0) floats per ns_gpu for it (allocated at ns_gpu_open, 1 GiB) */
 int ns_llm_minimaxm3_attend(ns_gpu* g, const float* q, const uint16_t* kc, const uint16_t* vc, const int32_t* sel, int64_t K, float* out, int64_t T,
                             int64_t H, int64_t G, int64_t pos0, float scale);
 
@@ -253,8 +253,10 @@ void ns_q35_graph_free(void* h);
 /* Tuning knobs for sweeps and tests (this library's own): knob 0 work-groups a decode pass aims for, 1 key splits and
  * 2 waves a work-group (4 or 8) of a prompt pass, 3 work-groups an MLA pass aims for, 4 heads a wave of the
  * pre-attention kernel, 5 = 1: a prompt pass over a bfloat16, q8_0 or q4_0 cache keeps the rows' own form in the kernel
- * instead of widening them to half rows first, 5 = 2: it widens them whenever they fit; value 0 = the library's own choice. Each knob starts from its environment variable
- * (NS_DEC_WGS, NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW, NS_PREFILL_BF16), read once a process */
+ * instead of widening them to half rows first, 5 = 2: it widens them whenever they fit; 6 the MiB of the library's own
+ * scratch a pass may plan with (tests of the paths a pass takes when its rows or partials outgrow it); value 0 = the
+ * library's own choice. Each knob starts from its environment variable
+ * (NS_DEC_WGS, NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW, NS_PREFILL_BF16, NS_SCRATCH_MIB), read once a process */
 int ns_attn_tune(int knob, int64_t value);
 
 #ifdef __cplusplus

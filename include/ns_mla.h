@@ -32,7 +32,7 @@ int ns_mla_decode_latent(ns_gpu* g, int qt, const void* qa, const uint16_t* cach
 
 /* MLA at decode widths in one call: q [T][H][128 nope + 64 rope] (rope part rotated), k_b [H][512][128] and v_b
  * [H][128][512] half, cache [n][576] half -> out [T][H][128] = v_b u. Runs absorb, the latent decode and the value
- * up-projection; its scratch is the library's own (kept per ns_gpu, 256 MiB). Replaces:
+ * up-projection; its scratch is the library's own (kept per ns_gpu, 1 GiB). Replaces:
  * kernels/llm/deepseek2/ds2.h:32-37 (ds2.cpp:139-258, 262-270) */
 int ns_ds2_mla_decode(ns_gpu* g, const float* q, const uint16_t* kb, const uint16_t* vb, const uint16_t* cache, float* out, int64_t T, int64_t H,
                       int64_t pos0, float scale);

@@ -13,7 +13,7 @@ from .sys import P, f32, i32, i64
 
 F32, F16, BF16 = 0, 1, 2                       # q / out element types (NS_F32, NS_F16, NS_BF16)
 # ns_attn_tune's knobs
-TUNE_DEC_WGS, TUNE_PREFILL_SPLITS, TUNE_PREFILL_WAVES, TUNE_MLA_WGS, TUNE_PRE_HPW, TUNE_PREFILL_BF16 = 0, 1, 2, 3, 4, 5
+TUNE_DEC_WGS, TUNE_PREFILL_SPLITS, TUNE_PREFILL_WAVES, TUNE_MLA_WGS, TUNE_PRE_HPW, TUNE_PREFILL_BF16, TUNE_SCRATCH_MIB = 0, 1, 2, 3, 4, 5, 6
 KV_F16, KV_Q8_0, KV_Q4_0, KV_BF16 = 0, 1, 2, 3   # cache forms
 ELT = {F32: 4, F16: 2, BF16: 2}
 

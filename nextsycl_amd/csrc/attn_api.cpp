@@ -162,7 +162,7 @@ static int mm3_attend(ns_gpu* g, const char* who, const float* q, const uint16_t
     if (!(scale > 0.0f)) return ns_fail(w + ": a positive scale");
     if (pos0 < 0) return ns_fail(w + ": a position");
     float* sc = g->own_scratch;
-    int64_t sc_floats = (int64_t) g->own_scratch_floats;
+    int64_t sc_floats = (int64_t) ns_own_floats(g);
     if (sel) {
         if (part && part_floats >= T * H * K * 130) sc = part, sc_floats = part_floats;      // (splits of at least 128 keys: at most K of them)
         return ns_attn_decode_sel(g, who, q, kc, vc, sel, K, out, T, H, G, pos0, scale, sc, (size_t) sc_floats);
@@ -229,7 +229,7 @@ int ns_mm3s_attend_block(ns_gpu* g, const float* q, const uint16_t* kc, const ui
 // ---- tuning knobs (tests and sweeps): read from the environment once, then only changed through ns_attn_tune
 
 namespace {
-const char* const TUNE_ENV[NS_TUNE_KNOBS] = {"NS_DEC_WGS", "NS_PREFILL_SPLITS", "NS_PREFILL_WAVES", "NS_MLA_WGS", "NS_PRE_HPW", "NS_PREFILL_BF16"};
+const char* const TUNE_ENV[NS_TUNE_KNOBS] = {"NS_DEC_WGS", "NS_PREFILL_SPLITS", "NS_PREFILL_WAVES", "NS_MLA_WGS", "NS_PRE_HPW", "NS_PREFILL_BF16", "NS_SCRATCH_MIB"};
 std::atomic<int64_t>* tune_table() {
     static std::atomic<int64_t> t[NS_TUNE_KNOBS];
     static const bool once = [] {
@@ -249,7 +249,7 @@ int64_t ns_tune_get(int knob) { return knob >= 0 && knob < NS_TUNE_KNOBS ? tune_
 extern "C" {
 
 int ns_attn_tune(int knob, int64_t value) {
-    if (knob < 0 || knob >= NS_TUNE_KNOBS || value < 0) return ns_fail("ns_attn_tune: a knob 0..5 and a value of 0 (the default) or more");
+    if (knob < 0 || knob >= NS_TUNE_KNOBS || value < 0) return ns_fail("ns_attn_tune: a knob 0..6 and a value of 0 (the default) or more");
     tune_table()[knob].store(value, std::memory_order_relaxed);
     return 0;
 }

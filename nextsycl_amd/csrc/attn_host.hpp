@@ -1,9 +1,10 @@
 // attn_host.hpp: the host-side entry points the attention translation units share (not part of the C ABI).
 #pragma once
+#include <algorithm>
 #include <cstddef>
 #include <cstdint>
 
-struct ns_gpu;
+#include "ns_internal.hpp"
 
 // What a decode pass may differ in beyond its shapes: causal 0 = every row sees to the pass's last key (a draft block);
 // kfirst >= 0 = every row starts at that key (a block with one first key for all its rows) instead of at its own
@@ -34,8 +35,14 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
 // Tuning knobs, 0 = the library's own choice: work-groups a decode pass aims for, key splits and waves of a prompt pass,
 // work-groups an MLA pass aims for, heads a wave of the pre-attention kernel, and whether a prompt pass over a bfloat16,
 // q8_0 or q4_0 cache keeps the rows' own form in the kernel (1) or widens them to half first whenever they fit (2). Each starts from its environment variable
-// (NS_DEC_WGS, NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW, NS_PREFILL_BF16), read once, and changes only
+// (NS_DEC_WGS, NS_PREFILL_SPLITS, NS_PREFILL_WAVES, NS_MLA_WGS, NS_PRE_HPW, NS_PREFILL_BF16, NS_SCRATCH_MIB), read once, and changes only
 // through ns_attn_tune
 enum { NS_TUNE_DEC_WGS = 0, NS_TUNE_PREFILL_SPLITS = 1, NS_TUNE_PREFILL_WAVES = 2, NS_TUNE_MLA_WGS = 3, NS_TUNE_PRE_HPW = 4, NS_TUNE_PREFILL_BF16 = 5,
-       NS_TUNE_KNOBS = 6 };
+       NS_TUNE_SCRATCH_MIB = 6, NS_TUNE_KNOBS = 7 };
 int64_t ns_tune_get(int knob);
+// floats of the library's own scratch a pass may plan with: all of it, or knob 6's MiB (NS_SCRATCH_MIB: tests of the paths
+// a pass takes when its rows or partials outgrow the scratch)
+inline size_t ns_own_floats(const ns_gpu* g) {
+    const int64_t mib = ns_tune_get(NS_TUNE_SCRATCH_MIB);
+    return mib > 0 ? std::min<size_t>(g->own_scratch_floats, (size_t) mib << 18) : g->own_scratch_floats;
+}

@@ -921,18 +921,18 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
         const int64_t by_keys = p0 < 2 * T || !filled || pairs > 64 ? keys / 1024 : pairs < 32 ? root : std::max(keys / 1024, root / 2);
         const int64_t aim = 512;
         int64_t ns = std::min<int64_t>({(aim + pairs - 1) / pairs, by_keys, 64,
-                                        (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
+                                        (int64_t) (ns_own_floats(g) / (size_t) (T * Hq * (D + 2)))});
         // (a pass the context dominates - equal work-groups - whose count would fill the chip's 512 places unevenly, say 640:
         // cut further, to about two and a half rounds. 1024 rows x 40 heads behind 32768 keys: 740 -> 652 us; 2048 rows: 1467 -> 1280)
         if (p0 >= T && keys / 1024 >= 2) {
             const int64_t n0 = std::max<int64_t>(ns, 1), wg = pairs * n0;
             if ((double) wg / (double) ((wg + 511) / 512 * 512) < 0.85) {
-                const int64_t cap_ns = std::min<int64_t>({keys / 1024, 64, (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
+                const int64_t cap_ns = std::min<int64_t>({keys / 1024, 64, (int64_t) (ns_own_floats(g) / (size_t) (T * Hq * (D + 2)))});
                 ns = std::max(ns, std::min<int64_t>((1280 + pairs - 1) / pairs, cap_ns));
             }
         }
         // (a forced count - tests - stays within what the scratch and the merge kernel hold)
-        if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_SPLITS)) ns = std::min<int64_t>({forced, 2048, (int64_t) (g->own_scratch_floats / (size_t) (T * Hq * (D + 2)))});
+        if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_SPLITS)) ns = std::min<int64_t>({forced, 2048, (int64_t) (ns_own_floats(g) / (size_t) (T * Hq * (D + 2)))});
         if (ns >= 2) {
             sk0 = kf / KT_TILE * KT_TILE;
             skbs = ((p0 + T - sk0 + ns - 1) / ns + KT_TILE - 1) / KT_TILE * KT_TILE;
@@ -956,7 +956,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     const int64_t key_reads = ((T + 127) / 128) * (Hq / Hkv);
     const bool own_form = ns_tune_get(NS_TUNE_PREFILL_BF16) == 1 ||
                           (ns_tune_get(NS_TUNE_PREFILL_BF16) == 0 && (kt == 3 ? qt == 2 && key_reads <= D / 32 : kt == 2 && D == 128 && key_reads <= 8));
-    const bool widen = kt != 0 && !own_form && part_bytes + 2 * wone <= g->own_scratch_floats * 4 && wn * D * 2 < (int64_t) 1 << 32;
+    const bool widen = kt != 0 && !own_form && part_bytes + 2 * wone <= ns_own_floats(g) * 4 && wn * D * 2 < (int64_t) 1 << 32;
     int PWs = D == 128 ? (sns == 1 && ((T + 255) / 256) * Hq >= 512 ? 8 : 4) : (T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
     if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_WAVES); forced == 4 || forced == 8) PWs = (int) forced;
     if (kt == 2 && D == 128 && !widen) PWs = 4;                              // (a q4_0 tile of 128-value rows has chunks for 256 threads)

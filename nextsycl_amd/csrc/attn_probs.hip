@@ -10,6 +10,7 @@
 #include "ns_internal.hpp"
 #include "ns_attn.h"
 #include "attn_common.hpp"
+#include "attn_host.hpp"
 #include "kv_formats.hpp"
 
 #include <cmath>
@@ -88,7 +89,7 @@ int ns_q35_attn_probs(ns_gpu* g, int kt, const float* q, const void* kc, int64_t
         return ns_fail("ns_q35_attn_probs: keys past the cache, heads that do not share, or not heads of 128 or 256");
     if (!q || !kc || !scratch || !out) return ns_fail("ns_q35_attn_probs: a null buffer");
     if (Hkv > 65535) return ns_fail("ns_q35_attn_probs: at most 65535 key heads");
-    if ((size_t) (Hq * n) > g->own_scratch_floats) return ns_fail("ns_q35_attn_probs: more scores (heads x keys) than the library's scratch holds");
+    if ((size_t) (Hq * n) > ns_own_floats(g)) return ns_fail("ns_q35_attn_probs: more scores (heads x keys) than the library's scratch holds");
     NS_HIP(hipSetDevice(g->dev));
     float* scores = g->own_scratch;
     const float scale = 1.0f / sqrtf((float) D);

@@ -1156,7 +1156,7 @@ static int ds2_decode(ns_gpu* g, const char* who, const float* q, const uint16_t
         const int64_t n = std::min<int64_t>(16, T - t0);
         // the library's own scratch (the reference's signature has none): the absorbed queries, u, then the partials
         const size_t rows = (size_t) (n * H), qa_f = (rows * (ML + 64) + 3) / 4 * 4, u_f = rows * ML;
-        if (qa_f + u_f + rows * PSTRIDE > g->own_scratch_floats) return ns_fail(w + ": the pass needs more scratch than the library keeps");
+        if (qa_f + u_f + rows * PSTRIDE > ns_own_floats(g)) return ns_fail(w + ": the pass needs more scratch than the library keeps");
         float* qa = g->own_scratch;
         float* u = qa + qa_f;
         float* part = u + u_f;
@@ -1165,7 +1165,7 @@ static int ds2_decode(ns_gpu* g, const char* who, const float* q, const uint16_t
         if (kvb) mla_absorb_q6k_kernel<<<(unsigned) rows, 256, 0, g->q>>>(qp, kvb, qa, H);
         else mla_absorb_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(qp, kb, qa, H);
         NS_LAUNCHED("mla_absorb");
-        if (mla_latent(g, who, 0, 0, 64, false, qa, cache, u, n, H, pos0 + t0, scale, part, g->own_scratch_floats - qa_f - u_f)) return -1;
+        if (mla_latent(g, who, 0, 0, 64, false, qa, cache, u, n, H, pos0 + t0, scale, part, ns_own_floats(g) - qa_f - u_f)) return -1;
         if (kvb) mla_vb_q6k_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(u, kvb, op, H);
         else mla_vb_kernel<<<dim3((unsigned) rows, 4), 256, 0, g->q>>>(u, vb, op, H);
         NS_LAUNCHED("mla_vb");
@@ -1237,7 +1237,7 @@ int ns_mla_attend_sel(ns_gpu* g, const float* qa, const uint16_t* c, float* u, i
     if (T <= 0) return 0;
     // (both of the reference's widths, kernels/llm/glm5next/glm.cpp:1254-1266, each an instance of the latent kernel)
     if (L != 256 && L != 512) return ns_fail("ns_mla_attend_sel: latent width 256 or 512");
-    return mla_sel_rows(g, "ns_mla_attend_sel", false, qa, c, u, T, H, pos0, scale, sel, sel_cnt, K, g->own_scratch, g->own_scratch_floats, (int) L);
+    return mla_sel_rows(g, "ns_mla_attend_sel", false, qa, c, u, T, H, pos0, scale, sel, sel_cnt, K, g->own_scratch, ns_own_floats(g), (int) L);
     NS_CATCH
 }
 
@@ -1246,7 +1246,7 @@ int ns_mla_attend_sel_q8(ns_gpu* g, const float* qa, const void* c, float* u, in
     NS_TRY
     if (T <= 0) return 0;
     if (L != 512) return ns_fail("ns_mla_attend_sel_q8: latent width 512");
-    return mla_sel_rows(g, "ns_mla_attend_sel_q8", true, qa, c, u, T, H, pos0, scale, sel, sel_cnt, K, g->own_scratch, g->own_scratch_floats);
+    return mla_sel_rows(g, "ns_mla_attend_sel_q8", true, qa, c, u, T, H, pos0, scale, sel, sel_cnt, K, g->own_scratch, ns_own_floats(g));
     NS_CATCH
 }
 
@@ -1259,14 +1259,14 @@ int ns_mla_attend(ns_gpu* g, const float* qa, const float* c, float* u, int64_t 
     if (pos0 < 0 || !c) return ns_fail("ns_mla_attend: a position and a cache");
     if ((uintptr_t) c % 16) return ns_fail("ns_mla_attend: the cache 16-byte aligned");
     const int64_t cells = pos0 + T, ch_floats = (cells * L / 2 + 3) / 4 * 4;      // the half rows, counted in floats
-    if ((size_t) ch_floats + (size_t) (H > 0 ? 16 * H * PSTRIDE : 0) > g->own_scratch_floats)
+    if ((size_t) ch_floats + (size_t) (H > 0 ? 16 * H * PSTRIDE : 0) > ns_own_floats(g))
         return ns_fail("ns_mla_attend: more cells than the library's scratch holds as half rows (use a half cache and ns_mla_attend_sel)");
     NS_HIP(hipSetDevice(g->dev));
     uint16_t* ch = (uint16_t*) g->own_scratch;
     to_half_kernel<<<(unsigned) ((cells * L / 8 + 255) / 256), 256, 0, g->q>>>(c, ch, cells * L / 8);
     NS_LAUNCHED("to_half");
     return mla_sel_rows(g, "ns_mla_attend", false, qa, ch, u, T, H, pos0, scale, nullptr, nullptr, 0, g->own_scratch + ch_floats,
-                        g->own_scratch_floats - (size_t) ch_floats, (int) L);
+                        ns_own_floats(g) - (size_t) ch_floats, (int) L);
     NS_CATCH
 }
 

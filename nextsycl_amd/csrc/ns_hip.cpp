@@ -7,7 +7,7 @@
 namespace {
 thread_local std::string g_err;
 constexpr size_t EV_RING = 1 << 16;
-constexpr size_t OWN_SCRATCH_FLOATS = (size_t) 64 << 20;   // 256 MiB
+constexpr size_t OWN_SCRATCH_FLOATS = (size_t) 256 << 20;   // 1 GiB of the card's 288
 
 // the event of a ticket the ring still holds, or null: tickets are 0 .. next_ev - 1, the ring keeps the last EV_RING
 hipEvent_t ticket_event(ns_gpu* g, int64_t t) {
