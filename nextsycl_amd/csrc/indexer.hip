@@ -23,8 +23,10 @@ constexpr int BLK = 128;
 // a query is reduced over the two waves
 constexpr int QCH = 16;     // queries staged in LDS at a time
 
+// (a prompt's thousands of queries are dealt to grid.y slices of qper queries each: a work-group is two waves, and one
+// a key block - 272 of them behind 32768 keys - left three SIMDs in four idle: 2048 rows x 4 heads 6.5 ms)
 __global__ __launch_bounds__(BLK) void idx_scores_kernel(const float* __restrict__ iq, const uint16_t* __restrict__ ik, float* __restrict__ bs, int64_t TG,
-                                                         int64_t G, int64_t nblk, int64_t pos0, int64_t local) {
+                                                         int64_t G, int64_t nblk, int64_t pos0, int64_t local, int64_t qper) {
     __shared__ float qs[QCH][BLK];
     __shared__ float red[QCH][2];
     const int64_t b = blockIdx.x;
@@ -43,13 +45,16 @@ __global__ __launch_bounds__(BLK) void idx_scores_kernel(const float* __restrict
             for (int e = 0; e < 8; ++e) kf[c * 8 + e] = f16_to_f32((uint16_t) (ww[e >> 1] >> (16 * (e & 1))));
         }
     }
-    for (int64_t q0 = 0; q0 < TG; q0 += QCH) {
-        const int nq = (int) std::min<int64_t>(QCH, TG - q0);
+    const int64_t qbeg = (int64_t) blockIdx.y * qper, qend = std::min(TG, qbeg + qper);
+    for (int64_t q0 = qbeg; q0 < qend; q0 += QCH) {
+        const int nq = (int) std::min<int64_t>(QCH, qend - q0);
         __syncthreads();
         for (int i = 0; i < nq; ++i) qs[i][lid] = iq[(q0 + i) * BLK + lid];
         __syncthreads();
         for (int i = 0; i < nq; ++i) {
             const int64_t pos = pos0 + (q0 + i) / G;
+            // (the query's features as scalar operands straight from memory instead - they are the same for every lane -
+            // were measured twice as slow: every multiply-add then waits for the scalar load in front of it)
             float s = 0.0f;
 #pragma unroll
             for (int d = 0; d < BLK; ++d) s += qs[i][d] * kf[d];
@@ -578,7 +583,11 @@ int ns_llm_minimaxm3_idx_scores(ns_gpu* g, const float* iq, const uint16_t* ik, 
     if ((uintptr_t) ik % 16) return ns_fail("ns_llm_minimaxm3_idx_scores: key rows 16-byte aligned");
     if (T * G * nblk > (int64_t) 1 << 31) return ns_fail("ns_llm_minimaxm3_idx_scores: too many blocks");
     NS_HIP(hipSetDevice(g->dev));
-    idx_scores_kernel<<<(unsigned) nblk, BLK, 0, g->q>>>(iq, ik, bs, T * G, G, nblk, pos0, local);
+    // slices of whole 16-query stages, enough of them for ~4096 work-groups (16 a CU)
+    const int64_t TG = T * G, stages = (TG + QCH - 1) / QCH;
+    const int64_t slices = std::max<int64_t>(1, std::min<int64_t>({stages, (4096 + nblk - 1) / nblk, 65535}));
+    const int64_t qper = (stages + slices - 1) / slices * QCH;
+    idx_scores_kernel<<<dim3((unsigned) nblk, (unsigned) ((TG + qper - 1) / qper)), BLK, 0, g->q>>>(iq, ik, bs, TG, G, nblk, pos0, local, qper);
     NS_LAUNCHED("idx_scores");
     return 0;
     NS_CATCH
