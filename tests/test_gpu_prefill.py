@@ -328,6 +328,20 @@ def test_prefill_work_groups_holding_several_heads(ops, T, Hq, Hkv, D, p0, win, 
     check_close(got, ref, qt, "prefill, several heads a work-group", kt=kt)
 
 
+@pytest.mark.parametrize("T,Hq,Hkv,D,p0", [(20, 16, 2, 128, 3000), (64, 8, 2, 128, 500), (100, 4, 2, 128, 9000), (10, 8, 1, 256, 700), (30, 8, 2, 256, 0)])
+def test_prefill_8_wave_work_groups_holding_several_heads(ops, tune, T, Hq, Hkv, D, p0):
+    """The 8-wave form (knob 2) over passes of few rows: 8, 4 or 2 heads a work-group; the same results as the 4-wave
+    form's to the bound (their key splits differ with the heads a work-group holds)."""
+    cap = p0 + T + 1
+    kc, vc = make_kv(0, Hkv, D, cap, p0 + T, cfg=1)
+    qd, qf = make_q(F16, T, Hq, D, cfg=3)
+    ref = orc.attn_f64(qf, kc, vc, 0, T, Hq, Hkv, D, cap, p0)
+    for waves in (8, 4):
+        tune(TUNE_PREFILL_WAVES, waves)
+        got, _ = gpu_prompt(ops, F16, 0, qd, kc, vc, T, Hq, Hkv, D, cap, p0)
+        check_close(got, ref, F16, "prefill, %d waves, several heads a work-group" % waves)
+
+
 def _own_form_cases():
     """Every case of the tables above over a cache that is not half, as (T, Hq, Hkv, D, p0, win, kt, qt)."""
     out = [(T, Hq, Hkv, 128, p0, win, kt, qt) for T, Hq, Hkv, p0, win, kt, qt in SMALL + QROWS128]
