@@ -958,6 +958,16 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
                           (ns_tune_get(NS_TUNE_PREFILL_BF16) == 0 && (kt == 3 ? qt == 2 && key_reads <= D / 32 : kt == 2 && D == 128 && key_reads <= 8));
     const bool widen = kt != 0 && !own_form && part_bytes + 2 * wone <= ns_own_floats(g) * 4 && wn * D * 2 < (int64_t) 1 << 32;
     int PWs = D == 128 ? (sns == 1 && ((T + 255) / 256) * Hq >= 512 ? 8 : 4) : (T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
+    // (a pass cut into key splits takes 8 waves after all where its rows - some heads of them to a work-group - fill
+    // every 256-row block to 70 % and the blocks the chip, one a CU: a staged tile then serves twice the rows. 128 rows x 64 / 4
+    // heads behind 32768 keys 142 -> 131 us, 256 rows 260 -> 240; x 32 / 8 heads 192 rows 141 -> 130)
+    if (D == 128 && sns > 1 && T >= 96) {
+        const int64_t pk8 = pack_of(T, Hq / Hkv, D, 8), rb8 = 256 / pk8, blocks8 = (T + rb8 - 1) / rb8;
+        const int64_t last8 = T - (blocks8 - 1) * rb8, wg8 = blocks8 * (Hq / pk8) * sns;
+        // (the last block filled like the others - 384 rows = a block and a half: 233 -> 286 us - and whole rounds of the
+        // 256 CUs - 520 work-groups, 40 heads x 13 splits, are three rounds: 74 -> 80 us)
+        if (10 * last8 >= 7 * rb8 && wg8 >= 256 && 100 * wg8 >= 85 * ((wg8 + 255) / 256 * 256)) PWs = 8;
+    }
     if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_WAVES); forced == 4 || forced == 8) PWs = (int) forced;
     if (kt == 2 && D == 128 && !widen) PWs = 4;                              // (a q4_0 tile of 128-value rows has chunks for 256 threads)
     const int64_t ROWS = rows_of((int) D, PWs);
