@@ -916,7 +916,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
         // A pass about as long as its context is mostly diagonal - its row blocks see different key counts, and equal cuts
         // of the keys leave them unequal work - and is cut as a long pass is, by 1024 keys; so is a pass whose work-groups
         // hold one head's few rows, three waves of four idle: 17 rows x 40 / 8 heads behind 8192 keys 42 us in 8 splits, 49 in 13)
-        const bool filled = pack_of(T, Hq / Hkv, D, 4) > 1 || T >= 96;
+        const bool filled = pack_of(T, Hq / Hkv, D, 4) > 1 || T >= (D == 128 ? 96 : 48);      // (4 waves of 32 rows, or of 16)
         const int64_t root = keys < 512 ? 1 : (int64_t) (0.177 * std::sqrt((double) keys));
         const int64_t by_keys = p0 < 2 * T || !filled || pairs > 64 ? keys / 1024 : pairs < 32 ? root : std::max(keys / 1024, root / 2);
         const int64_t aim = 512;
@@ -961,6 +961,9 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // (a pass cut into key splits takes 8 waves after all where its rows - some heads of them to a work-group - fill
     // every 256-row block to 70 % and the blocks the chip, one a CU: a staged tile then serves twice the rows. 128 rows x 64 / 4
     // heads behind 32768 keys 142 -> 131 us, 256 rows 260 -> 240; x 32 / 8 heads 192 rows 141 -> 130)
+    // (heads of 256: 33 - 64 rows behind a long context - 128 rows of two heads to an 8-wave work-group, one staging of the
+    // keys for both - 16 / 2 heads behind 32768 keys 92 -> 70 us, 32 / 8 heads 131 -> 94; behind 8192 keys the 4-wave form)
+    if (D == 256 && T > 32 && T <= 64 && sns > 1 && p0 + T >= 16384) PWs = 8;
     if (D == 128 && sns > 1 && T >= 96) {
         const int64_t pk8 = pack_of(T, Hq / Hkv, D, 8), rb8 = 256 / pk8, blocks8 = (T + rb8 - 1) / rb8;
         const int64_t last8 = T - (blocks8 - 1) * rb8, wg8 = blocks8 * (Hq / pk8) * sns;
