@@ -916,7 +916,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
         // A pass about as long as its context is mostly diagonal - its row blocks see different key counts, and equal cuts
         // of the keys leave them unequal work - and is cut as a long pass is, by 1024 keys; so is a pass whose work-groups
         // hold one head's few rows, three waves of four idle: 17 rows x 40 / 8 heads behind 8192 keys 42 us in 8 splits, 49 in 13)
-        const bool filled = pack_of(T, Hq / Hkv, D, 4) > 1 || T >= (D == 128 ? 96 : 48);      // (4 waves of 32 rows, or of 16)
+        const bool filled = pack_of(T, Hq / Hkv, D, 4) > 1 || T > (D == 128 ? 64 : 32);      // (rows for three of 4 waves of 32 rows, or of 16)
         const int64_t root = keys < 512 ? 1 : (int64_t) (0.177 * std::sqrt((double) keys));
         const int64_t by_keys = p0 < 2 * T || !filled || pairs > 64 ? keys / 1024 : pairs < 32 ? root : std::max(keys / 1024, root / 2);
         const int64_t aim = 512;
@@ -924,6 +924,13 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
                                         (int64_t) (ns_own_floats(g) / (size_t) (T * Hq * (D + 2)))});
         // (a pass the context dominates - equal work-groups - whose count would fill the chip's 512 places unevenly, say 640:
         // cut further, to about two and a half rounds. 1024 rows x 40 heads behind 32768 keys: 740 -> 652 us; 2048 rows: 1467 -> 1280)
+        // (a pass of few pairs whose splits overfill a round of the chip's places - heads of 256: one work-group a CU; 24
+        // heads x 16 splits = a round and a half - is cut into fewer, to whole rounds: 33 rows x 24 / 4 heads of 256 behind
+        // 8192 keys 59 -> 45 us)
+        {
+            const int64_t slots = D == 128 ? 512 : 256, wg = pairs * std::max<int64_t>(ns, 1);
+            if (ns > 1 && wg > slots && wg <= 2 * slots && 100 * wg < 85 * ((wg + slots - 1) / slots * slots)) ns = std::max<int64_t>(1, slots / pairs);
+        }
         if (p0 >= T && keys / 1024 >= 2) {
             const int64_t n0 = std::max<int64_t>(ns, 1), wg = pairs * n0;
             if ((double) wg / (double) ((wg + 511) / 512 * 512) < 0.85) {
