@@ -126,7 +126,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // padded to a multiple of 8 units; the work-groups of the padding leave at once.
     const int pid = blockIdx.x, xcd = pid % 8, xi = pid / 8;
     const int pk = p.pack, wh = w % pk, wr = w / pk;              // (scalars: this wave's head of the work-group's, its rows' place)
-    const int RB = ROWS / pk;                                     // rows of a head a work-group holds
+    const int wslots = PW / pk;                                   // waves a head (a wave past pk x wslots has no rows: 5 heads to 8 waves)
+    const int RB = wslots * WROWS;                                // rows of a head a work-group holds
     const int nblk = (p.T + RB - 1) / RB;
     const int Hkv = p.Hq / p.G;
     // (with key splits a split is one more factor of the units, the slowest: a pass of fewer than 8 units still puts work on
@@ -139,6 +140,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     const int blk = nblk - 1 - unit / Hkv;
     const int r0 = blk * RB;
     const int rl = std::min(r0 + RB, p.T) - 1;                    // the block's last row
+    const int wbase = wr < wslots ? r0 + wr * WROWS : p.T;        // this wave's first row (none: past the pass's last)
     // keys [kbeg, kend) cover every row of the block; with key splits, the part of them in this work-group's split
     const int split = u2 / nun;
     int64_t kend = p.causal ? p.p0 + rl + 1 : p.p0 + p.T;
@@ -153,7 +155,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     s8v qreg[RT][KB];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        const int row = r0 + wr * WROWS + rt * 16 + n;
+        const int row = wbase + rt * 16 + n;
         const bool live = row < p.T;
         const int rr = live ? row : p.T - 1;
         const int64_t pos = p.p0 + rr;
@@ -201,13 +203,13 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     int lo32[RT], hi32[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-        const bool live = r0 + wr * WROWS + rt * 16 + n < p.T;
+        const bool live = wbase + rt * 16 + n < p.T;
         lo32[rt] = live ? (int) (lo_r[rt] - base) : 1;
         hi32[rt] = live ? (int) (hi_r[rt] - base) : 0;
     }
     // the wave's own steps: from its first row's first key to its last row's last; steps in between that no row's edge
     // crosses need no mask
-    const int wrow0 = r0 + wr * WROWS, wrow1 = std::min(wrow0 + WROWS - 1, p.T - 1);
+    const int wrow0 = wbase, wrow1 = std::min(wrow0 + WROWS - 1, p.T - 1);
     const int w_full_end = (int) ((p.causal ? p.p0 + wrow0 + 1 : p.p0 + p.T) - base);
     const int w_full_beg = p.kfirst >= 0 ? (int) (p.kfirst - base) : p.win > 0 ? (int) (std::max<int64_t>(0, p.p0 + wrow1 + 1 - p.win) - base) : 0;
 
@@ -744,13 +746,13 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             const uint32_t at = (uint32_t) n * rowp + (uint32_t) (g4 * 16);
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) *reinterpret_cast<__attribute__((address_space(3))) f4v*>(OB + at + dt * 64) = o[rt][dt];
-            const int row = r0 + wr * WROWS + rt * 16 + n;
+            const int row = wbase + rt * 16 + n;
             if (g4 == 0 && row < p.T) {
                 float* pr = p.part + (((int64_t) row * p.Hq + hq) * p.ns + split) * (D + 2);
                 *reinterpret_cast<float2*>(pr + D) = float2{thr[rt] < 0.0f ? -INFINITY : -nbr[rt], lsum};
             }
             for (int c = lane; c < 16 * (D / 2); c += 64) {
-                const int rl_ = c / (D / 2), piece = c % (D / 2), prow = r0 + wr * WROWS + rt * 16 + rl_;
+                const int rl_ = c / (D / 2), piece = c % (D / 2), prow = wbase + rt * 16 + rl_;
                 if (prow < p.T) {
                     typedef uint32_t u2v __attribute__((ext_vector_type(2)));
                     const u2v x = *reinterpret_cast<const __attribute__((address_space(3))) u2v*>(OB + (uint32_t) rl_ * rowp + (uint32_t) piece * 8);
@@ -785,7 +787,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             }
             // the wave reads back its own block only: no barrier, the LDS queue keeps a wave's accesses in order
             for (int c = lane; c < 16 * ppr; c += 64) {
-                const int rl_ = c / ppr, piece = c % ppr, row = r0 + wr * WROWS + rt * 16 + rl_;
+                const int rl_ = c / ppr, piece = c % ppr, row = wbase + rt * 16 + rl_;
                 if (row < p.T) {
                     const u4v x = *reinterpret_cast<const __attribute__((address_space(3))) u4v*>(OB + (uint32_t) rl_ * rowp + (uint32_t) piece * 16);
                     *reinterpret_cast<u4v*>(orow + (int64_t) row * p.Hq * rowb + piece * 16) = x;
@@ -848,11 +850,12 @@ __global__ __launch_bounds__(256) void kv_quant_to_half_kernel(const WidenParams
 // Query heads a work-group holds (PrefillParams::pack): a pass of so few rows that they fill only some of a work-group's
 // waves gives the other waves further heads of the same key head - 32 rows and fewer: 4 heads to 4 waves - and every
 // staged tile then serves them all (17 rows x 32 / 8 heads behind 32768 keys: each head's work-group re-staged the keys
-// for one live wave). A power of two that divides the group.
+// for one live wave). A divisor of the group: 5 heads take 5 of 8 waves.
 int64_t pack_of(int64_t T, int64_t G, int64_t D, int64_t PW) {
     const int64_t need = (T + (D == 128 ? 32 : 16) - 1) / (D == 128 ? 32 : 16);       // waves the rows of one head fill
     int64_t pack = 1;
-    while (pack * 2 * need <= PW && G % (pack * 2) == 0) pack *= 2;
+    for (int64_t c = 2; c * need <= PW; ++c)
+        if (G % c == 0) pack = c;
     return pack;
 }
 
@@ -899,6 +902,11 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     if (((uintptr_t) kc | (uintptr_t) vc) % (rb % 16 ? 8 : 16)) return ns_fail(w + (rb % 16 ? ": caches 8-byte aligned" : ": caches 16-byte aligned"));
     // (512 work-groups of 256 rows: two for each of the chip's 256 CUs; NS_PREFILL_WAVES = 4 or 8 overrides: tuning, tests)
     int64_t sns = 1, skbs = 0, sk0 = 0;
+    // heads a work-group of a short pass holds (pack_of): with 4 waves, or - where only 8 waves let a group share at all,
+    // 5 or 7 heads - with 8
+    const int64_t pk4 = pack_of(T, Hq / Hkv, D, 4), pk8 = pack_of(T, Hq / Hkv, D, 8);
+    const bool wide_pack = pk8 > 2 * pk4 && (pk4 == 1 || p0 + T >= 8192);     // (a group that shares with 4 waves too: only behind a long context)
+    const int64_t pkp = wide_pack ? pk8 : pk4;
     // Key splits. A pass of few rows over a long context - a chunk of a prompt behind 32K tokens, a long draft block - has
     // too few (row block, head) pairs to fill the chip, each walking every key: its keys are cut into ns splits of whole
     // tiles, a work-group a (row block, head, split), the partials merged by the decode path's merge kernel. ns is
@@ -907,7 +915,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // scratch (the prompt entry points have no scratch argument): what fits bounds ns.
     {
         const int64_t kf = kfirst >= 0 ? kfirst : win > 0 ? std::max<int64_t>(0, p0 + 1 - win) : 0, keys = p0 + T - kf;
-        const int64_t pairs = ((T + 127) / 128) * Hq / pack_of(T, Hq / Hkv, D, 4);
+        const int64_t pairs = ((T + 127) / 128) * Hq / pkp;
         // (how far a context is worth cutting grows with its root where the (row block, head) pairs are few - under 32:
         // splits of about 256 keys at 2048, 512 at 8192, 1024 at 32768, 2048 at 131072; shorter ones cost more in partials
         // and their merge than they save, longer ones leave a work-group a long chain of tiles; under 512 keys none. Up to
@@ -916,7 +924,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
         // A pass about as long as its context is mostly diagonal - its row blocks see different key counts, and equal cuts
         // of the keys leave them unequal work - and is cut as a long pass is, by 1024 keys; so is a pass whose work-groups
         // hold one head's few rows, three waves of four idle: 17 rows x 40 / 8 heads behind 8192 keys 42 us in 8 splits, 49 in 13)
-        const bool filled = pack_of(T, Hq / Hkv, D, 4) > 1 || T > (D == 128 ? 64 : 32);      // (rows for three of 4 waves of 32 rows, or of 16)
+        const bool filled = pkp > 1 || T > (D == 128 ? 64 : 32);      // (rows for three of 4 waves of 32 rows, or of 16)
         const int64_t root = keys < 512 ? 1 : (int64_t) (0.177 * std::sqrt((double) keys));
         const int64_t by_keys = p0 < 2 * T || !filled || pairs > 64 ? keys / 1024 : pairs < 32 ? root : std::max(keys / 1024, root / 2);
         const int64_t aim = 512;
@@ -972,12 +980,13 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // keys for both - 16 / 2 heads behind 32768 keys 92 -> 70 us, 32 / 8 heads 131 -> 94; behind 8192 keys the 4-wave form)
     if (D == 256 && T > 32 && T <= 64 && sns > 1 && p0 + T >= 16384) PWs = 8;
     if (D == 128 && sns > 1 && T >= 96) {
-        const int64_t pk8 = pack_of(T, Hq / Hkv, D, 8), rb8 = 256 / pk8, blocks8 = (T + rb8 - 1) / rb8;
+        const int64_t rb8 = (8 / pk8) * 32, blocks8 = (T + rb8 - 1) / rb8;
         const int64_t last8 = T - (blocks8 - 1) * rb8, wg8 = blocks8 * (Hq / pk8) * sns;
         // (the last block filled like the others - 384 rows = a block and a half: 233 -> 286 us - and whole rounds of the
         // 256 CUs - 520 work-groups, 40 heads x 13 splits, are three rounds: 74 -> 80 us)
         if (10 * last8 >= 7 * rb8 && wg8 >= 256 && 100 * wg8 >= 85 * ((wg8 + 255) / 256 * 256)) PWs = 8;
     }
+    if (wide_pack) PWs = 8;
     if (const int64_t forced = ns_tune_get(NS_TUNE_PREFILL_WAVES); forced == 4 || forced == 8) PWs = (int) forced;
     if (kt == 2 && D == 128 && !widen) PWs = 4;                              // (a q4_0 tile of 128-value rows has chunks for 256 threads)
     const int64_t ROWS = rows_of((int) D, PWs);
@@ -1055,7 +1064,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     }
     p.pack = (int) pack_of(T, Hq / Hkv, D, PWs);
     p.gw = (int) (Hq / Hkv) / p.pack;
-    const int64_t RB = ROWS / p.pack;
+    const int64_t RB = (PWs / p.pack) * (ROWS / PWs);
     const int64_t units = ((T + RB - 1) / RB) * Hkv * p.ns;            // (split, row block, key head); padded to the 8 XCDs
     if ((units + 7) / 8 * 8 * p.gw >= (int64_t) 1 << 31) return ns_fail(w + ": too many work-groups");
     dim3 grid((unsigned) ((units + 7) / 8 * 8 * p.gw));

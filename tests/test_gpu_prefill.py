@@ -313,7 +313,12 @@ PACKED = [
     (64, 6, 1, 128, 2000, 0, 2, F32),           # q4_0 rows of 128 in the kernel's own staging, 2 heads
     (17, 12, 2, 256, 4000, 0, 0, F32),          # heads of 256: 17 rows fill two of four waves
     (5, 8, 2, 256, 1000, 0, 1, F16),            # ... 5 rows: 4 heads a work-group
-    (16, 10, 2, 128, 100, 0, 0, F32),           # G 5 has no power of two to share: one head a work-group
+    (16, 10, 2, 128, 100, 0, 0, F32),           # G 5: five heads to an 8-wave work-group, three waves without rows
+    (30, 20, 4, 128, 6000, 0, 3, BF16),         # ... behind key splits, bfloat16
+    (40, 14, 2, 128, 900, 0, 0, F16),           # G 7, two waves a head: no divisor fits - one head a work-group
+    (9, 14, 2, 256, 900, 0, 0, F16),            # G 7 at heads of 256: seven heads to 8 waves
+    (20, 6, 2, 128, 3000, 0, 1, F32),           # G 3: three heads to 4 waves
+    (33, 20, 2, 128, 2000, 100, 0, F32),        # G 10, two waves a head: 2 heads (4 waves); a window
     (40, 4, 1, 128, 0, 0, 0, F16),              # no context: the last rows' blocks see few keys
 ]
 
