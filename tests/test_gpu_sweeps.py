@@ -20,7 +20,7 @@ def test_prompt_sweep(ops, tune):
         D = int(rng.choice([128, 128, 256]))
         kt = int(rng.choice([0, 3, 1, 2]))
         Hkv = int(rng.integers(1, 3))
-        G = int(rng.choice([1, 2, 4, 5, 8, 10]))
+        G = int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 10]))
         Hq = Hkv * G
         T = int(rng.choice([rng.integers(17, 70), rng.integers(70, 300), rng.integers(300, 900)]))
         p0 = int(rng.choice([0, rng.integers(1, 100), rng.integers(100, 2500)]))
