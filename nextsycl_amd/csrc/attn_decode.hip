@@ -807,15 +807,17 @@ __global__ __launch_bounds__(256) void attn_merge_rows_kernel(const float* __res
 // is written and read again for every query row on it - T x G rows of D + 2 floats against the split's 2 kbs rows of
 // keys and values - so 16-bit caches whose key heads serve 8 or more query heads take half as many, twice as long
 // splits (G = 8, 64K keys, 4 rows: 30.9 -> 29.7 us; G = 16, 4 rows: 44.7 -> 40.5; one row: within 0.5 us either way);
-// quantized rows keep the two work-groups a CU their arithmetic needs (128K keys of q8_0: 35.0 against 37.8 us).
+// quantized rows keep the two work-groups a CU their arithmetic needs (128K keys of q8_0: 35.0 against 37.8 us) - but
+// for one or two key heads, whose 256 or 512 partials a query head cost the merge more than that (8 / 1 heads over
+// 131072 q8_0 keys: 21.9 -> 18.7 us, 16 / 2 heads 23.7 -> 22.3).
 // The rule may depend on the heads and the cache form, never on the rows of a pass. NS_DEC_WGS overrides (tuning)
-int64_t target_wgs(int64_t D, int64_t G, int kt) {
+int64_t target_wgs(int64_t D, int64_t G, int kt, int64_t Hkv) {
     const int64_t v = ns_tune_get(NS_TUNE_DEC_WGS);
-    return v > 0 ? v : D == 256 || (G >= 8 && (kt == 0 || kt == 3)) ? 256 : 512;
+    return v > 0 ? v : D == 256 || (G >= 8 && (kt == 0 || kt == 3)) || (kt == 1 && Hkv <= 2) ? 256 : 512;
 }
 // keys a split for a row that sees `keys` keys: a multiple of 128 (4 waves x 32-key tiles)
 int64_t dec_kbs(int64_t keys, int64_t Hkv, int64_t D, int64_t G, int kt) {
-    const int64_t t = target_wgs(D, G, kt), want = (keys * Hkv + t - 1) / t;
+    const int64_t t = target_wgs(D, G, kt, Hkv), want = (keys * Hkv + t - 1) / t;
     return std::max<int64_t>(128, (want + 127) / 128 * 128);
 }
 inline int64_t row_first(int64_t pos, int64_t win) { return win > 0 ? std::max<int64_t>(0, pos - win + 1) : 0; }
