@@ -677,9 +677,12 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
 // pieces) and the four sums are added as (0 + 1) + (2 + 3): a fixed shape, so the result does not depend on how many
 // empty splits a pass appends to a row's own (their weight is 0). Every wave works out all the weights itself (no
 // barrier before the sums), and its first 32 splits' values are requested before the weights exist.
-constexpr int MERGE_MAX_NS = 2048, MERGE_W = 4;
+// (MERGE_W waves: 4, or 8 for passes over one or two key heads, whose rows have 256 partials and more - chosen by the heads,
+// never by the rows or the splits of a pass, so a row is summed in the same shape whatever pass it is in: 8 / 1 heads over
+// 131072 keys, merge 6.1 -> 4.6 us)
+constexpr int MERGE_MAX_NS = 2048;
 
-template <int D>
+template <int D, int MERGE_W>
 __global__ __launch_bounds__(MERGE_W * 64) void attn_merge_kernel(const float* __restrict__ part, int ns, int qt, void* __restrict__ out) {
     constexpr int C = D / 128, PS = D + 2, PF = 32, B = 16;
     __shared__ float wsh[MERGE_W][MERGE_MAX_NS + MERGE_W * PF];
@@ -750,7 +753,12 @@ __global__ __launch_bounds__(MERGE_W * 64) void attn_merge_kernel(const float* _
 #pragma unroll
     for (int c = 0; c < C; ++c) {
         const float2 s0 = sums[0][c][lane], s1 = sums[1][c][lane], s2 = sums[2][c][lane], s3 = sums[3][c][lane];
-        const float ax = (s0.x + s1.x) + (s2.x + s3.x), ay = (s0.y + s1.y) + (s2.y + s3.y);
+        float ax = (s0.x + s1.x) + (s2.x + s3.x), ay = (s0.y + s1.y) + (s2.y + s3.y);
+        if constexpr (MERGE_W == 8) {
+            const float2 s4 = sums[4][c][lane], s5 = sums[5][c][lane], s6 = sums[6][c][lane], s7 = sums[7][c][lane];
+            ax += (s4.x + s5.x) + (s6.x + s7.x);
+            ay += (s4.y + s5.y) + (s6.y + s7.y);
+        }
         const float a = ls > 0.0f ? ax / ls : 0.0f, b = ls > 0.0f ? ay / ls : 0.0f;
         const int64_t i = rh * D + 2 * (lane + 64 * c);
         if (qt == 0) *reinterpret_cast<float2*>(reinterpret_cast<float*>(out) + i) = float2{a, b};
@@ -851,9 +859,10 @@ int launch_kt(ns_gpu* g, int kt, const DecodeParams& p, int rows, dim3 grid_xy) 
 }
 
 template <int D>
-int launch_merge(ns_gpu* g, const float* part, int ns, int qt, int64_t rh, void* out) {
+int launch_merge(ns_gpu* g, const float* part, int ns, int qt, int64_t rh, void* out, bool wide = false) {
     if (ns > MERGE_MAX_NS) return ns_fail("ns_attn_decode: more key splits than the merge holds");
-    attn_merge_kernel<D><<<(unsigned) rh, MERGE_W * 64, 0, g->q>>>(part, ns, qt, out);
+    if (wide) attn_merge_kernel<D, 8><<<(unsigned) rh, 8 * 64, 0, g->q>>>(part, ns, qt, out);
+    else attn_merge_kernel<D, 4><<<(unsigned) rh, 4 * 64, 0, g->q>>>(part, ns, qt, out);
     NS_LAUNCHED("attn_merge");
     return 0;
 }
@@ -904,7 +913,7 @@ int decode_typed(ns_gpu* g, int kt, int pm, const void* q, int64_t qs, const voi
         if (x.marks && ns_profile_mark(g, 0)) return -1;
         if (launch_kt<D>(g, kt, c, (int) (nr * c.G), dim3((unsigned) ns, (unsigned) Hkv))) return -1;
         if (x.marks && ns_profile_mark(g, 1)) return -1;
-        if (launch_merge<D>(g, c.part, (int) ns, QT, nr * Hq, (uint8_t*) out + r0 * Hq * D * esz)) return -1;
+        if (launch_merge<D>(g, c.part, (int) ns, QT, nr * Hq, (uint8_t*) out + r0 * Hq * D * esz, Hkv <= 2)) return -1;
         return x.marks ? ns_profile_mark(g, 2) : 0;
     };
     if (!causal) return launch(0, T, dec_kbs(last + 1 - first_of(0), Hkv, D, Hq / Hkv, kt));
@@ -1095,8 +1104,8 @@ int ns_attn_decode_static(ns_gpu* g, int qt, int kt, int pm, const void* q, int6
 int64_t ns_attn_decode_scratch(int64_t T, int64_t Hq, int64_t Hkv, int64_t D, int64_t p0, int64_t win) {
     if (T <= 0 || Hq <= 0 || Hkv <= 0) return 0;
     int64_t ns = 1;
-    // (the cache form is not an argument: the count holds for the 16-bit rule and the quantized one)
-    for (int kt = 0; kt < 2; ++kt) {
+    // (the cache form is not an argument: the count holds for the 16-bit rule, q8_0's and q4_0's)
+    for (int kt = 0; kt < 3; ++kt) {
         auto kbs = [&](int64_t keys) { return dec_kbs(keys, Hkv, D, Hq / Hkv, kt); };
         // a run of rows launched on its own: the row's own split size over its own first key to the pass's last
         // the pass in one launch: from its first row's first key to its last row's last; causal or not, the last row's

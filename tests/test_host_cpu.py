@@ -46,11 +46,9 @@ def test_pure_functions_without_a_gpu(handle):
     # one row, 32 / 8 heads, 4096 keys: splits of 128 -> 32 partials of D + 2 floats a head
     assert f(1, 32, 8, 128, 4095, 0) == 32 * 32 * 130
     assert f(0, 32, 8, 128, 4095, 0) == 0
-    # heads of 256 aim for half as many work-groups: 32768 keys x 2 heads in 256 splits of 256 keys -> 128 a head; so do
-    # heads of 128 with one or two key heads (16-bit rows of 8 query heads a key head, q8_0 rows of any) - with 4 key heads
-    # of 4 query heads each the quantized forms keep 512: 128 a head as well
-    assert f(1, 16, 2, 256, 32767, 0) == 16 * 128 * 258 and f(1, 16, 2, 128, 32767, 0) == 16 * 128 * 130
-    assert f(1, 16, 4, 128, 32767, 0) == 16 * 128 * 130 and f(1, 64, 4, 128, 32767, 0) == 64 * 128 * 130
+    # heads of 256 aim for half as many work-groups: 32768 keys x 2 heads in 256 splits of 256 keys -> 128 a head; heads of
+    # 128 are sized for the cache form that splits finest (q4_0 rows: 512 work-groups -> 256 a head)
+    assert f(1, 16, 2, 256, 32767, 0) == 16 * 128 * 258 and f(1, 16, 2, 128, 32767, 0) == 16 * 256 * 130
     # a verify pass needs at least its rows' own
     assert f(4, 32, 4, 128, 65536, 0) >= 4 * f(1, 32, 4, 128, 65536, 0)
     # a window bounds the splits whatever the position
