@@ -129,7 +129,8 @@ def test_mm3s_attend_block(ops, T, H, G, pos0, w0):
 
 
 @pytest.mark.parametrize("kt,Hq,Hkv,D,cap,n", [(0, 12, 2, 256, 3000, 2777), (1, 12, 2, 256, 900, 900), (2, 6, 1, 256, 500, 333),
-                                               (0, 32, 8, 128, 1500, 1499), (1, 8, 8, 128, 70, 1)])
+                                               (0, 32, 8, 128, 1500, 1499), (1, 8, 8, 128, 70, 1),
+                                               (3, 8, 2, 128, 41000, 40001), (0, 6, 1, 256, 17000, 16999)])   # a head's statistics over 4 and 2 key slices
 def test_q35_attn_probs(ops, kt, Hq, Hkv, D, cap, n):
     g = ops.gpu
     k = orc.randn(70 + kt, (cap, Hkv * D))
