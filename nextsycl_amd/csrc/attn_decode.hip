@@ -91,8 +91,12 @@ struct TileRegs {
     uint32_t vsc[DMA ? 1 : NLV];
 };
 
-template <int D, int RT, int KT>
+// QS (bfloat16 rows only): query rows that are not bfloat16 enter the first product as two bfloat16 numbers - the rounded
+// value and the rounded rest, 16 significant bits, as the weights enter the second - so a float32 or half row loses
+// nothing a half operand would keep (one bfloat16 number a feature cost such rows ~2e-3 of absolute error)
+template <int D, int RT, int KT, bool QS = false>
 __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kernel(const DecodeParams p) {
+    static_assert(!QS || KT == 3, "query rows in two parts: bfloat16 operands only");
     constexpr bool BF = KT == 3;
     using R = TileRegs<D, KT>;
     constexpr bool DMA = R::DMA;
@@ -337,7 +341,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
     // ---- this lane's rows (one per row tile): their key ranges and Q^T operands
     int lo_r[RT], hi_r[RT];     // the row's first and last key in this split, relative to the split's first (none: 1, 0)
     bool live_r[RT];
-    s8v qreg[RT][KB];
+    s8v qreg[RT][KB], qlo[QS ? RT : 1][KB];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         const int ri = (z * RT + rt) * 16 + n;
@@ -365,7 +369,11 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             for (int kb = 0; kb < KB; ++kb) {
                 const float f[8] = {raw[kb][0].x, raw[kb][0].y, raw[kb][0].z, raw[kb][0].w, raw[kb][1].x, raw[kb][1].y, raw[kb][1].z, raw[kb][1].w};
 #pragma unroll
-                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = live ? to16<BF>(f[i]) : (short) 0;
+                for (int i = 0; i < 8; ++i) {
+                    const short hi = to16<BF>(f[i]);
+                    qreg[rt][kb][i] = live ? hi : (short) 0;
+                    if constexpr (QS) qlo[rt][kb][i] = live ? to16<true>(f[i] - bf16_to_f32((uint16_t) hi)) : (short) 0;
+                }
             }
         } else {
             uint4 raw[KB];
@@ -380,6 +388,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                     // the same 16-bit type as the kernel's operands passes through; the other is converted
                     const short v = (p.qt == 2) == BF ? (short) b16 : to16<BF>(p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16));
                     qreg[rt][kb][i] = live ? v : (short) 0;
+                    if constexpr (QS) qlo[rt][kb][i] = live && p.qt == 1 ? to16<true>(f16_to_f32(b16) - bf16_to_f32((uint16_t) v)) : (short) 0;
                 }
             }
         }
@@ -455,7 +464,10 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                     for (int rt = 0; rt < RT; ++rt) {
                         f4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                        for (int kb = 0; kb < KB; ++kb) acc = mfma16<BF>(kall[kt2][kb], qreg[rt][kb], acc);
+                        for (int kb = 0; kb < KB; ++kb) {
+                            acc = mfma16<BF>(kall[kt2][kb], qreg[rt][kb], acc);
+                            if constexpr (QS) acc = mfma16<BF>(kall[kt2][kb], qlo[rt][kb], acc);
+                        }
                         s[rt][h0 + kt2] = acc;
                     }
             }
@@ -836,12 +848,22 @@ template <int D, int KT>
 int launch_rt(ns_gpu* g, const DecodeParams& p, int rows, dim3 grid_xy) {
     // (quantized rows of 256 as two row tiles take the whole register file - 512 with a few spilled - and still beat two
     // chunks that each lift and widen the tile: 24 / 4 heads x 4 rows behind 131072 q8_0 keys 110.8 -> 76.4 us, q4_0 106.4 -> 72.7)
-    const int RT = rows <= 16 ? 1 : 2;
+    // (rows of 256 in two bfloat16 parts stay one row tile a chunk: two tiles of them would spill a fifth of the kernel's registers)
+    const bool parts = KT == 3 && p.qt != 2;
+    const int RT = rows <= 16 || (parts && D == 256) ? 1 : 2;
     DecodeParams c = p;
     c.nz = (rows + RT * 16 - 1) / (RT * 16);
     const int64_t pairs = (int64_t) grid_xy.x * grid_xy.y, wgs = (pairs + 7) / 8 * 8 * c.nz;
     if (wgs >= (int64_t) 1 << 31) return ns_fail("ns_attn_decode: too many work-groups");
     const dim3 grid((unsigned) wgs);
+    if constexpr (KT == 3) {
+        if (parts) {
+            if (RT == 1) attn_decode_kernel<D, 1, KT, true><<<grid, WAVES * 64, 0, g->q>>>(c);
+            else if constexpr (D == 128) attn_decode_kernel<D, 2, KT, true><<<grid, WAVES * 64, 0, g->q>>>(c);
+            NS_LAUNCHED("attn_decode");
+            return 0;
+        }
+    }
     if (RT == 1) attn_decode_kernel<D, 1, KT><<<grid, WAVES * 64, 0, g->q>>>(c);
     else attn_decode_kernel<D, 2, KT><<<grid, WAVES * 64, 0, g->q>>>(c);
     NS_LAUNCHED("attn_decode");

@@ -96,7 +96,8 @@ def tolerances(ref64, qt=F32, kt=0, bf16_queries=False):
     roundoff u moves by up to u |v1 - v2| / 2 <= u |v|max, so the absolute bound 2e-3 can hold only while |out| < 4 (half).
     A bfloat16 rounding is 8 times coarser: each adds 2^-9 to the relative bound as well (a correctly rounded bfloat16
     copy of the exact result sits at ~1.6e-3 relative L2). bf16_queries: float32 / half query rows against a bfloat16
-    cache on a path that multiplies them as bfloat16 (they are rounded once to 8 bits for the first product)."""
+    cache on a prompt pass that keeps bfloat16 operands (they are rounded once to 8 bits for the first product; a decode
+    pass enters them as two bfloat16 numbers and takes no allowance)."""
     n_half = 1 + (kt in (1, 2)) + (qt == F16)
     n_bf16 = (qt == BF16) + (1 if bf16_queries else 0)
     big = float(np.abs(ref64).max())

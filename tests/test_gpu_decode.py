@@ -23,6 +23,9 @@ SMALL = [
     (1, 64, 4, 128, 5000, 0, 1, F16),      # q8_0, G 16
     (2, 12, 2, 128, 3000, 0, 2, F32),      # q4_0
     (3, 8, 2, 128, 4000, 0, 3, BF16),      # bfloat16 cache and rows
+    (2, 8, 2, 128, 166, 0, 3, F32),        # bfloat16 cache, float32 rows: the rows in two bfloat16 parts
+    (5, 16, 2, 128, 3000, 0, 3, F16),      # ... half rows, two row tiles
+    (1, 6, 1, 256, 700, 0, 3, F32),        # ... heads of 256
     (1, 12, 2, 256, 1500, 0, 0, F32),      # qwen35's head size, G 6
     (2, 12, 2, 256, 900, 0, 1, F32),       # ... with a q8_0 cache
     (2, 8, 2, 256, 700, 0, 2, F32),        # ... with a q4_0 cache
