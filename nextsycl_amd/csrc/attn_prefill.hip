@@ -78,11 +78,14 @@ typedef uint32_t u4v __attribute__((ext_vector_type(4)));
 // the same at an address that is only 8-byte aligned (q8_0 / q4_0 rows of 128 values are 136 / 72 bytes long)
 typedef uint32_t u4a8 __attribute__((ext_vector_type(4), aligned(8)));
 
-// BF: bfloat16 operands (a bfloat16 cache too long to be widened to half first), else half.
-template <int D, bool BF, int KT, int PW>
+// BF: bfloat16 operands (a bfloat16 cache too long to be widened to half first), else half. QS (bfloat16 operands only):
+// query rows of another type enter the first product as two bfloat16 numbers - the rounded row and the rounded rest, 16
+// significant bits between them - a second matrix instruction a key block.
+template <int D, bool BF, int KT, int PW, bool QS = false>
 __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_prefill_kernel(const PrefillParams p) {
     static_assert(D == 128 || D == 256, "head size 128 or 256");
     static_assert(KT == 0 || !BF, "quantized rows are widened to half");
+    static_assert(!QS || BF, "query rows in two parts: bfloat16 operands only");
     // a wave owns RT row tiles of 16: 32 rows at D = 128; 16 at D = 256, whose accumulators are twice as wide
     constexpr int RT = D == 128 ? 2 : 1, WROWS = RT * 16, ROWS = PW * WROWS;
     constexpr int KB = D / 32, DT = D / 16;
@@ -152,7 +155,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
 
     // ---- this lane's two rows: positions, key ranges, Q^T operands
     int64_t lo_r[RT], hi_r[RT];
-    s8v qreg[RT][KB];
+    s8v qreg[RT][KB], qlo[QS ? RT : 1][KB];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         const int row = wbase + rt * 16 + n;
@@ -173,7 +176,10 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
             for (int kb = 0; kb < KB; ++kb) {
                 const float f[8] = {raw[kb][0].x, raw[kb][0].y, raw[kb][0].z, raw[kb][0].w, raw[kb][1].x, raw[kb][1].y, raw[kb][1].z, raw[kb][1].w};
 #pragma unroll
-                for (int i = 0; i < 8; ++i) qreg[rt][kb][i] = to16<BF>(PRESCALE ? f[i] * p.sl2 : f[i]);
+                for (int i = 0; i < 8; ++i) {
+                    qreg[rt][kb][i] = to16<BF>(PRESCALE ? f[i] * p.sl2 : f[i]);
+                    if constexpr (QS) qlo[rt][kb][i] = to16<true>(f[i] - bf16_to_f32((uint16_t) qreg[rt][kb][i]));
+                }
             }
         } else {
             uint4 raw[KB];
@@ -189,6 +195,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                     // the row x the scale, rounded once
                     if constexpr (PRESCALE) qreg[rt][kb][i] = to16<BF>((p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16)) * p.sl2);
                     else qreg[rt][kb][i] = (p.qt == 2) == BF ? (short) b16 : to16<BF>(p.qt == 1 ? f16_to_f32(b16) : bf16_to_f32(b16));
+                    if constexpr (QS) qlo[rt][kb][i] = p.qt == 1 ? to16<true>(f16_to_f32(b16) - bf16_to_f32((uint16_t) qreg[rt][kb][i])) : (short) 0;
                 }
             }
         }
@@ -437,7 +444,10 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                 for (int kt2 = 0; kt2 < 2; ++kt2)
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt)
+                    {
                         s[rt][kt2] = mfma16<BF>(kpre[kt2][kb], qreg[rt][kb], kb == 0 ? ntile[rt] : s[rt][kt2]);
+                        if constexpr (QS) s[rt][kt2] = mfma16<BF>(kpre[kt2][kb], qlo[rt][kb], s[rt][kt2]);
+                    }
         } else {
 #pragma unroll
             for (int kt2 = 0; kt2 < 2; ++kt2) {
@@ -450,6 +460,10 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
                     f4v acc = mfma16<BF>(ka[0], qreg[rt][0], ntile[rt]);
 #pragma unroll
                     for (int kb = 1; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qreg[rt][kb], acc);
+                    if constexpr (QS) {
+#pragma unroll
+                        for (int kb = 0; kb < KB; ++kb) acc = mfma16<BF>(ka[kb], qlo[rt][kb], acc);
+                    }
                     s[rt][kt2] = acc;
                 }
             }
@@ -865,7 +879,8 @@ int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
     if (kt == 0) {
         attn_prefill_kernel<D, false, 0, PW><<<grid, TH, 0, g->q>>>(p);
     } else if (kt == 3) {
-        attn_prefill_kernel<D, true, 0, PW><<<grid, TH, 0, g->q>>>(p);
+        if (p.qt != 2) attn_prefill_kernel<D, true, 0, PW, true><<<grid, TH, 0, g->q>>>(p);
+        else attn_prefill_kernel<D, true, 0, PW><<<grid, TH, 0, g->q>>>(p);
     } else if (kt == 1) {
         attn_prefill_kernel<D, false, 1, PW><<<grid, TH, 0, g->q>>>(p);
     } else if constexpr (D == 256 || PW == 4) {

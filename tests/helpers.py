@@ -80,7 +80,7 @@ def gpu_prompt(ops, qt, kt, q_dev_arr, kc, vc, T, Hq, Hkv, D, cap, p0, win=0, pm
 U_HALF, U_BF16 = 2.0 ** -11, 2.0 ** -8      # unit roundoffs: half carries 11 significant bits, bfloat16 8
 
 
-def tolerances(ref64, qt=F32, kt=0, bf16_queries=False):
+def tolerances(ref64, qt=F32, kt=0):
     """The path's bar against the float64 closed form, as ONE rule for every cache form and row type.
 
     relative L2 <= 1e-3 and max-abs <= max(2e-3, sum of u |ref|max over the 16-bit roundings between the stored values
@@ -95,19 +95,18 @@ def tolerances(ref64, qt=F32, kt=0, bf16_queries=False):
     Why max-abs scales with |ref|max: an output that is the mean of two values v1, v2 under weights rounded with unit
     roundoff u moves by up to u |v1 - v2| / 2 <= u |v|max, so the absolute bound 2e-3 can hold only while |out| < 4 (half).
     A bfloat16 rounding is 8 times coarser: each adds 2^-9 to the relative bound as well (a correctly rounded bfloat16
-    copy of the exact result sits at ~1.6e-3 relative L2). bf16_queries: float32 / half query rows against a bfloat16
-    cache on a prompt pass that keeps bfloat16 operands (they are rounded once to 8 bits for the first product; a decode
-    pass enters them as two bfloat16 numbers and takes no allowance)."""
+    copy of the exact result sits at ~1.6e-3 relative L2). Float32 / half query rows against bfloat16 operands
+    enter the first product as two bfloat16 numbers (the rounded row and the rounded rest) and add no rounding of their own."""
     n_half = 1 + (kt in (1, 2)) + (qt == F16)
-    n_bf16 = (qt == BF16) + (1 if bf16_queries else 0)
+    n_bf16 = int(qt == BF16)
     big = float(np.abs(ref64).max())
     return max(MAX_ABS, (n_half * U_HALF + n_bf16 * U_BF16) * big), REL_L2 + n_bf16 * BF16_ROUND
 
 
-def check_close(got, ref64, qt=F32, what="", kt=0, bf16_queries=False):
+def check_close(got, ref64, qt=F32, what="", kt=0):
     """got against the float64 closed form under `tolerances`; returns (max-abs, relative L2)."""
     mx, rel, cos = orc.compare(got, ref64)
-    tol_abs, tol_rel = tolerances(ref64, qt, kt, bf16_queries)
+    tol_abs, tol_rel = tolerances(ref64, qt, kt)
     assert np.isfinite(got).all(), "%s: non-finite output" % what
     assert mx <= tol_abs and rel <= tol_rel, "%s: max-abs %.3g (<= %.3g), rel-L2 %.3g (<= %.3g), cosine %.6f" % (what, mx, tol_abs, rel, tol_rel, cos)
     return mx, rel

@@ -146,8 +146,8 @@ def test_prompt_that_keeps_bfloat16_operands(ops, tune):
     """A prompt pass over a bfloat16 cache whose rows do not fit the library's scratch keeps bfloat16 operands in both
     products (forced here by knob 5): its weights enter the second product as two bfloat16 numbers - the rounded weight and
     the rounded rest - so it meets the same bound as the widened pass over the same inputs, whose bfloat16 rows are the
-    rounding of its float32 rows. Query rows of another type are rounded to the cache's 8 bits for the first product
-    there (`bf16_queries`), which the widened pass avoids."""
+    rounding of its float32 rows. Query rows of another type enter the first product the same way, as two bfloat16
+    numbers: every row type under the plain bound."""
     T, Hq, Hkv, D, p0 = 600, 10, 2, 128, 400
     cap = p0 + T
     kc, vc = make_kv(3, Hkv, D, cap, cap, cfg=2)
@@ -181,4 +181,4 @@ def test_prompt_that_keeps_bfloat16_operands(ops, tune):
         got, _ = gpu_prompt(ops, qt, 3, qd, kc, vc, T, Hkv * G, Hkv, D, n + 2, p0, win=win)
         ref = orc.attn_f64(qf, kc, vc, 3, T, Hkv * G, Hkv, D, n + 2, p0, win=win)
         check_close(got, ref, qt, "bfloat16 operands, pass %d: T %d, heads %d / %d of %d, p0 %d, window %d, rows of type %d" % (it, T, Hkv * G, Hkv, D, p0, win, qt),
-                    kt=3, bf16_queries=qt != BF16)
+                    kt=3)
