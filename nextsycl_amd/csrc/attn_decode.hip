@@ -11,18 +11,21 @@
 // being independent) makes a row's arithmetic the same whatever rows share its pass - the verify invariant.
 //
 // A wave's tile step (32 keys), all in the transposed orientation so no row statistic ever crosses lanes through LDS:
-//   K:  global -> registers straight in MFMA A-operand layout (lane = key, 16 bytes of its row per k-block)
+//   K:  half / bfloat16 rows: global -> LDS directly, read back as the MFMA A operand (ds_read_b128: lane = key, 16
+//       bytes of its row per k-block); q8_0 rows and q4_0 rows of 256: the raw rows global -> LDS, lifted into registers
+//       and widened to half there; q4_0 rows of 128: global -> registers
 //   S^T[key][row] = K Q^T           v_mfma_f32_16x16x32 (rows padded to 16-row tiles; Q^T lives in registers)
 //   online softmax, base 2, float32: a lane holds 8 keys of one row; row max / sum = 8 in-lane + 2 xor-shuffles
 //   P^T -> 16 bit: it already IS the B operand of the next product (k-slot i of lane group g <-> key 4 g + i | 16 + 4 g + i)
 //   V:  half / bfloat16 rows: global -> LDS directly (global_load_lds_dwordx4, 1 KiB contiguous per instruction), the
 //       16-byte chunks of a row XOR-swizzled by the key so the transposing reads meet no bank conflicts; q8_0 / q4_0
-//       rows: global -> registers -> dequantized -> LDS [key][D] (rows padded by 32 bytes);
+//       rows: lifted as the keys are, widened to half in registers -> LDS [key][D] (rows padded by 32 bytes);
 //       then ds_read_b64_tr_b16 gives V^T in A-operand layout
 //   O^T[d][row] = O^T c + V^T P^T   v_mfma_f32_16x16x32, float32 accumulators in registers
-// The next tile's K (registers) and V (second LDS buffer) loads are issued before the current tile's math: ~16 KiB in
-// flight per wave, 8 waves a CU. The 4 waves' (O, m, l) are merged through LDS in a fixed order and written as the split's partial
-// {O[D], m (log2 units), l}; a second kernel merges the splits: out = sum O_s 2^(m_s - M) / sum l_s 2^(m_s - M).
+// The next tile's K and V loads are issued as soon as this tile's have been read out of their buffers: ~16 KiB in
+// flight per wave, 8 waves a CU. Float32 / half query rows over a bfloat16 cache enter the first product as two bfloat16
+// numbers (the rounded row and the rounded rest), the softmax weights the second product likewise. The 4 waves'
+// (O, m, l) are merged through LDS in a fixed order and written as the split's partial {O[D], m (log2 units), l}; a second kernel merges the splits: out = sum O_s 2^(m_s - M) / sum l_s 2^(m_s - M).
 //
 // Reference behaviour kept: kernels/llm/qwen35/silo/attn.cpp:100-104,261-290,321-370 (split form, partial layout,
 // merge, one launch when the rows' split sizes agree - here: a launch a run of rows whose sizes agree), kernels/llm/museglimmer/silo/attn.cpp:51-55,

@@ -14,6 +14,11 @@
 // leaving the newest tile's transfers in flight; the 4-wave form (two work-groups a CU) one tile ahead into two buffers a
 // stream, requested right behind the barrier that frees them. The other forms (quantized rows, D = 256) go global ->
 // registers two tiles ahead -> LDS one tile ahead: two register sets, two padded LDS buffers.
+// A pass of few rows packs several query heads of one key head into a work-group (a wave slot a head: the tile staged
+// once serves them all), and a pass of few rows over a long context is cut into key splits whose partials a merge
+// kernel puts together. bfloat16, q8_0 and q4_0 rows read many times are first widened to half rows in the library's
+// scratch (bit for bit the halfs the kernel would stage); the kernel's own forms of them serve short passes and caches
+// the scratch does not hold.
 //
 // A wave's tile step, in the transposed orientation (a lane owns one query row of each row tile, so the row maximum,
 // the rescale and the normalisation never leave the lane):
@@ -87,7 +92,7 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     static_assert(KT == 0 || !BF, "quantized rows are widened to half");
     static_assert(!QS || BF, "query rows in two parts: bfloat16 operands only");
     // a wave owns RT row tiles of 16: 32 rows at D = 128; 16 at D = 256, whose accumulators are twice as wide
-    constexpr int RT = D == 128 ? 2 : 1, WROWS = RT * 16, ROWS = PW * WROWS;
+    constexpr int RT = D == 128 ? 2 : 1, WROWS = RT * 16;
     constexpr int KB = D / 32, DT = D / 16;
     // Half operands: the query enters the first product scaled by the softmax scale x log2 e and rounded once to half - what
     // the reference's kernels do (qwen35/silo/attn.cpp:112,147: qh = half(q x qscale)) - and the product starts from minus

@@ -845,7 +845,7 @@ __global__ __launch_bounds__(256) void mla_vb_q6k_kernel(const float* __restrict
     float uv[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) uv[e] = u[th * ML + lane * 8 + e];
-    for (int r = blockIdx.y * 32 + w; r < blockIdx.y * 32 + 32; r += 4) {
+    for (int r = (int) blockIdx.y * 32 + w; r < (int) blockIdx.y * 32 + 32; r += 4) {
         float v[8];
         q6k_cols8(kvb + ((size_t) h * (NOPE + V) + NOPE + r) * ROWB, lane, v);
         float a = 0.0f;
