@@ -10,9 +10,8 @@
 // heads - a wave 16 of them (one 16-row MFMA tile: 72 registers of queries, 128 of accumulators), and a split of the
 // cells in 32-cell tiles; short passes of at most 128 rows run 4 waves = 64 pairs a work-group (mla_waves). Half rows go
 // global -> LDS directly two tiles ahead into three LDS buffers (the 4-wave form: three ahead into four), one barrier a
-// tile; GLM's q8 rows are fetched through
-// registers and widened to half on the way. The tile is shared by the work-group's waves. LDS
-// rows are 74 chunks of 16 bytes (72 of data, 2 of padding): rows 32 bytes apart modulo 256 spread both access patterns
+// tile; GLM's q8 rows are fetched through registers and widened to half on the way. The tile is shared by the
+// work-group's waves. LDS rows are 74 chunks of 16 bytes (72 of data, 2 of padding): rows 32 bytes apart modulo 256 spread both access patterns
 // over the banks - 16 rows x 16 bytes of one column (the score product's operand) and 8 rows x 32 bytes (the
 // transposing read); both measured at the full LDS rate, where rows a multiple of 128 bytes apart halve the first.
 //
@@ -21,8 +20,9 @@
 //   base-2 online softmax in float32 (scale folded in), causal edge masked per row
 //   P^T -> half = the B operand of the second product
 //   O^T[latent][row] += C^T P^T     A = the same tile through ds_read_b64_tr_b16; 128 float32 accumulators a lane
-// Each wave owns its rows outright, so a split's partial {O[L], m (log2 units), l} goes from registers to scratch
-// [row][split][L + 4]; the splits are merged by a second kernel.
+// Each wave owns its rows outright, so a split's partial {O[L] / l as halfs, m (log2 units), l} goes from registers
+// (through LDS, as 512-byte runs) to scratch [row][split]; the splits are merged by a second kernel, and a pass of one
+// split writes its rows' results itself.
 //
 // Reference behaviour kept: kernels/llm/deepseek2/ds2.cpp:139-258 (q~, scores over [latent | rope] x scale, online
 // softmax, u = sum p c / sum p, out = v_b u; L 512, R 64, nope = V = 128), :85-112 (cache rows), and
