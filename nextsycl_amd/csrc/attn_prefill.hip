@@ -413,9 +413,9 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
     // S^T of one 32-key half (LDS byte offset kl) against the wave's 32 rows: the raw dot products
     // (the operands of a block's first matrix instructions are read a block earlier - kread / vread - so that their LDS
     // latency passes under the other block's work instead of at the head of this one)
-    constexpr int VPRE = D == 128 ? DT : 4;                       // value operands read ahead
+    // (rows in two parts: the registers of half the value operands read ahead go to the rows' second part - no spills)
+    constexpr int VPRE = D == 128 && !QS ? DT : 4;                // value operands read ahead
     constexpr int KPRE = D == 128 ? 2 : 1;                        // 16-key halves whose key operands are read ahead
-    // (kl / vl: where the 32-key half starts - a pointer into the tile buffers)
     auto kread = [&](s8v (&ka)[KPRE][KB], const lds_u8* kl) __attribute__((always_inline)) {
 #pragma unroll
         for (int kt2 = 0; kt2 < KPRE; ++kt2)
@@ -986,11 +986,15 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // (what widening costs is read once a key; a pass of few rows reads a key only once a row block and query head of its
     // group: up to 128 rows x 4 heads over bfloat16 rows of 128 - 8 heads over rows of 256 - and up to 256 x 4 over q4_0
     // rows of 128 the kernel's own staging is the shorter way - 32768 keys behind 64 rows, 8 key heads: 108 against 121 us,
-    // q4_0 86 against 106; q8_0 rows are widened always: 123 against 112. Query rows that are not bfloat16 would be rounded
-    // to it for a bfloat16 first product: their passes widen. Knob 5: 1 keeps the rows' form, 2 widens.)
+    // q4_0 86 against 106; q8_0 rows are widened always: 123 against 112. Query rows that are not bfloat16 enter a bfloat16
+    // first product in two parts, twice its matrix instructions: the own form then pays up to 2 D rows a key head - 64
+    // float32 rows x 32 / 8 heads behind 32768 keys 84 against 107 us, 17 rows behind 131072 keys 164 against 333; 128 rows
+    // x 32 / 8 heads 122 against 120. Behind fewer than 4096 keys the widening costs next to nothing and its pass is the
+    // shorter (17 rows x 8 / 8 heads behind 2048 keys: 35 against 38 us). Knob 5: 1 keeps the rows' form, 2 widens.)
     const int64_t key_reads = ((T + 127) / 128) * (Hq / Hkv);
     const bool own_form = ns_tune_get(NS_TUNE_PREFILL_BF16) == 1 ||
-                          (ns_tune_get(NS_TUNE_PREFILL_BF16) == 0 && (kt == 3 ? qt == 2 && key_reads <= D / 32 : kt == 2 && D == 128 && key_reads <= 8));
+                          (ns_tune_get(NS_TUNE_PREFILL_BF16) == 0 &&
+                           (kt == 3 ? wn >= 4096 && key_reads <= D / 32 && (qt == 2 || T * (Hq / Hkv) <= 2 * D) : kt == 2 && D == 128 && key_reads <= 8));
     const bool widen = kt != 0 && !own_form && part_bytes + 2 * wone <= ns_own_floats(g) * 4 && wn * D * 2 < (int64_t) 1 << 32;
     int PWs = D == 128 ? (sns == 1 && ((T + 255) / 256) * Hq >= 512 ? 8 : 4) : (T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
     // (a pass cut into key splits takes 8 waves after all where its rows - some heads of them to a work-group - fill

@@ -370,7 +370,7 @@ def test_prefill_over_the_caches_own_form(ops, tune, T, Hq, Hkv, D, p0, win, kt,
     own, _ = gpu_prompt(ops, qt, kt, qd, kc, vc, T, Hq, Hkv, D, cap, p0, win=win)
     ref = orc.attn_f64(qf, kc, vc, kt, T, Hq, Hkv, D, cap, p0, win=win)
     check_close(wide, ref, qt, "prefill, rows widened first", kt=kt)
-    # (bfloat16 operands: query rows of another type are rounded to bfloat16 on their way into the first product)
+    # (bfloat16 operands: query rows of another type enter the first product as two bfloat16 numbers - the same bound)
     check_close(own, ref, qt, "prefill, the cache's own form in the kernel", kt=kt)
     if kt in (1, 2) and not (kt == 2 and D == 128):
         assert np.array_equal(np.asarray(wide).view(np.uint8), np.asarray(own).view(np.uint8))
