@@ -878,6 +878,30 @@ int64_t pack_of(int64_t T, int64_t G, int64_t D, int64_t PW) {
     return pack;
 }
 
+// Whether a pass over rows that are not half keeps their form in the kernel instead of widening them to half rows first
+// (knob 5 = 0: the measured rule). What widening costs is read and written once a key; a pass of few rows reads a key
+// only once a row block and query head of its group, and the kernel's own staging of it is then the shorter way. T rows x
+// G heads a key head behind `keys` keys, float32 query rows, widened / own form in us:
+//   bfloat16 (bfloat16 query rows up to 128 rows x D / 32 heads; rows of another type, which enter the first product in
+//     two parts - twice its matrix instructions - up to 2 D rows a key head; behind fewer than 4096 keys the widening
+//     costs next to nothing and its pass is the shorter): 64 x 4 of 128 behind 32768 keys 107 / 84, 17 x 4 behind 131072
+//     333 / 164, 128 x 4 behind 32768 120 / 122; 17 bfloat16 rows x 1 behind 2048 35 / 38
+//   q8_0 rows of 128 behind 32768 keys and more, up to 8 reads a key: 17 x 4 behind 131072 294 / 158, 128 x 4 behind
+//     32768 111 / 86, 64 x 4 behind 8192 42 / 54; 17 x 16 behind 131072 217 / 215. Rows of 256: widened (17 x 8 behind
+//     32768 76 / 95)
+//   q4_0 rows of 128 up to 1024 rows a key head: 64 x 4 behind 32768 92 / 67, 17 x 16 behind 131072 214 / 157, 128 x 16
+//     behind 32768 143 / 148. Rows of 256 behind 32768 keys and more, past 32 rows, up to 8 reads a key: 64 x 8 behind
+//     131072 232 / 187, 17 x 8 there 230 / 246
+bool own_form_pays(int kt, int qt, int64_t D, int64_t T, int64_t G, int64_t keys) {
+    const int64_t key_reads = ((T + 127) / 128) * G;
+    switch (kt) {
+        case 3: return keys >= 4096 && key_reads <= D / 32 && (qt == 2 || T * G <= 2 * D);
+        case 1: return D == 128 && keys >= 32768 && key_reads <= 8;
+        case 2: return D == 128 ? T * G <= 1024 : keys >= 32768 && T > 32 && key_reads <= 8;
+        default: return false;
+    }
+}
+
 template <int D, int PW>
 int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
     constexpr int TH = PW * 64;
@@ -983,18 +1007,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     const int64_t wkf = kfirst >= 0 ? kfirst : win > 0 ? std::max<int64_t>(0, p0 + 1 - win) : 0, wn = p0 + T - wkf;
     const size_t part_bytes = sns > 1 ? ((size_t) (T * Hq * sns * (D + 2)) * 4 + 255) / 256 * 256 : 0;
     const size_t wone = (size_t) (Hkv * wn * D * 2);
-    // (what widening costs is read once a key; a pass of few rows reads a key only once a row block and query head of its
-    // group: up to 128 rows x 4 heads over bfloat16 rows of 128 - 8 heads over rows of 256 - and up to 256 x 4 over q4_0
-    // rows of 128 the kernel's own staging is the shorter way - 32768 keys behind 64 rows, 8 key heads: 108 against 121 us,
-    // q4_0 86 against 106; q8_0 rows are widened always: 123 against 112. Query rows that are not bfloat16 enter a bfloat16
-    // first product in two parts, twice its matrix instructions: the own form then pays up to 2 D rows a key head - 64
-    // float32 rows x 32 / 8 heads behind 32768 keys 84 against 107 us, 17 rows behind 131072 keys 164 against 333; 128 rows
-    // x 32 / 8 heads 122 against 120. Behind fewer than 4096 keys the widening costs next to nothing and its pass is the
-    // shorter (17 rows x 8 / 8 heads behind 2048 keys: 35 against 38 us). Knob 5: 1 keeps the rows' form, 2 widens.)
-    const int64_t key_reads = ((T + 127) / 128) * (Hq / Hkv);
-    const bool own_form = ns_tune_get(NS_TUNE_PREFILL_BF16) == 1 ||
-                          (ns_tune_get(NS_TUNE_PREFILL_BF16) == 0 &&
-                           (kt == 3 ? wn >= 4096 && key_reads <= D / 32 && (qt == 2 || T * (Hq / Hkv) <= 2 * D) : kt == 2 && D == 128 && key_reads <= 8));
+    const bool own_form = ns_tune_get(NS_TUNE_PREFILL_BF16) == 1 || (ns_tune_get(NS_TUNE_PREFILL_BF16) == 0 && own_form_pays(kt, qt, D, T, Hq / Hkv, wn));
     const bool widen = kt != 0 && !own_form && part_bytes + 2 * wone <= ns_own_floats(g) * 4 && wn * D * 2 < (int64_t) 1 << 32;
     int PWs = D == 128 ? (sns == 1 && ((T + 255) / 256) * Hq >= 512 ? 8 : 4) : (T > 64 && ((T + 127) / 128) * Hq * sns >= 128 ? 8 : 4);
     // (a pass cut into key splits takes 8 waves after all where its rows - some heads of them to a work-group - fill
