@@ -950,7 +950,10 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // 5 or 7 heads - with 8
     const int64_t pk4 = pack_of(T, Hq / Hkv, D, 4), pk8 = pack_of(T, Hq / Hkv, D, 8);
     const bool wide_pack = pk8 > 2 * pk4 && (pk4 == 1 || p0 + T >= 8192);     // (a group that shares with 4 waves too: only behind a long context)
-    const int64_t pkp = wide_pack ? pk8 : pk4;
+    // (heads of 256, up to 64 rows behind a long context: 8 waves - twice the heads a work-group, and one work-group a CU
+    // is all its LDS admits - 17 rows x 16 / 2 heads behind 131072 keys 130 -> 92 us)
+    const bool long256 = D == 256 && T <= 64 && p0 + T >= 16384;
+    const int64_t pkp = wide_pack || long256 ? pk8 : pk4;
     // Key splits. A pass of few rows over a long context - a chunk of a prompt behind 32K tokens, a long draft block - has
     // too few (row block, head) pairs to fill the chip, each walking every key: its keys are cut into ns splits of whole
     // tiles, a work-group a (row block, head, split), the partials merged by the decode path's merge kernel. ns is
@@ -970,9 +973,18 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
         // hold one head's few rows, three waves of four idle: 17 rows x 40 / 8 heads behind 8192 keys 42 us in 8 splits, 49 in 13)
         const bool filled = pkp > 1 || T > (D == 128 ? 64 : 32);      // (rows for three of 4 waves of 32 rows, or of 16)
         const int64_t root = keys < 512 ? 1 : (int64_t) (0.177 * std::sqrt((double) keys));
-        const int64_t by_keys = p0 < 2 * T || !filled || pairs > 64 ? keys / 1024 : pairs < 32 ? root : std::max(keys / 1024, root / 2);
+        // (few pairs: at least the splits that give every CU a work-group, down to a tile or 2 T keys a split - the partials
+        // grow with the rows - 17 rows x 8 / 1 heads behind 32768 keys in 32 splits 30.0 us, in 128 20.3; 32 / 8 heads behind
+        // 8192 keys in 16 24.7, in 32 21.3; 17 rows x 4 / 4 heads, a head's few rows a work-group, behind 8192 keys in 8
+        // 32.4, in 64 15.4. Heads of 256 - one work-group a CU - take exactly those: 40 rows x 16 / 2 heads behind 131072
+        // keys in 32 splits 163 us, in 64 175)
+        const int64_t fill = keys < 512 ? 1 : std::min<int64_t>((256 + pairs - 1) / pairs, keys / std::max<int64_t>(KT_TILE, 2 * T));
+        const int64_t by_keys = p0 < 2 * T || pairs > 64 ? keys / 1024
+                                : pairs < 32         ? (D == 256 ? std::max<int64_t>(fill, 1) : std::max(root, fill))
+                                : !filled            ? keys / 1024
+                                                     : std::max(keys / 1024, root / 2);
         const int64_t aim = 512;
-        int64_t ns = std::min<int64_t>({(aim + pairs - 1) / pairs, by_keys, 64,
+        int64_t ns = std::min<int64_t>({(aim + pairs - 1) / pairs, by_keys, 128,
                                         (int64_t) (ns_own_floats(g) / (size_t) (T * Hq * (D + 2)))});
         // (a pass the context dominates - equal work-groups - whose count would fill the chip's 512 places unevenly, say 640:
         // cut further, to about two and a half rounds. 1024 rows x 40 heads behind 32768 keys: 740 -> 652 us; 2048 rows: 1467 -> 1280)
@@ -984,10 +996,10 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
             if (ns > 1 && wg > slots && wg <= 2 * slots && 100 * wg < 85 * ((wg + slots - 1) / slots * slots)) ns = std::max<int64_t>(1, slots / pairs);
         }
         if (p0 >= T && keys / 1024 >= 2) {
-            const int64_t n0 = std::max<int64_t>(ns, 1), wg = pairs * n0;
-            if ((double) wg / (double) ((wg + 511) / 512 * 512) < 0.85) {
+            const int64_t slots = D == 128 ? 512 : 256, n0 = std::max<int64_t>(ns, 1), wg = pairs * n0;
+            if ((double) wg / (double) ((wg + slots - 1) / slots * slots) < 0.85) {
                 const int64_t cap_ns = std::min<int64_t>({keys / 1024, 64, (int64_t) (ns_own_floats(g) / (size_t) (T * Hq * (D + 2)))});
-                ns = std::max(ns, std::min<int64_t>((1280 + pairs - 1) / pairs, cap_ns));
+                ns = std::max(ns, std::min<int64_t>((5 * slots / 2 + pairs - 1) / pairs, cap_ns));
             }
         }
         // (a forced count - tests - stays within what the scratch and the merge kernel hold)
@@ -1015,7 +1027,7 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     // heads behind 32768 keys 142 -> 131 us, 256 rows 260 -> 240; x 32 / 8 heads 192 rows 141 -> 130)
     // (heads of 256: 33 - 64 rows behind a long context - 128 rows of two heads to an 8-wave work-group, one staging of the
     // keys for both - 16 / 2 heads behind 32768 keys 92 -> 70 us, 32 / 8 heads 131 -> 94; behind 8192 keys the 4-wave form)
-    if (D == 256 && T > 32 && T <= 64 && sns > 1 && p0 + T >= 16384) PWs = 8;
+    if (long256 && sns > 1) PWs = 8;
     if (D == 128 && sns > 1 && T >= 96) {
         const int64_t rb8 = (8 / pk8) * 32, blocks8 = (T + rb8 - 1) / rb8;
         const int64_t last8 = T - (blocks8 - 1) * rb8, wg8 = blocks8 * (Hq / pk8) * sns;
