@@ -887,17 +887,18 @@ int64_t pack_of(int64_t T, int64_t G, int64_t D, int64_t PW) {
 //     costs next to nothing and its pass is the shorter): 64 x 4 of 128 behind 32768 keys 107 / 84, 17 x 4 behind 131072
 //     333 / 164, 128 x 4 behind 32768 120 / 122; 17 bfloat16 rows x 1 behind 2048 35 / 38
 //   q8_0 rows of 128 behind 32768 keys and more, up to 8 reads a key: 17 x 4 behind 131072 294 / 158, 128 x 4 behind
-//     32768 111 / 86, 64 x 4 behind 8192 42 / 54; 17 x 16 behind 131072 217 / 215. Rows of 256: widened (17 x 8 behind
-//     32768 76 / 95)
+//     32768 111 / 86, 64 x 4 behind 8192 42 / 54; 17 x 16 behind 131072 217 / 215. Rows of 256 behind 65536 keys and
+//     more, up to 256 rows a key head: 17 x 4 behind 131072 130 / 86, 32 x 8 154 / 139, 64 x 8 220 / 240; 17 x 8 behind
+//     32768 54 / 62
 //   q4_0 rows of 128 up to 1024 rows a key head: 64 x 4 behind 32768 92 / 67, 17 x 16 behind 131072 214 / 157, 128 x 16
-//     behind 32768 143 / 148. Rows of 256 behind 32768 keys and more, past 32 rows, up to 8 reads a key: 64 x 8 behind
-//     131072 232 / 187, 17 x 8 there 230 / 246
+//     behind 32768 143 / 148. Rows of 256 behind 32768 keys and more, up to 8 reads a key: 64 x 8 behind 131072 217 /
+//     176, 17 x 8 there 147 / 95, 17 x 8 behind 8192 36 / 43
 bool own_form_pays(int kt, int qt, int64_t D, int64_t T, int64_t G, int64_t keys) {
     const int64_t key_reads = ((T + 127) / 128) * G;
     switch (kt) {
         case 3: return keys >= 4096 && key_reads <= D / 32 && (qt == 2 || T * G <= 2 * D);
-        case 1: return D == 128 && keys >= 32768 && key_reads <= 8;
-        case 2: return D == 128 ? T * G <= 1024 : keys >= 32768 && T > 32 && key_reads <= 8;
+        case 1: return D == 128 ? keys >= 32768 && key_reads <= 8 : keys >= 65536 && T * G <= 256;
+        case 2: return D == 128 ? T * G <= 1024 : keys >= 32768 && key_reads <= 8;
         default: return false;
     }
 }
