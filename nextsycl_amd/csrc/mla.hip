@@ -1003,10 +1003,28 @@ int64_t mla_target_wgs() {
     const int64_t v = ns_tune_get(NS_TUNE_MLA_WGS);
     return v > 0 ? v : 256;
 }
-// cells a split: ~mla_target_wgs() work-groups over the pass, whole 32-cell tiles, at least 2 tiles
+// cells a split: ~mla_target_wgs() work-groups over the pass, whole 32-cell tiles, at least 2 tiles. A CU holds one
+// work-group and a split's row groups sit on one XCD (an eighth of the places), splits dealt round the XCDs: 3 row groups
+// x 86 splits are 11 splits = 33 work-groups an XCD with 32 places - two rounds, the second all but empty, and a round
+// that is nearly empty costs as much as a full one. Where the rule's count fills its rounds to less than 85 % the count is
+// chosen by cost instead: in units of a tile step a work-group costs its tiles + 5 (its queries, its first tile's latency,
+// its partials' stores) and the merge 0.032 a partial of a row group; the count whose rounds and merge add up to the least
 int64_t mla_kbs(int64_t cells, int64_t groups) {
     const int64_t t = mla_target_wgs(), want = (cells * groups + t - 1) / t;
-    return std::max<int64_t>(2 * MTILE, (want + MTILE - 1) / MTILE * MTILE);
+    const int64_t kbs = std::max<int64_t>(2 * MTILE, (want + MTILE - 1) / MTILE * MTILE), ns0 = (cells + kbs - 1) / kbs;
+    // (rounds: fewer than 8 splits deal their row groups over the whole chip)
+    auto rounds_of = [&](int64_t ns) { return ns < 8 || t < 8 ? (ns * groups + t - 1) / t : ((ns + 7) / 8 * groups + t / 8 - 1) / (t / 8); };
+    if (100 * ns0 * groups >= 85 * rounds_of(ns0) * t || ns0 * groups <= t / 2) return kbs;
+    const int64_t tiles = (cells + MTILE - 1) / MTILE, most = std::max<int64_t>(1, std::min<int64_t>(tiles / 2, 4 * t));
+    int64_t best = 1;
+    double cost = 0.0;
+    for (int64_t ns = 1; ns <= most; ++ns) {
+        const int64_t len = (tiles + ns - 1) / ns;
+        const double c = (double) (rounds_of(ns) * (len + 5)) + 0.032 * (double) (groups * ns);
+        if (ns == 1 || c < cost) best = ns, cost = c;
+    }
+    const int64_t per = (cells + best - 1) / best;
+    return std::max<int64_t>(2 * MTILE, (per + MTILE - 1) / MTILE * MTILE);
 }
 
 int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const void* qa, const void* cache, void* u, int64_t T, int64_t H,
@@ -1102,10 +1120,13 @@ extern "C" {
 // later ones masked), so a pass is 128 rows (behind a short context the masked work is small in absolute terms and a
 // pass costs its two launches), 256 = MLA_PASS_MAX once the masked part stays under a quarter. The scratch is
 // the largest pass's.
-static int64_t mla_pass_rows(int64_t before, int64_t left) {
+// (17 to 27 row groups of 128 (row, head) pairs fill an XCD's 32 places once and little more: behind 4096 cells and more
+// such a pass is cut at 16 groups - 17 rows x 128 heads behind 32768 cells: 274 us as one pass, 152 + 27 as two)
+static int64_t mla_pass_rows(int64_t before, int64_t left, int64_t H) {
     int64_t w = 128;
     while (w < MLA_PASS_MAX && 8 * w <= before) w *= 2;
-    return std::min(w, left);
+    const int64_t n = std::min(w, left), groups = (n * H + 127) / 128;
+    return before >= 4096 && groups >= 17 && groups <= 27 && 16 * 128 / H >= 1 ? std::min<int64_t>(n, 16 * 128 / H) : n;
 }
 static int64_t mla_pass_scratch(int64_t T, int64_t H, int64_t pos0) {
     const int64_t rows = T * H, cells = pos0 + T, MROWS = mla_waves(rows, cells) * 16, nz = (rows + MROWS - 1) / MROWS, kbs = mla_kbs(cells, nz);
@@ -1117,7 +1138,7 @@ int64_t ns_mla_decode_latent_scratch(int64_t T, int64_t H, int64_t pos0) {
     if (T <= 16) return mla_pass_scratch(T, H, pos0);
     int64_t need = 0;
     for (int64_t t0 = 0, n; t0 < T; t0 += n) {
-        n = mla_pass_rows(pos0 + t0, T - t0);
+        n = mla_pass_rows(pos0 + t0, T - t0, H);
         need = std::max(need, mla_pass_scratch(n, H, pos0 + t0));
     }
     return need;
@@ -1133,7 +1154,7 @@ int ns_mla_decode_latent(ns_gpu* g, int qt, const void* qa, const uint16_t* cach
     if (!qa || !u) return ns_fail("ns_mla_decode_latent: a null buffer");
     const int64_t e = qt == 0 ? 4 : 2;
     for (int64_t t0 = 0, n; t0 < T; t0 += n) {
-        n = T <= 16 ? T : mla_pass_rows(pos0 + t0, T - t0);
+        n = T <= 16 ? T : mla_pass_rows(pos0 + t0, T - t0, H);
         if (mla_latent(g, "ns_mla_decode_latent", qt, qt, (int) R, false, (const char*) qa + t0 * H * (ML + R) * e, cache, (char*) u + t0 * H * ML * e, n, H,
                        pos0 + t0, scale, scratch, (size_t) mla_pass_scratch(n, H, pos0 + t0)))
             return -1;
@@ -1225,7 +1246,7 @@ static int mla_sel_rows(ns_gpu* g, const char* who, bool q8, const float* qa, co
     if (H <= 0 || pos0 < 0) return ns_fail(std::string(who) + ": heads and a position");
     if (!qa || !u) return ns_fail(std::string(who) + ": a null buffer");
     for (int64_t t0 = 0, n; t0 < T; t0 += n) {
-        n = T <= 16 ? T : sel_cnt ? std::min<int64_t>(16, T - t0) : mla_pass_rows(pos0 + t0, T - t0);
+        n = T <= 16 ? T : sel_cnt ? std::min<int64_t>(16, T - t0) : mla_pass_rows(pos0 + t0, T - t0, H);
         if (mla_latent(g, who, 0, 0, 0, q8, qa + t0 * H * LW, c, u + t0 * H * LW, n, H, pos0 + t0, scale, scratch, scratch_floats,
                        sel_cnt ? sel + t0 * K : nullptr, sel_cnt ? sel_cnt + t0 : nullptr, K, LW))
             return -1;

@@ -44,7 +44,9 @@ def test_latent_decode_small(ops, T, H, R, pos0, qt):
         _close(orc.mla_decode_u(qf, cache, T, H, pos0, scale), ref, "the restatement itself")
 
 
-@pytest.mark.parametrize("T,H,pos0,qt", [(1, 16, 49999, F32), (2, 32, 100000, F16), (1, 16, 131071, F16), (1, 16, 131072, F32)])
+@pytest.mark.parametrize("T,H,pos0,qt", [(1, 16, 49999, F32), (2, 32, 100000, F16), (1, 16, 131071, F16), (1, 16, 131072, F32),
+                                         # 3 and 5 row groups: split counts chosen so that an XCD's places take whole splits
+                                         (5, 64, 12000, F32), (5, 128, 6000, F16)])
 def test_latent_decode_long_contexts(ops, T, H, pos0, qt):
     """One or two rows behind long contexts: the passes either side of the cell count at which the kernel's 64-row form
     gives way to the 128-row one, many tiles a split."""
@@ -81,11 +83,14 @@ def test_latent_decode_seeded_shapes(ops, T, H, R, pos0, qt):
 
 
 @pytest.mark.parametrize("T,H,R,pos0,qt", [(40, 16, 64, 100, F16), (33, 128, 64, 0, F32), (17, 8, 0, 2000, F32), (64, 20, 64, 37, F16),
-                                            (300, 16, 64, 250, F16), (1100, 8, 64, 0, F32), (70, 16, 0, 5000, F32), (300, 4, 64, 1900, F16)])
+                                            (300, 16, 64, 250, F16), (1100, 8, 64, 0, F32), (70, 16, 0, 5000, F32), (300, 4, 64, 1900, F16),
+                                            # 20 and 23 row groups behind 4096 cells and more: cut at 16 groups, the rest a pass of its own
+                                            (20, 128, 64, 4500, F16), (45, 64, 0, 6000, F32)])
 def test_latent_prompt_widths(ops, T, H, R, pos0, qt):
     """A prompt's rows through the same entry point (the reference's GEMM chain + masked softmax over these rows:
     llm/deepseek2/src/engine.rs:1165-1253): row t over cells 0 .. pos0 + t, against the float64 closed form. The passes
-    are 128 rows, 256 behind long enough contexts: the cases cross both widths."""
+    are 128 rows, 256 behind long enough contexts, and end at 16 row groups where 17 to 27 would follow: the cases cross
+    all of these."""
     n = pos0 + T
     cache = orc.f2h(orc.randn(9, (n, 512 + R), 0.5))
     qa = orc.randn(10, (T, H, 512 + R))
