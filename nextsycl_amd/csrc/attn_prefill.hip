@@ -997,10 +997,20 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
             if (ns > 1 && wg > slots && wg <= 2 * slots && 100 * wg < 85 * ((wg + slots - 1) / slots * slots)) ns = std::max<int64_t>(1, slots / pairs);
         }
         if (p0 >= T && keys / 1024 >= 2) {
-            const int64_t slots = D == 128 ? 512 : 256, n0 = std::max<int64_t>(ns, 1), wg = pairs * n0;
-            if ((double) wg / (double) ((wg + slots - 1) / slots * slots) < 0.85) {
-                const int64_t cap_ns = std::min<int64_t>({keys / 1024, 64, (int64_t) (ns_own_floats(g) / (size_t) (T * Hq * (D + 2)))});
-                ns = std::max(ns, std::min<int64_t>((5 * slots / 2 + pairs - 1) / pairs, cap_ns));
+            const int64_t slots = D == 128 ? 512 : 256;
+            const int64_t cap_ns = std::min<int64_t>({keys / 1024, 64, (int64_t) (ns_own_floats(g) / (size_t) (T * Hq * (D + 2)))});
+            auto fill_of = [&](int64_t n) { const int64_t w = pairs * n; return (double) w / (double) ((w + slots - 1) / slots * slots); };
+            if (fill_of(std::max<int64_t>(ns, 1)) < 0.85) ns = std::max(ns, std::min<int64_t>((5 * slots / 2 + pairs - 1) / pairs, cap_ns));
+            // (and from there the count - up to three more - whose rounds are fullest, a split more charged what its
+            // partials cost against the pass, 620 / keys: 5000 rows x 32 heads behind 32768 keys are 1280 work-groups, two
+            // rounds and a half; in two splits five whole ones: 2657 -> 2505 us, x 40 heads 3613 -> 3178)
+            const int64_t from = std::max<int64_t>(ns, 1);
+            if (p0 >= 2 * T && fill_of(from) < 0.92) {      // (behind less than two passes' keys the diagonal makes the work-groups unequal)
+                double best = 0.0;
+                for (int64_t n = from; n <= std::min(from + 3, std::max(cap_ns, from)); ++n) {
+                    const double fill = fill_of(n) - 620.0 / (double) keys * (double) (n - from);
+                    if (n == from || fill > best + 0.02) best = fill, ns = n;
+                }
             }
         }
         // (a forced count - tests - stays within what the scratch and the merge kernel hold)
