@@ -1009,12 +1009,15 @@ int64_t mla_target_wgs() {
 // that is nearly empty costs as much as a full one. Where the rule's count fills its rounds to less than 85 % the count is
 // chosen by cost instead: in units of a tile step a work-group costs its tiles + 5 (its queries, its first tile's latency,
 // its partials' stores) and the merge 0.032 a partial of a row group; the count whose rounds and merge add up to the least
-int64_t mla_kbs(int64_t cells, int64_t groups) {
+int64_t mla_kbs(int64_t cells, int64_t groups, bool lists = false) {
     const int64_t t = mla_target_wgs(), want = (cells * groups + t - 1) / t;
     const int64_t kbs = std::max<int64_t>(2 * MTILE, (want + MTILE - 1) / MTILE * MTILE), ns0 = (cells + kbs - 1) / kbs;
     // (rounds: fewer than 8 splits deal their row groups over the whole chip)
     auto rounds_of = [&](int64_t ns) { return ns < 8 || t < 8 ? (ns * groups + t - 1) / t : ((ns + 7) / 8 * groups + t / 8 - 1) / (t / 8); };
-    if (100 * ns0 * groups >= 85 * rounds_of(ns0) * t || ns0 * groups <= t / 2) return kbs;
+    // (rows with cell lists of their own, splits of fewer than 12 tiles: mostly their fixed cost, and a second round's few
+    // work-groups run beside the first's last - the plain rule stands: 12 rows' 2051 listed cells x 128 heads 48 us, by
+    // cost 54)
+    if (100 * ns0 * groups >= 85 * rounds_of(ns0) * t || ns0 * groups <= t / 2 || (lists && kbs < 12 * MTILE)) return kbs;
     const int64_t tiles = (cells + MTILE - 1) / MTILE, most = std::max<int64_t>(1, std::min<int64_t>(tiles / 2, 4 * t));
     int64_t best = 1;
     double cost = 0.0;
@@ -1052,7 +1055,7 @@ int mla_latent(ns_gpu* g, const char* who, int qt, int ot, int R, bool q8, const
     const int MW = mla_waves(per_t ? H : rows, pos0 + T), MROWS = MW * 16;
     const int64_t nz = per_t ? T * ((H + MROWS - 1) / MROWS) : (rows + MROWS - 1) / MROWS;
     const int64_t listed = 4 * K + 3, cells = per_t ? std::max(listed, std::min<int64_t>(pos0 + T, SEL_DENSE_MAX)) : pos0 + T;
-    int64_t kbs = mla_kbs(cells, nz);
+    int64_t kbs = mla_kbs(cells, nz, per_t);
     int64_t ns = (cells + kbs - 1) / kbs;
     // a caller's scratch may be smaller than the rule asks (the library's own, for the reference-named entry points):
     // fewer, longer splits then
