@@ -201,6 +201,14 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
         cpk = cp ^ kr0;
         cpv = cp ^ (2 * kr0);
     }
+    // (a pass of several row chunks reads a split's keys once a chunk, the chunks side by side on one XCD: its loads keep
+    // the ordinary policy, so that the chunks after the first find the lines in that XCD's L2 - 16 rows x 32 / 8 heads
+    // behind 131072 keys 148.5 -> 118.9 us; a pass of one chunk reads every key once and streams)
+    const bool stream = p.nz == 1;
+    auto to_lds = [&](const uint8_t* src, uint8_t* dst) __attribute__((always_inline)) {
+        if (stream) __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) src, (__attribute__((address_space(3))) void*) dst, 16, 0, NT_AUX);
+        else __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) src, (__attribute__((address_space(3))) void*) dst, 16, 0, 0);
+    };
     auto dma_tile = [&](int64_t ti, int which) __attribute__((always_inline)) {
         const int j0 = (int) (ti * TILE - jb);                 // the tile's first key relative to the split's
         if constexpr (FAST) {
@@ -209,12 +217,10 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
 #pragma unroll
                 for (int i = 0; i < R::NLV; ++i) {
                     if constexpr (FAST_KEPT) {
-                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (base + (which ? voff[i] : koff[i])),
-                                                         (__attribute__((address_space(3))) void*) (stage + which * VTILE + i * 1024), 16, 0, NT_AUX);
+                        to_lds(base + (which ? voff[i] : koff[i]), stage + which * VTILE + i * 1024);
                     } else {
                         const uint32_t off = lane_row + ((which ? cpv ^ (uint32_t) ((2 * R::KPI * i) & 14) : cpk ^ (uint32_t) ((R::KPI * i) & 15)) << 4);
-                        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (base + (int64_t) (R::KPI * i) * p.row_stride + off),
-                                                         (__attribute__((address_space(3))) void*) (stage + which * VTILE + i * 1024), 16, 0, NT_AUX);
+                        to_lds(base + (int64_t) (R::KPI * i) * p.row_stride + off, stage + which * VTILE + i * 1024);
                     }
                 }
                 return;
@@ -226,8 +232,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
             const int kk = kr0 + R::KPI * i;
             const uint8_t* row = (which ? vbase : kbase) + tile_off(ti, j0, kk);
             const int c = which ? cp ^ (2 * (kk & 7)) : cp ^ (kk & 15);
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*) (row + c * 16),
-                                             (__attribute__((address_space(3))) void*) (stage + which * VTILE + i * 1024), 16, 0, NT_AUX);
+            to_lds(row + c * 16, stage + which * VTILE + i * 1024);
         }
     };
     // quantized rows: the tile's keys (MFMA A layout) and values raw into registers
@@ -307,6 +312,7 @@ __global__ __launch_bounds__(WAVES * 64, D == 128 ? 2 : 1) void attn_decode_kern
                 const uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t) (uintptr_t) (stage + VTILE + which * QRAW + i * 1024));
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
+                // (quantized rows stream whatever the chunks: their passes of several chunks gain nothing from the other policy)
                 asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m), "v"(off), "s"(base) : "memory", "m0");
 #pragma clang diagnostic pop
             }
