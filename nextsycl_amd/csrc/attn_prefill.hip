@@ -86,7 +86,9 @@ typedef uint32_t u4a8 __attribute__((ext_vector_type(4), aligned(8)));
 // BF: bfloat16 operands (a bfloat16 cache too long to be widened to half first), else half. QS (bfloat16 operands only):
 // query rows of another type enter the first product as two bfloat16 numbers - the rounded row and the rounded rest, 16
 // significant bits between them - a second matrix instruction a key block.
-template <int D, bool BF, int KT, int PW, bool QS = false>
+// NTS (16-bit rows of 128 only): the tiles' transfers carry the streaming cache policy - a pass whose keys are each read
+// by one work-group, once.
+template <int D, bool BF, int KT, int PW, bool QS = false, bool NTS = false>
 __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_prefill_kernel(const PrefillParams p) {
     static_assert(D == 128 || D == 256, "head size 128 or 256");
     static_assert(KT == 0 || !BF, "quantized rows are widened to half");
@@ -351,7 +353,8 @@ __global__ __launch_bounds__(PW * 64, PW == 4 && D == 128 ? 2 : 1) void attn_pre
         const uint32_t m = __builtin_amdgcn_readfirstlane((uint32_t) (uintptr_t) dst);
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"                   // (m0 is reserved: nothing of the compiler's lives in it across this)
-        asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m), "v"(off), "s"(base_) : "memory", "m0");
+        if constexpr (NTS) asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(m), "v"(off), "s"(base_) : "memory", "m0");
+        else asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m), "v"(off), "s"(base_) : "memory", "m0");
 #pragma clang diagnostic pop
     };
     auto dma = [&](lds_u8* dst, const uint8_t* cache, int krel, auto which_c) __attribute__((always_inline)) {
@@ -904,8 +907,22 @@ bool own_form_pays(int kt, int qt, int64_t D, int64_t T, int64_t G, int64_t keys
 }
 
 template <int D, int PW>
-int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid) {
+int launch_prefill(ns_gpu* g, int kt, const PrefillParams& p, dim3 grid, bool stream) {
     constexpr int TH = PW * 64;
+    if constexpr (D == 128) {
+        // (the streaming forms: half rows with either work-group size, bfloat16 rows - short passes keep them - with 4 waves)
+        if (stream && kt == 0) {
+            attn_prefill_kernel<D, false, 0, PW, false, true><<<grid, TH, 0, g->q>>>(p);
+            return 0;
+        }
+        if constexpr (PW == 4) {
+            if (stream && kt == 3) {
+                if (p.qt != 2) attn_prefill_kernel<D, true, 0, PW, true, true><<<grid, TH, 0, g->q>>>(p);
+                else attn_prefill_kernel<D, true, 0, PW, false, true><<<grid, TH, 0, g->q>>>(p);
+                return 0;
+            }
+        }
+    }
     if (kt == 0) {
         attn_prefill_kernel<D, false, 0, PW><<<grid, TH, 0, g->q>>>(p);
     } else if (kt == 3) {
@@ -1129,8 +1146,12 @@ int ns_attn_prompt_any(ns_gpu* g, const char* who, int qt, int kt, int pm, const
     if ((units + 7) / 8 * 8 * p.gw >= (int64_t) 1 << 31) return ns_fail(w + ": too many work-groups");
     dim3 grid((unsigned) ((units + 7) / 8 * 8 * p.gw));
     if (ns_profile_mark(g, 0)) return -1;
-    if ((D == 256 ? (PWs == 8 ? launch_prefill<256, 8>(g, kt_run, p, grid) : launch_prefill<256, 4>(g, kt_run, p, grid))
-                  : PWs == 8 ? launch_prefill<128, 8>(g, kt_run, p, grid) : launch_prefill<128, 4>(g, kt_run, p, grid)) != 0)
+    // (a pass whose keys are each read by one work-group - all the group's heads in it, one row block - behind a long
+    // context streams them: 17 rows x 32 / 8 heads behind 131072 keys 110 -> 97 us; where several work-groups read a key
+    // the streaming policy loses what they share in L2: x 64 / 4 heads 142 -> 156)
+    const bool stream = p.gw == 1 && T <= RB && p0 + T >= 32768;
+    if ((D == 256 ? (PWs == 8 ? launch_prefill<256, 8>(g, kt_run, p, grid, false) : launch_prefill<256, 4>(g, kt_run, p, grid, false))
+                  : PWs == 8 ? launch_prefill<128, 8>(g, kt_run, p, grid, stream) : launch_prefill<128, 4>(g, kt_run, p, grid, stream)) != 0)
         return -1;
     NS_LAUNCHED("attn_prefill");
     if (ns_profile_mark(g, 1)) return -1;

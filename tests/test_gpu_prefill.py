@@ -113,6 +113,10 @@ SPLIT = [
     (40, 4, 2, 256, 4000, 0, 0, F32),
     (130, 6, 2, 256, 2500, 0, 1, F16),          # quantized rows at head size 256
     (17, 2, 1, 128, 40000, 0, 0, F32),
+    # a key head's rows all in one work-group behind 32768 keys and more: the tiles' transfers stream
+    (20, 4, 1, 128, 33000, 0, 3, BF16),         # ... bfloat16 rows kept as they are
+    (24, 4, 1, 128, 33000, 0, 3, F32),          # ... float32 query rows over them, in two parts
+    (17, 5, 1, 128, 33000, 0, 0, F16),          # ... five heads to an 8-wave work-group
 ]
 
 
