@@ -845,9 +845,17 @@ int64_t target_wgs(int64_t D, int64_t G, int kt, int64_t Hkv) {
     return v > 0 ? v : D == 256 || (G >= 8 && (kt == 0 || kt == 3)) || (kt == 1 && Hkv <= 2) ? 256 : 512;
 }
 // keys a split for a row that sees `keys` keys: a multiple of 128 (4 waves x 32-key tiles)
+// (quantized rows whose rule aims for 512 work-groups: short contexts take 256 of splits up to 384 or 512 keys first - a split's
+// fixed cost and its partial weigh more than the second work-group a CU gains; 64 / 4 heads over 16383 q8_0 keys: one row
+// 13.8 -> 12.5 us, four rows 28.2 -> 20.7. 16-bit rows gained in one layout of the caches and lost in another: unchanged)
 int64_t dec_kbs(int64_t keys, int64_t Hkv, int64_t D, int64_t G, int kt) {
     const int64_t t = target_wgs(D, G, kt, Hkv), want = (keys * Hkv + t - 1) / t;
-    return std::max<int64_t>(128, (want + 127) / 128 * 128);
+    const int64_t kbs = std::max<int64_t>(128, (want + 127) / 128 * 128);
+    if (t != 512 || ns_tune_get(NS_TUNE_DEC_WGS) > 0 || kt == 0 || kt == 3) return kbs;
+    const int64_t want2 = (keys * Hkv + 255) / 256, kbs2 = std::max<int64_t>(128, (want2 + 127) / 128 * 128);
+    // (up to 512 keys a split where a key head serves 8 query heads and more - their partials weigh most - else 384: 32 / 8
+    // heads over 12500 q8_0 keys in 256 splits of 512 keys 14.7 us, in 392 of 256 keys 13.9)
+    return kbs2 <= (G >= 8 ? 512 : 384) ? kbs2 : kbs;
 }
 inline int64_t row_first(int64_t pos, int64_t win) { return win > 0 ? std::max<int64_t>(0, pos - win + 1) : 0; }
 

@@ -47,8 +47,10 @@ def test_pure_functions_without_a_gpu(handle):
     assert f(1, 32, 8, 128, 4095, 0) == 32 * 32 * 130
     assert f(0, 32, 8, 128, 4095, 0) == 0
     # heads of 256 aim for half as many work-groups: 32768 keys x 2 heads in 256 splits of 256 keys -> 128 a head; heads of
-    # 128 are sized for the cache form that splits finest (q4_0 rows: 512 work-groups -> 256 a head)
-    assert f(1, 16, 2, 256, 32767, 0) == 16 * 128 * 258 and f(1, 16, 2, 128, 32767, 0) == 16 * 256 * 130
+    # 128 are sized for the cache form that splits finest (q4_0 rows: 512 work-groups, but 256 of them first while a split
+    # stays within 512 keys -> 128 a head here, 256 a head of 512 keys at four times the keys)
+    assert f(1, 16, 2, 256, 32767, 0) == 16 * 128 * 258 and f(1, 16, 2, 128, 32767, 0) == 16 * 128 * 130
+    assert f(1, 16, 2, 128, 131071, 0) == 16 * 256 * 130
     # a verify pass needs at least its rows' own
     assert f(4, 32, 4, 128, 65536, 0) >= 4 * f(1, 32, 4, 128, 65536, 0)
     # a window bounds the splits whatever the position
