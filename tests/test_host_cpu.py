@@ -65,6 +65,11 @@ def test_pure_functions_without_a_gpu(handle):
     m.restype, m.argtypes = C.c_int64, [C.c_int64] * 3
     assert m(1, 128, 32767) == 128 * 128 * 260 and m(0, 128, 5) == 0     # two 64-row groups x 128 splits of 256 cells; a partial: 512 halfs + m, l (+ 2)
     assert m(2, 128, 32766) == 256 * 128 * 260                           # two 128-row groups x 128 splits
+    # whole rounds of an XCD's 32 places: 3 row groups take 79 splits (10 an XCD = 30 work-groups; 86 would be 11 = 33, a
+    # second round for three of them), 5 groups 47; 17 rows end at 16 groups x 16 splits, the 17th row a pass of its own; 33
+    # groups, fewer than 8 splits, are dealt over the whole chip: 7 splits = 231 work-groups
+    assert m(3, 128, 131069) == 3 * 128 * 79 * 260 and m(5, 128, 32763) == 5 * 128 * 47 * 260
+    assert m(17, 128, 32751) == m(16, 128, 32751) == 16 * 128 * 16 * 260 and m(33, 128, 32735) == 33 * 128 * 7 * 260
     handle.ns_version.restype = C.c_char_p
     assert b"gfx950" in handle.ns_version()
     handle.ns_last_error.restype = C.c_char_p
